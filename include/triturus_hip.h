@@ -1,0 +1,127 @@
+/*
+ * triturus_hip.h -- C ABI of the gfx950 (MI355X) log-space contraction library.
+ *
+ * Every entry point takes raw DEVICE pointers, sizes, element strides and a
+ * hipStream_t (as void*).  The library allocates nothing, keeps no state,
+ * never synchronises and never throws: each call enqueues its kernels on the
+ * given stream and returns an int status
+ *      0            success
+ *      < 0          argument / layout error (TRT_E_*), nothing was enqueued
+ *      > 0          a hipError_t reported by the launch
+ * Outputs and workspaces are owned by the caller.
+ *
+ * The reference (loreloc/triturus) has no FFI: its boundary for this path is
+ * the Triton kernel launch made by each Python wrapper.  Each function below
+ * names the reference launch site it replaces (path:line in the reference).
+ *
+ * Letters: R = batch; lm2exp contracts J; lt2exp contracts (I, J); K is the
+ * trailing, contiguous "column" axis of every log-space operand.
+ */
+#ifndef TRITURUS_HIP_H
+#define TRITURUS_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TRT_ABI_VERSION 1
+
+#define TRT_OK 0
+#define TRT_E_INVALID (-1)   /* null pointer, non-positive size, bad enum   */
+#define TRT_E_LAYOUT (-2)    /* stride pattern the kernels do not handle    */
+#define TRT_E_WORKSPACE (-3) /* workspace missing or smaller than required  */
+#define TRT_E_RANGE (-4)     /* a size exceeds what the index math supports */
+
+/* Element types of the max reductions (triturus/max.py:37,98,178 accept any
+ * floating dtype). */
+#define TRT_F32 0
+#define TRT_F64 1
+#define TRT_F16 2
+#define TRT_BF16 3
+
+/* lt2exp launch modes (triturus/lt2exp.py:534-541). */
+#define TRT_MODE_AUTO 0
+#define TRT_MODE_SPLIT 1
+#define TRT_MODE_UNSPLIT 2
+
+/* ABI version of the loaded library (== TRT_ABI_VERSION it was built with). */
+int trt_version(void);
+
+/* Static, human-readable text for a status returned by any call below. */
+const char *trt_error_string(int status);
+
+/*
+ * c[r,i,k] = log sum_j a[r,i,j] * exp(b[r,j,k])            (fp32)
+ * a: R x I x J linear-space, b: R x J x K log-space, c: R x I x K.
+ * sa/sb/sc: element strides of the three axes.  The trailing stride of each
+ * tensor must be 1 (TRT_E_LAYOUT otherwise); the two leading strides are
+ * free.  Replaces the `_ker_lm2exp[grid](...)` launch, triturus/lm2exp.py:186-205;
+ * arithmetic contract baselines/lm2exp.py:11-14 (column max clamped to
+ * +-1e38, an all -inf column gives -inf, never NaN).
+ * variant: 0 = choose by shape; other values pick a tile shape for
+ * experiments (see trt_lm2exp_variant_count).
+ */
+int trt_lm2exp_f32(const float *a, const float *b, float *c,
+                   int64_t R, int64_t I, int64_t J, int64_t K,
+                   const int64_t sa[3], const int64_t sb[3], const int64_t sc[3],
+                   int variant, void *stream);
+int trt_lm2exp_variant_count(void);
+
+/*
+ * c[r,s,k] = log sum_{i,j} w[r,s,i,j] * exp(a[r,i,k]) * exp(b[r,j,k])   (fp32)
+ * w: R x S x (I*J) linear-space (the reference flattens the two trailing axes
+ * with w.view(batch, m, -1), triturus/lt2exp.py:549, so sw has 3 entries),
+ * a: R x I x K, b: R x J x K log-space, c: R x S x K.  Trailing strides must
+ * be 1.  Replaces the `_ker_lt2exp_unsplit[grid](...)` launch,
+ * triturus/lt2exp.py:601-629, and the `_ker_lt2exp_split[grid](...)` launch,
+ * triturus/lt2exp.py:564-597; arithmetic contract baselines/lt2exp.py:15-25.
+ * mode: TRT_MODE_*.  AUTO applies the reference heuristic
+ * (R*S*K < 1048576 and I*J > 512, triturus/lt2exp.py:535).  SPLIT partitions
+ * the contracted (i,j) range over several workgroups and merges the partial
+ * sums deterministically; it needs a workspace of
+ * trt_lt2exp_workspace_bytes(...) bytes (UNSPLIT needs none: pass NULL, 0).
+ */
+int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c,
+                   int64_t R, int64_t S, int64_t I, int64_t J, int64_t K,
+                   const int64_t sw[3], const int64_t sa[3], const int64_t sb[3],
+                   const int64_t sc[3], int mode, int variant,
+                   void *workspace, size_t workspace_bytes, void *stream);
+size_t trt_lt2exp_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t J,
+                                  int64_t K, int mode);
+int trt_lt2exp_variant_count(void);
+
+/*
+ * Max of a contiguous m x n row-major matrix along axis 0 (y has n entries)
+ * or axis 1 (y has m entries).  NaN propagates as in torch.amax.  Replaces the
+ * multi-launch `_ker_matmax` tree, triturus/max.py:190-225.  workspace:
+ * trt_matmax_workspace_bytes(m, n, axis, dtype) bytes (may be 0).
+ */
+int trt_matmax(const void *x, void *y, int64_t m, int64_t n, int axis, int dtype,
+               void *workspace, size_t workspace_bytes, void *stream);
+size_t trt_matmax_workspace_bytes(int64_t m, int64_t n, int axis, int dtype);
+
+/*
+ * Max and first-occurrence argmax (int64) of a contiguous vector of n
+ * elements; a NaN wins and reports the first NaN, as torch.max(x, 0) does.
+ * out_idx may be NULL (value only: the reference's vamax).  Replaces the
+ * `_ker_vmax` / `_ker_vamax` launch loops, triturus/max.py:108-121 and
+ * :46-58.  workspace: trt_vmax_workspace_bytes(n, dtype) bytes.
+ */
+int trt_vmax(const void *x, int64_t n, int dtype, void *out_val, int64_t *out_idx,
+             void *workspace, size_t workspace_bytes, void *stream);
+size_t trt_vmax_workspace_bytes(int64_t n, int dtype);
+
+/*
+ * Plain device-to-device copy kernel of nbytes (multiple of 16, 16-byte
+ * aligned pointers).  No counterpart in the reference: it is the known-size
+ * kernel that hardware byte counters are calibrated against.
+ */
+int trt_copy_bytes(const void *src, void *dst, size_t nbytes, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TRITURUS_HIP_H */

@@ -1,0 +1,6 @@
+"""Drop-in import path of the reference: ``from triturus.utils import ...``."""
+from triturus_amd.utils import (  # noqa: F401
+    ensure_reproducibility,
+    is_triturus_tf32_enabled,
+    set_tf32_enabled,
+)

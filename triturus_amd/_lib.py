@@ -1,0 +1,113 @@
+"""ctypes binding of the C-ABI library (include/triturus_hip.h).
+
+The library is the only compute path.  If it has not been built, or a call
+reports a non-zero status, a RuntimeError is raised: there is no fallback.
+"""
+
+from __future__ import annotations
+
+import ctypes
+import threading
+from ctypes import POINTER, c_char_p, c_int, c_int64, c_size_t, c_void_p
+from pathlib import Path
+
+import torch
+
+LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtriturus_hip.so"
+ABI_VERSION = 1
+
+TRT_F32, TRT_F64, TRT_F16, TRT_BF16 = 0, 1, 2, 3
+MODE_AUTO, MODE_SPLIT, MODE_UNSPLIT = 0, 1, 2
+
+DTYPE_CODES = {
+    torch.float32: TRT_F32,
+    torch.float64: TRT_F64,
+    torch.float16: TRT_F16,
+    torch.bfloat16: TRT_BF16,
+}
+
+_I64x3 = c_int64 * 3
+
+# name -> (restype, argtypes); mirrors include/triturus_hip.h one to one
+SIGNATURES = {
+    "trt_version": (c_int, []),
+    "trt_error_string": (c_char_p, [c_int]),
+    "trt_lm2exp_f32": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+         POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int, c_void_p],
+    ),
+    "trt_lm2exp_variant_count": (c_int, []),
+    "trt_lt2exp_f32": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+         POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
+         c_int, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "trt_lt2exp_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int]),
+    "trt_lt2exp_variant_count": (c_int, []),
+    "trt_matmax": (
+        c_int,
+        [c_void_p, c_void_p, c_int64, c_int64, c_int, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "trt_matmax_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int, c_int]),
+    "trt_vmax": (
+        c_int,
+        [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p],
+    ),
+    "trt_vmax_workspace_bytes": (c_size_t, [c_int64, c_int]),
+    "trt_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+}
+
+_lock = threading.Lock()
+_lib: ctypes.CDLL | None = None
+
+
+def load() -> ctypes.CDLL:
+    """Load the HIP library once; raise if it is missing or of another ABI."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    with _lock:
+        if _lib is not None:
+            return _lib
+        if not LIB_PATH.exists():
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build it with `python -m triturus_amd.build` "
+                "(hipcc, gfx950). There is no CPU or eager fallback."
+            )
+        lib = ctypes.CDLL(str(LIB_PATH))
+        for name, (restype, argtypes) in SIGNATURES.items():
+            fn = getattr(lib, name)  # AttributeError if a declared symbol is absent
+            fn.restype = restype
+            fn.argtypes = argtypes
+        if lib.trt_version() != ABI_VERSION:
+            raise RuntimeError(
+                f"{LIB_PATH} has ABI version {lib.trt_version()}, expected {ABI_VERSION}: rebuild it"
+            )
+        _lib = lib
+        return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        text = load().trt_error_string(status)
+        raise RuntimeError(f"{what} failed with status {status}: {text.decode() if text else '?'}")
+
+
+def strides3(t: torch.Tensor):
+    return _I64x3(*t.stride())
+
+
+def current_stream(device: torch.device) -> c_void_p:
+    return c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def require_gpu(*tensors: torch.Tensor) -> None:
+    """The kernels run on HIP device memory only."""
+    for t in tensors:
+        if t.device.type != "cuda":
+            raise RuntimeError(
+                f"triturus_amd runs on the GPU only: got a tensor on '{t.device}'. "
+                "Move the inputs to the HIP device (there is no CPU fallback)."
+            )

@@ -1,0 +1,433 @@
+// lt2exp for gfx950:  c[r,s,k] = log sum_{i,j} w[r,s,i,j] exp(a[r,i,k]) exp(b[r,j,k])
+//
+// One workgroup owns a (32*RT rows of S) x (32*CT*NWAVES columns of K) tile of
+// c[r]; each wavefront owns 32*CT of those columns for all rows.  The
+// contraction runs on v_mfma_f32_32x32x2_f32 with
+//   A operand = w tile, staged global -> registers -> LDS (double buffered),
+//               read back 16 bytes per lane (4 consecutive j);
+//   B operand = the shifted Khatri-Rao product exp(a[i,n]-ma[n]) * exp(b[j,n]-mb[n]),
+//               formed in registers with ONE multiply per MFMA operand: a lane
+//               owns one column n, keeps exp(b[j,n]-mb[n]) for the j of the
+//               current j-chunk in VGPRs and multiplies by the scalar
+//               exp(a[i,n]-ma[n]) of the current i.
+// The I*J*K intermediate of the torch recipe (baselines/lt2exp.py:21-22)
+// never exists; every exp is evaluated once per (workgroup, column).
+//
+// MFMA k-slot mapping (the contraction order is free): within a chunk of
+// JC = 8*NQ values of j, MFMA number (q,u) in lane-half h = lane/32 consumes
+// j = 8q + 4h + u, so one 16-byte LDS read feeds 4 MFMAs.
+//
+// Replaces _ker_lt2exp_unsplit / _ker_lt2exp_split, triturus/lt2exp.py:227-357,365-506.
+
+#include "common.hpp"
+
+namespace trt {
+
+struct Lt2Args {
+    const float *w, *a, *b;
+    float *c;         // output (unsplit) -- or partial sums (split)
+    float *shift;     // split only: [2][R][K] clamped column maxima
+    int R, S, I, J, K;
+    int64_t sw0, sw1, sa0, sa1, sb0, sb1, sc0, sc1;
+    int s_tiles, n_tiles, splits;
+    int iters_per_split;  // (j-chunk, i) iterations per split
+    int64_t total_wgs, padded_wgs;
+};
+
+template <int RT, int CT, int NQ, int NWAVES, bool VEC, bool SPLIT>
+__global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args p) {
+    constexpr int NT = NWAVES * kWave;
+    constexpr int TS = 32 * RT;           // rows of S per workgroup
+    constexpr int JC = 8 * NQ;            // j per chunk
+    constexpr int LDW = JC + 4;           // padded LDS row (floats): conflict-free 16-byte reads
+    constexpr int F4_PER_ROW = JC / 4;
+    constexpr int SLOTS = TS * F4_PER_ROW / NT;  // float4 tile slots per thread
+    static_assert(TS * F4_PER_ROW % NT == 0, "tile must divide over the threads");
+    constexpr int TN = 32 * CT * NWAVES;
+
+    __shared__ __attribute__((aligned(16))) float wt[2][TS * LDW];
+
+    const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
+    if (L >= p.total_wgs) return;
+    const int nt = (int)(L % p.n_tiles);
+    int64_t rest = L / p.n_tiles;
+    const int split = (int)(rest % p.splits);
+    rest /= p.splits;
+    const int st = (int)(rest % p.s_tiles);
+    const int r = (int)(rest / p.s_tiles);
+
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int lane = tid % kWave;
+    const int h = lane / 32;
+    const int m = lane % 32;
+    const int s0 = st * TS;
+    const int n0 = nt * TN + wave * 32 * CT;
+
+    int ncol[CT], ncl[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        ncol[ct] = n0 + 32 * ct + m;
+        ncl[ct] = ncol[ct] < p.K ? ncol[ct] : p.K - 1;
+    }
+    const float *ar = p.a + (int64_t)r * p.sa0;
+    const float *br = p.b + (int64_t)r * p.sb0;
+    const float *wr = p.w + (int64_t)r * p.sw0;
+
+    // ---- column maxima over the contracted axes (both lane halves share a
+    // column: each takes every other row, then they exchange).
+    float ma[CT], mb[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        float x = -__builtin_inff();
+#pragma unroll 8
+        for (int i = h; i < p.I; i += 2) x = max_nan(x, ar[(int64_t)i * p.sa1 + ncl[ct]]);
+        x = max_nan(x, __shfl_xor(x, 32, kWave));
+        ma[ct] = clamp_shift(x);
+        float y = -__builtin_inff();
+#pragma unroll 8
+        for (int j = h; j < p.J; j += 2) y = max_nan(y, br[(int64_t)j * p.sb1 + ncl[ct]]);
+        y = max_nan(y, __shfl_xor(y, 32, kWave));
+        mb[ct] = clamp_shift(y);
+    }
+
+    const int n_jc = (p.J + JC - 1) / JC;
+    const int total_iters = n_jc * p.I;
+    int it = split * p.iters_per_split;
+    int it_end = it + p.iters_per_split;
+    if (it_end > total_iters) it_end = total_iters;
+
+    floatx16 acc[RT][CT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[rt][ct][v] = 0.f;
+
+    // ---- tile staging helpers
+    floatx4 stage[SLOTS];
+    auto load_tile = [&](int i, int jc) {
+#pragma unroll
+        for (int sidx = 0; sidx < SLOTS; ++sidx) {
+            const int f = tid + sidx * NT;
+            const int row = f / F4_PER_ROW;
+            const int c4 = f % F4_PER_ROW;
+            const int j = jc * JC + 4 * c4;
+            const bool row_ok = (s0 + row) < p.S;
+            const float *src = wr + (int64_t)(s0 + row) * p.sw1 + (int64_t)i * p.J + j;
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (VEC) {
+                if (row_ok && j < p.J) v = *reinterpret_cast<const floatx4 *>(src);
+            } else {
+                if (row_ok) {
+                    if (j + 0 < p.J) v[0] = src[0];
+                    if (j + 1 < p.J) v[1] = src[1];
+                    if (j + 2 < p.J) v[2] = src[2];
+                    if (j + 3 < p.J) v[3] = src[3];
+                }
+            }
+            stage[sidx] = v;
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int sidx = 0; sidx < SLOTS; ++sidx) {
+            const int f = tid + sidx * NT;
+            const int row = f / F4_PER_ROW;
+            const int c4 = f % F4_PER_ROW;
+            *reinterpret_cast<floatx4 *>(&wt[buf][row * LDW + 4 * c4]) = stage[sidx];
+        }
+    };
+
+    float eb[CT][4 * NQ];
+    auto load_eb = [&](int jc) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const int j = jc * JC + 8 * q + 4 * h + u;
+                    float raw = -__builtin_inff();
+                    if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl[ct]];
+                    eb[ct][4 * q + u] = expf(raw - mb[ct]);
+                }
+    };
+
+    float ea[CT], ea_raw[CT];
+
+    if (it < it_end) {
+        int jc = it / p.I;
+        int i = it - jc * p.I;
+        load_tile(i, jc);
+        load_eb(jc);
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) ea[ct] = expf(ar[(int64_t)i * p.sa1 + ncl[ct]] - ma[ct]);
+        store_tile(0);
+        __syncthreads();
+
+        int cur = 0;
+        for (; it < it_end; ++it) {
+            int ni = i + 1, njc = jc;
+            if (ni == p.I) {
+                ni = 0;
+                njc = jc + 1;
+            }
+            const bool has_next = (it + 1) < it_end;
+            if (has_next) {
+                load_tile(ni, njc);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) ea_raw[ct] = ar[(int64_t)ni * p.sa1 + ncl[ct]];
+            }
+            // ---- MFMA block over this (i, j-chunk)
+            const float *tile = wt[cur];
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                floatx4 af[RT];
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    af[rt] = *reinterpret_cast<const floatx4 *>(&tile[(32 * rt + m) * LDW + 8 * q + 4 * h]);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+#pragma unroll
+                    for (int ct = 0; ct < CT; ++ct) {
+                        const float bop = ea[ct] * eb[ct][4 * q + u];
+#pragma unroll
+                        for (int rt = 0; rt < RT; ++rt)
+                            acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[rt][u], bop, acc[rt][ct], 0, 0, 0);
+                    }
+                }
+            }
+            if (has_next) {
+                store_tile(cur ^ 1);
+                if (njc != jc) load_eb(njc);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) ea[ct] = expf(ea_raw[ct] - ma[ct]);
+            }
+            __syncthreads();
+            cur ^= 1;
+            i = ni;
+            jc = njc;
+        }
+    }
+
+    // ---- epilogue.  D layout of 32x32x2: register v of lane (h, m) holds
+    // row 8*(v/4) + 4*h + v%4, column m.
+    if (SPLIT) {
+        // partial sums (all splits share ma, mb: they depend on the column only)
+        float *part = p.c + ((int64_t)split * p.R + r) * (int64_t)p.S * p.K;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            if (ncol[ct] >= p.K) continue;
+            if (split == 0 && st == 0 && h == 0) {
+                p.shift[(int64_t)r * p.K + ncol[ct]] = ma[ct];
+                p.shift[((int64_t)p.R + r) * p.K + ncol[ct]] = mb[ct];
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = s0 + 32 * rt + 8 * (v / 4) + 4 * h + (v % 4);
+                    if (row < p.S) part[(int64_t)row * p.K + ncol[ct]] = acc[rt][ct][v];
+                }
+        }
+    } else {
+        float *cr = p.c + (int64_t)r * p.sc0;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            if (ncol[ct] >= p.K) continue;
+            const float mm = ma[ct] + mb[ct];
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int row = s0 + 32 * rt + 8 * (v / 4) + 4 * h + (v % 4);
+                    if (row < p.S) cr[(int64_t)row * p.sc1 + ncol[ct]] = mm + logf(acc[rt][ct][v]);
+                }
+        }
+    }
+}
+
+// c = (ma + mb) + log(sum over splits of the partial sums), in split order.
+__global__ __launch_bounds__(256) void lt2exp_merge_kernel(const float *__restrict__ part,
+                                                           const float *__restrict__ shift, float *__restrict__ c,
+                                                           int R, int S, int K, int splits, int64_t sc0,
+                                                           int64_t sc1) {
+    const int64_t total = (int64_t)R * S * K;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+        const int k = (int)(e % K);
+        const int64_t rs = e / K;
+        const int s = (int)(rs % S);
+        const int r = (int)(rs / S);
+        float sum = 0.f;
+        for (int sp = 0; sp < splits; ++sp) sum += part[(int64_t)sp * total + e];
+        const float mm = shift[(int64_t)r * K + k] + shift[((int64_t)R + r) * K + k];
+        c[(int64_t)r * sc0 + (int64_t)s * sc1 + k] = mm + logf(sum);
+    }
+}
+
+// ------------------------------------------------------------------ host
+struct Lt2Variant {
+    int rt, ct, nq;
+};
+// variant ids (1-based in the C ABI; 0 = choose by shape)
+static const Lt2Variant kVariants[] = {
+    {2, 2, 8},  // 64 x 256 tile, j-chunks of 64
+    {2, 2, 4},  // 64 x 256 tile, j-chunks of 32
+    {1, 2, 8},  // 32 x 256 tile
+    {1, 2, 4},
+    {2, 1, 8},  // 64 x 128 tile
+    {2, 1, 4},
+    {1, 1, 8},  // 32 x 128 tile
+    {1, 1, 4},
+};
+constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
+constexpr int kLt2Waves = 4;
+
+static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
+    (void)I;
+    const int rt = S > 32 ? 2 : 1;
+    const int nq = J > 32 ? 8 : 4;
+    // narrow column tiles when the wide one cannot fill the 256 CUs twice over
+    const int64_t wide_wgs = R * ceil_div(S, 32 * rt) * ceil_div(K, 256);
+    const int ct = (wide_wgs >= 512) ? 2 : 1;
+    for (int v = 0; v < kNumVariants; ++v)
+        if (kVariants[v].rt == rt && kVariants[v].ct == ct && kVariants[v].nq == nq) return v;
+    return 0;
+}
+
+template <int RT, int CT, int NQ, bool VEC, bool SPLIT>
+static void launch_one(const Lt2Args &args, hipStream_t stream) {
+    hipLaunchKernelGGL((lt2exp_kernel<RT, CT, NQ, kLt2Waves, VEC, SPLIT>), dim3((unsigned)args.padded_wgs),
+                       dim3(kLt2Waves * kWave), 0, stream, args);
+}
+
+template <int RT, int CT, int NQ>
+static void launch_vs(const Lt2Args &args, bool vec, bool split, hipStream_t stream) {
+    if (vec) {
+        if (split) launch_one<RT, CT, NQ, true, true>(args, stream);
+        else launch_one<RT, CT, NQ, true, false>(args, stream);
+    } else {
+        if (split) launch_one<RT, CT, NQ, false, true>(args, stream);
+        else launch_one<RT, CT, NQ, false, false>(args, stream);
+    }
+}
+
+static void launch_variant(int v, const Lt2Args &args, bool vec, bool split, hipStream_t stream) {
+    switch (v) {
+        case 0: launch_vs<2, 2, 8>(args, vec, split, stream); break;
+        case 1: launch_vs<2, 2, 4>(args, vec, split, stream); break;
+        case 2: launch_vs<1, 2, 8>(args, vec, split, stream); break;
+        case 3: launch_vs<1, 2, 4>(args, vec, split, stream); break;
+        case 4: launch_vs<2, 1, 8>(args, vec, split, stream); break;
+        case 5: launch_vs<2, 1, 4>(args, vec, split, stream); break;
+        case 6: launch_vs<1, 1, 8>(args, vec, split, stream); break;
+        default: launch_vs<1, 1, 4>(args, vec, split, stream); break;
+    }
+}
+
+struct SplitPlan {
+    bool split;
+    int splits;
+    int iters_per_split;
+};
+
+static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode, int variant) {
+    const Lt2Variant &v = kVariants[variant];
+    bool split;
+    if (mode == TRT_MODE_AUTO)
+        split = (R * S * K < 1048576) && (I * J > 512);  // triturus/lt2exp.py:535
+    else
+        split = (mode == TRT_MODE_SPLIT);
+    const int64_t iters = ceil_div(J, 8 * v.nq) * I;
+    if (!split) return {false, 1, (int)iters};
+    const int64_t base = R * ceil_div(S, 32 * v.rt) * ceil_div(K, 32 * v.ct * kLt2Waves);
+    int64_t splits = ceil_div(1024, base);
+    if (splits > 32) splits = 32;
+    if (splits > iters) splits = iters;
+    if (splits < 1) splits = 1;
+    const int64_t per = ceil_div(iters, splits);
+    splits = ceil_div(iters, per);
+    return {true, (int)splits, (int)per};
+}
+
+}  // namespace trt
+
+using namespace trt;
+
+extern "C" int trt_lt2exp_variant_count(void) { return kNumVariants; }
+
+static int resolve_variant(int variant, int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
+    if (variant >= 1 && variant <= kNumVariants) return variant - 1;
+    return choose_variant(R, S, I, J, K);
+}
+
+extern "C" size_t trt_lt2exp_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode) {
+    if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return 0;
+    // the split count depends on the tile shape: size for the largest possible
+    size_t need = 0;
+    for (int v = 0; v < kNumVariants; ++v) {
+        SplitPlan sp = plan_split(R, S, I, J, K, mode, v);
+        if (!sp.split) continue;
+        size_t b = ((size_t)sp.splits * R * S * K + (size_t)2 * R * K) * sizeof(float);
+        if (b > need) need = b;
+    }
+    return need;
+}
+
+extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c, int64_t R, int64_t S,
+                              int64_t I, int64_t J, int64_t K, const int64_t sw[3], const int64_t sa[3],
+                              const int64_t sb[3], const int64_t sc[3], int mode, int variant, void *workspace,
+                              size_t workspace_bytes, void *stream) {
+    if (!w || !a || !b || !c || !sw || !sa || !sb || !sc) return TRT_E_INVALID;
+    if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
+    if (mode != TRT_MODE_AUTO && mode != TRT_MODE_SPLIT && mode != TRT_MODE_UNSPLIT) return TRT_E_INVALID;
+    if (variant < 0 || variant > kNumVariants) return TRT_E_INVALID;
+    if (sw[2] != 1 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
+    for (int d = 0; d < 2; ++d)
+        if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
+    const int64_t lim = (int64_t)1 << 30;
+    if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
+
+    const int v = resolve_variant(variant, R, S, I, J, K);
+    const Lt2Variant &vr = kVariants[v];
+    const SplitPlan sp = plan_split(R, S, I, J, K, mode, v);
+
+    Lt2Args args;
+    args.w = w; args.a = a; args.b = b;
+    args.R = (int)R; args.S = (int)S; args.I = (int)I; args.J = (int)J; args.K = (int)K;
+    args.sw0 = sw[0]; args.sw1 = sw[1];
+    args.sa0 = sa[0]; args.sa1 = sa[1];
+    args.sb0 = sb[0]; args.sb1 = sb[1];
+    args.sc0 = sc[0]; args.sc1 = sc[1];
+    args.s_tiles = (int)ceil_div(S, 32 * vr.rt);
+    args.n_tiles = (int)ceil_div(K, 32 * vr.ct * kLt2Waves);
+    args.splits = sp.splits;
+    args.iters_per_split = sp.iters_per_split;
+    args.total_wgs = (int64_t)R * args.s_tiles * args.n_tiles * sp.splits;
+    args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+    args.shift = nullptr;
+    args.c = c;
+    if (sp.split) {
+        const size_t need = ((size_t)sp.splits * R * S * K + (size_t)2 * R * K) * sizeof(float);
+        if (!workspace || workspace_bytes < need) return TRT_E_WORKSPACE;
+        args.c = static_cast<float *>(workspace);
+        args.shift = args.c + (size_t)sp.splits * R * S * K;
+    }
+    // 16-byte loads of w need aligned rows
+    const bool vec = (J % 4 == 0) && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) &&
+                     ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    launch_variant(v, args, vec, sp.split, s);
+    if (sp.split) {
+        const int64_t total = R * S * K;
+        int64_t blocks = ceil_div(total, 256);
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(lt2exp_merge_kernel, dim3((unsigned)blocks), dim3(256), 0, s, args.c, args.shift, c,
+                           (int)R, (int)S, (int)K, sp.splits, sc[0], sc[1]);
+    }
+    return (int)hipGetLastError();
+}

@@ -1,0 +1,52 @@
+"""lm2exp: batched ``log(a @ exp(b))`` on MI355X.
+
+Same contract as the reference wrapper, triturus/lm2exp.py:167-206:
+a is R x I x J (linear space), b is R x J x K (log space), both fp32 on one
+device; returns a fresh R x I x K tensor, enqueued on the current stream
+without synchronising.
+"""
+
+from __future__ import annotations
+
+from ctypes import c_void_p
+
+import torch
+
+from triturus_amd import _lib
+
+
+def _unit_inner(t: torch.Tensor) -> torch.Tensor:
+    # The kernels take free batch/row strides but a unit trailing stride (and
+    # no negative or zero-broadcast strides); anything else is materialised.
+    if t.stride(-1) == 1 and all(s > 0 for s in t.stride()):
+        return t
+    return t.contiguous()
+
+
+def lm2exp(a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0) -> torch.Tensor:
+    assert len(a.shape) == len(b.shape) == 3
+    assert a.shape[0] == b.shape[0]
+    assert a.shape[2] == b.shape[1]
+    assert a.dtype == b.dtype == torch.float32
+    assert a.device == b.device
+    _lib.require_gpu(a, b)
+    lib = _lib.load()
+
+    R, I, J = a.shape
+    K = b.shape[2]
+    c = torch.empty((R, I, K), dtype=a.dtype, device=a.device)
+    if c.numel() == 0:
+        return c
+    if J == 0:
+        # empty contraction: log(0)
+        return c.fill_(float("-inf"))
+    a = _unit_inner(a)
+    b = _unit_inner(b)
+    with torch.cuda.device(a.device):
+        status = lib.trt_lm2exp_f32(
+            c_void_p(a.data_ptr()), c_void_p(b.data_ptr()), c_void_p(c.data_ptr()),
+            R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
+            _variant, _lib.current_stream(a.device),
+        )
+    _lib.check(status, "trt_lm2exp_f32")
+    return c

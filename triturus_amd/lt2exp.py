@@ -1,0 +1,75 @@
+"""lt2exp: batched log-space Tucker-2 contraction on MI355X.
+
+Same contract as the reference wrapper, triturus/lt2exp.py:519-630:
+w is R x S x I x J (linear space), a is R x I x K, b is R x J x K (log space),
+all fp32 on one device; returns a fresh R x S x K tensor.  ``mode`` is
+"auto" | "split" | "unsplit"; anything else raises ValueError.  w must be
+viewable as R x S x (I*J) (``w.view`` raises RuntimeError otherwise, as in the
+reference).
+"""
+
+from __future__ import annotations
+
+from ctypes import c_void_p
+
+import torch
+
+from triturus_amd import _lib
+from triturus_amd.lm2exp import _unit_inner
+
+_MODES = {"auto": _lib.MODE_AUTO, "split": _lib.MODE_SPLIT, "unsplit": _lib.MODE_UNSPLIT}
+
+
+def launches_split(R: int, S: int, I: int, J: int, K: int, mode: str) -> bool:
+    """The reference's mode rule, triturus/lt2exp.py:534-541."""
+    if mode == "auto":
+        return R * S * K < 1048576 and I * J > 512
+    if mode == "split":
+        return True
+    if mode == "unsplit":
+        return False
+    raise ValueError(f"Uknown mode '{mode}' for the l2exp kernel")
+
+
+def lt2exp(
+    w: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, mode: str = "auto", _variant: int = 0
+) -> torch.Tensor:
+    assert len(w.shape) == 4
+    assert len(a.shape) == len(b.shape) == 3
+    assert w.shape[0] == a.shape[0] == b.shape[0]
+    assert w.shape[2] == a.shape[1]
+    assert w.shape[3] == b.shape[1]
+    assert a.shape[2] == b.shape[2]
+    assert w.dtype == a.dtype == b.dtype == torch.float32
+    assert w.device == a.device == b.device
+    R, S, I, J = w.shape
+    K = a.shape[2]
+    launches_split(R, S, I, J, K, mode)  # validates mode
+    _lib.require_gpu(w, a, b)
+    lib = _lib.load()
+
+    c = torch.empty((R, S, K), dtype=a.dtype, device=a.device)
+    w = w.view(R, S, -1)
+    if c.numel() == 0:
+        return c
+    if I * J == 0:
+        return c.fill_(float("-inf"))
+    w = _unit_inner(w)
+    a = _unit_inner(a)
+    b = _unit_inner(b)
+    mode_code = _MODES[mode]
+    ws_bytes = lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, mode_code)
+    ws = None
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+    with torch.cuda.device(a.device):
+        status = lib.trt_lt2exp_f32(
+            c_void_p(w.data_ptr()), c_void_p(a.data_ptr()), c_void_p(b.data_ptr()),
+            c_void_p(c.data_ptr()), R, S, I, J, K,
+            _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
+            mode_code, _variant,
+            c_void_p(ws.data_ptr() if ws is not None else None), ws_bytes,
+            _lib.current_stream(a.device),
+        )
+    _lib.check(status, "trt_lt2exp_f32")
+    return c
