@@ -1,0 +1,268 @@
+#!/usr/bin/env python3
+"""Benchmark of the log-space contraction path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A step is one ``lt2exp`` call on the large configuration (R=64, S=I=J=64, K=4096,
+fp32, seeded synthetic inputs already resident in HBM).  W untimed steps, then
+exactly K steps bracketed by ``torch.cuda.synchronize()``; rank 0 prints ONE
+JSON line on stdout (progress goes to stderr).  The same line carries
+
+  roofline      fp32-MFMA roofline of the dominant kernel: algorithmic flops per
+                launch / average launch duration from HIP events recorded on the
+                launch stream around the timed region;
+  cpu_baseline  the reference's torch recipe (restated in oracle/torch_baseline.py)
+                timed on this host's cores on a bounded sample of the same workload;
+  lm2exp, max   the other kernels of the path, each measured the same way
+                (lm2exp R=64, I=J=256, K=4096; matmax / vmax on the 64x64x4096
+                operand), with their own roofline objects.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+import torch
+
+PEAK_FP32_MFMA_TFLOPS = 157.3  # 256 CU x 4 SIMD x 64 flop/clk x 2.4 GHz
+PEAK_HBM_GBPS = 8000.0
+
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by
+# the same counters over trt_copy_bytes of known size; None until measured.
+MEASURED_TRAFFIC_BYTES = {"lt2exp_c5": None, "lm2exp_c3": None}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+def timed_region(fn, steps: int, warmup: int):
+    """(wall seconds, HIP-event seconds) over exactly `steps` calls."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    start.record()  # on the current stream: the stream the kernels are launched on
+    for _ in range(steps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    return wall, start.elapsed_time(stop) * 1e-3
+
+
+def do_bench(fn, *, warmup_ms=150.0, rep_ms=1000.0, flush_bytes=512 << 20):
+    """Median / q10 / q90 milliseconds of single calls, each preceded by a cache flush
+    (the protocol of the reference's benchmarks: benchmarks/lm2exp.py:94)."""
+    flush = torch.empty(flush_bytes, dtype=torch.uint8, device="cuda")
+    fn()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(5):
+        fn()
+    e.record()
+    torch.cuda.synchronize()
+    est = max(s.elapsed_time(e) / 5, 1e-3)
+    n_warm = max(1, int(warmup_ms / est))
+    n_rep = max(5, min(2000, int(rep_ms / est)))
+    for _ in range(n_warm):
+        fn()
+    ss = [torch.cuda.Event(enable_timing=True) for _ in range(n_rep)]
+    ee = [torch.cuda.Event(enable_timing=True) for _ in range(n_rep)]
+    for i in range(n_rep):
+        flush.zero_()
+        ss[i].record()
+        fn()
+        ee[i].record()
+    torch.cuda.synchronize()
+    ts = sorted(a.elapsed_time(b) for a, b in zip(ss, ee))
+    q = lambda f: ts[min(len(ts) - 1, int(f * len(ts)))]
+    return {"median_ms": q(0.5), "q10_ms": q(0.1), "q90_ms": q(0.9), "reps": n_rep}
+
+
+def graph_time(fn, calls: int = 20, reps: int = 20) -> float:
+    """Average seconds per call of a short kernel: `calls` launches captured in one HIP
+    graph (no host launch gaps), replayed `reps` times between HIP events."""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(3):
+            fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for _ in range(calls):
+            fn()
+    g.replay()
+    torch.cuda.synchronize()
+    s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    s.record()
+    for _ in range(reps):
+        g.replay()
+    e.record()
+    torch.cuda.synchronize()
+    return s.elapsed_time(e) * 1e-3 / (calls * reps)
+
+
+def cpu_time(fn, budget_s: float = 10.0):
+    """Median seconds of fn() on the host: 1 warm-up, then >= 3 repetitions (bounded)."""
+    t0 = time.perf_counter()
+    fn()
+    first = time.perf_counter() - t0
+    reps = max(3, min(10, int(budget_s / max(first, 1e-3))))
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return statistics.median(ts), reps
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-extras", action="store_true", help="skip lm2exp / max / do_bench sections")
+    args = ap.parse_args()
+    if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        log("bench.py: this path is built and measured on ONE GPU; R and K shard without any "
+            "exchange step, so a multi-GPU figure would be N independent copies of this run. "
+            "Run with --gpus 1.")
+        return 2
+    if not torch.cuda.is_available():
+        log("bench.py: no HIP device visible")
+        return 3
+
+    from triturus_amd import workloads as W
+    from triturus_amd.lm2exp import lm2exp
+    from triturus_amd.lt2exp import lt2exp
+    from triturus_amd.max import matmax, vmax
+
+    dev = torch.device("cuda", 0)
+    torch.cuda.set_device(dev)
+    log(f"device: {torch.cuda.get_device_name(0)}; torch {torch.__version__}")
+
+    # ------------------------------------------------------------ lt2exp, large
+    R, S, I, J, K = 64, 64, 64, 64, 4096
+    cfg = W.c5(R, S, I, J, K)
+    w, a, b = (cfg[k].to(dev) for k in "wab")
+    flops = W.lt2exp_flops(R, S, I, J, K)
+    step = lambda: lt2exp(w, a, b)
+    wall, ev = timed_region(step, args.steps, args.warmup)
+    ms_per_step = wall / args.steps * 1e3
+    value = flops * args.steps / wall / 1e9
+    achieved = flops / (ev / args.steps) / 1e12
+    log(f"lt2exp large: {ms_per_step:.4f} ms/step wall, {ev / args.steps * 1e3:.4f} ms/launch (HIP events), "
+        f"{achieved:.1f} TFLOP/s = {achieved / PEAK_FP32_MFMA_TFLOPS * 100:.1f}% of fp32 MFMA peak")
+    result = {
+        "metric": "lt2exp GFLOP/s (fp32, 2*R*S*I*J*K flops per call)",
+        "value": round(value, 1),
+        "unit": "GFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic (seeded: w ~ Dirichlet(1) over i*j, a,b ~ N(-30,10)), resident in HBM",
+        "config": {"workload": "lt2exp R=64 S=64 I=64 J=64 K=4096 (unsplit)", "R": R, "S": S, "I": I, "J": J,
+                   "K": K, "algorithmic_bytes": W.lt2exp_bytes(R, S, I, J, K), "algorithmic_flops": flops},
+        "roofline": {
+            "bound": "mfma",
+            "achieved": round(achieved, 2),
+            "peak": PEAK_FP32_MFMA_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
+            "traffic": MEASURED_TRAFFIC_BYTES["lt2exp_c5"],
+            "kernel": "lt2exp_kernel<2,2,8,4,vec,unsplit>",
+        },
+    }
+
+    from oracle import torch_baseline  # CPU competitor lines only; never on the GPU path
+
+    if not args.no_cpu_baseline:
+        torch.set_num_threads(max(1, min(16, os.cpu_count() or 1)))
+        nb = 2  # batches in the sample; the recipe materialises R x (I*J) x K floats
+        wc, ac, bc = cfg["w"][:nb], cfg["a"][:nb], cfg["b"][:nb]
+        sec, reps = cpu_time(lambda: torch_baseline.lt2exp_fp32_chunked(wc, ac, bc, 1))
+        cpu_gflops = W.lt2exp_flops(nb, S, I, J, K) / sec / 1e9
+        result["cpu_baseline"] = {
+            "value": round(cpu_gflops, 2),
+            "unit": "GFLOP/s",
+            "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{nb} of {R} batches of the same inputs, torch fp32 recipe (amax/clamp/exp/outer/bmm/log) "
+                      f"one batch at a time, median of {reps} runs after 1 warm-up; host has {os.cpu_count()} logical CPUs",
+            "speedup_gpu_over_cpu": round(value / cpu_gflops, 1),
+        }
+        log(f"cpu baseline lt2exp: {cpu_gflops:.1f} GFLOP/s on {torch.get_num_threads()} threads")
+
+    if not args.no_extras:
+        result["do_bench_lt2exp"] = do_bench(step)
+        del w, a, b
+        # ------------------------------------------------------- lm2exp, rectangular
+        R2, I2, J2, K2 = 64, 256, 256, 4096
+        cfg3 = W.c3(R2, I2, J2, K2)
+        a3, b3 = cfg3["a"].to(dev), cfg3["b"].to(dev)
+        fl3 = W.lm2exp_flops(R2, I2, J2, K2)
+        step3 = lambda: lm2exp(a3, b3)
+        wall3, ev3 = timed_region(step3, args.steps, args.warmup)
+        ach3 = fl3 / (ev3 / args.steps) / 1e12
+        lm = {
+            "workload": "lm2exp R=64 I=256 J=256 K=4096 (b ~ N(-50,20), 5% -inf)",
+            "value": round(fl3 * args.steps / wall3 / 1e9, 1),
+            "unit": "GFLOP/s",
+            "ms_per_step": round(wall3 / args.steps * 1e3, 5),
+            "algorithmic_bytes": W.lm2exp_bytes(R2, I2, J2, K2),
+            "roofline": {"bound": "mfma", "achieved": round(ach3, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(ach3 / PEAK_FP32_MFMA_TFLOPS, 4),
+                         "traffic": MEASURED_TRAFFIC_BYTES["lm2exp_c3"]},
+            "do_bench": do_bench(step3),
+        }
+        log(f"lm2exp rect: {ev3 / args.steps * 1e3:.4f} ms/launch, {ach3:.1f} TFLOP/s = "
+            f"{ach3 / PEAK_FP32_MFMA_TFLOPS * 100:.1f}% of fp32 MFMA peak")
+        if not args.no_cpu_baseline:
+            nb = 8
+            sec, reps = cpu_time(lambda: torch_baseline.lm2exp_fp32(cfg3["a"][:nb], cfg3["b"][:nb]))
+            g = W.lm2exp_flops(nb, I2, J2, K2) / sec / 1e9
+            lm["cpu_baseline"] = {"value": round(g, 2), "unit": "GFLOP/s", "cores": torch.get_num_threads(),
+                                  "kind": "port", "sample": f"{nb} of {R2} batches, median of {reps} runs",
+                                  "speedup_gpu_over_cpu": round(lm["value"] / g, 1)}
+            log(f"cpu baseline lm2exp: {g:.1f} GFLOP/s")
+        result["lm2exp"] = lm
+        del a3, b3
+
+        # ------------------------------------------------ max reductions (HBM bound)
+        x = cfg["b"].to(dev)  # 64 x 64 x 4096
+        nbytes = x.numel() * 4
+        flat, mat = x.view(-1), x.view(4096, 4096)
+        mx = {"bytes": nbytes, "unit": "GB/s", "peak": PEAK_HBM_GBPS}
+        for name, fn in (("vmax", lambda: vmax(flat)), ("matmax_axis0", lambda: matmax(mat, 0)),
+                         ("matmax_axis1", lambda: matmax(mat, 1)),
+                         ("torch_max", lambda: torch.max(flat, 0)), ("torch_amax_axis0", lambda: torch.amax(mat, 0)),
+                         ("torch_amax_axis1", lambda: torch.amax(mat, 1))):
+            sec = graph_time(fn)
+            mx[name] = {"us": round(sec * 1e6, 2), "achieved": round(nbytes / sec / 1e9, 1),
+                        "frac": round(nbytes / sec / 1e9 / PEAK_HBM_GBPS, 4)}
+            log(f"{name}: {sec * 1e6:.2f} us, {nbytes / sec / 1e9:.0f} GB/s")
+        result["max"] = mx
+
+    print(json.dumps(result), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -1,0 +1,193 @@
+"""The drop-in boundary, without a GPU: the C-ABI library loads and exports what
+include/triturus_hip.h declares, argument errors are reported as statuses before
+anything is enqueued, and the Python wrappers raise what the reference wrappers
+raise (triturus/lm2exp.py:168-172, triturus/lt2exp.py:522-541,549,
+triturus/max.py:97-99,177-180)."""
+
+import ctypes
+import re
+from ctypes import c_void_p
+from pathlib import Path
+
+import pytest
+import torch
+
+from triturus_amd import _lib
+from triturus_amd.lm2exp import lm2exp
+from triturus_amd.lt2exp import launches_split, lt2exp
+from triturus_amd.max import matmax, vamax, vmax
+from triturus_amd.utils import ensure_reproducibility, is_triturus_tf32_enabled, set_tf32_enabled
+
+ROOT = Path(__file__).resolve().parents[1]
+HEADER = (ROOT / "include" / "triturus_hip.h").read_text()
+
+
+def declared_functions():
+    body = re.sub(r"/\*.*?\*/", "", HEADER, flags=re.S)
+    return sorted(set(re.findall(r"\b(trt_[a-z0-9_]+)\s*\(", body)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert "trt_lm2exp_f32" in names and "trt_lt2exp_f32" in names and len(names) >= 10
+    raw = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in names:
+        assert hasattr(raw, name), f"{name} declared in the header but not exported"
+    # the ctypes table binds exactly the declared set
+    assert sorted(_lib.SIGNATURES) == names
+
+
+def test_version_and_error_strings():
+    lib = _lib.load()
+    assert lib.trt_version() == _lib.ABI_VERSION
+    assert int(re.search(r"#define TRT_ABI_VERSION (\d+)", HEADER).group(1)) == _lib.ABI_VERSION
+    assert lib.trt_error_string(0) == b"success"
+    for code in (-1, -2, -3, -4):
+        assert lib.trt_error_string(code) not in (b"success", b"unknown status")
+    assert lib.trt_error_string(-99) == b"unknown status"
+
+
+def test_header_constants_match_python():
+    def const(name):
+        return int(re.search(rf"#define {name} \(?(-?\d+)\)?", HEADER).group(1))
+
+    assert (const("TRT_F32"), const("TRT_F64"), const("TRT_F16"), const("TRT_BF16")) == (0, 1, 2, 3)
+    assert (const("TRT_MODE_AUTO"), const("TRT_MODE_SPLIT"), const("TRT_MODE_UNSPLIT")) == (
+        _lib.MODE_AUTO, _lib.MODE_SPLIT, _lib.MODE_UNSPLIT)
+
+
+def test_c_abi_argument_errors_are_statuses():
+    lib = _lib.load()
+    s3 = (ctypes.c_int64 * 3)
+    ok = s3(12, 4, 1)
+    one = c_void_p(16)  # never dereferenced: every call below is rejected first
+    null = c_void_p(None)
+    # lm2exp
+    assert lib.trt_lm2exp_f32(null, one, one, 1, 1, 1, 1, ok, ok, ok, 0, null) == -1
+    assert lib.trt_lm2exp_f32(one, one, one, 0, 1, 1, 1, ok, ok, ok, 0, null) == -1
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, ok, 99, null) == -1
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, s3(12, 1, 4), ok, ok, 0, null) == -2
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, s3(-12, 4, 1), ok, 0, null) == -2
+    assert lib.trt_lm2exp_f32(one, one, one, 1 << 31, 1, 1, 1, ok, ok, ok, 0, null) == -4
+    # lt2exp
+    args = (1, 1, 1, 1, 1, ok, ok, ok, ok)
+    assert lib.trt_lt2exp_f32(one, null, one, one, *args, 0, 0, null, 0, null) == -1
+    assert lib.trt_lt2exp_f32(one, one, one, one, *args, 7, 0, null, 0, null) == -1
+    assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, s3(1, 1, 2), ok, 0, 0, null, 0, null) == -2
+    assert lib.trt_lt2exp_f32(one, one, one, one, *args, _lib.MODE_SPLIT, 0, null, 0, null) == -3
+    # max
+    assert lib.trt_vmax(null, 5, 0, one, one, one, 1 << 20, null) == -1
+    assert lib.trt_vmax(one, 0, 0, one, one, one, 1 << 20, null) == -1
+    assert lib.trt_vmax(one, 5, 9, one, one, one, 1 << 20, null) == -1
+    assert lib.trt_vmax(one, 5, 0, one, one, null, 0, null) == -3
+    assert lib.trt_matmax(one, one, 4, 4, 2, 0, null, 0, null) == -1
+    assert lib.trt_matmax(one, one, 0, 4, 0, 0, null, 0, null) == -1
+    assert lib.trt_copy_bytes(one, one, 24, null) == -1
+
+
+def test_workspace_queries_are_host_only_and_follow_the_mode_rule():
+    lib = _lib.load()
+    assert lib.trt_vmax_workspace_bytes(1000, _lib.TRT_F32) >= 2048 * 16
+    assert lib.trt_vmax_workspace_bytes(1000, 9) == 0
+    assert lib.trt_matmax_workspace_bytes(4096, 4096, 1, _lib.TRT_F32) == 0
+    assert lib.trt_matmax_workspace_bytes(4096, 4096, 0, _lib.TRT_F32) > 0
+    assert lib.trt_matmax_workspace_bytes(2, 1 << 24, 1, _lib.TRT_F32) > 0
+    shapes = [(3, 75, 50, 50, 100), (16, 64, 32, 32, 2048), (64, 64, 64, 64, 4096), (1, 16, 16, 16, 16),
+              (1, 1024, 32, 32, 1023), (1, 1024, 32, 32, 1024), (4, 8, 2, 256, 100), (4, 8, 23, 23, 100)]
+    for R, S, I, J, K in shapes:
+        assert lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, _lib.MODE_UNSPLIT) == 0
+        assert lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, _lib.MODE_SPLIT) >= 4 * (R * S * K + 2 * R * K)
+        auto = lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, _lib.MODE_AUTO) > 0
+        assert auto == launches_split(R, S, I, J, K, "auto")
+    # the reference rule itself, triturus/lt2exp.py:535: at the benchmark configurations it is unsplit
+    assert not launches_split(16, 64, 32, 32, 2048, "auto")
+    assert not launches_split(64, 64, 64, 64, 4096, "auto")
+    assert launches_split(3, 75, 50, 50, 100, "auto")
+    assert not launches_split(1, 1024, 32, 32, 1024, "auto")  # 2**20 is not < 2**20
+    assert not launches_split(1, 16, 16, 32, 16, "auto")  # I*J = 512 is not > 512
+
+
+def test_lm2exp_wrapper_validation():
+    a, b = torch.rand(2, 3, 4), torch.rand(2, 4, 5)
+    with pytest.raises(AssertionError):
+        lm2exp(a[0], b)
+    with pytest.raises(AssertionError):
+        lm2exp(a, b[:1])
+    with pytest.raises(AssertionError):
+        lm2exp(a, torch.rand(2, 5, 5))
+    with pytest.raises(AssertionError):
+        lm2exp(a.double(), b)
+    with pytest.raises(AssertionError):
+        lm2exp(a, b.to("meta"))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        lm2exp(a, b)
+
+
+def test_lt2exp_wrapper_validation():
+    w, a, b = torch.rand(2, 3, 4, 5), torch.rand(2, 4, 6), torch.rand(2, 5, 6)
+    with pytest.raises(AssertionError):
+        lt2exp(w[0], a, b)
+    with pytest.raises(AssertionError):
+        lt2exp(w, a[:1], b)
+    with pytest.raises(AssertionError):
+        lt2exp(w, b, a)  # I/J swapped
+    with pytest.raises(AssertionError):
+        lt2exp(w, a, torch.rand(2, 5, 7))
+    with pytest.raises(AssertionError):
+        lt2exp(w, a.half(), b)
+    with pytest.raises(ValueError):
+        lt2exp(w, a, b, mode="stream-k")
+    with pytest.raises(RuntimeError, match="GPU only"):
+        lt2exp(w, a, b, mode="split")
+
+
+def test_max_wrapper_validation():
+    x = torch.randn(10, 12)
+    with pytest.raises(AssertionError):
+        vmax(x)
+    with pytest.raises(AssertionError):
+        vamax(torch.arange(5))
+    with pytest.raises(AssertionError):
+        vmax(x[0, ::2])
+    with pytest.raises(AssertionError):
+        matmax(x[0])
+    with pytest.raises(AssertionError):
+        matmax(x.T)
+    with pytest.raises(AssertionError):
+        matmax(x, axis=2)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        matmax(x, axis=1, block_size=2)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        vmax(x[0], block_size=2)
+
+
+def test_flags():
+    set_tf32_enabled(True)
+    assert is_triturus_tf32_enabled()
+    set_tf32_enabled(False)
+    assert not is_triturus_tf32_enabled()
+    ensure_reproducibility(seed=7, device="cpu")
+    x = torch.rand(3)
+    ensure_reproducibility(seed=7, device="cpu")
+    assert torch.equal(x, torch.rand(3))
+
+
+def test_reference_import_paths_exist():
+    from triturus.lm2exp import lm2exp as f1
+    from triturus.lt2exp import lt2exp as f2
+    from triturus.max import matmax as f3, vamax as f4, vmax as f5
+    from triturus.utils import ensure_reproducibility as f6, set_tf32_enabled as f7
+
+    assert f1 is lm2exp and f2 is lt2exp and (f3, f4, f5) == (matmax, vamax, vmax)
+    assert callable(f6) and callable(f7)
+    import triturus
+
+    assert not hasattr(triturus, "__all__")  # the reference's __init__ is empty
+
+
+def test_product_never_imports_the_oracle():
+    for pkg in ("triturus_amd", "triturus"):
+        for f in (ROOT / pkg).rglob("*"):
+            if f.suffix in {".py", ".hip", ".hpp", ".h"}:
+                text = f.read_text()
+                assert "oracle" not in text.replace("the oracle the reference tests use", ""), f

@@ -1,0 +1,200 @@
+"""lm2exp on the GPU against the float64 oracle and the fp32 torch recipe.
+
+Accuracy gate: |x - y| <= 1e-5 + 1e-4 |y| against float64, -inf positions exact,
+no NaN (oracle64.compare); at the reference's own test shape additionally the
+reference's bar, torch.allclose defaults (rtol 1e-5, atol 1e-8, tests/lm2exp.py:23)
+against the fp32 torch recipe."""
+
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle64, torch_baseline
+from triturus.lm2exp import lm2exp
+from triturus.utils import set_tf32_enabled
+from triturus_amd import _lib, workloads
+
+pytestmark = pytest.mark.gpu
+GOLDEN = Path(__file__).resolve().parent / "golden"
+NINF = float("-inf")
+N_VARIANTS = 7
+
+
+def _check(out, a, b, **kw):
+    r = oracle64.compare(out, oracle64.lm2exp64(a, b), **kw)
+    assert r["ok"], r
+    return r
+
+
+@pytest.mark.parametrize("allow_tf32", [False, True])
+def test_lm2exp(dev, allow_tf32):
+    """The reference's test (tests/lm2exp.py:10-23): same shape, inputs and tolerances."""
+    set_tf32_enabled(allow_tf32)
+    batch, m, k, n = 24, 150, 100, 200
+    a = torch.rand(batch, m, k)
+    b = torch.randn(batch, k, n)
+    gt = torch_baseline.lm2exp_fp32(a, b)
+    c = lm2exp(a.to(dev), b.to(dev))
+    assert c.shape == (batch, m, n) and c.dtype == torch.float32 and c.device.type == "cuda"
+    if allow_tf32:
+        assert torch.allclose(gt, c.cpu(), rtol=5e-4)
+    else:
+        assert torch.allclose(gt, c.cpu())
+    # and the same recipe evaluated by torch on the GPU
+    assert torch.allclose(torch_baseline.lm2exp_fp32(a.to(dev), b.to(dev)), c)
+    _check(c, a, b)
+
+
+@pytest.mark.parametrize("name", ["lm2exp_small", "lm2exp_ragged"])
+def test_golden(dev, name):
+    z = np.load(GOLDEN / f"{name}.npz")
+    out = lm2exp(torch.from_numpy(z["a"]).to(dev), torch.from_numpy(z["b"]).to(dev))
+    r = oracle64.compare(out, z["c"])
+    assert r["ok"] and r["n_neg_inf"] > 0, r
+
+
+@pytest.mark.parametrize("variant", range(1, N_VARIANTS + 1))
+@pytest.mark.parametrize("shape", [(3, 37, 41, 70), (2, 300, 52, 129), (1, 64, 64, 64), (2, 33, 7, 31)])
+def test_every_tile_variant_on_ragged_shapes(dev, variant, shape):
+    assert _lib.load().trt_lm2exp_variant_count() == N_VARIANTS
+    R, I, J, K = shape
+    g = torch.Generator().manual_seed(variant * 100 + I)
+    a = torch.rand(R, I, J, generator=g)
+    b = -5 + 4 * torch.randn(R, J, K, generator=g)
+    b[torch.rand(b.shape, generator=g) < 0.1] = NINF
+    out = lm2exp(a.to(dev), b.to(dev), _variant=variant)
+    _check(out, a, b)
+
+
+@pytest.mark.parametrize(
+    "shape",
+    [(1, 1, 1, 1), (1, 1, 5, 1), (2, 1, 1, 9), (1, 5, 1, 3), (3, 2, 3, 1), (1, 31, 33, 35), (2, 257, 4, 65),
+     (1, 513, 130, 260), (5, 16, 1000, 24), (1, 8, 4097, 16)],
+)
+def test_edge_shapes(dev, shape):
+    R, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(R, I, J, generator=g)
+    b = 2 * torch.randn(R, J, K, generator=g)
+    _check(lm2exp(a.to(dev), b.to(dev)), a, b)
+
+
+def test_empty_inputs(dev):
+    assert lm2exp(torch.rand(0, 3, 4, device=dev), torch.rand(0, 4, 5, device=dev)).shape == (0, 3, 5)
+    assert lm2exp(torch.rand(2, 0, 4, device=dev), torch.rand(2, 4, 5, device=dev)).shape == (2, 0, 5)
+    assert lm2exp(torch.rand(2, 3, 4, device=dev), torch.rand(2, 4, 0, device=dev)).shape == (2, 3, 0)
+    out = lm2exp(torch.rand(2, 3, 0, device=dev), torch.rand(2, 0, 5, device=dev))
+    assert out.shape == (2, 3, 5) and torch.all(out == NINF)
+
+
+def test_neg_inf_columns_zero_rows_and_range(dev):
+    g = torch.Generator().manual_seed(5)
+    a = torch.rand(3, 70, 90, generator=g)
+    b = -50 + 20 * torch.randn(3, 90, 150, generator=g)
+    b[torch.rand(b.shape, generator=g) < 0.3] = NINF
+    b[0, :, 17] = NINF
+    b[2, :, 149] = NINF
+    a[1, 33, :] = 0.0
+    out = lm2exp(a.to(dev), b.to(dev))
+    r = _check(out, a, b)
+    assert r["n_neg_inf"] >= 2 * 70 + 150
+    assert torch.all(out[0, :, 17] == NINF) and torch.all(out[1, 33, :] == NINF)
+    assert not torch.isnan(out).any()
+    # extreme magnitudes: columns near the clamp, and a column whose max is huge
+    b = torch.full((1, 4, 64), -9e37)
+    b[0, :, 1] = torch.tensor([-1e30, -2e30, NINF, -1e30])
+    b[0, :, 2] = torch.tensor([80.0, -80.0, 0.0, 3.0])
+    a = torch.rand(1, 6, 4, generator=g)
+    out = lm2exp(a.to(dev), b.to(dev))
+    _check(out, a, b)
+    assert torch.isfinite(out).all()
+
+
+def test_nan_input_propagates_like_the_torch_recipe(dev):
+    a = torch.rand(1, 8, 8)
+    b = torch.randn(1, 8, 40)
+    b[0, 3, 5] = float("nan")
+    out = lm2exp(a.to(dev), b.to(dev)).cpu()
+    ref = torch_baseline.lm2exp_fp32(a, b)
+    assert torch.equal(torch.isnan(out), torch.isnan(ref))
+    assert torch.isnan(out[0, :, 5]).all() and not torch.isnan(out[0, :, :5]).any()
+
+
+def test_strided_inputs(dev):
+    g = torch.Generator().manual_seed(6)
+    a_big = torch.rand(4, 80, 96, generator=g)
+    b_big = torch.randn(4, 96, 200, generator=g)
+    # row / batch strided views with unit inner stride go to the kernel as they are
+    a = a_big[::2, 5:61, 8:72]
+    b = b_big[::2, 16:80, 3:143]
+    out = lm2exp(a_big.to(dev)[::2, 5:61, 8:72], b_big.to(dev)[::2, 16:80, 3:143])
+    _check(out, a, b)
+    # transposed operands (inner stride != 1) and broadcast views
+    at = torch.rand(2, 64, 56, generator=g)
+    out = lm2exp(at.to(dev).transpose(1, 2), b_big.to(dev)[:2, :64])
+    _check(out, at.transpose(1, 2), b_big[:2, :64])
+    a1 = torch.rand(1, 56, 64, generator=g)
+    out = lm2exp(a1.to(dev).expand(2, 56, 64), b_big.to(dev)[:2, :64])
+    _check(out, a1.expand(2, 56, 64), b_big[:2, :64])
+    # inputs are never modified
+    ag, bg = a_big.to(dev), b_big.to(dev)
+    lm2exp(ag[:, :, :96], bg)
+    assert torch.equal(ag.cpu(), a_big) and torch.equal(bg.cpu(), b_big)
+
+
+def test_algebraic_properties_on_the_gpu(dev):
+    g = torch.Generator().manual_seed(7)
+    R, I, J, K = 2, 128, 96, 256
+    a = torch.rand(R, I, J, generator=g).to(dev)
+    b = (3 * torch.randn(R, J, K, generator=g)).to(dev)
+    c = lm2exp(a, b)
+    # identity weights return b
+    eye = torch.eye(J, device=dev).expand(R, J, J).contiguous()
+    assert torch.allclose(lm2exp(eye, b), b, rtol=1e-5, atol=1e-5)
+    # power-of-two column shifts and row scalings are exact in floating point
+    shift = 64.0 * torch.arange(K, device=dev).remainder(5)
+    assert torch.allclose(lm2exp(a, b + shift), c + shift, rtol=1e-5, atol=1e-4)
+    assert torch.allclose(lm2exp(4 * a, b), c + np.log(4.0), rtol=1e-5, atol=1e-5)
+    # convex weights stay between the column extremes
+    an = a / a.sum(2, keepdim=True)
+    cn = lm2exp(an, b)
+    assert torch.all(cn <= b.amax(1, keepdim=True) + 1e-4) and torch.all(cn >= b.amin(1, keepdim=True) - 1e-4)
+    # deterministic
+    assert torch.equal(lm2exp(a, b), c)
+
+
+@pytest.mark.parametrize("name", ["c1", "c2"])
+def test_benchmark_configurations_small(dev, name):
+    cfg = workloads.CONFIGS[name]()
+    a, b = cfg["a"], cfg["b"]
+    out = lm2exp(a.to(dev), b.to(dev))
+    r = _check(out, a, b)
+    if name == "c2":
+        assert r["n_neg_inf"] >= 16 * 512
+        for rr in range(16):
+            assert torch.all(out[rr, :, cfg["neg_inf_cols"][rr]] == NINF)
+        assert torch.allclose(torch_baseline.lm2exp_fp32(a, b), out.cpu(), rtol=1e-5, atol=1e-6)
+
+
+def test_benchmark_configuration_c3_full_size(dev):
+    """R=64, I=J=256, K=4096, b ~ N(-50, 20) with 5% -inf: every output against float64."""
+    cfg = workloads.c3()
+    a, b = cfg["a"], cfg["b"]
+    ag, bg = a.to(dev), b.to(dev)
+    out = lm2exp(ag, bg)
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()
+    worst = 0.0
+    for r0 in range(0, 64, 8):  # float64 oracle, 8 batches at a time
+        r = oracle64.compare(out[r0:r0 + 8], oracle64.lm2exp64(a[r0:r0 + 8], b[r0:r0 + 8]))
+        assert r["ok"], (r0, r)
+        worst = max(worst, r["worst_err_over_tol"])
+    # size-independent properties on the whole output
+    assert torch.all(out <= bg.amax(1, keepdim=True) + 1e-3)
+    for variant in (1, 2, 3):
+        alt = lm2exp(ag, bg, _variant=variant)
+        assert torch.allclose(alt, out, rtol=1e-5, atol=1e-5)
+    shifted = lm2exp(ag, bg + 128.0)
+    assert torch.allclose(shifted, out + 128.0, rtol=1e-5, atol=1e-3)

@@ -1,0 +1,190 @@
+"""lt2exp on the GPU against the float64 oracle and the fp32 torch recipe.
+
+Accuracy gate as for lm2exp (oracle64.compare: rtol 1e-4, atol 1e-5, -inf exact,
+no NaN); at the reference's test shape additionally torch.allclose defaults
+against the fp32 torch recipe (tests/lt2exp.py:36-40), for every ``mode``."""
+
+import itertools
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import oracle64, torch_baseline
+from triturus.lm2exp import lm2exp
+from triturus.lt2exp import lt2exp
+from triturus.utils import set_tf32_enabled
+from triturus_amd import _lib, workloads
+
+pytestmark = pytest.mark.gpu
+GOLDEN = Path(__file__).resolve().parent / "golden"
+NINF = float("-inf")
+N_VARIANTS = 8
+
+
+def _check(out, w, a, b, **kw):
+    r = oracle64.compare(out, oracle64.lt2exp64(w, a, b), **kw)
+    assert r["ok"], r
+    return r
+
+
+@pytest.mark.parametrize("mode,allow_tf32", itertools.product(["auto", "split", "unsplit"], [False, True]))
+def test_lt2exp(dev, mode, allow_tf32):
+    """The reference's test (tests/lt2exp.py:14-40): same shape, inputs and tolerances."""
+    set_tf32_enabled(allow_tf32)
+    batch, m, j, k, n = 3, 75, 50, 50, 100
+    w = torch.rand(batch, m, j, k)
+    a = torch.randn(batch, j, n)
+    b = torch.randn(batch, k, n)
+    gt = torch_baseline.lt2exp_fp32(w, a, b)
+    c = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode)
+    assert c.shape == (batch, m, n) and c.dtype == torch.float32 and c.device.type == "cuda"
+    if allow_tf32:
+        assert torch.allclose(gt, c.cpu(), rtol=5e-4)
+    else:
+        assert torch.allclose(gt, c.cpu())
+    assert torch.allclose(torch_baseline.lt2exp_fp32(w.to(dev), a.to(dev), b.to(dev)), c)
+    _check(c, w, a, b)
+
+
+@pytest.mark.parametrize("name", ["lt2exp_small", "lt2exp_ragged"])
+@pytest.mark.parametrize("mode", ["unsplit", "split"])
+def test_golden(dev, name, mode):
+    z = np.load(GOLDEN / f"{name}.npz")
+    out = lt2exp(*(torch.from_numpy(z[k]).to(dev) for k in "wab"), mode=mode)
+    r = oracle64.compare(out, z["c"])
+    assert r["ok"] and r["n_neg_inf"] > 0, r
+
+
+@pytest.mark.parametrize("variant", range(1, N_VARIANTS + 1))
+@pytest.mark.parametrize("mode", ["unsplit", "split"])
+@pytest.mark.parametrize("shape", [(2, 35, 9, 13, 45), (1, 70, 20, 33, 300), (2, 16, 5, 72, 64), (1, 33, 3, 3, 31)])
+def test_every_tile_variant_on_ragged_shapes(dev, variant, mode, shape):
+    assert _lib.load().trt_lt2exp_variant_count() == N_VARIANTS
+    R, S, I, J, K = shape
+    g = torch.Generator().manual_seed(variant * 100 + S)
+    w = torch.rand(R, S, I, J, generator=g)
+    a = -3 + 2 * torch.randn(R, I, K, generator=g)
+    b = -3 + 2 * torch.randn(R, J, K, generator=g)
+    a[torch.rand(a.shape, generator=g) < 0.1] = NINF
+    b[torch.rand(b.shape, generator=g) < 0.1] = NINF
+    out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _variant=variant)
+    _check(out, w, a, b)
+
+
+@pytest.mark.parametrize(
+    "shape",
+    [(1, 1, 1, 1, 1), (2, 1, 3, 1, 5), (1, 3, 1, 4, 1), (1, 65, 2, 2, 257), (3, 8, 64, 4, 40), (1, 8, 4, 64, 40),
+     (1, 129, 17, 65, 33), (1, 4, 300, 3, 16), (1, 4, 3, 300, 16)],
+)
+@pytest.mark.parametrize("mode", ["auto", "split"])
+def test_edge_shapes(dev, shape, mode):
+    R, S, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    w = torch.rand(R, S, I, J, generator=g)
+    a = 2 * torch.randn(R, I, K, generator=g)
+    b = 2 * torch.randn(R, J, K, generator=g)
+    _check(lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode), w, a, b)
+
+
+def test_empty_inputs(dev):
+    def z(*shape):
+        return torch.rand(*shape, device=dev)
+
+    assert lt2exp(z(0, 3, 4, 5), z(0, 4, 6), z(0, 5, 6)).shape == (0, 3, 6)
+    assert lt2exp(z(2, 0, 4, 5), z(2, 4, 6), z(2, 5, 6)).shape == (2, 0, 6)
+    assert lt2exp(z(2, 3, 4, 5), z(2, 4, 0), z(2, 5, 0)).shape == (2, 3, 0)
+    out = lt2exp(z(2, 3, 0, 5), z(2, 0, 6), z(2, 5, 6))
+    assert out.shape == (2, 3, 6) and torch.all(out == NINF)
+
+
+def test_neg_inf_and_zero_weights(dev):
+    g = torch.Generator().manual_seed(8)
+    R, S, I, J, K = 2, 40, 24, 40, 130
+    w = torch.rand(R, S, I, J, generator=g)
+    a = -30 + 10 * torch.randn(R, I, K, generator=g)
+    b = -30 + 10 * torch.randn(R, J, K, generator=g)
+    a[torch.rand(a.shape, generator=g) < 0.3] = NINF
+    b[torch.rand(b.shape, generator=g) < 0.3] = NINF
+    a[0, :, 11] = NINF
+    b[1, :, 129] = NINF
+    w[1, 7] = 0.0
+    for mode in ("unsplit", "split"):
+        out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode)
+        _check(out, w, a, b)
+        assert torch.all(out[0, :, 11] == NINF) and torch.all(out[1, :, 129] == NINF)
+        assert torch.all(out[1, 7] == NINF) and not torch.isnan(out).any()
+
+
+def test_non_viewable_weights_raise_like_the_reference(dev):
+    w = torch.rand(2, 3, 5, 4, device=dev).transpose(2, 3)  # I and J not jointly contiguous
+    with pytest.raises(RuntimeError):
+        lt2exp(w, torch.rand(2, 4, 6, device=dev), torch.rand(2, 5, 6, device=dev))
+
+
+def test_strided_inputs(dev):
+    g = torch.Generator().manual_seed(9)
+    w_big = torch.rand(4, 50, 12, 20, generator=g)
+    a_big = torch.randn(4, 12, 100, generator=g)
+    b_big = torch.randn(4, 40, 100, generator=g)
+    sl = (slice(None, None, 2), slice(3, 45))
+    w, a, b = w_big[sl], a_big[::2, :, 7:90], b_big[::2, 10:30, 7:90]
+    out = lt2exp(w_big.to(dev)[sl], a_big.to(dev)[::2, :, 7:90], b_big.to(dev)[::2, 10:30, 7:90])
+    _check(out, w, a, b)
+    # inner-strided log operands are materialised by the wrapper
+    at = torch.randn(2, 83, 12, generator=g)
+    out = lt2exp(w_big.to(dev)[sl], at.to(dev).transpose(1, 2), b_big.to(dev)[::2, 10:30, 7:90])
+    _check(out, w, at.transpose(1, 2), b)
+
+
+def test_reduces_to_lm2exp_and_factorises(dev):
+    g = torch.Generator().manual_seed(10)
+    R, S, I, J, K = 2, 64, 16, 24, 192
+    w = torch.rand(R, S, I, J, generator=g).to(dev)
+    a = (2 * torch.randn(R, I, K, generator=g)).to(dev)
+    b = (2 * torch.randn(R, J, K, generator=g)).to(dev)
+    c = lt2exp(w, a, b)
+    ab = (a[:, :, None, :] + b[:, None, :, :]).reshape(R, I * J, K)
+    assert torch.allclose(c, lm2exp(w.view(R, S, I * J), ab), rtol=1e-5, atol=1e-5)
+    u = torch.rand(R, S, I, generator=g).to(dev)
+    v = torch.rand(R, S, J, generator=g).to(dev)
+    w1 = (u[:, :, :, None] * v[:, :, None, :]).contiguous()
+    assert torch.allclose(lt2exp(w1, a, b), lm2exp(u, a) + lm2exp(v, b), rtol=1e-5, atol=1e-5)
+    # split and unsplit agree, and both are deterministic
+    cs = lt2exp(w, a, b, mode="split")
+    assert torch.allclose(cs, c, rtol=1e-6, atol=1e-6)
+    assert torch.equal(lt2exp(w, a, b, mode="split"), cs) and torch.equal(lt2exp(w, a, b), c)
+
+
+def test_benchmark_configuration_c4(dev):
+    cfg = workloads.c4()
+    w, a, b = cfg["w"], cfg["a"], cfg["b"]
+    out = lt2exp(w.to(dev), a.to(dev), b.to(dev))
+    _check(out, w, a, b)
+    assert torch.allclose(torch_baseline.lt2exp_fp32(w, a, b), out.cpu(), rtol=1e-5, atol=1e-5)
+
+
+def test_benchmark_configuration_c5_full_size(dev):
+    """R=64, S=I=J=64, K=4096: float64 oracle on 8 of the 64 batches, the lm2exp
+    identity and shift equivariance on the whole output."""
+    cfg = workloads.c5()
+    w, a, b = cfg["w"], cfg["a"], cfg["b"]
+    wg, ag, bg = w.to(dev), a.to(dev), b.to(dev)
+    out = lt2exp(wg, ag, bg)
+    torch.cuda.synchronize()
+    assert out.shape == (64, 64, 4096) and torch.isfinite(out).all()
+    for r in (0, 9, 18, 27, 36, 45, 54, 63):
+        res = oracle64.compare(out[r:r + 1], oracle64.lt2exp64(w[r:r + 1], a[r:r + 1], b[r:r + 1]))
+        assert res["ok"], (r, res)
+    # the same contraction through the other kernel, 16 batches at a time (1 GiB intermediate each)
+    for r0 in range(0, 64, 16):
+        sl = slice(r0, r0 + 16)
+        ab = (ag[sl, :, None, :] + bg[sl, None, :, :]).reshape(16, 64 * 64, 4096)
+        via = lm2exp(wg[sl].view(16, 64, 64 * 64), ab)
+        assert torch.allclose(out[sl], via, rtol=1e-5, atol=1e-4)
+        del ab, via
+    assert torch.allclose(lt2exp(wg, ag + 64.0, bg - 32.0), out + 32.0, rtol=1e-5, atol=1e-3)
+    for variant in (2, 5):
+        assert torch.allclose(lt2exp(wg, ag, bg, _variant=variant), out, rtol=1e-5, atol=1e-5)
+    assert torch.allclose(lt2exp(wg, ag, bg, mode="split"), out, rtol=1e-5, atol=1e-5)

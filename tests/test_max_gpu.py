@@ -1,0 +1,197 @@
+"""matmax / vmax / vamax on the GPU: bit-exact against torch.amax / torch.max
+(the reference's own ground truth, tests/max.py:13,22,32) and against the
+brute-force NumPy rule in oracle/max_ref.py."""
+
+import itertools
+import math
+from pathlib import Path
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import max_ref
+from triturus.max import matmax, vamax, vmax
+
+pytestmark = pytest.mark.gpu
+GOLDEN = Path(__file__).resolve().parent / "golden"
+
+
+def _same(got: torch.Tensor, want: torch.Tensor):
+    got = got.cpu()
+    assert got.shape == want.shape and got.dtype == want.dtype
+    assert torch.equal(torch.isnan(got), torch.isnan(want))
+    assert torch.equal(torch.nan_to_num(got, nan=0.0), torch.nan_to_num(want, nan=0.0))
+
+
+# ---- the reference's own tests (tests/max.py), same shapes and parameters
+@pytest.mark.parametrize("block_size", [2, 32, 128])
+def test_max_vamax(dev, block_size):
+    x = torch.randn(2000)
+    m = vamax(x.to(dev), block_size=block_size)
+    assert m.shape == () and torch.all(torch.amax(x, dim=0) == m.cpu())
+
+
+@pytest.mark.parametrize("block_size", [2, 32, 128])
+def test_max_vmax(dev, block_size):
+    x = torch.randn(2000)
+    gt_m, gt_i = torch.max(x, dim=0)
+    m, i = vmax(x.to(dev), block_size=block_size)
+    assert m.shape == () and i.shape == () and i.dtype == torch.int64
+    assert torch.all(gt_m == m.cpu()) and torch.all(gt_i == i.cpu())
+
+
+@pytest.mark.parametrize("block_size,axis", itertools.product([2, 32, 128], [0, 1]))
+def test_max_matmax(dev, block_size, axis):
+    x = torch.randn(200, 150)
+    m = matmax(x.to(dev), axis=axis, block_size=block_size)
+    assert torch.all(torch.amax(x, dim=axis) == m.cpu())
+
+
+# ---- sizes, alignment, ties, special values
+@pytest.mark.parametrize("n", [1, 2, 3, 4, 5, 63, 64, 65, 255, 1023, 1025, 4099, 100003, 1 << 20, (1 << 22) + 7])
+def test_vmax_sizes(dev, n):
+    x = torch.randn(n)
+    v, i = vmax(x.to(dev))
+    rv, ri = max_ref.vmax_ref_fast(x.numpy())
+    assert (v.item(), i.item()) == (rv, ri)
+    assert vamax(x.to(dev)).item() == rv
+
+
+@pytest.mark.parametrize("offset", [1, 2, 3, 5])
+def test_vmax_unaligned_views(dev, offset):
+    base = torch.randn(5000)
+    xg = base.to(dev)[offset:]
+    gv, gi = torch.max(base[offset:], 0)
+    v, i = vmax(xg)
+    assert (v.item(), i.item()) == (gv.item(), gi.item())
+    assert vamax(xg[: 4096 - offset]).item() == base[offset:4096].max().item()
+
+
+def test_vmax_ties_go_to_the_lowest_index(dev):
+    z = np.load(GOLDEN / "vmax_ties.npz")
+    v, i = vmax(torch.from_numpy(z["x"]).to(dev))
+    assert v.item() == z["value"] and i.item() == z["index"]
+    # the maximum repeated across wavefronts, workgroups and vector lanes
+    x = torch.zeros(1 << 20)
+    for first in (0, 3, 64, 255, 256, 1027, 70001, (1 << 20) - 1):
+        y = x.clone()
+        y[first:] = 1.0
+        y[first::7] = 2.0
+        v, i = vmax(y.to(dev))
+        assert (v.item(), i.item()) == (2.0, first)
+    v, i = vmax(torch.full((300001,), -3.5).to(dev))
+    assert (v.item(), i.item()) == (-3.5, 0)
+
+
+def test_vmax_special_values(dev):
+    ninf = float("-inf")
+    v, i = vmax(torch.full((70000,), ninf).to(dev))
+    assert (v.item(), i.item()) == (ninf, 0)
+    x = torch.full((70000,), ninf)
+    x[69999] = -1e38
+    v, i = vmax(x.to(dev))
+    assert (v.item(), i.item()) == (x[69999].item(), 69999)
+    x = torch.randn(100000)
+    x[[777, 50000]] = float("inf")
+    v, i = vmax(x.to(dev))
+    assert (v.item(), i.item()) == (float("inf"), 777)
+    # NaN wins and reports the first NaN, like torch.max
+    x = torch.randn(100000)
+    x[[99999, 4242, 65000]] = float("nan")
+    x[10] = float("inf")
+    gv, gi = torch.max(x, 0)
+    v, i = vmax(x.to(dev))
+    assert math.isnan(v.item()) and math.isnan(gv.item()) and i.item() == gi.item() == 4242
+    assert math.isnan(vamax(x.to(dev)).item())
+    x = torch.tensor([0.0, -0.0, 0.0])
+    v, i = vmax(x.to(dev))
+    assert v.item() == 0.0 and i.item() == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float16, torch.bfloat16])
+def test_other_float_dtypes(dev, dtype):
+    x = torch.randn(50001).to(dtype)
+    gv, gi = torch.max(x.float() if dtype != torch.float64 else x, 0)
+    v, i = vmax(x.to(dev))
+    assert v.dtype == dtype and v.item() == gv.item() and i.item() == gi.item()
+    assert vamax(x.to(dev)).item() == gv.item()
+    m = torch.randn(301, 257).to(dtype)
+    for axis in (0, 1):
+        _same(matmax(m.to(dev), axis), torch.amax(m, axis))
+    m = torch.randn(256, 512).to(dtype)
+    for axis in (0, 1):
+        _same(matmax(m.to(dev), axis), torch.amax(m, axis))
+
+
+@pytest.mark.parametrize(
+    "shape",
+    [(1, 1), (1, 7), (7, 1), (23, 31), (64, 64), (65, 127), (200, 150), (1000, 3), (3, 1000), (2, 300000),
+     (300000, 2), (513, 1024), (4096, 256), (5, 65536), (65537, 5)],
+)
+def test_matmax_shapes(dev, shape):
+    x = torch.randn(*shape)
+    for axis in (0, 1):
+        y = matmax(x.to(dev), axis)
+        assert y.is_contiguous()
+        _same(y, torch.amax(x, axis))
+        assert np.array_equal(y.cpu().numpy(), max_ref.matmax_ref(x.numpy(), axis))
+
+
+def test_matmax_golden_and_views(dev):
+    z = np.load(GOLDEN / "matmax_small.npz")
+    x = torch.from_numpy(z["x"]).to(dev)
+    assert np.array_equal(matmax(x, 0).cpu().numpy(), z["axis0"])
+    assert np.array_equal(matmax(x, 1).cpu().numpy(), z["axis1"])
+    # contiguous but 4-byte aligned storage (a view into a larger buffer)
+    base = torch.randn(1 + 300 * 129)
+    v = base[1:].view(300, 129)
+    for axis in (0, 1):
+        _same(matmax(base.to(dev)[1:].view(300, 129), axis), torch.amax(v, axis))
+
+
+def test_matmax_special_values(dev):
+    x = torch.randn(300, 500)
+    x[5, :] = float("-inf")
+    x[:, 7] = float("-inf")
+    x[17, 33] = float("nan")
+    x[200, 400] = float("inf")
+    for axis in (0, 1):
+        _same(matmax(x.to(dev), axis), torch.amax(x, axis))
+
+
+def test_max_on_the_large_lt2exp_operand(dev):
+    """matmax along both axes and vmax with indices on the 64 x 64 x 4096 log-space
+    operand of the large lt2exp configuration, bit-exact against torch."""
+    from triturus_amd import workloads
+
+    b = workloads.c5()["b"]
+    bg = b.to(dev)
+    flat = b.view(4096, 4096)
+    for axis in (0, 1):
+        _same(matmax(bg.view(4096, 4096), axis), torch.amax(flat, axis))
+    for r in (0, 31, 63):
+        for axis in (0, 1):
+            _same(matmax(bg[r], axis), torch.amax(b[r], axis))
+    gv, gi = torch.max(b.view(-1), 0)
+    v, i = vmax(bg.view(-1))
+    assert (v.item(), i.item()) == (gv.item(), gi.item())
+    # duplicate the maximum later in the vector: the first one must still win
+    b2 = b.clone().view(-1)
+    b2[-1] = gv
+    v, i = vmax(b2.to(dev))
+    assert (v.item(), i.item()) == (gv.item(), gi.item())
+    assert vamax(bg.view(-1)).item() == gv.item()
+
+
+def test_runs_on_the_current_stream_without_synchronising(dev):
+    x = torch.randn(1 << 20)
+    xg = x.to(dev)
+    s = torch.cuda.Stream(device=dev)
+    s.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(s):
+        v, i = vmax(xg)
+        y = matmax(xg.view(1024, 1024), 1)
+    s.synchronize()
+    assert (v.item(), i.item()) == tuple(t.item() for t in torch.max(x, 0))
+    _same(y, torch.amax(x.view(1024, 1024), 1))

@@ -409,7 +409,7 @@ struct MatPlan {
     int64_t chunk;   // reduced-axis elements per partial
 };
 
-constexpr int64_t kTargetWaves = 8192;
+constexpr int64_t kTargetWaves = 4096;
 
 static MatPlan rowmax_plan(int64_t m, int64_t n, int vn) {
     // enough (row, chunk) wavefronts to fill 256 CUs; chunks of >= 2048

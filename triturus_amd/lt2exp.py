@@ -49,7 +49,9 @@ def lt2exp(
     lib = _lib.load()
 
     c = torch.empty((R, S, K), dtype=a.dtype, device=a.device)
-    w = w.view(R, S, -1)
+    # the reference flattens with w.view(batch, m, -1) (triturus/lt2exp.py:549); naming the
+    # size keeps the same RuntimeError for non-viewable w and also accepts empty tensors
+    w = w.view(R, S, I * J)
     if c.numel() == 0:
         return c
     if I * J == 0:
