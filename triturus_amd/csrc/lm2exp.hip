@@ -1,18 +1,29 @@
 // lm2exp for gfx950:  c[r,i,k] = log sum_j a[r,i,j] exp(b[r,j,k])
 //
 // A workgroup of WM x WN wavefronts owns a (32*RT*WM rows of I) x
-// (32*CT*WN columns of K) tile of c[r].  Each wavefront first takes the
-// maximum of its b columns over all J (every lane owns one column, the two
-// lane halves take alternate rows and exchange once), then walks J in chunks
-// of JC = 8*NQ:
+// (32*CT*WN columns of K) tile of c[r] and walks J in chunks of JC = 8*NQ:
 //   B operand = exp(b[j,n] - m[n]), evaluated once per (wavefront, element)
-//               straight into the VGPRs the MFMA reads: b never visits LDS;
+//               straight into the VGPRs the MFMA reads: every lane owns one
+//               column n, b never visits LDS;
 //   A operand = the a tile, staged global -> registers -> LDS (double
 //               buffered) and read back 16 bytes per lane.
 // The contraction runs on v_mfma_f32_32x32x2_f32 (IEEE fp32 in, fp32 accumulate),
 // MFMA (q,u) of lane-half h consuming j = 8q + 4h + u of the chunk.
-// Epilogue: m[n] + log(acc); acc == 0 (all -inf column, or zero row of a)
-// gives -inf, never NaN, because m is clamped to +-1e38 first.
+//
+// The shift m[n].  The result m + log(sum_j a exp(b - m)) does not depend on m,
+// only overflow/underflow do, so m need not be the exact column maximum:
+//   ONLINE = true   one sweep over b.  m starts as the maximum of the first
+//                   chunk of the column; when a later chunk's maximum exceeds
+//                   m by more than kRescaleMargin the accumulators of that
+//                   column are multiplied by exp(m_old - m_new) and m moves
+//                   up.  exp(b - m) therefore never exceeds e^kRescaleMargin,
+//                   and b is read from HBM exactly once.
+//   ONLINE = false  two sweeps, as the reference kernel does
+//                   (triturus/lm2exp.py:125-127): the exact column maximum
+//                   first (wavefront reduction: the two lane halves take
+//                   alternate rows and exchange once), then the contraction.
+// In both, m is clamped to +-1e38 (baselines/lm2exp.py:12) so an all -inf
+// column gives exp(-inf) = 0, log(0) = -inf: -inf out, never NaN.
 //
 // Replaces _ker_lm2exp, triturus/lm2exp.py:63-164.  Ragged contracted-axis
 // tails are padded with a = 0 and b = -inf (the reference pads b with 0.0,
@@ -21,6 +32,9 @@
 #include "common.hpp"
 
 namespace trt {
+
+constexpr float kRescaleMargin = 8.0f;
+constexpr int kValuPerMfma = 4;  // VALU instructions scheduled under each MFMA of the steady state
 
 struct Lm2Args {
     const float *a, *b;
@@ -31,13 +45,14 @@ struct Lm2Args {
     int64_t total_wgs, padded_wgs;
 };
 
-template <int RT, int CT, int WM, int WN, int NQ, bool VEC>
+template <int RT, int CT, int WM, int WN, int NQ, bool VEC, bool ONLINE>
 __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args p) {
     constexpr int NT = WM * WN * kWave;
     constexpr int TM = 32 * RT * WM;  // rows of I per workgroup
     constexpr int TN = 32 * CT * WN;  // columns of K per workgroup
     constexpr int JC = 8 * NQ;
-    constexpr int LDA = JC + 4;  // padded LDS row (floats)
+    constexpr int NB = 4 * NQ;   // b values per lane, column tile and chunk
+    constexpr int LDA = JC + 4;  // padded LDS row (floats): conflict-free 16-byte reads
     constexpr int F4_PER_ROW = JC / 4;
     constexpr int SLOTS = TM * F4_PER_ROW / NT;
     static_assert(TM * F4_PER_ROW % NT == 0, "tile must divide over the threads");
@@ -63,32 +78,15 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     const int wrow0 = wm * 32 * RT;  // first tile row of this wavefront
 
     int ncol[CT], ncl[CT];
+    uint32_t boff[CT];  // per-lane byte offset inside a wave-uniform row group of b
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         ncol[ct] = n0 + 32 * ct + m;
         ncl[ct] = ncol[ct] < p.K ? ncol[ct] : p.K - 1;
+        boff[ct] = ((uint32_t)(4 * h) * (uint32_t)p.sb1 + (uint32_t)ncl[ct]) * 4u;
     }
     const float *ar = p.a + (int64_t)r * p.sa0;
     const float *br = p.b + (int64_t)r * p.sb0;
-
-    // ---- sweep 1: column maxima of b over all J
-    float mx[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        float x0 = -__builtin_inff(), x1 = x0, x2 = x0, x3 = x0;
-        int j = h;
-        for (; j + 6 < p.J; j += 8) {
-            const float *bp = br + (int64_t)j * p.sb1 + ncl[ct];
-            x0 = max_nan(x0, bp[0]);
-            x1 = max_nan(x1, bp[2 * p.sb1]);
-            x2 = max_nan(x2, bp[4 * p.sb1]);
-            x3 = max_nan(x3, bp[6 * p.sb1]);
-        }
-        for (; j < p.J; j += 2) x0 = max_nan(x0, br[(int64_t)j * p.sb1 + ncl[ct]]);
-        float x = max_nan(max_nan(x0, x1), max_nan(x2, x3));
-        x = max_nan(x, __shfl_xor(x, 32, kWave));
-        mx[ct] = clamp_shift(x);
-    }
 
     floatx16 acc[RT][CT];
 #pragma unroll
@@ -98,43 +96,70 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[rt][ct][v] = 0.f;
 
+    // ---- a tile: global -> registers -> LDS.  Rows past I are clamped to the last
+    // valid row instead of masked: they only feed accumulator rows that are never
+    // stored.  Columns past J (ragged tail chunk only) must be exact zeros.
     floatx4 stage[SLOTS];
-    auto load_tile = [&](int jc) {
+    constexpr int ROWS_PER_SLOT = NT / F4_PER_ROW;
+    const int trow = tid / F4_PER_ROW;  // tile row of this thread's first slot
+    const int tc4 = tid % F4_PER_ROW;
+    uint32_t aoff[SLOTS];  // per-lane byte offsets from the (wave-uniform) tile origin
+#pragma unroll
+    for (int sidx = 0; sidx < SLOTS; ++sidx) {
+        int row = i0 + trow + sidx * ROWS_PER_SLOT;
+        row = row < p.I ? row : p.I - 1;
+        aoff[sidx] = ((uint32_t)(row - i0) * (uint32_t)p.sa1 + 4u * tc4) * 4u;
+    }
+    const float *atile0 = ar + (int64_t)i0 * p.sa1;
+    auto load_tile_full = [&](int jc) {
+        const char *org = reinterpret_cast<const char *>(atile0 + jc * JC);  // uniform
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
-            const int f = tid + sidx * NT;
-            const int row = f / F4_PER_ROW;
-            const int c4 = f % F4_PER_ROW;
-            const int j = jc * JC + 4 * c4;
-            const bool row_ok = (i0 + row) < p.I;
-            const float *src = ar + (int64_t)(i0 + row) * p.sa1 + j;
-            floatx4 v = {0.f, 0.f, 0.f, 0.f};
             if (VEC) {
-                if (row_ok && j < p.J) v = *reinterpret_cast<const floatx4 *>(src);
+                stage[sidx] = *reinterpret_cast<const floatx4 *>(org + aoff[sidx]);
             } else {
-                if (row_ok) {
-                    if (j + 0 < p.J) v[0] = src[0];
-                    if (j + 1 < p.J) v[1] = src[1];
-                    if (j + 2 < p.J) v[2] = src[2];
-                    if (j + 3 < p.J) v[3] = src[3];
-                }
+                const float *src = reinterpret_cast<const float *>(org + aoff[sidx]);
+                floatx4 v = {src[0], src[1], src[2], src[3]};
+                stage[sidx] = v;
             }
+        }
+    };
+    auto load_tile_masked = [&](int jc) {
+        const char *org = reinterpret_cast<const char *>(atile0 + jc * JC);
+        const int j = jc * JC + 4 * tc4;
+#pragma unroll
+        for (int sidx = 0; sidx < SLOTS; ++sidx) {
+            const float *src = reinterpret_cast<const float *>(org + aoff[sidx]);
+            floatx4 v = {0.f, 0.f, 0.f, 0.f};
+            if (j + 0 < p.J) v[0] = src[0];
+            if (j + 1 < p.J) v[1] = src[1];
+            if (j + 2 < p.J) v[2] = src[2];
+            if (j + 3 < p.J) v[3] = src[3];
             stage[sidx] = v;
         }
     };
     auto store_tile = [&](int buf) {
-        float *dst = at + buf * (TM * LDA);
+        float *dst = at + buf * (TM * LDA) + trow * LDA + 4 * tc4;
 #pragma unroll
-        for (int sidx = 0; sidx < SLOTS; ++sidx) {
-            const int f = tid + sidx * NT;
-            const int row = f / F4_PER_ROW;
-            const int c4 = f % F4_PER_ROW;
-            *reinterpret_cast<floatx4 *>(&dst[row * LDA + 4 * c4]) = stage[sidx];
-        }
+        for (int sidx = 0; sidx < SLOTS; ++sidx)
+            *reinterpret_cast<floatx4 *>(&dst[sidx * ROWS_PER_SLOT * LDA]) = stage[sidx];
     };
 
-    float braw[CT][4 * NQ], eb[CT][4 * NQ];
-    auto load_b = [&](int jc) {
+    // ---- b chunk: global -> registers.  Lane (h, m) takes rows 8q + 4h + u.
+    // Full chunks use a wave-uniform row pointer plus a 32-bit per-lane offset.
+    float braw[CT][NB], eb[CT][NB];
+    auto load_b_full = [&](int jc) {
+#pragma unroll
+        for (int q = 0; q < NQ; ++q)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const char *rowp = reinterpret_cast<const char *>(br + (int64_t)(jc * JC + 8 * q + u) * p.sb1);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+                    braw[ct][4 * q + u] = *reinterpret_cast<const float *>(rowp + boff[ct]);
+            }
+    };
+    auto load_b_masked = [&](int jc) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
@@ -147,78 +172,235 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
                     braw[ct][4 * q + u] = raw;
                 }
     };
-    auto exp_b = [&]() {
+    auto chunk_max = [&](int ct) {
+        float x0 = max_nan(braw[ct][0], braw[ct][1]), x1 = max_nan(braw[ct][2], braw[ct][3]);
+#pragma unroll
+        for (int e = 4; e < NB; e += 4) {
+            x0 = max_nan(x0, max_nan(braw[ct][e], braw[ct][e + 1]));
+            x1 = max_nan(x1, max_nan(braw[ct][e + 2], braw[ct][e + 3]));
+        }
+        float x = max_nan(x0, x1);
+        return max_nan(x, __shfl_xor(x, 32, kWave));
+    };
+
+    // ---- the shift and the MFMA operands of a chunk.  The work for chunk jc+1 is cut
+    // into pieces that are issued between the MFMAs of chunk jc (the matrix pipe runs
+    // a 32x32x2 MFMA for 64 cycles; the VALU work hides underneath):
+    //   plan_shift   decide the shift of the next chunk (once its loads have landed);
+    //   exp_quarter  one quarter of the exps, into the spare operand registers ebn;
+    //   commit       at the chunk boundary: rescale the accumulators if the shift
+    //                moved (rare, wave-uniform), then swap operands.
+    float mref[CT], mnext[CT], ebn[CT][NB];
+    bool moved = false;
+    auto plan_shift = [&]() {
+        moved = false;
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            mnext[ct] = mref[ct];
+            if (ONLINE) {
+                const float cm = chunk_max(ct);
+                const bool need = cm > mref[ct] + kRescaleMargin;  // false for NaN
+                mnext[ct] = need ? clamp_shift(cm) : mref[ct];
+                moved = moved || (__builtin_amdgcn_ballot_w64(need) != 0);
+            }
+        }
+    };
+    auto exp_quarter = [&](int q) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
-            for (int e = 0; e < 4 * NQ; ++e) eb[ct][e] = expf(braw[ct][e] - mx[ct]);
+            for (int u = 0; u < 4; ++u) {
+                float e = expf(braw[ct][4 * q + u] - mnext[ct]);
+                asm volatile("" : "+v"(e));  // evaluate here, under the MFMAs, not at the use
+                ebn[ct][4 * q + u] = e;
+            }
+    };
+    auto commit = [&]() {
+        if (ONLINE && moved) {
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const float sc = expf(mref[ct] - mnext[ct]);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[rt][ct][v] *= sc;
+            }
+        }
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            mref[ct] = mnext[ct];
+#pragma unroll
+            for (int e = 0; e < NB; ++e) eb[ct][e] = ebn[ct][e];
+        }
     };
 
-    const int n_jc = (p.J + JC - 1) / JC;
-    load_tile(0);
-    load_b(0);
+    const int n_full = p.J / JC;              // chunks with no ragged tail
+    const bool has_tail = (p.J % JC) != 0;    // one more, masked
+    const int n_jc = n_full + (has_tail ? 1 : 0);
+
+    if (!ONLINE) {
+        // ---- sweep 1: exact column maxima over all J
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            float x[8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) x[e] = -__builtin_inff();
+            int j = h;
+            for (; j + 14 < p.J; j += 16) {
+                const float *bp = br + (int64_t)j * p.sb1 + ncl[ct];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) x[e] = max_nan(x[e], bp[(int64_t)(2 * e) * p.sb1]);
+            }
+            for (; j < p.J; j += 2) x[0] = max_nan(x[0], br[(int64_t)j * p.sb1 + ncl[ct]]);
+            float y = max_nan(max_nan(max_nan(x[0], x[1]), max_nan(x[2], x[3])),
+                              max_nan(max_nan(x[4], x[5]), max_nan(x[6], x[7])));
+            y = max_nan(y, __shfl_xor(y, 32, kWave));
+            mref[ct] = clamp_shift(y);
+        }
+    }
+
+    // ---- prologue: chunk 0
+    if (n_full > 0) {
+        load_tile_full(0);
+        load_b_full(0);
+    } else {
+        load_tile_masked(0);
+        load_b_masked(0);
+    }
     store_tile(0);
-    exp_b();
+    if (ONLINE) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) mref[ct] = clamp_shift(chunk_max(ct));
+    }
+    plan_shift();  // chunk 0 cannot exceed its own maximum: the shift stays
+#pragma unroll
+    for (int q = 0; q < NQ; ++q) exp_quarter(q);
+    commit();
     __syncthreads();
 
-    int cur = 0;
-    for (int jc = 0; jc < n_jc; ++jc) {
-        const bool has_next = (jc + 1) < n_jc;
-        if (has_next) {
-            load_tile(jc + 1);
-            load_b(jc + 1);
-        }
-        const float *tile = at + cur * (TM * LDA) + wrow0 * LDA;
+    // Row tiles are taken two at a time so that consecutive MFMAs alternate between
+    // two accumulators while only two A fragments are live.
+    constexpr int RP = RT >= 2 ? 2 : 1;
+    auto mfma_q = [&](const float *tile, int q, int rt0) {
+        floatx4 af[RP];
 #pragma unroll
-        for (int q = 0; q < NQ; ++q) {
-            floatx4 af[RT];
+        for (int k = 0; k < RP; ++k)
+            af[k] = *reinterpret_cast<const floatx4 *>(&tile[(32 * (rt0 + k) + m) * LDA + 8 * q + 4 * h]);
 #pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-                af[rt] = *reinterpret_cast<const floatx4 *>(&tile[(32 * rt + m) * LDA + 8 * q + 4 * h]);
+        for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
             for (int u = 0; u < 4; ++u)
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
+                for (int k = 0; k < RP; ++k)
+                    acc[rt0 + k][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[k][u], eb[ct][4 * q + u],
+                                                                          acc[rt0 + k][ct], 0, 0, 0);
+    };
+    // Contract chunk `cur` while preparing the operands of the next one.
+    auto contract_and_prepare = [&](const float *tile) {
 #pragma unroll
-                    for (int rt = 0; rt < RT; ++rt)
-                        acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[rt][u], eb[ct][4 * q + u],
-                                                                          acc[rt][ct], 0, 0, 0);
+        for (int q = 0; q < NQ; ++q) {
+#pragma unroll
+            for (int rt0 = 0; rt0 < RT; rt0 += RP) mfma_q(tile, q, rt0);
+            // The loads of the next chunk were issued just before this block: leave the
+            // first half of the block to hide their latency, prepare in the second half.
+            constexpr int QH = NQ / 2;
+            if (q == QH) plan_shift();
+            if (q >= QH) {
+                exp_quarter(2 * (q - QH));
+                exp_quarter(2 * (q - QH) + 1);
+            }
+            // issue order inside this piece: A fragments first, then the VALU work
+            // spread evenly under the MFMAs
+#pragma unroll
+            for (int g = 0; g < RT / RP; ++g) {
+                __builtin_amdgcn_sched_group_barrier(0x100, RP, 0);  // LDS reads
+#pragma unroll
+                for (int i = 0; i < 4 * RP * CT; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
+                    if (q >= QH) __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
         }
-        if (has_next) {
-            store_tile(cur ^ 1);
-            exp_b();
-        }
+    };
+
+    // ---- steady state: prefetch chunk jc+1 unconditionally, contract chunk jc, then
+    // consume the prefetch before the back edge; the ragged tail and the last chunk
+    // are peeled so the loop body carries no masks.
+    int cur = 0;
+    int jc = 0;
+    for (; jc + 1 < n_full; ++jc) {
+        load_tile_full(jc + 1);
+        load_b_full(jc + 1);
+        contract_and_prepare(at + cur * (TM * LDA) + wrow0 * LDA);
+        store_tile(cur ^ 1);
+        commit();
+        __syncthreads();
+        cur ^= 1;
+    }
+    if (jc + 1 < n_jc) {  // the next chunk is the masked tail
+        load_tile_masked(jc + 1);
+        load_b_masked(jc + 1);
+        contract_and_prepare(at + cur * (TM * LDA) + wrow0 * LDA);
+        store_tile(cur ^ 1);
+        commit();
         __syncthreads();
         cur ^= 1;
     }
 
-    // ---- epilogue: register v of lane (h, m) holds row 8*(v/4) + 4*h + v%4, column m
+    // ---- last chunk, row-tile major, with the epilogue of each finished pair of row
+    // tiles issued under the MFMAs of the next pair.  Register v of lane (h, m) holds
+    // row 8*(v/4) + 4*h + v%4, column m of its 32 x 32 tile.
     float *cr = p.c + (int64_t)r * p.sc0;
+    auto store_rows = [&](int rt0, int part) {  // a quarter of the rows of one pair
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        if (ncol[ct] >= p.K) continue;
+        for (int ct = 0; ct < CT; ++ct) {
+            if (ncol[ct] >= p.K) continue;
 #pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
+            for (int k = 0; k < RP; ++k)
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int row = i0 + wrow0 + 32 * rt + 8 * (v / 4) + 4 * h + (v % 4);
-                if (row < p.I) cr[(int64_t)row * p.sc1 + ncol[ct]] = mx[ct] + logf(acc[rt][ct][v]);
+                for (int vv = 0; vv < 4; ++vv) {
+                    const int v = 4 * part + vv;
+                    const int row = i0 + wrow0 + 32 * (rt0 + k) + 8 * (v / 4) + 4 * h + (v % 4);
+                    if (row < p.I)
+                        cr[(int64_t)row * p.sc1 + ncol[ct]] = mref[ct] + logf(acc[rt0 + k][ct][v]);
+                }
+        }
+    };
+    {
+        const float *tile = at + cur * (TM * LDA) + wrow0 * LDA;
+#pragma unroll
+        for (int rt0 = 0; rt0 < RT; rt0 += RP) {
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                mfma_q(tile, q, rt0);
+                if (rt0 > 0) {
+#pragma unroll
+                    for (int part = q * 4 / NQ; part < (q + 1) * 4 / NQ; ++part) store_rows(rt0 - RP, part);
+                }
             }
+        }
+#pragma unroll
+        for (int part = 0; part < 4; ++part) store_rows(RT - RP, part);
     }
 }
 
 // ------------------------------------------------------------------ host
 struct Lm2Variant {
     int rt, ct, wm, wn, nq;
+    bool online;
 };
+// variant ids are 1-based in the C ABI (0 = choose by shape)
 static const Lm2Variant kVariants[] = {
-    {8, 1, 1, 8, 4},  // 256 x 256 tile, 8 waves each 256 x 32
-    {4, 2, 2, 4, 4},  // 256 x 256 tile, 8 waves each 128 x 64
-    {8, 1, 1, 4, 4},  // 256 x 128 tile, 4 waves each 256 x 32
-    {4, 1, 1, 4, 4},  // 128 x 128 tile, 4 waves each 128 x 32
-    {2, 2, 1, 4, 4},  // 64 x 256 tile, 4 waves each 64 x 64
-    {2, 1, 1, 4, 4},  // 64 x 128 tile
-    {1, 1, 1, 4, 4},  // 32 x 128 tile
+    {8, 1, 1, 8, 4, true},   // 1: 256 x 256 tile, 8 waves each 256 x 32, one sweep
+    {8, 1, 1, 4, 4, true},   // 2: 256 x 128 tile, 4 waves each 256 x 32
+    {8, 1, 1, 8, 4, false},  // 3: as 1, two sweeps (exact column maximum first)
+    {4, 2, 2, 4, 4, true},   // 4: 256 x 256 tile, 8 waves each 128 x 64
+    {4, 1, 1, 4, 4, true},   // 5: 128 x 128 tile
+    {2, 2, 1, 4, 4, true},   // 6: 64 x 256 tile
+    {2, 1, 1, 4, 4, true},   // 7: 64 x 128 tile
+    {1, 1, 1, 4, 4, true},   // 8: 32 x 128 tile
+    {2, 1, 1, 4, 4, false},  // 9: as 7, two sweeps
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be opted into per kernel
@@ -227,39 +409,34 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     (void)J;
     int v;
     if (I > 128) v = 0;
-    else if (I > 64) v = 3;
-    else if (I > 32) v = 4;
-    else v = 6;
-    // fall back to narrower column tiles when the grid would leave CUs idle
-    if (v == 0 && R * ceil_div(I, 256) * ceil_div(K, 256) < 256) v = 2;
-    if (v == 4 && R * ceil_div(I, 64) * ceil_div(K, 256) < 256) v = 5;
+    else if (I > 64) v = 4;
+    else if (I > 32) v = 5;
+    else v = 7;
+    // narrower column tiles when the wide ones would leave CUs idle
+    if (v == 0 && R * ceil_div(I, 256) * ceil_div(K, 256) < 256) v = 1;
+    if (v == 5 && R * ceil_div(I, 64) * ceil_div(K, 256) < 256) v = 6;
     return v;
 }
 
-template <int RT, int CT, int WM, int WN, int NQ>
-static int launch_v(const Lm2Args &args, bool vec, hipStream_t stream) {
+template <int RT, int CT, int WM, int WN, int NQ, bool VEC, bool ONLINE>
+static int launch_k(const Lm2Args &args, hipStream_t stream) {
     constexpr int TM = 32 * RT * WM;
     constexpr int LDA = 8 * NQ + 4;
     constexpr size_t lds = (size_t)2 * TM * LDA * sizeof(float);
-    hipError_t e;
-    if (vec) {
-        auto k = lm2exp_kernel<RT, CT, WM, WN, NQ, true>;
-        if (lds > kDefaultLdsLimit) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return (int)e;
-        }
-        hipLaunchKernelGGL(k, dim3((unsigned)args.padded_wgs), dim3(WM * WN * kWave), lds, stream, args);
-    } else {
-        auto k = lm2exp_kernel<RT, CT, WM, WN, NQ, false>;
-        if (lds > kDefaultLdsLimit) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(k),
-                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return (int)e;
-        }
-        hipLaunchKernelGGL(k, dim3((unsigned)args.padded_wgs), dim3(WM * WN * kWave), lds, stream, args);
+    auto k = lm2exp_kernel<RT, CT, WM, WN, NQ, VEC, ONLINE>;
+    if (lds > kDefaultLdsLimit) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
     }
+    hipLaunchKernelGGL(k, dim3((unsigned)args.padded_wgs), dim3(WM * WN * kWave), lds, stream, args);
     return (int)hipGetLastError();
+}
+
+template <int RT, int CT, int WM, int WN, int NQ, bool ONLINE>
+static int launch_v(const Lm2Args &args, bool vec, hipStream_t stream) {
+    return vec ? launch_k<RT, CT, WM, WN, NQ, true, ONLINE>(args, stream)
+               : launch_k<RT, CT, WM, WN, NQ, false, ONLINE>(args, stream);
 }
 
 }  // namespace trt
@@ -279,6 +456,8 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         if (sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || I >= lim || J >= lim || K >= lim) return TRT_E_RANGE;
+    // per-lane byte offsets into b (4 rows + a column) and into an a tile (256 rows) are 32-bit
+    if (4 * sb[1] + K >= ((int64_t)1 << 30) || 256 * sa[1] + J >= ((int64_t)1 << 30)) return TRT_E_RANGE;
 
     const int v = (variant >= 1) ? variant - 1 : choose_variant(R, I, J, K);
     const Lm2Variant &vr = kVariants[v];
@@ -297,12 +476,14 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (v) {
-        case 0: return launch_v<8, 1, 1, 8, 4>(args, vec, s);
-        case 1: return launch_v<4, 2, 2, 4, 4>(args, vec, s);
-        case 2: return launch_v<8, 1, 1, 4, 4>(args, vec, s);
-        case 3: return launch_v<4, 1, 1, 4, 4>(args, vec, s);
-        case 4: return launch_v<2, 2, 1, 4, 4>(args, vec, s);
-        case 5: return launch_v<2, 1, 1, 4, 4>(args, vec, s);
-        default: return launch_v<1, 1, 1, 4, 4>(args, vec, s);
+        case 0: return launch_v<8, 1, 1, 8, 4, true>(args, vec, s);
+        case 1: return launch_v<8, 1, 1, 4, 4, true>(args, vec, s);
+        case 2: return launch_v<8, 1, 1, 8, 4, false>(args, vec, s);
+        case 3: return launch_v<4, 2, 2, 4, 4, true>(args, vec, s);
+        case 4: return launch_v<4, 1, 1, 4, 4, true>(args, vec, s);
+        case 5: return launch_v<2, 2, 1, 4, 4, true>(args, vec, s);
+        case 6: return launch_v<2, 1, 1, 4, 4, true>(args, vec, s);
+        case 7: return launch_v<1, 1, 1, 4, 4, true>(args, vec, s);
+        default: return launch_v<2, 1, 1, 4, 4, false>(args, vec, s);
     }
 }

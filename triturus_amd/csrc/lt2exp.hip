@@ -167,21 +167,8 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
         store_tile(0);
         __syncthreads();
 
-        int cur = 0;
-        for (; it < it_end; ++it) {
-            int ni = i + 1, njc = jc;
-            if (ni == p.I) {
-                ni = 0;
-                njc = jc + 1;
-            }
-            const bool has_next = (it + 1) < it_end;
-            if (has_next) {
-                load_tile(ni, njc);
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct) ea_raw[ct] = ar[(int64_t)ni * p.sa1 + ncl[ct]];
-            }
-            // ---- MFMA block over this (i, j-chunk)
-            const float *tile = wt[cur];
+        // ---- MFMA block over one (i, j-chunk): 4*NQ*RT*CT MFMAs per wavefront
+        auto mfma_block = [&](const float *tile) {
 #pragma unroll
             for (int q = 0; q < NQ; ++q) {
                 floatx4 af[RT];
@@ -199,17 +186,32 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
                     }
                 }
             }
-            if (has_next) {
-                store_tile(cur ^ 1);
-                if (njc != jc) load_eb(njc);
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct) ea[ct] = expf(ea_raw[ct] - ma[ct]);
+        };
+
+        // Steady state: every iteration prefetches the next tile unconditionally and
+        // consumes it before the back edge (no load is ever left in flight across the
+        // loop header); the last iteration is peeled.
+        int cur = 0;
+        for (; it + 1 < it_end; ++it) {
+            int ni = i + 1, njc = jc;
+            if (ni == p.I) {
+                ni = 0;
+                njc = jc + 1;
             }
+            load_tile(ni, njc);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) ea_raw[ct] = ar[(int64_t)ni * p.sa1 + ncl[ct]];
+            mfma_block(wt[cur]);
+            store_tile(cur ^ 1);
+            if (njc != jc) load_eb(njc);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) ea[ct] = expf(ea_raw[ct] - ma[ct]);
             __syncthreads();
             cur ^= 1;
             i = ni;
             jc = njc;
         }
+        mfma_block(wt[cur]);
     }
 
     // ---- epilogue.  D layout of 32x32x2: register v of lane (h, m) holds
