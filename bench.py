@@ -234,7 +234,7 @@ def main() -> int:
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
             "traffic": MEASURED_TRAFFIC_BYTES["lt2exp_c5"],
-            "kernel": "lt2exp_kernel<2,2,8,4,vec,unsplit>",
+            "kernel": "lt2exp_kernel<RT=2,CT=1,NQ=4,NWAVES=4,VEC,unsplit>",
         },
     }
 

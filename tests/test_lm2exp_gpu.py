@@ -19,7 +19,7 @@ from triturus_amd import _lib, workloads
 pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
-N_VARIANTS = 9
+N_VARIANTS = 10
 
 
 def _check(out, a, b, **kw):
@@ -193,7 +193,7 @@ def test_benchmark_configuration_c3_full_size(dev):
         worst = max(worst, r["worst_err_over_tol"])
     # size-independent properties on the whole output
     assert torch.all(out <= bg.amax(1, keepdim=True) + 1e-3)
-    for variant in (2, 3, 4):  # other tile shapes, and the two-sweep (exact maximum) kernel
+    for variant in (2, 3, 5, 10):  # other tile shapes, and the two-sweep (exact maximum) kernels
         alt = lm2exp(ag, bg, _variant=variant)
         assert torch.allclose(alt, out, rtol=1e-5, atol=1e-5)
     shifted = lm2exp(ag, bg + 128.0)

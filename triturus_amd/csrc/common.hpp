@@ -44,4 +44,48 @@ __device__ __forceinline__ float max_nan(float a, float b) {
     return (a > b || a != a) ? a : b;
 }
 
+// ---- buffer addressing: a 128-bit resource (base, byte extent) in scalar registers,
+// a 32-bit per-lane byte offset and a wave-uniform scalar byte offset.  No vector ALU
+// instruction is spent on the address, and accesses past the extent are dropped
+// (loads return 0) by the hardware.
+typedef uint32_t uintx4 __attribute__((ext_vector_type(4)));
+constexpr uint32_t kRsrcFlags = 0x00020000;  // raw buffer, 32-bit data format
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, bytes, kRsrcFlags);
+}
+__device__ __forceinline__ float buf_load_f32(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0));
+}
+__device__ __forceinline__ floatx4 buf_load_f32x4(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0));
+}
+__device__ __forceinline__ void buf_store_f32(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, voff, soff, 0);
+}
+
+// max of three without NaN canonicalisation moves (a NaN operand is ignored, which is
+// what the callers want: see the kernels).
+__device__ __forceinline__ float max3_raw(float a, float b, float c) {
+    float d;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(d) : "v"(a), "v"(b), "v"(c));
+    return d;
+}
+
+constexpr float kLog2e = 1.44269504088896340736f;
+constexpr float kLn2 = 0.69314718055994530942f;
+
+// exp(x) for a shifted log-value x = b - m (x <= ~8, possibly -inf or NaN) as one
+// multiply and the hardware 2^t instruction.  Relative error <= 2^-23 |x log2(e)| + 1 ulp:
+// exact near the maximum, where the sum is decided; results below 2^-126 flush to 0.
+// The subtraction b - m is done by the caller in plain fp32 (exact for b close to m);
+// folding it into an fma with a pre-scaled m * log2(e) would turn the rounding of that
+// product into an absolute exponent error of |m| 2^-24, fatal for |m| >~ 1e9.
+__device__ __forceinline__ float exp_shifted(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
+
+// m + log(s) from the hardware log2: log2(0) = -inf gives -inf (m is finite), NaN stays NaN.
+__device__ __forceinline__ float log_plus(float s, float m) {
+    return __builtin_fmaf(__builtin_amdgcn_logf(s), kLn2, m);
+}
+
 }  // namespace trt

@@ -34,7 +34,6 @@
 namespace trt {
 
 constexpr float kRescaleMargin = 8.0f;
-constexpr int kValuPerMfma = 4;  // VALU instructions scheduled under each MFMA of the steady state
 
 struct Lm2Args {
     const float *a, *b;
@@ -61,10 +60,13 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
 
     const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
     if (L >= p.total_wgs) return;
-    const int nt = (int)(L % p.n_tiles);
+    // The tile coordinates are wave-uniform; the 64-bit divisions below are expanded on
+    // the vector ALU, so pin the results back into scalar registers (they feed buffer
+    // resources and scalar offsets).
     const int64_t rest = L / p.n_tiles;
-    const int itile = (int)(rest % p.i_tiles);
-    const int r = (int)(rest / p.i_tiles);
+    const int nt = __builtin_amdgcn_readfirstlane((int)(L % p.n_tiles));
+    const int itile = __builtin_amdgcn_readfirstlane((int)(rest % p.i_tiles));
+    const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.i_tiles));
 
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
@@ -111,15 +113,21 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         aoff[sidx] = ((uint32_t)(row - i0) * (uint32_t)p.sa1 + 4u * tc4) * 4u;
     }
     const float *atile0 = ar + (int64_t)i0 * p.sa1;
+    const int arows = (p.I - i0) < TM ? (p.I - i0) : TM;  // valid rows of this tile
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        make_rsrc(atile0, (uint32_t)(((int64_t)(arows - 1) * p.sa1 + p.J) * 4));
     auto load_tile_full = [&](int jc) {
-        const char *org = reinterpret_cast<const char *>(atile0 + jc * JC);  // uniform
+        const uint32_t soff = (uint32_t)(jc * JC) * 4u;  // wave-uniform
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
             if (VEC) {
-                stage[sidx] = *reinterpret_cast<const floatx4 *>(org + aoff[sidx]);
+                stage[sidx] = buf_load_f32x4(a_rsrc, aoff[sidx], soff);
             } else {
-                const float *src = reinterpret_cast<const float *>(org + aoff[sidx]);
-                floatx4 v = {src[0], src[1], src[2], src[3]};
+                floatx4 v;
+                v[0] = buf_load_f32(a_rsrc, aoff[sidx], soff);
+                v[1] = buf_load_f32(a_rsrc, aoff[sidx], soff + 4);
+                v[2] = buf_load_f32(a_rsrc, aoff[sidx], soff + 8);
+                v[3] = buf_load_f32(a_rsrc, aoff[sidx], soff + 12);
                 stage[sidx] = v;
             }
         }
@@ -146,17 +154,21 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     };
 
     // ---- b chunk: global -> registers.  Lane (h, m) takes rows 8q + 4h + u.
-    // Full chunks use a wave-uniform row pointer plus a 32-bit per-lane offset.
+    // Full chunks use a wave-uniform row pointer (SGPRs) plus a 32-bit per-lane offset.
+    // FP32 MFMA and the vector ALU do not execute concurrently on this hardware, so
+    // every VALU instruction in the steady state costs matrix throughput: addresses
+    // are kept in scalar registers and exp/log use the bare hardware instructions.
     float braw[CT][NB], eb[CT][NB];
+    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(br, (uint32_t)(((int64_t)(p.J - 1) * p.sb1 + p.K) * 4));
+    const uint32_t b_row_bytes = (uint32_t)p.sb1 * 4u;
     auto load_b_full = [&](int jc) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q)
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                const char *rowp = reinterpret_cast<const char *>(br + (int64_t)(jc * JC + 8 * q + u) * p.sb1);
+                const uint32_t soff = (uint32_t)(jc * JC + 8 * q + u) * b_row_bytes;  // wave-uniform
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
-                    braw[ct][4 * q + u] = *reinterpret_cast<const float *>(rowp + boff[ct]);
+                for (int ct = 0; ct < CT; ++ct) braw[ct][4 * q + u] = buf_load_f32(b_rsrc, boff[ct], soff);
             }
     };
     auto load_b_masked = [&](int jc) {
@@ -172,65 +184,38 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
                     braw[ct][4 * q + u] = raw;
                 }
     };
+    // Maximum of the chunk's column.  A NaN need not survive here: exp(NaN - m) is NaN
+    // for any m and poisons the whole output column through the MFMA, which is what
+    // the torch recipe gives for a NaN in b.
     auto chunk_max = [&](int ct) {
-        float x0 = max_nan(braw[ct][0], braw[ct][1]), x1 = max_nan(braw[ct][2], braw[ct][3]);
+        float x = max3_raw(braw[ct][0], braw[ct][1], braw[ct][2]);
 #pragma unroll
-        for (int e = 4; e < NB; e += 4) {
-            x0 = max_nan(x0, max_nan(braw[ct][e], braw[ct][e + 1]));
-            x1 = max_nan(x1, max_nan(braw[ct][e + 2], braw[ct][e + 3]));
-        }
-        float x = max_nan(x0, x1);
-        return max_nan(x, __shfl_xor(x, 32, kWave));
+        for (int e = 3; e + 1 < NB; e += 2) x = max3_raw(x, braw[ct][e], braw[ct][e + 1]);
+        x = max3_raw(x, braw[ct][NB - 1], braw[ct][NB - 1]);
+        return max3_raw(x, __shfl_xor(x, 32, kWave), x);
     };
 
-    // ---- the shift and the MFMA operands of a chunk.  The work for chunk jc+1 is cut
-    // into pieces that are issued between the MFMAs of chunk jc (the matrix pipe runs
-    // a 32x32x2 MFMA for 64 cycles; the VALU work hides underneath):
-    //   plan_shift   decide the shift of the next chunk (once its loads have landed);
-    //   exp_quarter  one quarter of the exps, into the spare operand registers ebn;
-    //   commit       at the chunk boundary: rescale the accumulators if the shift
-    //                moved (rare, wave-uniform), then swap operands.
-    float mref[CT], mnext[CT], ebn[CT][NB];
-    bool moved = false;
-    auto plan_shift = [&]() {
-        moved = false;
+    float mref[CT];
+    // Turn the raw chunk in braw into MFMA operands in eb, moving the shift first if this
+    // chunk towers over it (rare, wave-uniform branch).
+    auto shift_and_exp = [&]() {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
-            mnext[ct] = mref[ct];
             if (ONLINE) {
                 const float cm = chunk_max(ct);
-                const bool need = cm > mref[ct] + kRescaleMargin;  // false for NaN
-                mnext[ct] = need ? clamp_shift(cm) : mref[ct];
-                moved = moved || (__builtin_amdgcn_ballot_w64(need) != 0);
+                const bool need = cm > mref[ct] + kRescaleMargin;
+                if (__builtin_amdgcn_ballot_w64(need) != 0) {
+                    const float mnew = need ? clamp_shift(cm) : mref[ct];
+                    const float sc = exp_shifted(mref[ct] - mnew);
+#pragma unroll
+                    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[rt][ct][v] *= sc;
+                    mref[ct] = mnew;
+                }
             }
-        }
-    };
-    auto exp_quarter = [&](int q) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-            for (int u = 0; u < 4; ++u) {
-                float e = expf(braw[ct][4 * q + u] - mnext[ct]);
-                asm volatile("" : "+v"(e));  // evaluate here, under the MFMAs, not at the use
-                ebn[ct][4 * q + u] = e;
-            }
-    };
-    auto commit = [&]() {
-        if (ONLINE && moved) {
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) {
-                const float sc = expf(mref[ct] - mnext[ct]);
-#pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[rt][ct][v] *= sc;
-            }
-        }
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            mref[ct] = mnext[ct];
-#pragma unroll
-            for (int e = 0; e < NB; ++e) eb[ct][e] = ebn[ct][e];
+            for (int e = 0; e < NB; ++e) eb[ct][e] = exp_shifted(braw[ct][e] - mref[ct]);
         }
     };
 
@@ -272,55 +257,30 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) mref[ct] = clamp_shift(chunk_max(ct));
     }
-    plan_shift();  // chunk 0 cannot exceed its own maximum: the shift stays
-#pragma unroll
-    for (int q = 0; q < NQ; ++q) exp_quarter(q);
-    commit();
+    shift_and_exp();
     __syncthreads();
 
     // Row tiles are taken two at a time so that consecutive MFMAs alternate between
     // two accumulators while only two A fragments are live.
     constexpr int RP = RT >= 2 ? 2 : 1;
-    auto mfma_q = [&](const float *tile, int q, int rt0) {
-        floatx4 af[RP];
-#pragma unroll
-        for (int k = 0; k < RP; ++k)
-            af[k] = *reinterpret_cast<const floatx4 *>(&tile[(32 * (rt0 + k) + m) * LDA + 8 * q + 4 * h]);
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
-#pragma unroll
-            for (int u = 0; u < 4; ++u)
-#pragma unroll
-                for (int k = 0; k < RP; ++k)
-                    acc[rt0 + k][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[k][u], eb[ct][4 * q + u],
-                                                                          acc[rt0 + k][ct], 0, 0, 0);
-    };
-    // Contract chunk `cur` while preparing the operands of the next one.
-    auto contract_and_prepare = [&](const float *tile) {
+    auto mfma_block = [&](const float *tile) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
 #pragma unroll
-            for (int rt0 = 0; rt0 < RT; rt0 += RP) mfma_q(tile, q, rt0);
-            // The loads of the next chunk were issued just before this block: leave the
-            // first half of the block to hide their latency, prepare in the second half.
-            constexpr int QH = NQ / 2;
-            if (q == QH) plan_shift();
-            if (q >= QH) {
-                exp_quarter(2 * (q - QH));
-                exp_quarter(2 * (q - QH) + 1);
-            }
-            // issue order inside this piece: A fragments first, then the VALU work
-            // spread evenly under the MFMAs
+            for (int rt0 = 0; rt0 < RT; rt0 += RP) {
+                floatx4 af[RP];
 #pragma unroll
-            for (int g = 0; g < RT / RP; ++g) {
-                __builtin_amdgcn_sched_group_barrier(0x100, RP, 0);  // LDS reads
+                for (int k = 0; k < RP; ++k)
+                    af[k] = *reinterpret_cast<const floatx4 *>(&tile[(32 * (rt0 + k) + m) * LDA + 8 * q + 4 * h]);
 #pragma unroll
-                for (int i = 0; i < 4 * RP * CT; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // one MFMA
-                    if (q >= QH) __builtin_amdgcn_sched_group_barrier(0x002, kValuPerMfma, 0);
-                }
+                for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+                    for (int u = 0; u < 4; ++u)
+#pragma unroll
+                        for (int k = 0; k < RP; ++k)
+                            acc[rt0 + k][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(
+                                af[k][u], eb[ct][4 * q + u], acc[rt0 + k][ct], 0, 0, 0);
             }
-            __builtin_amdgcn_sched_barrier(0);
         }
     };
 
@@ -332,56 +292,45 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     for (; jc + 1 < n_full; ++jc) {
         load_tile_full(jc + 1);
         load_b_full(jc + 1);
-        contract_and_prepare(at + cur * (TM * LDA) + wrow0 * LDA);
+        __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block, not sunk into it
+        mfma_block(at + cur * (TM * LDA) + wrow0 * LDA);
         store_tile(cur ^ 1);
-        commit();
+        shift_and_exp();
         __syncthreads();
         cur ^= 1;
     }
     if (jc + 1 < n_jc) {  // the next chunk is the masked tail
         load_tile_masked(jc + 1);
         load_b_masked(jc + 1);
-        contract_and_prepare(at + cur * (TM * LDA) + wrow0 * LDA);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma_block(at + cur * (TM * LDA) + wrow0 * LDA);
         store_tile(cur ^ 1);
-        commit();
+        shift_and_exp();
         __syncthreads();
         cur ^= 1;
     }
+    mfma_block(at + cur * (TM * LDA) + wrow0 * LDA);
 
-    // ---- last chunk, row-tile major, with the epilogue of each finished pair of row
-    // tiles issued under the MFMAs of the next pair.  Register v of lane (h, m) holds
-    // row 8*(v/4) + 4*h + v%4, column m of its 32 x 32 tile.
-    float *cr = p.c + (int64_t)r * p.sc0;
-    auto store_rows = [&](int rt0, int part) {  // a quarter of the rows of one pair
+    // ---- epilogue: c = m + log(acc).  Register v of lane (h, m) holds row
+    // 8*(v/4) + 4*h + v%4, column m of its 32 x 32 tile; the row part of the address
+    // is wave-uniform apart from the lane half, so it lives in scalar registers.
+    // Rows past I fall outside the buffer extent and are dropped by the hardware.
+    const int crows = p.I - (i0 + wrow0);  // valid rows below this wavefront's first row
+    const __amdgpu_buffer_rsrc_t c_rsrc =
+        make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)(i0 + wrow0) * p.sc1,
+                  crows > 0 ? (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4) : 0u);
+    const uint32_t c_row_bytes = (uint32_t)p.sc1 * 4u;
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            if (ncol[ct] >= p.K) continue;
+    for (int ct = 0; ct < CT; ++ct) {
+        if (ncol[ct] >= p.K) continue;
+        const uint32_t co = ((uint32_t)(4 * h) * (uint32_t)p.sc1 + (uint32_t)ncol[ct]) * 4u;
 #pragma unroll
-            for (int k = 0; k < RP; ++k)
+        for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-                for (int vv = 0; vv < 4; ++vv) {
-                    const int v = 4 * part + vv;
-                    const int row = i0 + wrow0 + 32 * (rt0 + k) + 8 * (v / 4) + 4 * h + (v % 4);
-                    if (row < p.I)
-                        cr[(int64_t)row * p.sc1 + ncol[ct]] = mref[ct] + logf(acc[rt0 + k][ct][v]);
-                }
-        }
-    };
-    {
-        const float *tile = at + cur * (TM * LDA) + wrow0 * LDA;
-#pragma unroll
-        for (int rt0 = 0; rt0 < RT; rt0 += RP) {
-#pragma unroll
-            for (int q = 0; q < NQ; ++q) {
-                mfma_q(tile, q, rt0);
-                if (rt0 > 0) {
-#pragma unroll
-                    for (int part = q * 4 / NQ; part < (q + 1) * 4 / NQ; ++part) store_rows(rt0 - RP, part);
-                }
+            for (int v = 0; v < 16; ++v) {
+                const uint32_t trow = 32 * rt + 8 * (v / 4) + (v % 4);  // + 4h in the lane offset
+                buf_store_f32(log_plus(acc[rt][ct][v], mref[ct]), c_rsrc, co, trow * c_row_bytes);
             }
-        }
-#pragma unroll
-        for (int part = 0; part < 4; ++part) store_rows(RT - RP, part);
     }
 }
 
@@ -392,30 +341,28 @@ struct Lm2Variant {
 };
 // variant ids are 1-based in the C ABI (0 = choose by shape)
 static const Lm2Variant kVariants[] = {
-    {8, 1, 1, 8, 4, true},   // 1: 256 x 256 tile, 8 waves each 256 x 32, one sweep
-    {8, 1, 1, 4, 4, true},   // 2: 256 x 128 tile, 4 waves each 256 x 32
-    {8, 1, 1, 8, 4, false},  // 3: as 1, two sweeps (exact column maximum first)
-    {4, 2, 2, 4, 4, true},   // 4: 256 x 256 tile, 8 waves each 128 x 64
-    {4, 1, 1, 4, 4, true},   // 5: 128 x 128 tile
+    {4, 1, 1, 4, 4, true},   // 1: 128 x 128 tile, 4 waves each 128 x 32, one sweep (3 waves/SIMD)
+    {4, 1, 1, 8, 4, true},   // 2: 128 x 256 tile, 8 waves each 128 x 32
+    {8, 1, 1, 8, 4, true},   // 3: 256 x 256 tile, 8 waves each 256 x 32
+    {8, 1, 1, 4, 4, true},   // 4: 256 x 128 tile, 4 waves each 256 x 32
+    {8, 1, 1, 8, 4, false},  // 5: as 3, two sweeps (exact column maximum first)
     {2, 2, 1, 4, 4, true},   // 6: 64 x 256 tile
     {2, 1, 1, 4, 4, true},   // 7: 64 x 128 tile
     {1, 1, 1, 4, 4, true},   // 8: 32 x 128 tile
     {2, 1, 1, 4, 4, false},  // 9: as 7, two sweeps
+    {4, 1, 1, 4, 4, false},  // 10: as 1, two sweeps
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be opted into per kernel
 
+// Measured on MI355X at R=64, I=J=256, K=4096: the 128-row tiles (64 accumulator
+// registers, 3-4 wavefronts per SIMD) beat the 256-row tiles (128 accumulator
+// registers, 2 per SIMD) although b is then exponentiated once per row tile.
 static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
-    (void)J;
-    int v;
-    if (I > 128) v = 0;
-    else if (I > 64) v = 4;
-    else if (I > 32) v = 5;
-    else v = 7;
-    // narrower column tiles when the wide ones would leave CUs idle
-    if (v == 0 && R * ceil_div(I, 256) * ceil_div(K, 256) < 256) v = 1;
-    if (v == 5 && R * ceil_div(I, 64) * ceil_div(K, 256) < 256) v = 6;
-    return v;
+    (void)R; (void)J; (void)K;
+    if (I > 64) return 0;
+    if (I > 32) return 6;
+    return 7;
 }
 
 template <int RT, int CT, int WM, int WN, int NQ, bool VEC, bool ONLINE>
@@ -456,8 +403,10 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         if (sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || I >= lim || J >= lim || K >= lim) return TRT_E_RANGE;
-    // per-lane byte offsets into b (4 rows + a column) and into an a tile (256 rows) are 32-bit
-    if (4 * sb[1] + K >= ((int64_t)1 << 30) || 256 * sa[1] + J >= ((int64_t)1 << 30)) return TRT_E_RANGE;
+    // byte offsets inside one batch slab of a, b and c are 32-bit (buffer addressing)
+    if (J * sb[1] + K >= ((int64_t)1 << 30) || I * sa[1] + J >= ((int64_t)1 << 30) ||
+        I * sc[1] + K >= ((int64_t)1 << 30))
+        return TRT_E_RANGE;
 
     const int v = (variant >= 1) ? variant - 1 : choose_variant(R, I, J, K);
     const Lm2Variant &vr = kVariants[v];
@@ -476,14 +425,15 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (v) {
-        case 0: return launch_v<8, 1, 1, 8, 4, true>(args, vec, s);
-        case 1: return launch_v<8, 1, 1, 4, 4, true>(args, vec, s);
-        case 2: return launch_v<8, 1, 1, 8, 4, false>(args, vec, s);
-        case 3: return launch_v<4, 2, 2, 4, 4, true>(args, vec, s);
-        case 4: return launch_v<4, 1, 1, 4, 4, true>(args, vec, s);
+        case 0: return launch_v<4, 1, 1, 4, 4, true>(args, vec, s);
+        case 1: return launch_v<4, 1, 1, 8, 4, true>(args, vec, s);
+        case 2: return launch_v<8, 1, 1, 8, 4, true>(args, vec, s);
+        case 3: return launch_v<8, 1, 1, 4, 4, true>(args, vec, s);
+        case 4: return launch_v<8, 1, 1, 8, 4, false>(args, vec, s);
         case 5: return launch_v<2, 2, 1, 4, 4, true>(args, vec, s);
         case 6: return launch_v<2, 1, 1, 4, 4, true>(args, vec, s);
         case 7: return launch_v<1, 1, 1, 4, 4, true>(args, vec, s);
-        default: return launch_v<2, 1, 1, 4, 4, false>(args, vec, s);
+        case 8: return launch_v<2, 1, 1, 4, 4, false>(args, vec, s);
+        default: return launch_v<4, 1, 1, 4, 4, false>(args, vec, s);
     }
 }

