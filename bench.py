@@ -32,9 +32,11 @@ import torch
 PEAK_FP32_MFMA_TFLOPS = 157.3  # 256 CU x 4 SIMD x 64 flop/clk x 2.4 GHz
 PEAK_HBM_GBPS = 8000.0
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE), scaled by
-# the same counters over trt_copy_bytes of known size; None until measured.
-MEASURED_TRAFFIC_BYTES = {"lt2exp_c5": None, "lm2exp_c3": None}
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, then WRITE_SIZE, one run
+# each over `bench.py --profile-pass`), scaled by what the same counters read for
+# trt_copy_bytes of 256 MiB (factors 2.000 and 1.000 to KiB); the summary of those runs is
+# profiles/lt2exp_lm2exp_max_counters.md.  A constant, not a live measurement.
+MEASURED_TRAFFIC_BYTES = {"lt2exp_c5": 438.1e6, "lm2exp_c3": 757.1e6}
 
 
 def log(*a):
