@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TRT_ABI_VERSION 1
+#define TRT_ABI_VERSION 2
 
 #define TRT_OK 0
 #define TRT_E_INVALID (-1)   /* null pointer, non-positive size, bad enum   */
@@ -61,13 +61,22 @@ const char *trt_error_string(int status);
  * free.  Replaces the `_ker_lm2exp[grid](...)` launch, triturus/lm2exp.py:186-205;
  * arithmetic contract baselines/lm2exp.py:11-14 (column max clamped to
  * +-1e38, an all -inf column gives -inf, never NaN).
- * variant: 0 = choose by shape; other values pick a tile shape for
- * experiments (see trt_lm2exp_variant_count).
+ * variant: 0 = choose by shape; 1..trt_lm2exp_variant_count() pick a tile shape
+ * (experiments, tests).
+ * splits: the contraction over J may be cut over several workgroups whose partial
+ * sums are merged by a second kernel in a fixed order (deterministic): 0 = decide
+ * by shape (small grids with a long contraction), 1 = never, n = n ways.  The
+ * reference has no such mode for lm2exp.  When it splits, the call needs a
+ * workspace of trt_lm2exp_workspace_bytes(R, I, J, K, variant, splits) bytes
+ * (0 when it does not split: pass NULL, 0).
  */
 int trt_lm2exp_f32(const float *a, const float *b, float *c,
                    int64_t R, int64_t I, int64_t J, int64_t K,
                    const int64_t sa[3], const int64_t sb[3], const int64_t sc[3],
-                   int variant, void *stream);
+                   int variant, int splits, void *workspace, size_t workspace_bytes,
+                   void *stream);
+size_t trt_lm2exp_workspace_bytes(int64_t R, int64_t I, int64_t J, int64_t K,
+                                  int variant, int splits);
 int trt_lm2exp_variant_count(void);
 
 /*
@@ -78,8 +87,9 @@ int trt_lm2exp_variant_count(void);
  * be 1.  Replaces the `_ker_lt2exp_unsplit[grid](...)` launch,
  * triturus/lt2exp.py:601-629, and the `_ker_lt2exp_split[grid](...)` launch,
  * triturus/lt2exp.py:564-597; arithmetic contract baselines/lt2exp.py:15-25.
- * mode: TRT_MODE_*.  AUTO applies the reference heuristic
- * (R*S*K < 1048576 and I*J > 512, triturus/lt2exp.py:535).  SPLIT partitions
+ * mode: TRT_MODE_*.  AUTO splits when the reference heuristic says so
+ * (R*S*K < 1048576 and I*J > 512, triturus/lt2exp.py:535) and also when the
+ * unsplit grid would leave most compute units idle.  SPLIT partitions
  * the contracted (i,j) range over several workgroups and merges the partial
  * sums deterministically; it needs a workspace of
  * trt_lt2exp_workspace_bytes(...) bytes (UNSPLIT needs none: pass NULL, 0).

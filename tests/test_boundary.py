@@ -63,12 +63,18 @@ def test_c_abi_argument_errors_are_statuses():
     one = c_void_p(16)  # never dereferenced: every call below is rejected first
     null = c_void_p(None)
     # lm2exp
-    assert lib.trt_lm2exp_f32(null, one, one, 1, 1, 1, 1, ok, ok, ok, 0, null) == -1
-    assert lib.trt_lm2exp_f32(one, one, one, 0, 1, 1, 1, ok, ok, ok, 0, null) == -1
-    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, ok, 99, null) == -1
-    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, s3(12, 1, 4), ok, ok, 0, null) == -2
-    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, s3(-12, 4, 1), ok, 0, null) == -2
-    assert lib.trt_lm2exp_f32(one, one, one, 1 << 31, 1, 1, 1, ok, ok, ok, 0, null) == -4
+    tail = (0, 0, null, 0, null)  # variant, splits, workspace, bytes, stream
+    assert lib.trt_lm2exp_f32(null, one, one, 1, 1, 1, 1, ok, ok, ok, *tail) == -1
+    assert lib.trt_lm2exp_f32(one, one, one, 0, 1, 1, 1, ok, ok, ok, *tail) == -1
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, ok, 99, 0, null, 0, null) == -1
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, ok, 0, -1, null, 0, null) == -1
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, s3(12, 1, 4), ok, ok, *tail) == -2
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, s3(-12, 4, 1), ok, *tail) == -2
+    assert lib.trt_lm2exp_f32(one, one, one, 1 << 31, 1, 1, 1, ok, ok, ok, *tail) == -4
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 2, 2, 8, ok, ok, s3(16, 4, 1), *tail) == -2  # overlapping output rows
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 2, 2, 8, ok, s3(1 << 31, 1 << 30, 1), s3(16, 8, 1), *tail) == -4
+    big = s3(1024 * 1024, 1024, 1)
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1024, 1024, 1024, big, big, big, 0, 4, null, 0, null) == -3  # split needs a workspace
     # lt2exp
     args = (1, 1, 1, 1, 1, ok, ok, ok, ok)
     assert lib.trt_lt2exp_f32(one, null, one, one, *args, 0, 0, null, 0, null) == -1
@@ -98,7 +104,16 @@ def test_workspace_queries_are_host_only_and_follow_the_mode_rule():
         assert lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, _lib.MODE_UNSPLIT) == 0
         assert lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, _lib.MODE_SPLIT) >= 4 * (R * S * K + 2 * R * K)
         auto = lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, _lib.MODE_AUTO) > 0
-        assert auto == launches_split(R, S, I, J, K, "auto")
+        if launches_split(R, S, I, J, K, "auto"):  # the reference rule implies a split here too
+            assert auto
+    # the large benchmark configurations fill the machine unsplit
+    assert lib.trt_lt2exp_workspace_bytes(64, 64, 64, 64, 4096, _lib.MODE_AUTO) == 0
+    # lm2exp: splits only for small grids with a long contraction, or on request
+    assert lib.trt_lm2exp_workspace_bytes(64, 256, 256, 4096, 0, 0) == 0
+    assert lib.trt_lm2exp_workspace_bytes(1, 1024, 1024, 1024, 0, 1) == 0
+    assert lib.trt_lm2exp_workspace_bytes(1, 1024, 1024, 1024, 0, 0) > 0
+    assert lib.trt_lm2exp_workspace_bytes(1, 128, 64, 128, 0, 0) == 0  # two chunks: nothing to share
+    assert lib.trt_lm2exp_workspace_bytes(2, 100, 256, 50, 0, 4) == 4 * (4 * 2 * 100 * 50 + 4 * 2 * 50)
     # the reference rule itself, triturus/lt2exp.py:535: at the benchmark configurations it is unsplit
     assert not launches_split(16, 64, 32, 32, 2048, "auto")
     assert not launches_split(64, 64, 64, 64, 4096, "auto")

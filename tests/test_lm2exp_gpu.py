@@ -81,6 +81,39 @@ def test_edge_shapes(dev, shape):
     _check(lm2exp(a.to(dev), b.to(dev)), a, b)
 
 
+@pytest.mark.parametrize("splits", [2, 3, 5, 32])
+@pytest.mark.parametrize("variant", [0, 1, 3, 7, 10])
+def test_split_contraction(dev, splits, variant):
+    """The contraction over J cut over several workgroups and merged (no counterpart in the
+    reference): same results as the single-workgroup path, also with -inf chunks, ragged J."""
+    g = torch.Generator().manual_seed(splits * 31 + variant)
+    R, I, J, K = 2, 70, 333, 150
+    a = torch.rand(R, I, J, generator=g)
+    b = -40 + 25 * torch.randn(R, J, K, generator=g)
+    b[torch.rand(b.shape, generator=g) < 0.2] = NINF
+    b[0, :, 3] = NINF            # all -inf column
+    b[1, :200, 7] = NINF         # -inf in every chunk of the first splits
+    b[1, 40:, 9] = NINF          # finite only in the first split
+    a[1, 5, :] = 0.0
+    ag, bg = a.to(dev), b.to(dev)
+    out = lm2exp(ag, bg, _variant=variant, _splits=splits)
+    r = _check(out, a, b)
+    assert r["n_neg_inf"] >= I + K
+    assert torch.equal(out, lm2exp(ag, bg, _variant=variant, _splits=splits))  # deterministic
+    assert torch.allclose(out, lm2exp(ag, bg, _variant=variant, _splits=1), rtol=1e-5, atol=1e-5)
+
+
+def test_small_grid_long_contraction_splits_by_itself(dev):
+    lib = _lib.load()
+    assert lib.trt_lm2exp_workspace_bytes(1, 512, 2048, 384, 0, 0) > 0
+    g = torch.Generator().manual_seed(77)
+    a = torch.rand(1, 512, 2048, generator=g)
+    b = torch.randn(1, 2048, 384, generator=g)
+    out = lm2exp(a.to(dev), b.to(dev))
+    _check(out, a, b)
+    assert torch.allclose(torch_baseline.lm2exp_fp32(a, b), out.cpu())  # the reference's bar
+
+
 def test_empty_inputs(dev):
     assert lm2exp(torch.rand(0, 3, 4, device=dev), torch.rand(0, 4, 5, device=dev)).shape == (0, 3, 5)
     assert lm2exp(torch.rand(2, 0, 4, device=dev), torch.rand(2, 4, 5, device=dev)).shape == (2, 0, 5)

@@ -38,9 +38,11 @@ constexpr float kRescaleMargin = 8.0f;
 struct Lm2Args {
     const float *a, *b;
     float *c;
+    float *part;   // splits > 1: [splits][R][I][K] partial sums
+    float *shift;  // splits > 1: [splits][R][K] the shift each partial sum is relative to
     int R, I, J, K;
     int64_t sa0, sa1, sb0, sb1, sc0, sc1;
-    int i_tiles, n_tiles;
+    int i_tiles, n_tiles, splits, chunks_per_split;
     int64_t total_wgs, padded_wgs;
 };
 
@@ -63,8 +65,10 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     // The tile coordinates are wave-uniform; the 64-bit divisions below are expanded on
     // the vector ALU, so pin the results back into scalar registers (they feed buffer
     // resources and scalar offsets).
-    const int64_t rest = L / p.n_tiles;
+    int64_t rest = L / p.n_tiles;
     const int nt = __builtin_amdgcn_readfirstlane((int)(L % p.n_tiles));
+    const int split = __builtin_amdgcn_readfirstlane((int)(rest % p.splits));
+    rest /= p.splits;
     const int itile = __builtin_amdgcn_readfirstlane((int)(rest % p.i_tiles));
     const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.i_tiles));
 
@@ -219,9 +223,13 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         }
     };
 
-    const int n_full = p.J / JC;              // chunks with no ragged tail
-    const bool has_tail = (p.J % JC) != 0;    // one more, masked
-    const int n_jc = n_full + (has_tail ? 1 : 0);
+    // Chunks [jc0, jc1) of this workgroup (all of them unless the contraction is split
+    // over several workgroups); chunks below n_full carry no ragged tail.
+    const int n_full = p.J / JC;
+    const int n_jc = n_full + ((p.J % JC) != 0 ? 1 : 0);
+    const int jc0 = split * p.chunks_per_split;
+    const int jc1 = (jc0 + p.chunks_per_split < n_jc) ? jc0 + p.chunks_per_split : n_jc;
+    const int full_end = jc1 < n_full ? jc1 : n_full;
 
     if (!ONLINE) {
         // ---- sweep 1: exact column maxima over all J
@@ -244,13 +252,13 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         }
     }
 
-    // ---- prologue: chunk 0
-    if (n_full > 0) {
-        load_tile_full(0);
-        load_b_full(0);
+    // ---- prologue: first chunk
+    if (jc0 < n_full) {
+        load_tile_full(jc0);
+        load_b_full(jc0);
     } else {
-        load_tile_masked(0);
-        load_b_masked(0);
+        load_tile_masked(jc0);
+        load_b_masked(jc0);
     }
     store_tile(0);
     if (ONLINE) {
@@ -288,8 +296,8 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     // consume the prefetch before the back edge; the ragged tail and the last chunk
     // are peeled so the loop body carries no masks.
     int cur = 0;
-    int jc = 0;
-    for (; jc + 1 < n_full; ++jc) {
+    int jc = jc0;
+    for (; jc + 1 < full_end; ++jc) {
         load_tile_full(jc + 1);
         load_b_full(jc + 1);
         __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block, not sunk into it
@@ -299,7 +307,7 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         __syncthreads();
         cur ^= 1;
     }
-    if (jc + 1 < n_jc) {  // the next chunk is the masked tail
+    if (jc + 1 < jc1) {  // the next chunk is the masked tail
         load_tile_masked(jc + 1);
         load_b_masked(jc + 1);
         __builtin_amdgcn_sched_barrier(0);
@@ -315,22 +323,52 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     // 8*(v/4) + 4*h + v%4, column m of its 32 x 32 tile; the row part of the address
     // is wave-uniform apart from the lane half, so it lives in scalar registers.
     // Rows past I fall outside the buffer extent and are dropped by the hardware.
+    // With a split contraction the raw sums and their shift go to the workspace instead.
+    const bool split_out = p.splits > 1;  // wave-uniform
     const int crows = p.I - (i0 + wrow0);  // valid rows below this wavefront's first row
+    float *obase = split_out ? p.part + (((int64_t)split * p.R + r) * p.I + (i0 + wrow0)) * (int64_t)p.K
+                             : p.c + (int64_t)r * p.sc0 + (int64_t)(i0 + wrow0) * p.sc1;
+    const uint32_t orow = split_out ? (uint32_t)p.K : (uint32_t)p.sc1;
     const __amdgpu_buffer_rsrc_t c_rsrc =
-        make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)(i0 + wrow0) * p.sc1,
-                  crows > 0 ? (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4) : 0u);
-    const uint32_t c_row_bytes = (uint32_t)p.sc1 * 4u;
+        make_rsrc(obase, crows > 0 ? (uint32_t)(((int64_t)(crows - 1) * orow + p.K) * 4) : 0u);
+    const uint32_t c_row_bytes = orow * 4u;
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct) {
         if (ncol[ct] >= p.K) continue;
-        const uint32_t co = ((uint32_t)(4 * h) * (uint32_t)p.sc1 + (uint32_t)ncol[ct]) * 4u;
+        const uint32_t co = ((uint32_t)(4 * h) * orow + (uint32_t)ncol[ct]) * 4u;
+        if (split_out && itile == 0 && wm == 0 && h == 0)
+            p.shift[((int64_t)split * p.R + r) * p.K + ncol[ct]] = mref[ct];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const uint32_t trow = 32 * rt + 8 * (v / 4) + (v % 4);  // + 4h in the lane offset
-                buf_store_f32(log_plus(acc[rt][ct][v], mref[ct]), c_rsrc, co, trow * c_row_bytes);
+                const float val = split_out ? acc[rt][ct][v] : log_plus(acc[rt][ct][v], mref[ct]);
+                buf_store_f32(val, c_rsrc, co, trow * c_row_bytes);
             }
+    }
+}
+
+// Merge of a split contraction: every split s holds sum_s (relative to its own shift m_s);
+// c = M + log(sum_s sum_s * exp(m_s - M)) with M = max_s m_s, in split order (deterministic).
+__global__ __launch_bounds__(256) void lm2exp_merge_kernel(const float *__restrict__ part,
+                                                           const float *__restrict__ shift, float *__restrict__ c,
+                                                           int R, int I, int K, int splits, int64_t sc0,
+                                                           int64_t sc1) {
+    const int64_t total = (int64_t)R * I * K;
+    const int64_t rk = (int64_t)R * K;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+        const int k = (int)(e % K);
+        const int64_t ri = e / K;
+        const int i = (int)(ri % I);
+        const int r = (int)(ri / I);
+        const float *sh = shift + (int64_t)r * K + k;
+        float M = sh[0];
+        for (int sp = 1; sp < splits; ++sp) M = max_nan(M, sh[sp * rk]);
+        float sum = 0.f;
+        for (int sp = 0; sp < splits; ++sp) sum += part[(int64_t)sp * total + e] * exp_shifted(sh[sp * rk] - M);
+        c[(int64_t)r * sc0 + (int64_t)i * sc1 + k] = log_plus(sum, M);
     }
 }
 
@@ -386,54 +424,117 @@ static int launch_v(const Lm2Args &args, bool vec, hipStream_t stream) {
                : launch_k<RT, CT, WM, WN, NQ, false, ONLINE>(args, stream);
 }
 
+struct Lm2Plan {
+    int variant;           // index into kVariants
+    int splits;            // workgroups sharing one output tile
+    int chunks_per_split;  // j-chunks each of them contracts
+};
+
+constexpr int kMaxSplits = 32;
+
+// splits_req: 0 = decide here, 1 = never split, n > 1 = split n ways (capped).
+// A small grid with a long contraction is cut over J so that the 256 CUs have work:
+// e.g. batch 1, I=J=K=1024 is 64 tiles of 128 x 128 but 32 chunks deep.
+static Lm2Plan make_plan(int64_t R, int64_t I, int64_t J, int64_t K, int variant, int splits_req) {
+    Lm2Plan pl;
+    pl.variant = (variant >= 1) ? variant - 1 : choose_variant(R, I, J, K);
+    const Lm2Variant &vr = kVariants[pl.variant];
+    const int64_t chunks = ceil_div(J, 8 * vr.nq);
+    const int64_t base = R * ceil_div(I, 32 * vr.rt * vr.wm) * ceil_div(K, 32 * vr.ct * vr.wn);
+    int64_t splits = 1;
+    if (splits_req == 0) {
+        if (base < 384 && chunks >= 8) {
+            splits = ceil_div(768, base);
+            if (splits > chunks / 4) splits = chunks / 4;
+        }
+    } else {
+        splits = splits_req;
+    }
+    if (splits > kMaxSplits) splits = kMaxSplits;
+    if (splits > chunks) splits = chunks;
+    if (splits < 1) splits = 1;
+    const int64_t per = ceil_div(chunks, splits);
+    pl.splits = (int)ceil_div(chunks, per);
+    pl.chunks_per_split = (int)per;
+    return pl;
+}
+
+static size_t plan_workspace(const Lm2Plan &pl, int64_t R, int64_t I, int64_t K) {
+    if (pl.splits <= 1) return 0;
+    return ((size_t)pl.splits * R * I * K + (size_t)pl.splits * R * K) * sizeof(float);
+}
+
 }  // namespace trt
 
 using namespace trt;
 
 extern "C" int trt_lm2exp_variant_count(void) { return kNumVariants; }
 
+extern "C" size_t trt_lm2exp_workspace_bytes(int64_t R, int64_t I, int64_t J, int64_t K, int variant,
+                                             int splits) {
+    if (R <= 0 || I <= 0 || J <= 0 || K <= 0 || variant < 0 || variant > kNumVariants || splits < 0) return 0;
+    return plan_workspace(make_plan(R, I, J, K, variant, splits), R, I, K);
+}
+
 extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J,
                               int64_t K, const int64_t sa[3], const int64_t sb[3], const int64_t sc[3],
-                              int variant, void *stream) {
+                              int variant, int splits, void *workspace, size_t workspace_bytes, void *stream) {
     if (!a || !b || !c || !sa || !sb || !sc) return TRT_E_INVALID;
     if (R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
-    if (variant < 0 || variant > kNumVariants) return TRT_E_INVALID;
+    if (variant < 0 || variant > kNumVariants || splits < 0) return TRT_E_INVALID;
     if (sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
+    if (sc[1] < K || sc[0] < 0) return TRT_E_LAYOUT;  // output rows must not overlap (stores rely on it)
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || I >= lim || J >= lim || K >= lim) return TRT_E_RANGE;
     // byte offsets inside one batch slab of a, b and c are 32-bit (buffer addressing)
-    if (J * sb[1] + K >= ((int64_t)1 << 30) || I * sa[1] + J >= ((int64_t)1 << 30) ||
-        I * sc[1] + K >= ((int64_t)1 << 30))
-        return TRT_E_RANGE;
+    if (J * sb[1] + K >= lim || I * sa[1] + J >= lim || I * sc[1] + K >= lim || I * K >= lim) return TRT_E_RANGE;
 
-    const int v = (variant >= 1) ? variant - 1 : choose_variant(R, I, J, K);
+    const Lm2Plan pl = make_plan(R, I, J, K, variant, splits);
+    const int v = pl.variant;
     const Lm2Variant &vr = kVariants[v];
     Lm2Args args;
     args.a = a; args.b = b; args.c = c;
+    args.part = nullptr; args.shift = nullptr;
     args.R = (int)R; args.I = (int)I; args.J = (int)J; args.K = (int)K;
     args.sa0 = sa[0]; args.sa1 = sa[1];
     args.sb0 = sb[0]; args.sb1 = sb[1];
     args.sc0 = sc[0]; args.sc1 = sc[1];
     args.i_tiles = (int)ceil_div(I, 32 * vr.rt * vr.wm);
     args.n_tiles = (int)ceil_div(K, 32 * vr.ct * vr.wn);
-    args.total_wgs = (int64_t)R * args.i_tiles * args.n_tiles;
+    args.splits = pl.splits;
+    args.chunks_per_split = pl.chunks_per_split;
+    args.total_wgs = (int64_t)R * args.i_tiles * args.n_tiles * pl.splits;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+    if (pl.splits > 1) {
+        const size_t need = plan_workspace(pl, R, I, K);
+        if (!workspace || workspace_bytes < need) return TRT_E_WORKSPACE;
+        args.part = static_cast<float *>(workspace);
+        args.shift = args.part + (size_t)pl.splits * R * I * K;
+    }
     const bool vec = (J % 4 == 0) && (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    int st;
     switch (v) {
-        case 0: return launch_v<4, 1, 1, 4, 4, true>(args, vec, s);
-        case 1: return launch_v<4, 1, 1, 8, 4, true>(args, vec, s);
-        case 2: return launch_v<8, 1, 1, 8, 4, true>(args, vec, s);
-        case 3: return launch_v<8, 1, 1, 4, 4, true>(args, vec, s);
-        case 4: return launch_v<8, 1, 1, 8, 4, false>(args, vec, s);
-        case 5: return launch_v<2, 2, 1, 4, 4, true>(args, vec, s);
-        case 6: return launch_v<2, 1, 1, 4, 4, true>(args, vec, s);
-        case 7: return launch_v<1, 1, 1, 4, 4, true>(args, vec, s);
-        case 8: return launch_v<2, 1, 1, 4, 4, false>(args, vec, s);
-        default: return launch_v<4, 1, 1, 4, 4, false>(args, vec, s);
+        case 0: st = launch_v<4, 1, 1, 4, 4, true>(args, vec, s); break;
+        case 1: st = launch_v<4, 1, 1, 8, 4, true>(args, vec, s); break;
+        case 2: st = launch_v<8, 1, 1, 8, 4, true>(args, vec, s); break;
+        case 3: st = launch_v<8, 1, 1, 4, 4, true>(args, vec, s); break;
+        case 4: st = launch_v<8, 1, 1, 8, 4, false>(args, vec, s); break;
+        case 5: st = launch_v<2, 2, 1, 4, 4, true>(args, vec, s); break;
+        case 6: st = launch_v<2, 1, 1, 4, 4, true>(args, vec, s); break;
+        case 7: st = launch_v<1, 1, 1, 4, 4, true>(args, vec, s); break;
+        case 8: st = launch_v<2, 1, 1, 4, 4, false>(args, vec, s); break;
+        default: st = launch_v<4, 1, 1, 4, 4, false>(args, vec, s); break;
     }
+    if (st != 0 || pl.splits <= 1) return st;
+    const int64_t total = R * I * K;
+    int64_t blocks = ceil_div(total, 256);
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(lm2exp_merge_kernel, dim3((unsigned)blocks), dim3(256), 0, s, args.part, args.shift, c,
+                       (int)R, (int)I, (int)K, pl.splits, sc[0], sc[1]);
+    return (int)hipGetLastError();
 }

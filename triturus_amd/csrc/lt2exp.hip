@@ -368,14 +368,16 @@ struct SplitPlan {
 
 static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode, int variant) {
     const Lt2Variant &v = kVariants[variant];
+    const int64_t iters = ceil_div(J, 8 * v.nq) * I;
+    const int64_t base = R * ceil_div(S, 32 * v.rt) * ceil_div(K, 32 * v.ct * kLt2Waves);
     bool split;
     if (mode == TRT_MODE_AUTO)
-        split = (R * S * K < 1048576) && (I * J > 512);  // triturus/lt2exp.py:535
+        // the reference rule (triturus/lt2exp.py:535), or a grid that would leave most of
+        // the 256 CUs idle while the contraction is long enough to share
+        split = ((R * S * K < 1048576) && (I * J > 512)) || (base < 384 && iters >= 16);
     else
         split = (mode == TRT_MODE_SPLIT);
-    const int64_t iters = ceil_div(J, 8 * v.nq) * I;
     if (!split) return {false, 1, (int)iters};
-    const int64_t base = R * ceil_div(S, 32 * v.rt) * ceil_div(K, 32 * v.ct * kLt2Waves);
     int64_t splits = ceil_div(1024, base);
     if (splits > 32) splits = 32;
     if (splits > iters) splits = iters;
@@ -420,6 +422,7 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     if (sw[2] != 1 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
+    if (sc[1] < K) return TRT_E_LAYOUT;  // output rows must not overlap (stores rely on it)
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
     // byte offsets inside one batch slab of w, a and c are 32-bit (buffer addressing)

@@ -23,7 +23,7 @@ def _unit_inner(t: torch.Tensor) -> torch.Tensor:
     return t.contiguous()
 
 
-def lm2exp(a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0) -> torch.Tensor:
+def lm2exp(a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0, _splits: int = 0) -> torch.Tensor:
     assert len(a.shape) == len(b.shape) == 3
     assert a.shape[0] == b.shape[0]
     assert a.shape[2] == b.shape[1]
@@ -42,11 +42,15 @@ def lm2exp(a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0) -> torch.Tens
         return c.fill_(float("-inf"))
     a = _unit_inner(a)
     b = _unit_inner(b)
+    # small grids with a long contraction are cut over J; the partial sums need a workspace
+    ws_bytes = lib.trt_lm2exp_workspace_bytes(R, I, J, K, _variant, _splits)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     with torch.cuda.device(a.device):
         status = lib.trt_lm2exp_f32(
             c_void_p(a.data_ptr()), c_void_p(b.data_ptr()), c_void_p(c.data_ptr()),
             R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-            _variant, _lib.current_stream(a.device),
+            _variant, _splits, c_void_p(ws.data_ptr() if ws is not None else None), ws_bytes,
+            _lib.current_stream(a.device),
         )
     _lib.check(status, "trt_lm2exp_f32")
     return c
