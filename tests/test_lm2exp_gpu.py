@@ -145,6 +145,46 @@ def test_neg_inf_columns_zero_rows_and_range(dev):
     assert torch.isfinite(out).all()
 
 
+@pytest.mark.parametrize("variant", [0, 3, 10])
+def test_shift_moves_during_the_sweep(dev, variant):
+    """Columns whose maximum keeps growing along J (ascending, step changes of 1e3 and 1e30,
+    finite values only in the last rows): the single-sweep kernel must rescale its sums on
+    the way and still match the two-sweep recipe."""
+    g = torch.Generator().manual_seed(11)
+    R, I, J, K = 2, 40, 300, 96
+    a = torch.rand(R, I, J, generator=g) + 0.01
+    b = torch.empty(R, J, K)
+    ramp = torch.linspace(-500.0, 500.0, J)
+    b[0] = ramp[:, None] + torch.randn(J, K, generator=g)              # ascending: rescales every chunk
+    b[1] = -ramp[:, None] + torch.randn(J, K, generator=g)             # descending: never
+    b[0, :, 5] = NINF
+    b[0, J - 1, 5] = 3.0                                               # first finite value in the last row
+    b[0, :, 6] = torch.where(torch.arange(J) < 150, -1e30, 1e30)       # jump of 2e30 mid-way
+    b[1, :, 7] = torch.where(torch.arange(J) % 64 < 32, -1e3, 1e3)     # alternating by chunk
+    b[1, :, 8] = NINF
+    b[1, 100, 8] = -1e38                                               # at the clamp
+    ag, bg = a.to(dev), b.to(dev)
+    out = lm2exp(ag, bg, _variant=variant, _splits=1)
+    r = _check(out, a, b)
+    assert torch.isfinite(out[0, :, 5]).all() and torch.isfinite(out[0, :, 6]).all()
+    assert torch.allclose(out.cpu(), torch_baseline.lm2exp_fp32(a, b), rtol=1e-5, atol=1e-5)
+    out3 = lm2exp(ag, bg, _variant=variant, _splits=3)
+    _check(out3, a, b)
+
+
+def test_positive_infinity_follows_the_torch_recipe(dev):
+    a = torch.rand(1, 4, 40) + 0.1
+    b = torch.randn(1, 40, 33)
+    b[0, 7, 2] = float("inf")
+    b[0, 35, 3] = float("inf")
+    out = lm2exp(a.to(dev), b.to(dev)).cpu()
+    ref = torch_baseline.lm2exp_fp32(a, b)
+    assert torch.equal(torch.isposinf(out), torch.isposinf(ref))
+    assert torch.isposinf(out[0, :, 2]).all() and torch.isposinf(out[0, :, 3]).all()
+    fin = torch.isfinite(ref)
+    assert torch.allclose(out[fin], ref[fin], rtol=1e-5, atol=1e-6)
+
+
 def test_nan_input_propagates_like_the_torch_recipe(dev):
     a = torch.rand(1, 8, 8)
     b = torch.randn(1, 8, 40)

@@ -117,6 +117,27 @@ def test_neg_inf_and_zero_weights(dev):
         assert torch.all(out[1, 7] == NINF) and not torch.isnan(out).any()
 
 
+def test_nan_and_extreme_inputs_follow_the_torch_recipe(dev):
+    g = torch.Generator().manual_seed(12)
+    w = torch.rand(1, 8, 6, 10, generator=g) + 0.1
+    a = torch.randn(1, 6, 70, generator=g)
+    b = torch.randn(1, 10, 70, generator=g)
+    a[0, 2, 4] = float("nan")
+    b[0, 9, 8] = float("nan")
+    a[0, :, 10] = -9e37
+    b[0, :, 11] = torch.linspace(-1e30, 1e30, 10)
+    a[0, :, 12] = NINF
+    a[0, 5, 12] = -1e38
+    for mode in ("unsplit", "split"):
+        out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode).cpu()
+        ref = torch_baseline.lt2exp_fp32(w, a, b)
+        assert torch.equal(torch.isnan(out), torch.isnan(ref))
+        assert torch.isnan(out[0, :, 4]).all() and torch.isnan(out[0, :, 8]).all()
+        ok = ~torch.isnan(ref)
+        r = oracle64.compare(out[ok], oracle64.lt2exp64(w, a, b)[ok])
+        assert r["ok"], r
+
+
 def test_non_viewable_weights_raise_like_the_reference(dev):
     w = torch.rand(2, 3, 5, 4, device=dev).transpose(2, 3)  # I and J not jointly contiguous
     with pytest.raises(RuntimeError):
@@ -188,3 +209,36 @@ def test_benchmark_configuration_c5_full_size(dev):
     for variant in (2, 5):
         assert torch.allclose(lt2exp(wg, ag, bg, _variant=variant), out, rtol=1e-5, atol=1e-5)
     assert torch.allclose(lt2exp(wg, ag, bg, mode="split"), out, rtol=1e-5, atol=1e-5)
+
+
+def test_capturable_in_a_hip_graph(dev):
+    """No allocation, synchronisation or host state inside the C ABI: a call captured in a
+    HIP graph replays with new input values (replayed several times, with eager work and
+    synchronisations in between, each replay checked against the eager result)."""
+    g = torch.Generator().manual_seed(13)
+    w = torch.rand(2, 64, 16, 32, generator=g).to(dev)
+    a = torch.randn(2, 16, 256, generator=g).to(dev)
+    b = torch.randn(2, 32, 256, generator=g).to(dev)
+    a2 = torch.randn(2, 256, 32, generator=g).to(dev)
+    side = torch.cuda.Stream(device=dev)
+    side.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            lt2exp(w, a, b)
+            lm2exp(a2, b)
+    torch.cuda.current_stream(dev).wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_t = lt2exp(w, a, b)
+        out_t_split = lt2exp(w, a, b, mode="split")
+        out_m = lm2exp(a2, b)
+    for rep in range(4):
+        a.copy_(torch.randn(2, 16, 256, generator=g))
+        b.copy_(torch.randn(2, 32, 256, generator=g) - rep)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out_t, lt2exp(w, a, b))
+        assert torch.equal(out_t_split, lt2exp(w, a, b, mode="split"))
+        assert torch.equal(out_m, lm2exp(a2, b))
+        torch.cuda.synchronize()
