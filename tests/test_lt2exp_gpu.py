@@ -219,7 +219,7 @@ def test_capturable_in_a_hip_graph(dev):
     w = torch.rand(2, 64, 16, 32, generator=g).to(dev)
     a = torch.randn(2, 16, 256, generator=g).to(dev)
     b = torch.randn(2, 32, 256, generator=g).to(dev)
-    a2 = torch.randn(2, 256, 32, generator=g).to(dev)
+    a2 = torch.rand(2, 256, 32, generator=g).to(dev)
     side = torch.cuda.Stream(device=dev)
     side.wait_stream(torch.cuda.current_stream(dev))
     with torch.cuda.stream(side):
