@@ -63,6 +63,13 @@ __device__ __forceinline__ floatx4 buf_load_f32x4(__amdgpu_buffer_rsrc_t r, uint
 __device__ __forceinline__ void buf_store_f32(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
     __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, voff, soff, 0);
 }
+// Write-once output: the non-temporal hint keeps the result stream from evicting the
+// operand panels that other workgroups still re-read from L2 (measured: 3 % on lm2exp).
+constexpr int kCacheNonTemporal = 2;
+__device__ __forceinline__ void buf_store_f32_stream(float v, __amdgpu_buffer_rsrc_t r, uint32_t voff,
+                                                     uint32_t soff) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, voff, soff, kCacheNonTemporal);
+}
 
 // max of three without NaN canonicalisation moves (a NaN operand is ignored, which is
 // what the callers want: see the kernels).

@@ -343,8 +343,10 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
 #pragma unroll
             for (int v = 0; v < 16; ++v) {
                 const uint32_t trow = 32 * rt + 8 * (v / 4) + (v % 4);  // + 4h in the lane offset
-                const float val = split_out ? acc[rt][ct][v] : log_plus(acc[rt][ct][v], mref[ct]);
-                buf_store_f32(val, c_rsrc, co, trow * c_row_bytes);
+                if (split_out)  // partial sums are read back by the merge kernel right away
+                    buf_store_f32(acc[rt][ct][v], c_rsrc, co, trow * c_row_bytes);
+                else
+                    buf_store_f32_stream(log_plus(acc[rt][ct][v], mref[ct]), c_rsrc, co, trow * c_row_bytes);
             }
     }
 }

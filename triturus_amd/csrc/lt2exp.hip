@@ -276,7 +276,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4);  // + 4h in the lane offset
-                    buf_store_f32(log_plus(acc[rt][ct][v], mm), c_rsrc, co, trow_c * c_row_bytes);
+                    buf_store_f32_stream(log_plus(acc[rt][ct][v], mm), c_rsrc, co, trow_c * c_row_bytes);
                 }
         }
     }
