@@ -87,9 +87,11 @@ int trt_lm2exp_variant_count(void);
  * be 1.  Replaces the `_ker_lt2exp_unsplit[grid](...)` launch,
  * triturus/lt2exp.py:601-629, and the `_ker_lt2exp_split[grid](...)` launch,
  * triturus/lt2exp.py:564-597; arithmetic contract baselines/lt2exp.py:15-25.
- * mode: TRT_MODE_*.  AUTO splits when the reference heuristic says so
- * (R*S*K < 1048576 and I*J > 512, triturus/lt2exp.py:535) and also when the
- * unsplit grid would leave most compute units idle.  SPLIT partitions
+ * mode: TRT_MODE_*.  AUTO decides like the reference does -- by the size of the
+ * output grid and the length of the contraction (triturus/lt2exp.py:535 uses
+ * R*S*K < 1048576 and I*J > 512) -- with thresholds measured on MI355X: it
+ * splits when the unsplit grid would leave many compute units idle and the
+ * contraction is long enough to pay for the merge.  SPLIT partitions
  * the contracted (i,j) range over several workgroups and merges the partial
  * sums deterministically; it needs a workspace of
  * trt_lt2exp_workspace_bytes(...) bytes (UNSPLIT needs none: pass NULL, 0).

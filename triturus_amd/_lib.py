@@ -104,6 +104,24 @@ def current_stream(device: torch.device) -> c_void_p:
     return c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def on_device(device: torch.device):
+    """Context that makes `device` current for the launch; free when it already is."""
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
+
+
 def require_gpu(*tensors: torch.Tensor) -> None:
     """The kernels run on HIP device memory only."""
     for t in tensors:

@@ -372,9 +372,12 @@ static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t 
     const int64_t base = R * ceil_div(S, 32 * v.rt) * ceil_div(K, 32 * v.ct * kLt2Waves);
     bool split;
     if (mode == TRT_MODE_AUTO)
-        // the reference rule (triturus/lt2exp.py:535), or a grid that would leave most of
-        // the 256 CUs idle while the contraction is long enough to share
-        split = ((R * S * K < 1048576) && (I * J > 512)) || (base < 384 && iters >= 16);
+        // the reference rule (triturus/lt2exp.py:535) when the grid is small, or a grid that
+        // would leave much of the 256 CUs idle while the contraction is long enough to pay
+        // for the partial sums' round trip through memory and the merge launch (measured:
+        // R=16 S=64 I=J=32 K=2048 -- 256 tiles, 32 iterations -- is 1.4x slower split;
+        // R=32 S=I=J=128..256 K=256 -- 128..256 tiles, 512..2048 iterations -- 1.3-2.3x faster)
+        split = (base < 64 && iters >= 16) || (base < 384 && iters >= 128);
     else
         split = (mode == TRT_MODE_SPLIT);
     if (!split) return {false, 1, (int)iters};

@@ -45,7 +45,7 @@ def lm2exp(a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0, _splits: int 
     # small grids with a long contraction are cut over J; the partial sums need a workspace
     ws_bytes = lib.trt_lm2exp_workspace_bytes(R, I, J, K, _variant, _splits)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
-    with torch.cuda.device(a.device):
+    with _lib.on_device(a.device):
         status = lib.trt_lm2exp_f32(
             c_void_p(a.data_ptr()), c_void_p(b.data_ptr()), c_void_p(c.data_ptr()),
             R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),

@@ -64,7 +64,7 @@ def lt2exp(
     ws = None
     if ws_bytes:
         ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
-    with torch.cuda.device(a.device):
+    with _lib.on_device(a.device):
         status = lib.trt_lt2exp_f32(
             c_void_p(w.data_ptr()), c_void_p(a.data_ptr()), c_void_p(b.data_ptr()),
             c_void_p(c.data_ptr()), R, S, I, J, K,

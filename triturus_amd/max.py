@@ -39,7 +39,7 @@ def _vmax_impl(x: torch.Tensor, with_index: bool):
     idx = torch.empty((), dtype=torch.int64, device=x.device) if with_index else None
     ws_bytes = lib.trt_vmax_workspace_bytes(n, code)
     ws = _workspace(ws_bytes, x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         status = lib.trt_vmax(
             c_void_p(x.data_ptr()), n, code, c_void_p(val.data_ptr()),
             c_void_p(idx.data_ptr() if idx is not None else None),
@@ -78,7 +78,7 @@ def matmax(x: torch.Tensor, axis: int = 0, *, block_size: int = 32) -> torch.Ten
     y = torch.empty(n if axis == 0 else m, dtype=x.dtype, device=x.device)
     ws_bytes = lib.trt_matmax_workspace_bytes(m, n, axis, code)
     ws = _workspace(ws_bytes, x.device)
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         status = lib.trt_matmax(
             c_void_p(x.data_ptr()), c_void_p(y.data_ptr()), m, n, axis, code,
             c_void_p(ws.data_ptr() if ws is not None else None), ws_bytes,
