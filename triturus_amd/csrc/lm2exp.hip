@@ -444,17 +444,12 @@ static Lm2Plan make_plan(int64_t R, int64_t I, int64_t J, int64_t K, int variant
     const int64_t chunks = ceil_div(J, 8 * vr.nq);
     const int64_t base = R * ceil_div(I, 32 * vr.rt * vr.wm) * ceil_div(K, 32 * vr.ct * vr.wn);
     int64_t splits = 1;
-    if (splits_req == 0) {
-        // Splitting costs a round trip of the partial sums through memory and a second
-        // launch, so it must buy a lot of idle machine: measured, R=16 I=J=K=512 (256 tiles,
-        // 16 chunks) is 1.5x slower split, batch-1 squares of 512..1536 are 1.2-1.9x faster.
-        if ((base < 64 && chunks >= 8) || (base < 256 && chunks >= 32)) {
-            splits = ceil_div(768, base);
-            if (splits > chunks / 4) splits = chunks / 4;
-        }
-    } else {
+    if (splits_req == 0)
+        // measured: R=16 I=J=K=512 (256 tiles, 16 chunks) is 1.5x slower split, batch-1
+        // squares of 512..1536 are 1.2-1.9x faster; the model below reproduces both
+        splits = choose_splits(base, chunks, 4 * vr.nq * vr.rt * vr.ct, R * I * K, 2, kMaxSplits, false);
+    else
         splits = splits_req;
-    }
     if (splits > kMaxSplits) splits = kMaxSplits;
     if (splits > chunks) splits = chunks;
     if (splits < 1) splits = 1;

@@ -366,27 +366,20 @@ struct SplitPlan {
     int iters_per_split;
 };
 
+// AUTO follows the reference in kind -- a small output grid with a long contraction is
+// split (triturus/lt2exp.py:535 tests R*S*K < 1048576 and I*J > 512) -- but decides with a
+// cost model fitted to this machine (measured: R=16 S=64 I=J=32 K=2048, 256 tiles of 32
+// iterations, is 1.4x slower split; R=32 S=I=J=48..256 K=256 is 1.3-2.8x faster).
 static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode, int variant) {
     const Lt2Variant &v = kVariants[variant];
     const int64_t iters = ceil_div(J, 8 * v.nq) * I;
+    if (mode == TRT_MODE_UNSPLIT) return {false, 1, (int)iters};
     const int64_t base = R * ceil_div(S, 32 * v.rt) * ceil_div(K, 32 * v.ct * kLt2Waves);
-    bool split;
-    if (mode == TRT_MODE_AUTO)
-        // the reference rule (triturus/lt2exp.py:535) when the grid is small, or a grid that
-        // would leave much of the 256 CUs idle while the contraction is long enough to pay
-        // for the partial sums' round trip through memory and the merge launch (measured:
-        // R=16 S=64 I=J=32 K=2048 -- 256 tiles, 32 iterations -- is 1.4x slower split;
-        // R=32 S=I=J=128..256 K=256 -- 128..256 tiles, 512..2048 iterations -- 1.3-2.3x faster)
-        split = (base < 64 && iters >= 16) || (base < 384 && iters >= 128);
-    else
-        split = (mode == TRT_MODE_SPLIT);
-    if (!split) return {false, 1, (int)iters};
-    int64_t splits = ceil_div(1024, base);
-    if (splits > 32) splits = 32;
-    if (splits > iters) splits = iters;
-    if (splits < 1) splits = 1;
+    int64_t splits = choose_splits(base, iters, 4 * v.nq * v.rt * v.ct, R * S * K, 4, 32, mode == TRT_MODE_SPLIT);
+    if (splits <= 1) return {false, 1, (int)iters};
     const int64_t per = ceil_div(iters, splits);
     splits = ceil_div(iters, per);
+    if (splits <= 1) return {false, 1, (int)iters};
     return {true, (int)splits, (int)per};
 }
 
