@@ -86,7 +86,7 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_vmax(null, 5, 0, one, one, one, 1 << 20, null) == -1
     assert lib.trt_vmax(one, 0, 0, one, one, one, 1 << 20, null) == -1
     assert lib.trt_vmax(one, 5, 9, one, one, one, 1 << 20, null) == -1
-    assert lib.trt_vmax(one, 5, 0, one, one, null, 0, null) == -3
+    assert lib.trt_vmax(one, 1 << 20, 0, one, one, null, 0, null) == -3
     assert lib.trt_matmax(one, one, 4, 4, 2, 0, null, 0, null) == -1
     assert lib.trt_matmax(one, one, 0, 4, 0, 0, null, 0, null) == -1
     assert lib.trt_copy_bytes(one, one, 24, null) == -1
@@ -94,7 +94,8 @@ def test_c_abi_argument_errors_are_statuses():
 
 def test_workspace_queries_are_host_only_and_follow_the_mode_rule():
     lib = _lib.load()
-    assert lib.trt_vmax_workspace_bytes(1000, _lib.TRT_F32) >= 2048 * 16
+    assert lib.trt_vmax_workspace_bytes(1000, _lib.TRT_F32) == 0  # one workgroup, one launch
+    assert lib.trt_vmax_workspace_bytes(1 << 20, _lib.TRT_F32) >= 2048 * 16
     assert lib.trt_vmax_workspace_bytes(1000, 9) == 0
     assert lib.trt_matmax_workspace_bytes(4096, 4096, 1, _lib.TRT_F32) == 0
     assert lib.trt_matmax_workspace_bytes(4096, 4096, 0, _lib.TRT_F32) > 0

@@ -104,6 +104,20 @@ def current_stream(device: torch.device) -> c_void_p:
     return c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
+try:  # the raw hipStream_t of torch's current stream without building a Stream object
+    _raw_stream = torch._C._cuda_getCurrentRawStream
+except AttributeError:  # pragma: no cover - older / newer torch without the helper
+    _raw_stream = None
+
+
+def raw_stream(device: torch.device) -> int:
+    """hipStream_t (as an integer) of torch's current stream on `device`."""
+    if _raw_stream is not None:
+        idx = device.index
+        return _raw_stream(torch.cuda.current_device() if idx is None else idx)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
 class _NoSwitch:
     def __enter__(self):
         return None

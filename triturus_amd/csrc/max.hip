@@ -112,10 +112,13 @@ constexpr int kVmaxThreads = 256;
 constexpr int kVmaxMaxBlocks = 2048;
 constexpr int kVmaxUnroll = 4;
 
-template <int DT, bool WITH_IDX>
+// FINAL: the launch has a single workgroup, which writes the result itself (short vectors
+// take one launch instead of two).
+template <int DT, bool WITH_IDX, bool FINAL>
 __global__ __launch_bounds__(kVmaxThreads) void vmax_stage1(
     const typename Elem<DT>::T *__restrict__ x, int64_t n, int64_t head, int64_t nvec,
-    typename Elem<DT>::C *__restrict__ pval, int64_t *__restrict__ pidx) {
+    typename Elem<DT>::C *__restrict__ pval, int64_t *__restrict__ pidx,
+    typename Elem<DT>::T *__restrict__ out_val, int64_t *__restrict__ out_idx) {
     using E = Elem<DT>;
     using T = typename E::T;
     using C = typename E::C;
@@ -182,8 +185,14 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_stage1(
                 best = vmax_nan(best, sval[w]);
             }
         }
-        pval[blockIdx.x] = best;
-        if (WITH_IDX) pidx[blockIdx.x] = bidx;
+        if (FINAL) {
+            *out_val = E::down(best);
+            // every element is -inf: the first one is the answer, as in torch.max
+            if (WITH_IDX) *out_idx = (bidx == kNoIdx) ? 0 : bidx;
+        } else {
+            pval[blockIdx.x] = best;
+            if (WITH_IDX) pidx[blockIdx.x] = bidx;
+        }
     }
 }
 
@@ -256,8 +265,15 @@ static size_t elem_size(int dtype) {
     }
 }
 
-// workspace layout: [kVmaxMaxBlocks x 8-byte value slots][kVmaxMaxBlocks x int64]
-static size_t vmax_ws_bytes() { return (size_t)kVmaxMaxBlocks * 16; }
+// workspace layout: [kVmaxMaxBlocks x 8-byte value slots][kVmaxMaxBlocks x int64]; vectors
+// short enough for one workgroup need none
+static bool vmax_single_block(int64_t n, int dtype) {
+    const int64_t vn = 16 / (int64_t)elem_size(dtype);
+    return n <= (int64_t)kVmaxThreads * kVmaxUnroll * vn * 2;
+}
+static size_t vmax_ws_bytes(int64_t n, int dtype) {
+    return vmax_single_block(n, dtype) ? 0 : (size_t)kVmaxMaxBlocks * 16;
+}
 
 template <int DT>
 static int vmax_launch(const void *x, int64_t n, void *out_val, int64_t *out_idx, void *ws,
@@ -272,19 +288,29 @@ static int vmax_launch(const void *x, int64_t n, void *out_val, int64_t *out_idx
     int64_t head = (int64_t)(((16 - (addr & 15)) & 15) / sizeof(T));
     if (head > n) head = n;
     const int64_t nvec = (n - head) / VN;
+    T *ov = static_cast<T *>(out_val);
+    if (vmax_single_block(n, DT)) {
+        if (out_idx)
+            hipLaunchKernelGGL((vmax_stage1<DT, true, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
+                               nvec, (C *)nullptr, (int64_t *)nullptr, ov, out_idx);
+        else
+            hipLaunchKernelGGL((vmax_stage1<DT, false, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
+                               nvec, (C *)nullptr, (int64_t *)nullptr, ov, out_idx);
+        return (int)hipGetLastError();
+    }
     const int blocks = vmax_blocks(nvec);
     C *pval = static_cast<C *>(ws);
     int64_t *pidx = reinterpret_cast<int64_t *>(static_cast<char *>(ws) + (size_t)kVmaxMaxBlocks * 8);
     if (out_idx) {
-        hipLaunchKernelGGL((vmax_stage1<DT, true>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n,
-                           head, nvec, pval, pidx);
+        hipLaunchKernelGGL((vmax_stage1<DT, true, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n,
+                           head, nvec, pval, pidx, ov, out_idx);
         hipLaunchKernelGGL((vmax_stage2<DT, true>), dim3(1), dim3(kVmaxThreads), 0, stream, pval, pidx,
-                           blocks, static_cast<T *>(out_val), out_idx);
+                           blocks, ov, out_idx);
     } else {
-        hipLaunchKernelGGL((vmax_stage1<DT, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n,
-                           head, nvec, pval, pidx);
+        hipLaunchKernelGGL((vmax_stage1<DT, false, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n,
+                           head, nvec, pval, pidx, ov, out_idx);
         hipLaunchKernelGGL((vmax_stage2<DT, false>), dim3(1), dim3(kVmaxThreads), 0, stream, pval, pidx,
-                           blocks, static_cast<T *>(out_val), out_idx);
+                           blocks, ov, out_idx);
     }
     return (int)hipGetLastError();
 }
@@ -519,14 +545,14 @@ static int matmax_launch(const void *xv, void *yv, int64_t m, int64_t n, int axi
 using namespace trt;
 
 extern "C" size_t trt_vmax_workspace_bytes(int64_t n, int dtype) {
-    (void)n;
-    return elem_size(dtype) ? vmax_ws_bytes() : 0;
+    return (elem_size(dtype) && n > 0) ? vmax_ws_bytes(n, dtype) : 0;
 }
 
 extern "C" int trt_vmax(const void *x, int64_t n, int dtype, void *out_val, int64_t *out_idx,
                         void *workspace, size_t workspace_bytes, void *stream) {
     if (!x || !out_val || n <= 0 || !elem_size(dtype)) return TRT_E_INVALID;
-    if (!workspace || workspace_bytes < vmax_ws_bytes()) return TRT_E_WORKSPACE;
+    const size_t need = vmax_ws_bytes(n, dtype);
+    if (need && (!workspace || workspace_bytes < need)) return TRT_E_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(x) % elem_size(dtype)) != 0) return TRT_E_LAYOUT;
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {

@@ -8,11 +8,12 @@ without synchronising.
 
 from __future__ import annotations
 
-from ctypes import c_void_p
-
 import torch
 
 from triturus_amd import _lib
+
+
+_ws_bytes: dict = {}  # (R, I, J, K, variant, splits) -> workspace bytes, as reported by the library
 
 
 def _unit_inner(t: torch.Tensor) -> torch.Tensor:
@@ -43,14 +44,18 @@ def lm2exp(a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0, _splits: int 
     a = _unit_inner(a)
     b = _unit_inner(b)
     # small grids with a long contraction are cut over J; the partial sums need a workspace
-    ws_bytes = lib.trt_lm2exp_workspace_bytes(R, I, J, K, _variant, _splits)
+    key = (R, I, J, K, _variant, _splits)
+    ws_bytes = _ws_bytes.get(key)
+    if ws_bytes is None:
+        ws_bytes = _ws_bytes[key] = lib.trt_lm2exp_workspace_bytes(R, I, J, K, _variant, _splits)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     with _lib.on_device(a.device):
         status = lib.trt_lm2exp_f32(
-            c_void_p(a.data_ptr()), c_void_p(b.data_ptr()), c_void_p(c.data_ptr()),
+            a.data_ptr(), b.data_ptr(), c.data_ptr(),
             R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-            _variant, _splits, c_void_p(ws.data_ptr() if ws is not None else None), ws_bytes,
-            _lib.current_stream(a.device),
+            _variant, _splits, ws.data_ptr() if ws_bytes else None, ws_bytes,
+            _lib.raw_stream(a.device),
         )
-    _lib.check(status, "trt_lm2exp_f32")
+    if status:
+        _lib.check(status, "trt_lm2exp_f32")
     return c

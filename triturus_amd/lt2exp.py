@@ -10,12 +10,12 @@ reference).
 
 from __future__ import annotations
 
-from ctypes import c_void_p
-
 import torch
 
 from triturus_amd import _lib
 from triturus_amd.lm2exp import _unit_inner
+
+_ws_bytes: dict = {}  # (R, S, I, J, K, mode) -> workspace bytes, as reported by the library
 
 _MODES = {"auto": _lib.MODE_AUTO, "split": _lib.MODE_SPLIT, "unsplit": _lib.MODE_UNSPLIT}
 
@@ -60,18 +60,18 @@ def lt2exp(
     a = _unit_inner(a)
     b = _unit_inner(b)
     mode_code = _MODES[mode]
-    ws_bytes = lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, mode_code)
-    ws = None
-    if ws_bytes:
-        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+    key = (R, S, I, J, K, mode_code)
+    ws_bytes = _ws_bytes.get(key)
+    if ws_bytes is None:
+        ws_bytes = _ws_bytes[key] = lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, mode_code)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     with _lib.on_device(a.device):
         status = lib.trt_lt2exp_f32(
-            c_void_p(w.data_ptr()), c_void_p(a.data_ptr()), c_void_p(b.data_ptr()),
-            c_void_p(c.data_ptr()), R, S, I, J, K,
+            w.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), R, S, I, J, K,
             _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-            mode_code, _variant,
-            c_void_p(ws.data_ptr() if ws is not None else None), ws_bytes,
-            _lib.current_stream(a.device),
+            mode_code, _variant, ws.data_ptr() if ws_bytes else None, ws_bytes,
+            _lib.raw_stream(a.device),
         )
-    _lib.check(status, "trt_lt2exp_f32")
+    if status:
+        _lib.check(status, "trt_lt2exp_f32")
     return c

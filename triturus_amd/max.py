@@ -10,11 +10,11 @@ NaN handling follows torch.amax / torch.max (NaN propagates).
 
 from __future__ import annotations
 
-from ctypes import c_void_p
-
 import torch
 
 from triturus_amd import _lib
+
+_ws_bytes: dict = {}  # (op, shape..., dtype code) -> workspace bytes, as reported by the library
 
 
 def _dtype_code(x: torch.Tensor) -> int:
@@ -24,10 +24,6 @@ def _dtype_code(x: torch.Tensor) -> int:
         raise NotImplementedError(f"max reductions support fp32/fp64/fp16/bf16, got {x.dtype}") from None
 
 
-def _workspace(nbytes: int, device: torch.device) -> torch.Tensor | None:
-    return torch.empty(nbytes, dtype=torch.uint8, device=device) if nbytes else None
-
-
 def _vmax_impl(x: torch.Tensor, with_index: bool):
     _lib.require_gpu(x)
     lib = _lib.load()
@@ -35,18 +31,21 @@ def _vmax_impl(x: torch.Tensor, with_index: bool):
     n = x.shape[0]
     if n == 0:
         raise RuntimeError("max of an empty vector")
-    val = torch.empty((), dtype=x.dtype, device=x.device)
-    idx = torch.empty((), dtype=torch.int64, device=x.device) if with_index else None
-    ws_bytes = lib.trt_vmax_workspace_bytes(n, code)
-    ws = _workspace(ws_bytes, x.device)
-    with _lib.on_device(x.device):
+    dev = x.device
+    val = torch.empty((), dtype=x.dtype, device=dev)
+    idx = torch.empty((), dtype=torch.int64, device=dev) if with_index else None
+    key = ("v", n, code)
+    ws_bytes = _ws_bytes.get(key)
+    if ws_bytes is None:
+        ws_bytes = _ws_bytes[key] = lib.trt_vmax_workspace_bytes(n, code)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    with _lib.on_device(dev):
         status = lib.trt_vmax(
-            c_void_p(x.data_ptr()), n, code, c_void_p(val.data_ptr()),
-            c_void_p(idx.data_ptr() if idx is not None else None),
-            c_void_p(ws.data_ptr() if ws is not None else None), ws_bytes,
-            _lib.current_stream(x.device),
+            x.data_ptr(), n, code, val.data_ptr(), idx.data_ptr() if with_index else None,
+            ws.data_ptr() if ws_bytes else None, ws_bytes, _lib.raw_stream(dev),
         )
-    _lib.check(status, "trt_vmax")
+    if status:
+        _lib.check(status, "trt_vmax")
     return val, idx
 
 
@@ -75,14 +74,18 @@ def matmax(x: torch.Tensor, axis: int = 0, *, block_size: int = 32) -> torch.Ten
     m, n = x.shape
     if m == 0 or n == 0:
         raise RuntimeError("max of an empty matrix")
-    y = torch.empty(n if axis == 0 else m, dtype=x.dtype, device=x.device)
-    ws_bytes = lib.trt_matmax_workspace_bytes(m, n, axis, code)
-    ws = _workspace(ws_bytes, x.device)
-    with _lib.on_device(x.device):
+    dev = x.device
+    y = torch.empty(n if axis == 0 else m, dtype=x.dtype, device=dev)
+    key = ("m", m, n, axis, code)
+    ws_bytes = _ws_bytes.get(key)
+    if ws_bytes is None:
+        ws_bytes = _ws_bytes[key] = lib.trt_matmax_workspace_bytes(m, n, axis, code)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    with _lib.on_device(dev):
         status = lib.trt_matmax(
-            c_void_p(x.data_ptr()), c_void_p(y.data_ptr()), m, n, axis, code,
-            c_void_p(ws.data_ptr() if ws is not None else None), ws_bytes,
-            _lib.current_stream(x.device),
+            x.data_ptr(), y.data_ptr(), m, n, axis, code,
+            ws.data_ptr() if ws_bytes else None, ws_bytes, _lib.raw_stream(dev),
         )
-    _lib.check(status, "trt_matmax")
+    if status:
+        _lib.check(status, "trt_matmax")
     return y
