@@ -112,8 +112,8 @@ def test_workspace_queries_are_host_only_and_follow_the_mode_rule():
     assert lib.trt_lt2exp_workspace_bytes(64, 64, 64, 64, 4096, _lib.MODE_AUTO) == 0
     # lm2exp: splits only for small grids with a long contraction, or on request
     assert lib.trt_lm2exp_workspace_bytes(64, 256, 256, 4096, 0, 0) == 0
-    assert lib.trt_lm2exp_workspace_bytes(1, 1024, 1024, 1024, 0, 1) == 0
-    assert lib.trt_lm2exp_workspace_bytes(1, 1024, 1024, 1024, 0, 0) > 0
+    assert lib.trt_lm2exp_workspace_bytes(1, 128, 4096, 128, 0, 1) == 0
+    assert lib.trt_lm2exp_workspace_bytes(1, 128, 4096, 128, 0, 0) > 0
     assert lib.trt_lm2exp_workspace_bytes(1, 128, 64, 128, 0, 0) == 0  # two chunks: nothing to share
     assert lib.trt_lm2exp_workspace_bytes(16, 512, 512, 512, 0, 0) == 0  # 256 tiles, 16 chunks: not worth a merge
     assert lib.trt_lm2exp_workspace_bytes(2, 100, 256, 50, 0, 4) == 4 * (4 * 2 * 100 * 50 + 4 * 2 * 50)

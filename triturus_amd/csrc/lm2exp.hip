@@ -398,11 +398,45 @@ constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be op
 // Measured on MI355X at R=64, I=J=256, K=4096: the 128-row tiles (64 accumulator
 // registers, 3-4 wavefronts per SIMD) beat the 256-row tiles (128 accumulator
 // registers, 2 per SIMD) although b is then exponentiated once per row tile.
+// Smaller grids want smaller row tiles: a 128-row tile amortises each exp over four
+// MFMAs, but it only pays when there are enough tiles to keep 256 CUs busy with more
+// than one workgroup each.  Rules fitted to a sweep of all variants over the shapes of
+// the reference's benchmark grid (batch-1 squares 128..2048; R=64/384, n=256):
+//   >= 1.5 tiles of 128 rows per CU        128 x 128  (128 x 256 when a[r] outgrows an
+//                                          XCD's L2 and the wide tiles still fill the chip:
+//                                          one LDS copy of the a tile then serves 8 waves)
+//   >= 1.5 tiles of 64 rows per CU         64 x 128   (+2..5 %)
+//   fewer, long contraction (J >= 1280)    the largest tile that leaves >= 128 tiles
+//   fewer, short contraction               32 x 128   (+12..36 %)
+static int find_variant(int rt, int wn, bool online) {
+    for (int v = 0; v < kNumVariants; ++v)
+        if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].wm == 1 && kVariants[v].wn == wn &&
+            kVariants[v].nq == 4 && kVariants[v].online == online)
+            return v;
+    return 0;
+}
+
 static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
-    (void)R; (void)J; (void)K;
-    if (I > 64) return 0;
-    if (I > 32) return 6;
-    return 7;
+    const int64_t kFill = 384;  // 1.5 workgroups per CU
+    const int64_t ct = ceil_div(K, 128);
+    const int64_t n128 = R * ceil_div(I, 128) * ct, n64 = R * ceil_div(I, 64) * ct;
+    int rt;
+    if (I <= 32) {
+        rt = 1;
+    } else if (I <= 64) {
+        rt = (n64 >= kFill || J >= 1280) ? 2 : 1;
+    } else if (n128 >= kFill) {
+        if (I * J >= ((int64_t)1 << 20) && K % 256 == 0 && R * ceil_div(I, 128) * (K / 256) >= 512)
+            return find_variant(4, 8, true);
+        rt = 4;
+    } else if (n64 >= kFill) {
+        rt = 2;
+    } else if (J >= 1280) {
+        rt = n128 >= 128 ? 4 : (n64 >= 128 ? 2 : 1);
+    } else {
+        rt = 1;
+    }
+    return find_variant(rt, 4, true);
 }
 
 template <int RT, int CT, int WM, int WN, int NQ, bool VEC, bool ONLINE>

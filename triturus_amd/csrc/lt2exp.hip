@@ -322,9 +322,17 @@ constexpr int kLt2Waves = 4;
 // Measured on MI355X at R=64, S=I=J=64, K=4096: the narrow wavefront tile (64 x 32,
 // 32 accumulator registers, j-chunks of 32) runs at 87% of the fp32 MFMA peak, the
 // 64 x 64 tiles at 81-85%: occupancy beats operand reuse here.
+// Small grids want the 32-row tile (measured +8..25 % on batch-1 squares of 64..128 and on
+// R=32..128, S=I=J=64, K=256): with fewer than half a workgroup per CU the chip is not full
+// either way and the shorter tile halves each workgroup's chain; up to 1.5 per CU it still
+// wins while the contraction is short (I*J <= 4096).  Long contractions on a filling grid keep
+// the 64-row tile, whose Khatri-Rao multiply is shared by two MFMAs.
 static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
-    (void)R; (void)I; (void)J; (void)K;
-    const int rt = S > 32 ? 2 : 1;
+    int rt = S > 32 ? 2 : 1;
+    if (rt == 2) {
+        const int64_t n64 = R * ceil_div(S, 64) * ceil_div(K, 128);
+        if (n64 < 128 || (n64 < 384 && I * J <= 4096)) rt = 1;
+    }
     for (int v = 0; v < kNumVariants; ++v)
         if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == 4) return v;
     return 0;
