@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TRT_ABI_VERSION 2
+#define TRT_ABI_VERSION 3
 
 #define TRT_OK 0
 #define TRT_E_INVALID (-1)   /* null pointer, non-positive size, bad enum   */
@@ -104,6 +104,25 @@ int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c,
 size_t trt_lt2exp_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t J,
                                   int64_t K, int mode);
 int trt_lt2exp_variant_count(void);
+
+/*
+ * The same contraction as trt_lt2exp_f32 (fp32 tensors in and out, same layouts, strides
+ * and status codes) on the bf16 matrix pipe: every fp32 operand is cut into `pieces` bf16
+ * pieces and a product is the sum of the piece products that matter, accumulated in fp32.
+ *   pieces = 2 (TRT_PIECES_BF16X3): 3 MFMAs per product, relative error ~2^-16 per product
+ *   pieces = 3 (TRT_PIECES_BF16X6): 6 MFMAs per product, relative error ~2^-23 per product
+ * This is the library's counterpart of the reference's reduced-precision mode
+ * (ALLOW_TF32 passed to tl.dot, triturus/lt2exp.py:345, flag triturus/utils.py:33-44):
+ * gfx950 has no TF32 matrix instruction; two bf16 pieces are more accurate than TF32
+ * (2^-11) and several times faster than the fp32 matrix pipe.  Always unsplit; needs no
+ * workspace.  variant: 0 = choose by shape, 1..4 pick a tile shape (experiments, tests).
+ */
+#define TRT_PIECES_BF16X3 2
+#define TRT_PIECES_BF16X6 3
+int trt_lt2exp_bf16(const float *w, const float *a, const float *b, float *c,
+                    int64_t R, int64_t S, int64_t I, int64_t J, int64_t K,
+                    const int64_t sw[3], const int64_t sa[3], const int64_t sb[3],
+                    const int64_t sc[3], int pieces, int variant, void *stream);
 
 /*
  * Max of a contiguous m x n row-major matrix along axis 0 (y has n entries)

@@ -14,7 +14,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtriturus_hip.so"
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 TRT_F32, TRT_F64, TRT_F16, TRT_BF16 = 0, 1, 2, 3
 MODE_AUTO, MODE_SPLIT, MODE_UNSPLIT = 0, 1, 2
@@ -44,6 +44,11 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
          POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
          c_int, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "trt_lt2exp_bf16": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+         POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int, c_int, c_void_p],
     ),
     "trt_lt2exp_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int]),
     "trt_lt2exp_variant_count": (c_int, []),

@@ -1,0 +1,427 @@
+// lt2exp on the bf16 matrix pipe of gfx950, fp32 in and out:
+//   c[r,s,k] = log sum_{i,j} w[r,s,i,j] exp(a[r,i,k]) exp(b[r,j,k])
+//
+// The reference has a reduced-precision mode (TF32 operands, triturus/utils.py:33-44,
+// passed to tl.dot at triturus/lt2exp.py:345); gfx950 has no TF32 matrix instruction.
+// Its bf16 matrix pipe is 16x faster than the fp32 one, so each fp32 operand is cut
+// into NS bf16 pieces (x = x0 + x1 [+ x2], each the bf16 rounding of what the previous
+// pieces left) and a product is the sum of the piece products that matter:
+//   NS = 2:  x0 y0 + x0 y1 + x1 y0                        3 MFMAs, error ~2^-16 per product
+//   NS = 3:  ... + x0 y2 + x1 y1 + x2 y0                  6 MFMAs, error ~2^-23 per product
+// accumulated in fp32 by v_mfma_f32_32x32x16_bf16.  Unlike the fp32 MFMA, the bf16 MFMA
+// runs beside the vector ALU, so the splitting work is hidden as long as it is shorter
+// than the MFMAs it feeds.  To keep it short the Khatri-Rao product is never formed:
+//   sum_{i,j} w[s,i,j] ea[i,n] eb[j,n] = sum_i ea[i,n] * ( sum_j w[s,i,j] eb[j,n] )
+// so the B operand is eb alone (split once per column tile and j-chunk, reused for every
+// i) and the per-i factor ea[i,n] scales the 32 x 32 result tile of each i on its way
+// into the running sum (one fma per accumulator register, in fp32).
+//
+// A workgroup of 4 wavefronts owns 32*RT rows of S and 128 columns of K.  For RT = 2 the
+// wavefronts are arranged 2 x 2 and each owns 32 rows x 64 columns, so that an LDS read of
+// the w tile feeds two MFMAs (LDS bandwidth, not the matrix pipe, is the nearest limit at
+// this MFMA rate); for RT = 1 they are 1 x 4.  w tiles go global -> registers -> split ->
+// LDS (double buffered).  MFMA k-slot mapping: element e of lane-half h in k-step ks
+// of a chunk is j = 16 ks + 8 h + e for both operands.
+
+#include "common.hpp"
+
+namespace trt {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
+
+struct Lt2BfArgs {
+    const float *w, *a, *b;
+    float *c;
+    int R, S, I, J, K;
+    int64_t sw0, sw1, sa0, sa1, sb0, sb1, sc0, sc1;
+    int s_tiles, n_tiles;
+    int64_t total_wgs, padded_wgs;
+};
+
+// two fp32 -> one register of two bf16 (round to nearest even), element 0 in the low half
+__device__ __forceinline__ uint32_t pack_bf16(float x0, float x1) {
+    floatx2 v = {x0, x1};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+__device__ __forceinline__ float bf16_lo_as_f32(uint32_t pk) { return __builtin_bit_cast(float, pk << 16); }
+__device__ __forceinline__ float bf16_hi_as_f32(uint32_t pk) { return __builtin_bit_cast(float, pk & 0xffff0000u); }
+
+// Cut (x0, x1) into NS bf16 pieces each: out[s] holds piece s of both.  The subtraction is
+// exact (the piece agrees with x in its leading bits).  An infinite x leaves inf - inf = NaN
+// in the later pieces; with KEEP_INF those are set to 0 so that inf stays inf (two more
+// instructions per value: used where the count does not matter).
+template <int NS, bool KEEP_INF>
+__device__ __forceinline__ void split_pair(float x0, float x1, uint32_t (&out)[NS]) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        out[s] = pack_bf16(x0, x1);
+        if (s + 1 < NS) {
+            const float f0 = bf16_lo_as_f32(out[s]), f1 = bf16_hi_as_f32(out[s]);
+            x0 = (KEEP_INF && __builtin_isinf(f0)) ? 0.f : x0 - f0;
+            x1 = (KEEP_INF && __builtin_isinf(f1)) ? 0.f : x1 - f1;
+        }
+    }
+}
+
+template <int RT, int KS, int NS, bool VEC>
+__global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) {
+    constexpr int NT = 256;
+    constexpr int TS = 32 * RT;    // rows of S per workgroup
+    constexpr int CT = RT;         // 32-column tiles per wavefront: RT = 2 arranges the 4 wavefronts
+                                   // 2 x 2 (each 32 rows x 64 columns), RT = 1 arranges them 1 x 4
+    constexpr int WN = 4 / RT;     // wavefronts along the columns
+    constexpr int JC = 16 * KS;    // j per chunk
+    constexpr int LDA = JC + 8;    // padded LDS row in bf16 (16 bytes of padding: conflict-free 16-byte reads)
+    constexpr int F4_PER_ROW = JC / 4;
+    constexpr int ROWS_PER_SLOT = NT / F4_PER_ROW;
+    constexpr int SLOTS = TS * F4_PER_ROW / NT;
+    static_assert(TS * F4_PER_ROW % NT == 0, "tile must divide over the threads");
+    constexpr int TN = 128;
+
+    __shared__ __attribute__((aligned(16))) __bf16 wt[2][NS][TS * LDA];
+
+    const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
+    if (L >= p.total_wgs) return;
+    int64_t rest = L / p.n_tiles;
+    const int nt = __builtin_amdgcn_readfirstlane((int)(L % p.n_tiles));
+    const int st = __builtin_amdgcn_readfirstlane((int)(rest % p.s_tiles));
+    const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.s_tiles));
+
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int lane = tid % kWave;
+    const int h = lane / 32;
+    const int m = lane % 32;
+    const int wm = wave / WN;  // row tile of this wavefront
+    const int wn = wave % WN;
+    const int s0 = st * TS;
+    int ncol[CT], ncl[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        ncol[ct] = nt * TN + wn * 32 * CT + 32 * ct + m;
+        ncl[ct] = ncol[ct] < p.K ? ncol[ct] : p.K - 1;
+    }
+
+    const float *ar = p.a + (int64_t)r * p.sa0;
+    const float *br = p.b + (int64_t)r * p.sb0;
+    const float *wr = p.w + (int64_t)r * p.sw0;
+
+    // ---- clamped column maxima (baselines/lt2exp.py:15-19): the lane halves take
+    // alternate rows and exchange once
+    float ma[CT], mb[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        float x = -__builtin_inff();
+#pragma unroll 8
+        for (int i = h; i < p.I; i += 2) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + ncl[ct]]);
+        x = __builtin_fmaxf(x, __shfl_xor(x, 32, kWave));
+        ma[ct] = clamp_shift(x);
+        float y = -__builtin_inff();
+#pragma unroll 8
+        for (int j = h; j < p.J; j += 2) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + ncl[ct]]);
+        y = __builtin_fmaxf(y, __shfl_xor(y, 32, kWave));
+        mb[ct] = clamp_shift(y);
+    }
+
+    const int n_jc = (p.J + JC - 1) / JC;
+    const int total_iters = n_jc * p.I;
+
+    floatx16 total[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) total[ct][v] = 0.f;
+
+    // ---- w tile staging (same addressing as the fp32 kernel: buffer resource whose
+    // extent ends at the last valid row, so rows past S read as zeros)
+    floatx4 stage[SLOTS];
+    const int trow = tid / F4_PER_ROW;
+    const int tc4 = tid % F4_PER_ROW;
+    const int wrows = (p.S - s0) < TS ? (p.S - s0) : TS;
+    const float *wtile0 = wr + (int64_t)s0 * p.sw1;
+    const __amdgpu_buffer_rsrc_t w_rsrc =
+        make_rsrc(wtile0, (uint32_t)(((int64_t)(wrows - 1) * p.sw1 + (int64_t)p.I * p.J) * 4));
+    uint32_t woff[SLOTS];
+#pragma unroll
+    for (int sidx = 0; sidx < SLOTS; ++sidx)
+        woff[sidx] = ((uint32_t)(trow + sidx * ROWS_PER_SLOT) * (uint32_t)p.sw1 + 4u * tc4) * 4u;
+    auto load_tile = [&](int i, int jc) {
+        const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
+        if (full) {
+            const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx) stage[sidx] = buf_load_f32x4(w_rsrc, woff[sidx], soff);
+        } else {
+            const int j = jc * JC + 4 * tc4;
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx) {
+                const int row = trow + sidx * ROWS_PER_SLOT;
+                const float *src = wtile0 + (int64_t)row * p.sw1 + (int64_t)i * p.J + j;
+                floatx4 v = {0.f, 0.f, 0.f, 0.f};
+                if (row < wrows) {
+                    if (j + 0 < p.J) v[0] = src[0];
+                    if (j + 1 < p.J) v[1] = src[1];
+                    if (j + 2 < p.J) v[2] = src[2];
+                    if (j + 3 < p.J) v[3] = src[3];
+                }
+                stage[sidx] = v;
+            }
+        }
+    };
+    // split the staged fp32 values and write the pieces to LDS (8 bytes per piece and slot)
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int sidx = 0; sidx < SLOTS; ++sidx) {
+            uint32_t p01[NS], p23[NS];
+            split_pair<NS, false>(stage[sidx][0], stage[sidx][1], p01);
+            split_pair<NS, false>(stage[sidx][2], stage[sidx][3], p23);
+            const int off = (trow + sidx * ROWS_PER_SLOT) * LDA + 4 * tc4;
+#pragma unroll
+            for (int sp = 0; sp < NS; ++sp) {
+                uintx2 v = {p01[sp], p23[sp]};
+                *reinterpret_cast<uintx2 *>(&wt[buf][sp][off]) = v;
+            }
+        }
+    };
+
+    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ar, (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + p.K) * 4));
+    const uint32_t a_row_bytes = (uint32_t)p.sa1 * 4u;
+    uint32_t aoff[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) aoff[ct] = (uint32_t)ncl[ct] * 4u;
+
+    // B operand: exp(b[j,n] - mb[n]) of the current j-chunk, split, in MFMA layout
+    uintx4 ebp[CT][NS][KS];
+    auto load_eb = [&](int jc) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) {
+                float e[8];
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const int j = jc * JC + 16 * ks + 8 * h + u;
+                    float raw = -__builtin_inff();
+                    if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl[ct]];
+                    e[u] = exp_shifted(raw - mb[ct]);
+                }
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    uint32_t pk[NS];
+                    split_pair<NS, true>(e[2 * u], e[2 * u + 1], pk);
+#pragma unroll
+                    for (int sp = 0; sp < NS; ++sp) ebp[ct][sp][ks][u] = pk[sp];
+                }
+            }
+    };
+
+    if (total_iters > 0) {
+        int jc = 0, i = 0;
+        load_tile(0, 0);
+        load_eb(0);
+        float ea[CT], ea_raw[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) ea[ct] = exp_shifted(ar[ncl[ct]] - ma[ct]);
+        store_tile(0);
+        __syncthreads();
+
+        // ---- one (i, j-chunk) and 32-column tile: inner = w tile x eb (3 or 6 MFMAs per
+        // k-step, starting from zero), then total += ea[i,n] * inner
+        bf16x8 af[NS][KS];
+        auto load_a = [&](int buf) {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int sp = 0; sp < NS; ++sp)
+                    af[sp][ks] = *reinterpret_cast<const bf16x8 *>(&wt[buf][sp][(32 * wm + m) * LDA + 16 * ks + 8 * h]);
+        };
+        auto mfma_cols = [&](int ct, floatx16 &inn) {
+            bool first = true;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int sa = 0; sa < NS; ++sa)
+#pragma unroll
+                    for (int sb = 0; sa + sb < NS; ++sb) {
+                        const bf16x8 bop = __builtin_bit_cast(bf16x8, ebp[ct][sb][ks]);
+                        if (first) {
+                            const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
+                                                   0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+                            inn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[sa][ks], bop, zero, 0, 0, 0);
+                        } else {
+                            inn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[sa][ks], bop, inn, 0, 0, 0);
+                        }
+                        first = false;
+                    }
+        };
+        // The empty asm pins the fmas to this place in the instruction stream: their results
+        // are not needed before the next step, and the compiler would otherwise sink them
+        // out of the MFMA block they are meant to overlap with.
+        auto scale_add = [&](floatx16 &tot, const floatx16 &inn, float e) {
+#pragma unroll
+            for (int v = 0; v < 16; ++v) tot[v] = __builtin_fmaf(inn[v], e, tot[v]);
+            asm volatile("" : "+v"(tot));
+        };
+
+        int cur = 0;
+        if constexpr (CT == 2) {
+            // Two half-steps per (i, j-chunk).  While the MFMAs of column tile 0 run, the vector
+            // ALU adds the previous step's column tile 1 into the running sum; while those of
+            // column tile 1 run, it adds column tile 0 and splits the prefetched w tile.
+            floatx16 inner0, inner1;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) inner1[v] = 0.f;
+            float ea_old = 0.f;
+            for (int it = 0; it + 1 < total_iters; ++it) {
+                int ni = i + 1, njc = jc;
+                if (ni == p.I) {
+                    ni = 0;
+                    njc = jc + 1;
+                }
+                load_tile(ni, njc);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct)
+                    ea_raw[ct] = buf_load_f32(a_rsrc, aoff[ct], (uint32_t)ni * a_row_bytes);
+                __builtin_amdgcn_sched_barrier(0);
+                load_a(cur);
+                mfma_cols(0, inner0);
+                scale_add(total[1], inner1, ea_old);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_cols(1, inner1);
+                scale_add(total[0], inner0, ea[0]);
+                store_tile(cur ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+                ea_old = ea[1];
+                if (njc != jc) load_eb(njc);
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) ea[ct] = exp_shifted(ea_raw[ct] - ma[ct]);
+                __syncthreads();
+                cur ^= 1;
+                i = ni;
+                jc = njc;
+            }
+            load_a(cur);
+            mfma_cols(0, inner0);
+            scale_add(total[1], inner1, ea_old);
+            mfma_cols(1, inner1);
+            scale_add(total[0], inner0, ea[0]);
+            scale_add(total[1], inner1, ea[1]);
+        } else {
+            floatx16 inner;
+            for (int it = 0; it + 1 < total_iters; ++it) {
+                int ni = i + 1, njc = jc;
+                if (ni == p.I) {
+                    ni = 0;
+                    njc = jc + 1;
+                }
+                load_tile(ni, njc);
+                ea_raw[0] = buf_load_f32(a_rsrc, aoff[0], (uint32_t)ni * a_row_bytes);
+                __builtin_amdgcn_sched_barrier(0);
+                load_a(cur);
+                mfma_cols(0, inner);
+                scale_add(total[0], inner, ea[0]);
+                store_tile(cur ^ 1);
+                if (njc != jc) load_eb(njc);
+                ea[0] = exp_shifted(ea_raw[0] - ma[0]);
+                __syncthreads();
+                cur ^= 1;
+                i = ni;
+                jc = njc;
+            }
+            load_a(cur);
+            mfma_cols(0, inner);
+            scale_add(total[0], inner, ea[0]);
+        }
+    }
+
+    // ---- epilogue: register v of lane (h, m) holds row 8*(v/4) + 4*h + v%4, column m of
+    // the wavefront's 32 x 32 tile
+    const int crows = p.S - s0;
+    const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)s0 * p.sc1,
+                                                    (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4));
+    const uint32_t c_row_bytes = (uint32_t)p.sc1 * 4u;
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        if (ncol[ct] >= p.K) continue;
+        const float mm = ma[ct] + mb[ct];
+        const uint32_t co = ((uint32_t)(32 * wm + 4 * h) * (uint32_t)p.sc1 + (uint32_t)ncol[ct]) * 4u;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const uint32_t trow_c = 8 * (v / 4) + (v % 4);
+            buf_store_f32_stream(log_plus(total[ct][v], mm), c_rsrc, co, trow_c * c_row_bytes);
+        }
+    }
+}
+
+template <int RT, int KS, int NS>
+static void launch_bf(const Lt2BfArgs &args, bool vec, hipStream_t stream) {
+    if (vec)
+        hipLaunchKernelGGL((lt2exp_bf16_kernel<RT, KS, NS, true>), dim3((unsigned)args.padded_wgs), dim3(256), 0,
+                           stream, args);
+    else
+        hipLaunchKernelGGL((lt2exp_bf16_kernel<RT, KS, NS, false>), dim3((unsigned)args.padded_wgs), dim3(256), 0,
+                           stream, args);
+}
+
+template <int NS>
+static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, hipStream_t stream) {
+    if (rt == 2) {
+        if (ks == 4) launch_bf<2, 4, NS>(args, vec, stream);
+        else launch_bf<2, 2, NS>(args, vec, stream);
+    } else {
+        if (ks == 4) launch_bf<1, 4, NS>(args, vec, stream);
+        else launch_bf<1, 2, NS>(args, vec, stream);
+    }
+}
+
+}  // namespace trt
+
+using namespace trt;
+
+extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, float *c, int64_t R, int64_t S,
+                               int64_t I, int64_t J, int64_t K, const int64_t sw[3], const int64_t sa[3],
+                               const int64_t sb[3], const int64_t sc[3], int pieces, int variant, void *stream) {
+    if (!w || !a || !b || !c || !sw || !sa || !sb || !sc) return TRT_E_INVALID;
+    if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
+    if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
+    if (variant < 0 || variant > 4) return TRT_E_INVALID;
+    if (sw[2] != 1 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
+    for (int d = 0; d < 2; ++d)
+        if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
+    if (sc[1] < K) return TRT_E_LAYOUT;
+    const int64_t lim = (int64_t)1 << 30;
+    if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
+    if (S * sw[1] + I * J >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
+
+    // 32-row tiles for small grids (same reasoning as the fp32 kernel), j-chunks of 64
+    // unless J fits 32
+    int rt = S > 32 ? 2 : 1;
+    if (rt == 2 && R * ceil_div(S, 64) * ceil_div(K, 128) < 384) rt = 1;
+    int ks = J > 32 ? 4 : 2;
+    if (variant >= 1) {  // 1: 64 rows, chunks of 64;  2: 64 rows, 32;  3: 32 rows, 64;  4: 32 rows, 32
+        rt = variant <= 2 ? 2 : 1;
+        ks = (variant & 1) ? 4 : 2;
+    }
+
+    Lt2BfArgs args;
+    args.w = w; args.a = a; args.b = b; args.c = c;
+    args.R = (int)R; args.S = (int)S; args.I = (int)I; args.J = (int)J; args.K = (int)K;
+    args.sw0 = sw[0]; args.sw1 = sw[1];
+    args.sa0 = sa[0]; args.sa1 = sa[1];
+    args.sb0 = sb[0]; args.sb1 = sb[1];
+    args.sc0 = sc[0]; args.sc1 = sc[1];
+    args.s_tiles = (int)ceil_div(S, 32 * rt);
+    args.n_tiles = (int)ceil_div(K, 128);
+    args.total_wgs = (int64_t)R * args.s_tiles * args.n_tiles;
+    args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+    const bool vec = (J % 4 == 0) && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) &&
+                     ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (pieces == 2) launch_bf_shape<2>(args, rt, ks, vec, s);
+    else launch_bf_shape<3>(args, rt, ks, vec, s);
+    return (int)hipGetLastError();
+}

@@ -14,6 +14,7 @@ import torch
 
 from triturus_amd import _lib
 from triturus_amd.lm2exp import _unit_inner
+from triturus_amd.utils import is_triturus_tf32_enabled
 
 _ws_bytes: dict = {}  # (R, S, I, J, K, mode) -> workspace bytes, as reported by the library
 
@@ -31,8 +32,12 @@ def launches_split(R: int, S: int, I: int, J: int, K: int, mode: str) -> bool:
     raise ValueError(f"Uknown mode '{mode}' for the l2exp kernel")
 
 
+_PIECES = {"bf16x3": 2, "bf16x6": 3}
+
+
 def lt2exp(
-    w: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, mode: str = "auto", _variant: int = 0
+    w: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, mode: str = "auto", _variant: int = 0,
+    _precision: str | None = None,
 ) -> torch.Tensor:
     assert len(w.shape) == 4
     assert len(a.shape) == len(b.shape) == 3
@@ -59,6 +64,18 @@ def lt2exp(
     w = _unit_inner(w)
     a = _unit_inner(a)
     b = _unit_inner(b)
+    if _precision is None:
+        _precision = "bf16x3" if is_triturus_tf32_enabled() else "fp32"
+    if _precision != "fp32":
+        with _lib.on_device(a.device):
+            status = lib.trt_lt2exp_bf16(
+                w.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), R, S, I, J, K,
+                _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
+                _PIECES[_precision], _variant, _lib.raw_stream(a.device),
+            )
+        if status:
+            _lib.check(status, "trt_lt2exp_bf16")
+        return c
     mode_code = _MODES[mode]
     key = (R, S, I, J, K, mode_code)
     ws_bytes = _ws_bytes.get(key)
