@@ -82,6 +82,12 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, s3(1, 1, 2), ok, 0, 0, null, 0, null) == -2
     big4 = (2, 8, 16, 16, 64, s3(2048, 256, 1), s3(1024, 64, 1), s3(1024, 64, 1), s3(512, 64, 1))
     assert lib.trt_lt2exp_f32(one, one, one, one, *big4, _lib.MODE_SPLIT, 0, null, 0, null) == -3  # split needs a workspace
+    # lt2exp on the bf16 matrix pipe: pieces must be 2 or 3, variant 0..4
+    assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 4, 0, null) == -1
+    assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 2, 9, null) == -1
+    assert lib.trt_lt2exp_bf16(null, one, one, one, *args, 2, 0, null) == -1
+    assert lib.trt_lt2exp_bf16(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, 2), ok, ok, ok, 2, 0, null) == -2
+    assert lib.trt_lt2exp_bf16(one, one, one, one, 1 << 31, 1, 1, 1, 1, ok, ok, ok, ok, 3, 0, null) == -4
     # max
     assert lib.trt_vmax(null, 5, 0, one, one, one, 1 << 20, null) == -1
     assert lib.trt_vmax(one, 0, 0, one, one, one, 1 << 20, null) == -1

@@ -21,6 +21,13 @@ pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
 N_VARIANTS = 8
+N_BF16_VARIANTS = 4
+# Accuracy gates of the split-bf16 paths against the float64 oracle.  Two pieces (3 MFMAs per
+# product) carry 16 significand bits: looser than fp32, ten times tighter than the rtol 5e-4
+# the reference allows its TF32 mode (tests/lt2exp.py:38).  Three pieces (6 MFMAs) carry 24
+# bits and must pass the fp32 gate unchanged.
+BF16X3_GATE = {"rtol": 1e-4, "atol": 5e-5}
+PRECISION_GATES = {"bf16x3": BF16X3_GATE, "bf16x6": {}}
 
 
 def _check(out, w, a, b, **kw):
@@ -41,11 +48,13 @@ def test_lt2exp(dev, mode, allow_tf32):
     c = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode)
     assert c.shape == (batch, m, n) and c.dtype == torch.float32 and c.device.type == "cuda"
     if allow_tf32:
+        # the flag selects the split-bf16 path (error ~2^-16 per product; TF32 has 2^-11)
         assert torch.allclose(gt, c.cpu(), rtol=5e-4)
+        _check(c, w, a, b, **BF16X3_GATE)
     else:
         assert torch.allclose(gt, c.cpu())
-    assert torch.allclose(torch_baseline.lt2exp_fp32(w.to(dev), a.to(dev), b.to(dev)), c)
-    _check(c, w, a, b)
+        assert torch.allclose(torch_baseline.lt2exp_fp32(w.to(dev), a.to(dev), b.to(dev)), c)
+        _check(c, w, a, b)
 
 
 @pytest.mark.parametrize("name", ["lt2exp_small", "lt2exp_ragged"])
@@ -242,3 +251,85 @@ def test_capturable_in_a_hip_graph(dev):
         assert torch.equal(out_t_split, lt2exp(w, a, b, mode="split"))
         assert torch.equal(out_m, lm2exp(a2, b))
         torch.cuda.synchronize()
+
+
+# ------------------------------------------------------------ split-bf16 matrix path
+@pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
+@pytest.mark.parametrize("variant", range(0, N_BF16_VARIANTS + 1))
+@pytest.mark.parametrize(
+    "shape", [(3, 75, 50, 50, 100), (2, 35, 9, 13, 45), (1, 70, 20, 33, 300), (2, 16, 5, 72, 64), (1, 33, 3, 3, 31),
+              (2, 64, 64, 64, 256), (1, 1, 1, 1, 1), (2, 130, 4, 128, 129)])
+def test_bf16_paths_on_ragged_shapes(dev, precision, variant, shape):
+    R, S, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape) + variant)
+    w = torch.rand(R, S, I, J, generator=g)
+    a = torch.randn(R, I, K, generator=g) * 4 - 3
+    b = torch.randn(R, J, K, generator=g) * 4 + 2
+    a[torch.rand(a.shape, generator=g) < 0.05] = NINF
+    b[:, :, 0] = NINF  # an all -inf column: -inf out, not NaN
+    w[:, 0] = 0.0  # a zero row of weights: -inf out
+    out = lt2exp(w.to(dev), a.to(dev), b.to(dev), _precision=precision, _variant=variant)
+    r = _check(out, w, a, b, **PRECISION_GATES[precision])
+    assert r["n_neg_inf"] > 0
+
+
+@pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
+def test_bf16_paths_strided_and_extreme(dev, precision):
+    g = torch.Generator().manual_seed(7)
+    R, S, I, J, K = 2, 40, 12, 20, 70
+    wbig = torch.rand(R, S + 3, I, J, generator=g)
+    abig = torch.randn(R, I + 2, K + 5, generator=g)
+    bbig = torch.randn(R, J, K + 9, generator=g)
+    w, a, b = wbig[:, 1 : S + 1], abig[:, 1 : I + 1, 2 : K + 2], bbig[:, :, 3 : K + 3]
+    out = lt2exp(w.to(dev), a.to(dev), b.to(dev), _precision=precision)
+    _check(out, w, a, b, **PRECISION_GATES[precision])
+    # large magnitudes and a huge dynamic range: the shifts keep every piece finite
+    a2 = a * 1e3 + 5e4
+    b2 = b * 30 - 9e6
+    out = lt2exp(w.to(dev), a2.contiguous().to(dev), b2.contiguous().to(dev), _precision=precision)
+    ref = oracle64.lt2exp64(w, a2, b2)
+    assert torch.isfinite(out).all()
+    assert torch.allclose(out.cpu().double(), ref, rtol=1e-6, atol=1e-3)
+    # NaN in a log-value poisons its column, nothing else
+    b3 = b.clone()
+    b3[0, 3, 5] = float("nan")
+    out = lt2exp(w.to(dev), a.to(dev), b3.to(dev), _precision=precision)
+    assert torch.isnan(out[0, :, 5]).all()
+    mask = torch.ones_like(out, dtype=torch.bool)
+    mask[0, :, 5] = False
+    assert not torch.isnan(out[mask]).any()
+
+
+def test_bf16x6_is_as_accurate_as_the_fp32_kernel(dev):
+    """Three bf16 pieces hold all 24 significand bits: against float64 the error of the
+    6-MFMA path must stay within twice that of the fp32 MFMA kernel on the same inputs."""
+    c = workloads.c4()
+    w, a, b = c["w"], c["a"], c["b"]
+    ref = oracle64.lt2exp64(w, a, b)
+    e32 = oracle64.compare(lt2exp(w.to(dev), a.to(dev), b.to(dev)), ref)
+    e6 = oracle64.compare(lt2exp(w.to(dev), a.to(dev), b.to(dev), _precision="bf16x6"), ref)
+    e3 = oracle64.compare(lt2exp(w.to(dev), a.to(dev), b.to(dev), _precision="bf16x3"), ref, **BF16X3_GATE)
+    assert e32["ok"] and e6["ok"] and e3["ok"], (e32, e6, e3)
+    assert e6["max_abs_err"] <= 2 * e32["max_abs_err"] + 1e-6, (e6, e32)
+
+
+@pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
+def test_bf16_paths_c5_full_size(dev, precision):
+    """Full-size check through properties that need no oracle: shifting a column of a or b
+    by t shifts the output column by t, scaling a row of w by 2^k adds k*log(2) exactly up
+    to rounding, and a sample of batches is compared with the float64 oracle."""
+    c = workloads.c5()
+    w, a, b = (c[k].to(dev) for k in "wab")
+    out = lt2exp(w, a, b, _precision=precision)
+    gate = PRECISION_GATES[precision]
+    for r in (0, 37, 63):
+        ref = oracle64.lt2exp64(c["w"][r : r + 1], c["a"][r : r + 1], c["b"][r : r + 1])
+        res = oracle64.compare(out[r : r + 1], ref, **gate)
+        assert res["ok"], (r, res)
+    t = torch.linspace(-7.0, 9.0, a.shape[2], device=dev)
+    out_shift = lt2exp(w, a + t, b - 2 * t, _precision=precision)
+    fin = torch.isfinite(out)
+    assert torch.equal(torch.isfinite(out_shift), fin)
+    assert torch.allclose(out_shift[fin], (out - t)[fin], rtol=1e-4, atol=2e-4)
+    out_scaled = lt2exp(w * 8.0, a, b, _precision=precision)
+    assert torch.allclose(out_scaled[fin], (out + float(np.log(8.0)))[fin], rtol=1e-6, atol=1e-5)

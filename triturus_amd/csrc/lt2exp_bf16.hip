@@ -16,11 +16,11 @@
 // i) and the per-i factor ea[i,n] scales the 32 x 32 result tile of each i on its way
 // into the running sum (one fma per accumulator register, in fp32).
 //
-// A workgroup of 4 wavefronts owns 32*RT rows of S and 128 columns of K.  For RT = 2 the
-// wavefronts are arranged 2 x 2 and each owns 32 rows x 64 columns, so that an LDS read of
-// the w tile feeds two MFMAs (LDS bandwidth, not the matrix pipe, is the nearest limit at
-// this MFMA rate); for RT = 1 they are 1 x 4.  w tiles go global -> registers -> split ->
-// LDS (double buffered).  MFMA k-slot mapping: element e of lane-half h in k-step ks
+// Tiling as in the fp32 kernel: a workgroup of 4 wavefronts owns 32*RT rows of S and 128
+// columns of K, a wavefront 32 of those columns for all rows; w tiles go global ->
+// registers -> split -> LDS (double buffered).  (A 2 x 2 arrangement of the wavefronts,
+// which halves the LDS reads per MFMA, was measured slower: it needs the B pieces of two
+// column tiles in registers and spills.)  MFMA k-slot mapping: element e of lane-half h in k-step ks
 // of a chunk is j = 16 ks + 8 h + e for both operands.
 
 #include "common.hpp"
@@ -70,9 +70,6 @@ template <int RT, int KS, int NS, bool VEC>
 __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) {
     constexpr int NT = 256;
     constexpr int TS = 32 * RT;    // rows of S per workgroup
-    constexpr int CT = RT;         // 32-column tiles per wavefront: RT = 2 arranges the 4 wavefronts
-                                   // 2 x 2 (each 32 rows x 64 columns), RT = 1 arranges them 1 x 4
-    constexpr int WN = 4 / RT;     // wavefronts along the columns
     constexpr int JC = 16 * KS;    // j per chunk
     constexpr int LDA = JC + 8;    // padded LDS row in bf16 (16 bytes of padding: conflict-free 16-byte reads)
     constexpr int F4_PER_ROW = JC / 4;
@@ -95,15 +92,9 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     const int lane = tid % kWave;
     const int h = lane / 32;
     const int m = lane % 32;
-    const int wm = wave / WN;  // row tile of this wavefront
-    const int wn = wave % WN;
     const int s0 = st * TS;
-    int ncol[CT], ncl[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        ncol[ct] = nt * TN + wn * 32 * CT + 32 * ct + m;
-        ncl[ct] = ncol[ct] < p.K ? ncol[ct] : p.K - 1;
-    }
+    const int ncol = nt * TN + wave * 32 + m;
+    const int ncl = ncol < p.K ? ncol : p.K - 1;
 
     const float *ar = p.a + (int64_t)r * p.sa0;
     const float *br = p.b + (int64_t)r * p.sb0;
@@ -111,32 +102,28 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 
     // ---- clamped column maxima (baselines/lt2exp.py:15-19): the lane halves take
     // alternate rows and exchange once
-    float ma[CT], mb[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        float x = -__builtin_inff();
+    float x = -__builtin_inff();
 #pragma unroll 8
-        for (int i = h; i < p.I; i += 2) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + ncl[ct]]);
-        x = __builtin_fmaxf(x, __shfl_xor(x, 32, kWave));
-        ma[ct] = clamp_shift(x);
-        float y = -__builtin_inff();
+    for (int i = h; i < p.I; i += 2) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + ncl]);
+    x = __builtin_fmaxf(x, __shfl_xor(x, 32, kWave));
+    const float ma = clamp_shift(x);
+    float y = -__builtin_inff();
 #pragma unroll 8
-        for (int j = h; j < p.J; j += 2) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + ncl[ct]]);
-        y = __builtin_fmaxf(y, __shfl_xor(y, 32, kWave));
-        mb[ct] = clamp_shift(y);
-    }
+    for (int j = h; j < p.J; j += 2) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + ncl]);
+    y = __builtin_fmaxf(y, __shfl_xor(y, 32, kWave));
+    const float mb = clamp_shift(y);
 
     const int n_jc = (p.J + JC - 1) / JC;
     const int total_iters = n_jc * p.I;
 
-    floatx16 total[CT];
+    floatx16 total[RT];
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct)
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-        for (int v = 0; v < 16; ++v) total[ct][v] = 0.f;
+        for (int v = 0; v < 16; ++v) total[rt][v] = 0.f;
 
-    // ---- w tile staging (same addressing as the fp32 kernel: buffer resource whose
-    // extent ends at the last valid row, so rows past S read as zeros)
+    // ---- w tile staging: a buffer resource whose extent ends at the last valid row (rows
+    // past S read as zeros), 32-bit lane offsets, the (i, j-chunk) offset in a scalar.
     floatx4 stage[SLOTS];
     const int trow = tid / F4_PER_ROW;
     const int tc4 = tid % F4_PER_ROW;
@@ -149,26 +136,22 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     for (int sidx = 0; sidx < SLOTS; ++sidx)
         woff[sidx] = ((uint32_t)(trow + sidx * ROWS_PER_SLOT) * (uint32_t)p.sw1 + 4u * tc4) * 4u;
     auto load_tile = [&](int i, int jc) {
+        const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
         const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
         if (full) {
-            const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) stage[sidx] = buf_load_f32x4(w_rsrc, woff[sidx], soff);
         } else {
+            // ragged chunk or unaligned rows: element loads; what lies past J belongs to the
+            // next i (or is outside the extent) and is replaced by zero
             const int j = jc * JC + 4 * tc4;
 #pragma unroll
-            for (int sidx = 0; sidx < SLOTS; ++sidx) {
-                const int row = trow + sidx * ROWS_PER_SLOT;
-                const float *src = wtile0 + (int64_t)row * p.sw1 + (int64_t)i * p.J + j;
-                floatx4 v = {0.f, 0.f, 0.f, 0.f};
-                if (row < wrows) {
-                    if (j + 0 < p.J) v[0] = src[0];
-                    if (j + 1 < p.J) v[1] = src[1];
-                    if (j + 2 < p.J) v[2] = src[2];
-                    if (j + 3 < p.J) v[3] = src[3];
+            for (int sidx = 0; sidx < SLOTS; ++sidx)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float v = buf_load_f32(w_rsrc, woff[sidx] + 4u * e, soff);
+                    stage[sidx][e] = (j + e < p.J) ? v : 0.f;
                 }
-                stage[sidx] = v;
-            }
         }
     };
     // split the staged fp32 values and write the pieces to LDS (8 bytes per piece and slot)
@@ -189,73 +172,65 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 
     const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ar, (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + p.K) * 4));
     const uint32_t a_row_bytes = (uint32_t)p.sa1 * 4u;
-    uint32_t aoff[CT];
-#pragma unroll
-    for (int ct = 0; ct < CT; ++ct) aoff[ct] = (uint32_t)ncl[ct] * 4u;
+    const uint32_t aoff = (uint32_t)ncl * 4u;
 
     // B operand: exp(b[j,n] - mb[n]) of the current j-chunk, split, in MFMA layout
-    uintx4 ebp[CT][NS][KS];
+    uintx4 ebp[NS][KS];
     auto load_eb = [&](int jc) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
+        for (int ks = 0; ks < KS; ++ks) {
+            float e[8];
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) {
-                float e[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int j = jc * JC + 16 * ks + 8 * h + u;
-                    float raw = -__builtin_inff();
-                    if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl[ct]];
-                    e[u] = exp_shifted(raw - mb[ct]);
-                }
-#pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    uint32_t pk[NS];
-                    split_pair<NS, true>(e[2 * u], e[2 * u + 1], pk);
-#pragma unroll
-                    for (int sp = 0; sp < NS; ++sp) ebp[ct][sp][ks][u] = pk[sp];
-                }
+            for (int u = 0; u < 8; ++u) {
+                const int j = jc * JC + 16 * ks + 8 * h + u;
+                float raw = -__builtin_inff();
+                if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl];
+                e[u] = exp_shifted(raw - mb);
             }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                uint32_t pk[NS];
+                split_pair<NS, true>(e[2 * u], e[2 * u + 1], pk);
+#pragma unroll
+                for (int sp = 0; sp < NS; ++sp) ebp[sp][ks][u] = pk[sp];
+            }
+        }
     };
 
     if (total_iters > 0) {
         int jc = 0, i = 0;
         load_tile(0, 0);
         load_eb(0);
-        float ea[CT], ea_raw[CT];
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) ea[ct] = exp_shifted(ar[ncl[ct]] - ma[ct]);
+        float ea = exp_shifted(ar[ncl] - ma);
+        float ea_raw;
         store_tile(0);
         __syncthreads();
 
-        // ---- one (i, j-chunk) and 32-column tile: inner = w tile x eb (3 or 6 MFMAs per
-        // k-step, starting from zero), then total += ea[i,n] * inner
-        bf16x8 af[NS][KS];
-        auto load_a = [&](int buf) {
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
-#pragma unroll
-                for (int sp = 0; sp < NS; ++sp)
-                    af[sp][ks] = *reinterpret_cast<const bf16x8 *>(&wt[buf][sp][(32 * wm + m) * LDA + 16 * ks + 8 * h]);
-        };
-        auto mfma_cols = [&](int ct, floatx16 &inn) {
+        // ---- one (i, j-chunk) and row tile: inner = w tile x eb (3 or 6 MFMAs per k-step,
+        // starting from zero), then total += ea[i,n] * inner
+        auto mfma_rows = [&](int buf, int rt, floatx16 &inn) {
             bool first = true;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks)
+            for (int ks = 0; ks < KS; ++ks) {
+                bf16x8 af[NS];
+#pragma unroll
+                for (int sp = 0; sp < NS; ++sp)
+                    af[sp] = *reinterpret_cast<const bf16x8 *>(&wt[buf][sp][(32 * rt + m) * LDA + 16 * ks + 8 * h]);
 #pragma unroll
                 for (int sa = 0; sa < NS; ++sa)
 #pragma unroll
                     for (int sb = 0; sa + sb < NS; ++sb) {
-                        const bf16x8 bop = __builtin_bit_cast(bf16x8, ebp[ct][sb][ks]);
+                        const bf16x8 bop = __builtin_bit_cast(bf16x8, ebp[sb][ks]);
                         if (first) {
                             const floatx16 zero = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f,
                                                    0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-                            inn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[sa][ks], bop, zero, 0, 0, 0);
+                            inn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[sa], bop, zero, 0, 0, 0);
                         } else {
-                            inn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[sa][ks], bop, inn, 0, 0, 0);
+                            inn = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[sa], bop, inn, 0, 0, 0);
                         }
                         first = false;
                     }
+            }
         };
         // The empty asm pins the fmas to this place in the instruction stream: their results
         // are not needed before the next step, and the compiler would otherwise sink them
@@ -267,10 +242,10 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
         };
 
         int cur = 0;
-        if constexpr (CT == 2) {
-            // Two half-steps per (i, j-chunk).  While the MFMAs of column tile 0 run, the vector
-            // ALU adds the previous step's column tile 1 into the running sum; while those of
-            // column tile 1 run, it adds column tile 0 and splits the prefetched w tile.
+        if constexpr (RT == 2) {
+            // Two half-steps per (i, j-chunk).  While the MFMAs of row tile 0 run, the vector
+            // ALU adds the previous step's row tile 1 into the running sum; while those of
+            // row tile 1 run, it adds row tile 0 and splits the prefetched w tile.
             floatx16 inner0, inner1;
 #pragma unroll
             for (int v = 0; v < 16; ++v) inner1[v] = 0.f;
@@ -282,33 +257,28 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
                     njc = jc + 1;
                 }
                 load_tile(ni, njc);
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct)
-                    ea_raw[ct] = buf_load_f32(a_rsrc, aoff[ct], (uint32_t)ni * a_row_bytes);
+                ea_raw = buf_load_f32(a_rsrc, aoff, (uint32_t)ni * a_row_bytes);
                 __builtin_amdgcn_sched_barrier(0);
-                load_a(cur);
-                mfma_cols(0, inner0);
+                mfma_rows(cur, 0, inner0);
                 scale_add(total[1], inner1, ea_old);
                 __builtin_amdgcn_sched_barrier(0);
-                mfma_cols(1, inner1);
-                scale_add(total[0], inner0, ea[0]);
+                mfma_rows(cur, 1, inner1);
+                scale_add(total[0], inner0, ea);
                 store_tile(cur ^ 1);
                 __builtin_amdgcn_sched_barrier(0);
-                ea_old = ea[1];
+                ea_old = ea;
                 if (njc != jc) load_eb(njc);
-#pragma unroll
-                for (int ct = 0; ct < CT; ++ct) ea[ct] = exp_shifted(ea_raw[ct] - ma[ct]);
+                ea = exp_shifted(ea_raw - ma);
                 __syncthreads();
                 cur ^= 1;
                 i = ni;
                 jc = njc;
             }
-            load_a(cur);
-            mfma_cols(0, inner0);
+            mfma_rows(cur, 0, inner0);
             scale_add(total[1], inner1, ea_old);
-            mfma_cols(1, inner1);
-            scale_add(total[0], inner0, ea[0]);
-            scale_add(total[1], inner1, ea[1]);
+            mfma_rows(cur, 1, inner1);
+            scale_add(total[0], inner0, ea);
+            scale_add(total[1], inner1, ea);
         } else {
             floatx16 inner;
             for (int it = 0; it + 1 < total_iters; ++it) {
@@ -318,42 +288,38 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
                     njc = jc + 1;
                 }
                 load_tile(ni, njc);
-                ea_raw[0] = buf_load_f32(a_rsrc, aoff[0], (uint32_t)ni * a_row_bytes);
+                ea_raw = buf_load_f32(a_rsrc, aoff, (uint32_t)ni * a_row_bytes);
                 __builtin_amdgcn_sched_barrier(0);
-                load_a(cur);
-                mfma_cols(0, inner);
-                scale_add(total[0], inner, ea[0]);
+                mfma_rows(cur, 0, inner);
+                scale_add(total[0], inner, ea);
                 store_tile(cur ^ 1);
                 if (njc != jc) load_eb(njc);
-                ea[0] = exp_shifted(ea_raw[0] - ma[0]);
+                ea = exp_shifted(ea_raw - ma);
                 __syncthreads();
                 cur ^= 1;
                 i = ni;
                 jc = njc;
             }
-            load_a(cur);
-            mfma_cols(0, inner);
-            scale_add(total[0], inner, ea[0]);
+            mfma_rows(cur, 0, inner);
+            scale_add(total[0], inner, ea);
         }
     }
 
-    // ---- epilogue: register v of lane (h, m) holds row 8*(v/4) + 4*h + v%4, column m of
-    // the wavefront's 32 x 32 tile
+    // ---- epilogue: register v of lane (h, m) holds row 8*(v/4) + 4*h + v%4, column m
+    if (ncol >= p.K) return;
     const int crows = p.S - s0;
     const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)s0 * p.sc1,
                                                     (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4));
     const uint32_t c_row_bytes = (uint32_t)p.sc1 * 4u;
+    const float mm = ma + mb;
+    const uint32_t co = ((uint32_t)(4 * h) * (uint32_t)p.sc1 + (uint32_t)ncol) * 4u;
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) {
-        if (ncol[ct] >= p.K) continue;
-        const float mm = ma[ct] + mb[ct];
-        const uint32_t co = ((uint32_t)(32 * wm + 4 * h) * (uint32_t)p.sc1 + (uint32_t)ncol[ct]) * 4u;
+    for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const uint32_t trow_c = 8 * (v / 4) + (v % 4);
-            buf_store_f32_stream(log_plus(total[ct][v], mm), c_rsrc, co, trow_c * c_row_bytes);
+            const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4);
+            buf_store_f32_stream(log_plus(total[rt][v], mm), c_rsrc, co, trow_c * c_row_bytes);
         }
-    }
 }
 
 template <int RT, int KS, int NS>
