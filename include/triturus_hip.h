@@ -125,6 +125,18 @@ int trt_lt2exp_bf16(const float *w, const float *a, const float *b, float *c,
                     const int64_t sc[3], int pieces, int variant, void *stream);
 
 /*
+ * trt_lm2exp_f32 on the bf16 matrix pipe, in the same way (ALLOW_TF32 at
+ * triturus/lm2exp.py:152 is the reference's counterpart): same tensors, layouts, strides and
+ * status codes; pieces as above; never splits the contraction, needs no workspace.
+ * variant: 0 = choose by shape, 1..trt_lm2exp_bf16_variant_count() pick a tile shape.
+ */
+int trt_lm2exp_bf16(const float *a, const float *b, float *c,
+                    int64_t R, int64_t I, int64_t J, int64_t K,
+                    const int64_t sa[3], const int64_t sb[3], const int64_t sc[3],
+                    int pieces, int variant, void *stream);
+int trt_lm2exp_bf16_variant_count(void);
+
+/*
  * Max of a contiguous m x n row-major matrix along axis 0 (y has n entries)
  * or axis 1 (y has m entries).  NaN propagates as in torch.amax.  Replaces the
  * multi-launch `_ker_matmax` tree, triturus/max.py:190-225.  workspace:

@@ -88,6 +88,13 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_lt2exp_bf16(null, one, one, one, *args, 2, 0, null) == -1
     assert lib.trt_lt2exp_bf16(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, 2), ok, ok, ok, 2, 0, null) == -2
     assert lib.trt_lt2exp_bf16(one, one, one, one, 1 << 31, 1, 1, 1, 1, ok, ok, ok, ok, 3, 0, null) == -4
+    # lm2exp on the bf16 matrix pipe
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, ok, ok, 1, 0, null) == -1
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, ok, ok, 2, lib.trt_lm2exp_bf16_variant_count() + 1, null) == -1
+    assert lib.trt_lm2exp_bf16(one, null, one, 1, 1, 1, 1, ok, ok, ok, 3, 0, null) == -1
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, s3(4, 1, 2), ok, 2, 0, null) == -2
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 2, 2, 8, ok, ok, s3(16, 4, 1), 2, 0, null) == -2
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1 << 30, 1, 1, ok, ok, ok, 2, 0, null) == -4
     # max
     assert lib.trt_vmax(null, 5, 0, one, one, one, 1 << 20, null) == -1
     assert lib.trt_vmax(one, 0, 0, one, one, one, 1 << 20, null) == -1

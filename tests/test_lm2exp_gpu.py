@@ -20,6 +20,13 @@ pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
 N_VARIANTS = 10
+N_BF16_VARIANTS = 6
+# Accuracy gates of the split-bf16 paths against the float64 oracle: two pieces (3 MFMAs per
+# product) carry 16 significand bits -- looser than fp32, ten times tighter than the rtol 5e-4
+# the reference allows its TF32 mode (tests/lm2exp.py:21); three pieces (6 MFMAs) carry 24 bits
+# and must pass the fp32 gate unchanged.
+BF16X3_GATE = {"rtol": 1e-4, "atol": 5e-5}
+PRECISION_GATES = {"bf16x3": BF16X3_GATE, "bf16x6": {}}
 
 
 def _check(out, a, b, **kw):
@@ -39,12 +46,14 @@ def test_lm2exp(dev, allow_tf32):
     c = lm2exp(a.to(dev), b.to(dev))
     assert c.shape == (batch, m, n) and c.dtype == torch.float32 and c.device.type == "cuda"
     if allow_tf32:
+        # the flag selects the split-bf16 path (error ~2^-16 per product; TF32 has 2^-11)
         assert torch.allclose(gt, c.cpu(), rtol=5e-4)
+        _check(c, a, b, **BF16X3_GATE)
     else:
         assert torch.allclose(gt, c.cpu())
-    # and the same recipe evaluated by torch on the GPU
-    assert torch.allclose(torch_baseline.lm2exp_fp32(a.to(dev), b.to(dev)), c)
-    _check(c, a, b)
+        # and the same recipe evaluated by torch on the GPU
+        assert torch.allclose(torch_baseline.lm2exp_fp32(a.to(dev), b.to(dev)), c)
+        _check(c, a, b)
 
 
 @pytest.mark.parametrize("name", ["lm2exp_small", "lm2exp_ragged"])
@@ -270,4 +279,100 @@ def test_benchmark_configuration_c3_full_size(dev):
         alt = lm2exp(ag, bg, _variant=variant)
         assert torch.allclose(alt, out, rtol=1e-5, atol=1e-5)
     shifted = lm2exp(ag, bg + 128.0)
+    assert torch.allclose(shifted, out + 128.0, rtol=1e-5, atol=1e-3)
+
+
+# ------------------------------------------------------------ split-bf16 matrix path
+@pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
+@pytest.mark.parametrize("variant", range(0, N_BF16_VARIANTS + 1))
+@pytest.mark.parametrize(
+    "shape", [(24, 150, 100, 200), (3, 37, 41, 70), (2, 300, 52, 129), (1, 64, 64, 64), (2, 33, 7, 31),
+              (1, 1, 1, 1), (2, 130, 128, 257)])
+def test_bf16_paths_on_ragged_shapes(dev, precision, variant, shape):
+    R, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape) + variant)
+    a = torch.rand(R, I, J, generator=g)
+    b = torch.randn(R, J, K, generator=g) * 6 - 2
+    b[torch.rand(b.shape, generator=g) < 0.05] = NINF
+    b[:, :, 0] = NINF  # an all -inf column: -inf out, not NaN
+    a[:, 0] = 0.0  # a zero row of weights: -inf out
+    out = lm2exp(a.to(dev), b.to(dev), _precision=precision, _variant=variant)
+    r = _check(out, a, b, **PRECISION_GATES[precision])
+    assert r["n_neg_inf"] > 0
+
+
+@pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
+@pytest.mark.parametrize("variant", [0, 1, 4])
+def test_bf16_paths_shift_moves_during_the_sweep(dev, precision, variant):
+    """The inputs of test_shift_moves_during_the_sweep: the running shift must move (and the
+    sums be rescaled) on the bf16 pipe as well."""
+    g = torch.Generator().manual_seed(11)
+    R, I, J, K = 2, 40, 300, 96
+    a = torch.rand(R, I, J, generator=g) + 0.01
+    b = torch.empty(R, J, K)
+    ramp = torch.linspace(-500.0, 500.0, J)
+    b[0] = ramp[:, None] + torch.randn(J, K, generator=g)
+    b[1] = -ramp[:, None] + torch.randn(J, K, generator=g)
+    b[0, :, 5] = NINF
+    b[0, J - 1, 5] = 3.0
+    b[0, :, 6] = torch.where(torch.arange(J) < 150, -1e30, 1e30)
+    b[1, :, 7] = torch.where(torch.arange(J) % 64 < 32, -1e3, 1e3)
+    b[1, :, 8] = NINF
+    b[1, 100, 8] = -1e38
+    out = lm2exp(a.to(dev), b.to(dev), _precision=precision, _variant=variant)
+    _check(out, a, b, **PRECISION_GATES[precision])
+    assert torch.isfinite(out[0, :, 5]).all() and torch.isfinite(out[0, :, 6]).all()
+
+
+@pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
+def test_bf16_paths_strided_nan_and_magnitude(dev, precision):
+    g = torch.Generator().manual_seed(5)
+    R, I, J, K = 2, 45, 36, 70
+    abig = torch.rand(R, I + 3, J + 4, generator=g)
+    bbig = torch.randn(R, J + 2, K + 9, generator=g) * 3
+    a, b = abig[:, 2 : I + 2, 4:], bbig[:, 1 : J + 1, 3 : K + 3]
+    out = lm2exp(a.to(dev), b.to(dev), _precision=precision)
+    _check(out, a, b, **PRECISION_GATES[precision])
+    b2 = (b * 1e3 - 7e8).contiguous()
+    out = lm2exp(a.to(dev), b2.to(dev), _precision=precision)
+    assert torch.isfinite(out).all()
+    assert torch.allclose(out.cpu().double(), oracle64.lm2exp64(a, b2), rtol=1e-6, atol=1e-3)
+    b3 = b.clone()
+    b3[1, 7, 9] = float("nan")
+    out = lm2exp(a.to(dev), b3.to(dev), _precision=precision)
+    assert torch.isnan(out[1, :, 9]).all()
+    mask = torch.ones_like(out, dtype=torch.bool)
+    mask[1, :, 9] = False
+    assert not torch.isnan(out[mask]).any()
+
+
+def test_bf16x6_is_as_accurate_as_the_fp32_kernel(dev):
+    """Three bf16 pieces hold all 24 significand bits: against float64 the error of the
+    6-MFMA path must stay within twice that of the fp32 MFMA kernel on the same inputs."""
+    cfg = workloads.c2()
+    a, b = cfg["a"], cfg["b"]
+    ref = oracle64.lm2exp64(a, b)
+    e32 = oracle64.compare(lm2exp(a.to(dev), b.to(dev)), ref)
+    e6 = oracle64.compare(lm2exp(a.to(dev), b.to(dev), _precision="bf16x6"), ref)
+    e3 = oracle64.compare(lm2exp(a.to(dev), b.to(dev), _precision="bf16x3"), ref, **BF16X3_GATE)
+    assert e32["ok"] and e6["ok"] and e3["ok"], (e32, e6, e3)
+    assert e6["max_abs_err"] <= 2 * e32["max_abs_err"] + 1e-6, (e6, e32)
+
+
+@pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
+def test_bf16_paths_c3_full_size(dev, precision):
+    """R=64, I=J=256, K=4096 on the bf16 pipe: every output against float64, plus the
+    size-independent bound c <= max_j b (rows of a sum to 1) and shift equivariance."""
+    cfg = workloads.c3()
+    a, b = cfg["a"], cfg["b"]
+    ag, bg = a.to(dev), b.to(dev)
+    out = lm2exp(ag, bg, _precision=precision)
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()
+    for r0 in range(0, 64, 8):
+        r = oracle64.compare(out[r0:r0 + 8], oracle64.lm2exp64(a[r0:r0 + 8], b[r0:r0 + 8]),
+                             **PRECISION_GATES[precision])
+        assert r["ok"], (r0, r)
+    assert torch.all(out <= bg.amax(1, keepdim=True) + 1e-3)
+    shifted = lm2exp(ag, bg + 128.0, _precision=precision)
     assert torch.allclose(shifted, out + 128.0, rtol=1e-5, atol=1e-3)

@@ -37,6 +37,12 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
          POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),
+    "trt_lm2exp_bf16": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
+         POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int, c_int, c_void_p],
+    ),
+    "trt_lm2exp_bf16_variant_count": (c_int, []),
     "trt_lm2exp_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int, c_int]),
     "trt_lm2exp_variant_count": (c_int, []),
     "trt_lt2exp_f32": (

@@ -1,0 +1,354 @@
+// lm2exp on the bf16 matrix pipe of gfx950, fp32 in and out:
+//   c[r,i,k] = log sum_j a[r,i,j] exp(b[r,j,k])
+//
+// Counterpart of the reference's reduced-precision mode (ALLOW_TF32 passed to tl.dot,
+// triturus/lm2exp.py:152, flag triturus/utils.py:33-44).  As in lt2exp_bf16.hip every fp32
+// operand is cut into NS bf16 pieces and a product is the sum of the 3 (NS = 2) or 6
+// (NS = 3) piece products that matter, accumulated in fp32 by v_mfma_f32_32x32x16_bf16.
+//
+// A workgroup of 4 wavefronts owns 32*RT rows of I and 128 columns of K; a wavefront owns
+// 32 of those columns for all rows.  J is walked in chunks of JC = 16*KS:
+//   B operand = exp(b[j,n] - m[n]), evaluated and split in registers (a lane owns one
+//               column; element e of lane-half h in k-step ks is j = 16 ks + 8 h + e);
+//   A operand = the a tile, global -> registers -> split -> LDS (double buffered).
+// The shift m[n] is found while sweeping (one pass over b): it starts as the maximum of the
+// column's first chunk and moves up, with the accumulators rescaled, when a later chunk
+// exceeds it by more than kBfRescaleMargin -- the scheme of the fp32 kernel (lm2exp.hip).
+// m is clamped to +-1e38 (baselines/lm2exp.py:12): an all -inf column gives -inf, not NaN.
+
+#include "common.hpp"
+
+namespace trt {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float floatx2 __attribute__((ext_vector_type(2)));
+typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
+
+constexpr float kBfRescaleMargin = 8.0f;
+
+struct Lm2BfArgs {
+    const float *a, *b;
+    float *c;
+    int R, I, J, K;
+    int64_t sa0, sa1, sb0, sb1, sc0, sc1;
+    int i_tiles, n_tiles;
+    int64_t total_wgs, padded_wgs;
+};
+
+// two fp32 -> one register of two bf16 (round to nearest even), element 0 in the low half
+__device__ __forceinline__ uint32_t lm_pack_bf16(float x0, float x1) {
+    floatx2 v = {x0, x1};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
+// Cut (x0, x1) into NS bf16 pieces each (out[s] holds piece s of both).  The subtraction is
+// exact.  An infinite x leaves inf - inf = NaN in the later pieces; with KEEP_INF those are
+// set to 0 so that inf stays inf.
+template <int NS, bool KEEP_INF>
+__device__ __forceinline__ void lm_split_pair(float x0, float x1, uint32_t (&out)[NS]) {
+#pragma unroll
+    for (int s = 0; s < NS; ++s) {
+        out[s] = lm_pack_bf16(x0, x1);
+        if (s + 1 < NS) {
+            const float f0 = __builtin_bit_cast(float, out[s] << 16);
+            const float f1 = __builtin_bit_cast(float, out[s] & 0xffff0000u);
+            x0 = (KEEP_INF && __builtin_isinf(f0)) ? 0.f : x0 - f0;
+            x1 = (KEEP_INF && __builtin_isinf(f1)) ? 0.f : x1 - f1;
+        }
+    }
+}
+
+template <int RT, int KS, int NS, bool VEC>
+__global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) {
+    constexpr int NT = 256;
+    constexpr int TM = 32 * RT;   // rows of I per workgroup
+    constexpr int TN = 128;
+    constexpr int JC = 16 * KS;
+    constexpr int LDA = JC + 8;   // padded LDS row in bf16: conflict-free 16-byte reads
+    constexpr int F4_PER_ROW = JC / 4;
+    constexpr int ROWS_PER_SLOT = NT / F4_PER_ROW;
+    constexpr int SLOTS = TM * F4_PER_ROW / NT;
+    static_assert(TM * F4_PER_ROW % NT == 0, "tile must divide over the threads");
+
+    extern __shared__ __attribute__((aligned(16))) __bf16 at[];  // [2][NS][TM * LDA]
+    auto tile_ptr = [&](int buf, int sp) { return at + (buf * NS + sp) * (TM * LDA); };
+
+    const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
+    if (L >= p.total_wgs) return;
+    int64_t rest = L / p.n_tiles;
+    const int nt = __builtin_amdgcn_readfirstlane((int)(L % p.n_tiles));
+    const int itile = __builtin_amdgcn_readfirstlane((int)(rest % p.i_tiles));
+    const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.i_tiles));
+
+    const int tid = threadIdx.x;
+    const int wave = tid / kWave;
+    const int lane = tid % kWave;
+    const int h = lane / 32;
+    const int m = lane % 32;
+    const int i0 = itile * TM;
+    const int ncol = nt * TN + wave * 32 + m;
+    const int ncl = ncol < p.K ? ncol : p.K - 1;
+
+    const float *ar = p.a + (int64_t)r * p.sa0;
+    const float *br = p.b + (int64_t)r * p.sb0;
+
+    floatx16 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[rt][v] = 0.f;
+
+    // ---- a tile: global -> registers.  Rows past I are clamped to the last valid row (they
+    // only feed accumulator rows that are never stored); columns past J must be zeros.
+    floatx4 stage[SLOTS];
+    const int trow = tid / F4_PER_ROW;
+    const int tc4 = tid % F4_PER_ROW;
+    uint32_t aoff[SLOTS];
+#pragma unroll
+    for (int sidx = 0; sidx < SLOTS; ++sidx) {
+        int row = i0 + trow + sidx * ROWS_PER_SLOT;
+        row = row < p.I ? row : p.I - 1;
+        aoff[sidx] = ((uint32_t)(row - i0) * (uint32_t)p.sa1 + 4u * tc4) * 4u;
+    }
+    const float *atile0 = ar + (int64_t)i0 * p.sa1;
+    const int arows = (p.I - i0) < TM ? (p.I - i0) : TM;
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        make_rsrc(atile0, (uint32_t)(((int64_t)(arows - 1) * p.sa1 + p.J) * 4));
+    auto load_tile = [&](int jc) {
+        const uint32_t soff = (uint32_t)(jc * JC) * 4u;  // wave-uniform
+        const bool full = VEC && (jc * JC + JC <= p.J);
+        if (full) {
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx) stage[sidx] = buf_load_f32x4(a_rsrc, aoff[sidx], soff);
+        } else {
+            const int j = jc * JC + 4 * tc4;
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float v = buf_load_f32(a_rsrc, aoff[sidx] + 4u * e, soff);
+                    stage[sidx][e] = (j + e < p.J) ? v : 0.f;
+                }
+        }
+    };
+    auto store_tile = [&](int buf) {
+#pragma unroll
+        for (int sidx = 0; sidx < SLOTS; ++sidx) {
+            uint32_t p01[NS], p23[NS];
+            lm_split_pair<NS, false>(stage[sidx][0], stage[sidx][1], p01);
+            lm_split_pair<NS, false>(stage[sidx][2], stage[sidx][3], p23);
+            const int off = (trow + sidx * ROWS_PER_SLOT) * LDA + 4 * tc4;
+#pragma unroll
+            for (int sp = 0; sp < NS; ++sp) {
+                uintx2 v = {p01[sp], p23[sp]};
+                *reinterpret_cast<uintx2 *>(tile_ptr(buf, sp) + off) = v;
+            }
+        }
+    };
+
+    // ---- b chunk: global -> registers; rows past J read as -inf
+    float braw[KS][8];
+    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(br, (uint32_t)(((int64_t)(p.J - 1) * p.sb1 + p.K) * 4));
+    const uint32_t b_row_bytes = (uint32_t)p.sb1 * 4u;
+    const uint32_t boff = ((uint32_t)(8 * h) * (uint32_t)p.sb1 + (uint32_t)ncl) * 4u;
+    auto load_b = [&](int jc) {
+        const bool full = jc * JC + JC <= p.J;  // wave-uniform
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float v = buf_load_f32(b_rsrc, boff, (uint32_t)(jc * JC + 16 * ks + e) * b_row_bytes);
+                braw[ks][e] = (full || jc * JC + 16 * ks + 8 * h + e < p.J) ? v : -__builtin_inff();
+            }
+    };
+    // Maximum of the chunk's column (both lane halves).  A NaN need not survive here:
+    // exp(NaN - m) is NaN for any m and poisons the column through the MFMA.
+    auto chunk_max = [&]() {
+        float x = max3_raw(braw[0][0], braw[0][1], braw[0][2]);
+#pragma unroll
+        for (int e = 3; e + 1 < 8 * KS; e += 2) x = max3_raw(x, braw[e / 8][e % 8], braw[(e + 1) / 8][(e + 1) % 8]);
+        x = max3_raw(x, braw[KS - 1][7], braw[KS - 1][7]);
+        return max3_raw(x, __shfl_xor(x, 32, kWave), x);
+    };
+
+    float mref;
+    uintx4 ebp[NS][KS];
+    // raw chunk -> split MFMA operands, moving the shift first if this chunk towers over it
+    auto shift_and_exp = [&]() {
+        const float cm = chunk_max();
+        const bool need = cm > mref + kBfRescaleMargin;
+        if (__builtin_amdgcn_ballot_w64(need) != 0) {
+            const float mnew = need ? clamp_shift(cm) : mref;
+            const float sc = exp_shifted(mref - mnew);
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[rt][v] *= sc;
+            mref = mnew;
+        }
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                uint32_t pk[NS];
+                lm_split_pair<NS, true>(exp_shifted(braw[ks][2 * u] - mref), exp_shifted(braw[ks][2 * u + 1] - mref),
+                                        pk);
+#pragma unroll
+                for (int sp = 0; sp < NS; ++sp) ebp[sp][ks][u] = pk[sp];
+            }
+    };
+
+    const int n_jc = (p.J + JC - 1) / JC;
+
+    // ---- prologue: first chunk
+    load_tile(0);
+    load_b(0);
+    store_tile(0);
+    mref = clamp_shift(chunk_max());
+    shift_and_exp();
+    __syncthreads();
+
+    // Row tiles are taken two at a time so that consecutive MFMAs alternate between two
+    // accumulators.
+    constexpr int RP = RT >= 2 ? 2 : 1;
+    auto mfma_block = [&](int buf) {
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+            for (int rt0 = 0; rt0 < RT; rt0 += RP) {
+                bf16x8 af[RP][NS];
+#pragma unroll
+                for (int k = 0; k < RP; ++k)
+#pragma unroll
+                    for (int sp = 0; sp < NS; ++sp)
+                        af[k][sp] = *reinterpret_cast<const bf16x8 *>(tile_ptr(buf, sp) + (32 * (rt0 + k) + m) * LDA +
+                                                                      16 * ks + 8 * h);
+#pragma unroll
+                for (int sa = 0; sa < NS; ++sa)
+#pragma unroll
+                    for (int sb = 0; sa + sb < NS; ++sb) {
+                        const bf16x8 bop = __builtin_bit_cast(bf16x8, ebp[sb][ks]);
+#pragma unroll
+                        for (int k = 0; k < RP; ++k)
+                            acc[rt0 + k] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[k][sa], bop, acc[rt0 + k], 0, 0, 0);
+                    }
+            }
+    };
+
+    int cur = 0;
+    for (int jc = 0; jc + 1 < n_jc; ++jc) {
+        load_tile(jc + 1);
+        load_b(jc + 1);
+        __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block
+        mfma_block(cur);
+        store_tile(cur ^ 1);
+        shift_and_exp();
+        __syncthreads();
+        cur ^= 1;
+    }
+    mfma_block(cur);
+
+    // ---- epilogue: c = m + log(acc); register v of lane (h, m) holds row 8*(v/4) + 4*h +
+    // v%4, column m of its 32 x 32 tile.  Rows past I fall outside the buffer extent.
+    if (ncol >= p.K) return;
+    const int crows = p.I - i0;
+    const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)i0 * p.sc1,
+                                                    (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4));
+    const uint32_t c_row_bytes = (uint32_t)p.sc1 * 4u;
+    const uint32_t co = ((uint32_t)(4 * h) * (uint32_t)p.sc1 + (uint32_t)ncol) * 4u;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4);
+            buf_store_f32_stream(log_plus(acc[rt][v], mref), c_rsrc, co, trow_c * c_row_bytes);
+        }
+}
+
+constexpr size_t kBfDefaultLdsLimit = 64 * 1024;
+
+template <int RT, int KS, int NS, bool VEC>
+static int launch_lm_bf_k(const Lm2BfArgs &args, hipStream_t stream) {
+    constexpr size_t lds = (size_t)2 * NS * (32 * RT) * (16 * KS + 8) * sizeof(__bf16);
+    auto k = lm2exp_bf16_kernel<RT, KS, NS, VEC>;
+    if (lds > kBfDefaultLdsLimit) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return (int)e;
+    }
+    hipLaunchKernelGGL(k, dim3((unsigned)args.padded_wgs), dim3(256), lds, stream, args);
+    return (int)hipGetLastError();
+}
+
+template <int RT, int KS>
+static int launch_lm_bf(const Lm2BfArgs &args, int pieces, bool vec, hipStream_t stream) {
+    if (pieces == 2) return vec ? launch_lm_bf_k<RT, KS, 2, true>(args, stream) : launch_lm_bf_k<RT, KS, 2, false>(args, stream);
+    return vec ? launch_lm_bf_k<RT, KS, 3, true>(args, stream) : launch_lm_bf_k<RT, KS, 3, false>(args, stream);
+}
+
+struct LmBfVariant {
+    int rt, ks;
+};
+// variant ids are 1-based in the C ABI (0 = choose by shape)
+static const LmBfVariant kLmBfVariants[] = {{4, 4}, {4, 2}, {2, 4}, {2, 2}, {1, 4}, {1, 2}};
+constexpr int kNumLmBfVariants = sizeof(kLmBfVariants) / sizeof(kLmBfVariants[0]);
+
+}  // namespace trt
+
+using namespace trt;
+
+extern "C" int trt_lm2exp_bf16_variant_count(void) { return kNumLmBfVariants; }
+
+extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
+                               const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], int pieces,
+                               int variant, void *stream) {
+    if (!a || !b || !c || !sa || !sb || !sc) return TRT_E_INVALID;
+    if (R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
+    if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
+    if (variant < 0 || variant > kNumLmBfVariants) return TRT_E_INVALID;
+    if (sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
+    for (int d = 0; d < 2; ++d)
+        if (sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
+    if (sc[1] < K) return TRT_E_LAYOUT;  // output rows must not overlap
+    const int64_t lim = (int64_t)1 << 30;
+    if (R >= lim || I >= lim || J >= lim || K >= lim) return TRT_E_RANGE;
+    // byte offsets inside one batch slab are 32-bit (buffer addressing)
+    if (I * sa[1] + J >= lim || J * sb[1] + K >= lim || I * sc[1] + K >= lim) return TRT_E_RANGE;
+
+    int v;
+    if (variant >= 1) {
+        v = variant - 1;
+    } else {
+        // row tile by grid fill, as for the fp32 kernel; chunks of 32 (more workgroups per CU fit)
+        const int64_t ct = ceil_div(K, 128);
+        int rt = 1;
+        if (I > 64 && R * ceil_div(I, 128) * ct >= 384) rt = 4;
+        else if (I > 32 && R * ceil_div(I, 64) * ct >= 384) rt = 2;
+        v = rt == 4 ? 1 : (rt == 2 ? 3 : 5);
+    }
+    const LmBfVariant &vr = kLmBfVariants[v];
+
+    Lm2BfArgs args;
+    args.a = a; args.b = b; args.c = c;
+    args.R = (int)R; args.I = (int)I; args.J = (int)J; args.K = (int)K;
+    args.sa0 = sa[0]; args.sa1 = sa[1];
+    args.sb0 = sb[0]; args.sb1 = sb[1];
+    args.sc0 = sc[0]; args.sc1 = sc[1];
+    args.i_tiles = (int)ceil_div(I, 32 * vr.rt);
+    args.n_tiles = (int)ceil_div(K, 128);
+    args.total_wgs = (int64_t)R * args.i_tiles * args.n_tiles;
+    args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+    const bool vec = (J % 4 == 0) && (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
+                     ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (v) {
+        case 0: return launch_lm_bf<4, 4>(args, pieces, vec, s);
+        case 1: return launch_lm_bf<4, 2>(args, pieces, vec, s);
+        case 2: return launch_lm_bf<2, 4>(args, pieces, vec, s);
+        case 3: return launch_lm_bf<2, 2>(args, pieces, vec, s);
+        case 4: return launch_lm_bf<1, 4>(args, pieces, vec, s);
+        default: return launch_lm_bf<1, 2>(args, pieces, vec, s);
+    }
+}

@@ -11,6 +11,7 @@ from __future__ import annotations
 import torch
 
 from triturus_amd import _lib
+from triturus_amd.utils import is_triturus_tf32_enabled
 
 
 _ws_bytes: dict = {}  # (R, I, J, K, variant, splits) -> workspace bytes, as reported by the library
@@ -24,7 +25,12 @@ def _unit_inner(t: torch.Tensor) -> torch.Tensor:
     return t.contiguous()
 
 
-def lm2exp(a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0, _splits: int = 0) -> torch.Tensor:
+_PIECES = {"bf16x3": 2, "bf16x6": 3}
+
+
+def lm2exp(
+    a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0, _splits: int = 0, _precision: str | None = None
+) -> torch.Tensor:
     assert len(a.shape) == len(b.shape) == 3
     assert a.shape[0] == b.shape[0]
     assert a.shape[2] == b.shape[1]
@@ -43,6 +49,18 @@ def lm2exp(a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0, _splits: int 
         return c.fill_(float("-inf"))
     a = _unit_inner(a)
     b = _unit_inner(b)
+    if _precision is None:
+        _precision = "bf16x3" if is_triturus_tf32_enabled() else "fp32"
+    if _precision != "fp32":
+        with _lib.on_device(a.device):
+            status = lib.trt_lm2exp_bf16(
+                a.data_ptr(), b.data_ptr(), c.data_ptr(),
+                R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
+                _PIECES[_precision], _variant, _lib.raw_stream(a.device),
+            )
+        if status:
+            _lib.check(status, "trt_lm2exp_bf16")
+        return c
     # small grids with a long contraction are cut over J; the partial sums need a workspace
     key = (R, I, J, K, _variant, _splits)
     ws_bytes = _ws_bytes.get(key)
