@@ -31,6 +31,7 @@ import torch
 
 PEAK_FP32_MFMA_TFLOPS = 157.3  # 256 CU x 4 SIMD x 64 flop/clk x 2.4 GHz
 PEAK_HBM_GBPS = 8000.0
+PEAK_BF16_MFMA_TFLOPS = 2516.6  # 16x the fp32 matrix rate
 
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, then WRITE_SIZE, one run
 # each over `bench.py --profile-pass`), scaled by what the same counters read for
@@ -207,7 +208,7 @@ def main() -> int:
     cfg = W.c5(R, S, I, J, K)
     w, a, b = (cfg[k].to(dev) for k in "wab")
     flops = W.lt2exp_flops(R, S, I, J, K)
-    step = lambda: lt2exp(w, a, b)
+    step = lambda: lt2exp(w, a, b, _precision="fp32")
     wall, ev = timed_region(step, args.steps, args.warmup)
     ms_per_step = wall / args.steps * 1e3
     value = flops * args.steps / wall / 1e9
@@ -259,15 +260,38 @@ def main() -> int:
         }
         log(f"cpu baseline lt2exp: {cpu_gflops:.1f} GFLOP/s on {torch.get_num_threads()} threads")
 
+    def split_bf16_line(fn_of_precision, flops_alg):
+        """The same call on the bf16 matrix pipe (fp32 in/out, operands cut into bf16 pieces):
+        not the headline figure -- the arithmetic is not the fp32 matrix instruction."""
+        out = {}
+        for prec, mfmas in (("bf16x3", 3), ("bf16x6", 6)):
+            fn = lambda: fn_of_precision(prec)
+            _, evp = timed_region(fn, args.steps, args.warmup)
+            t = evp / args.steps
+            out[prec] = {
+                "ms": round(t * 1e3, 5),
+                "equivalent_TFLOPs": round(flops_alg / t / 1e12, 2),
+                "speedup_over_fp32_pipe": None,
+                "roofline": {"bound": "mfma", "achieved": round(mfmas * flops_alg / t / 1e12, 1),
+                             "peak": PEAK_BF16_MFMA_TFLOPS, "unit": "TFLOP/s (bf16 MFMA issued)",
+                             "frac": round(mfmas * flops_alg / t / 1e12 / PEAK_BF16_MFMA_TFLOPS, 4)},
+            }
+            log(f"  {prec}: {t * 1e3:.4f} ms, {flops_alg / t / 1e12:.1f} TFLOP/s fp32-equivalent")
+        return out
+
     if not args.no_extras:
         result["do_bench_lt2exp"] = do_bench(step)
+        sb = split_bf16_line(lambda prec: lt2exp(w, a, b, _precision=prec), flops)
+        for v in sb.values():
+            v["speedup_over_fp32_pipe"] = round((ev / args.steps * 1e3) / v["ms"], 2)
+        result["lt2exp_split_bf16"] = sb
         del w, a, b
         # ------------------------------------------------------- lm2exp, rectangular
         R2, I2, J2, K2 = 64, 256, 256, 4096
         cfg3 = W.c3(R2, I2, J2, K2)
         a3, b3 = cfg3["a"].to(dev), cfg3["b"].to(dev)
         fl3 = W.lm2exp_flops(R2, I2, J2, K2)
-        step3 = lambda: lm2exp(a3, b3)
+        step3 = lambda: lm2exp(a3, b3, _precision="fp32")
         wall3, ev3 = timed_region(step3, args.steps, args.warmup)
         ach3 = fl3 / (ev3 / args.steps) / 1e12
         lm = {
@@ -291,6 +315,11 @@ def main() -> int:
                                   "kind": "port", "sample": f"{nb} of {R2} batches, median of {reps} runs",
                                   "speedup_gpu_over_cpu": round(lm["value"] / g, 1)}
             log(f"cpu baseline lm2exp: {g:.1f} GFLOP/s")
+        sb3 = split_bf16_line(lambda prec: lm2exp(a3, b3, _precision=prec), fl3)
+        for v in sb3.values():
+            v["speedup_over_fp32_pipe"] = round((ev3 / args.steps * 1e3) / v["ms"], 2)
+            v["algorithmic_GBps"] = round(lm["algorithmic_bytes"] / (v["ms"] * 1e-3) / 1e9, 1)
+        lm["split_bf16"] = sb3
         result["lm2exp"] = lm
         del a3, b3
 

@@ -197,6 +197,19 @@ def test_flags():
     assert is_triturus_tf32_enabled()
     set_tf32_enabled(False)
     assert not is_triturus_tf32_enabled()
+    # the arithmetic follows the flag unless it is pinned explicitly
+    from triturus_amd.utils import matrix_precision, set_matrix_precision
+    assert matrix_precision() == "fp32"
+    set_tf32_enabled(True)
+    assert matrix_precision() == "bf16x3"
+    set_matrix_precision("bf16x6")
+    assert matrix_precision() == "bf16x6"
+    set_tf32_enabled(False)
+    assert matrix_precision() == "bf16x6"
+    set_matrix_precision(None)
+    assert matrix_precision() == "fp32"
+    with pytest.raises(ValueError):
+        set_matrix_precision("tf32")
     ensure_reproducibility(seed=7, device="cpu")
     x = torch.rand(3)
     ensure_reproducibility(seed=7, device="cpu")

@@ -2,5 +2,7 @@
 from triturus_amd.utils import (  # noqa: F401
     ensure_reproducibility,
     is_triturus_tf32_enabled,
+    matrix_precision,
+    set_matrix_precision,
     set_tf32_enabled,
 )

@@ -11,7 +11,7 @@ from __future__ import annotations
 import torch
 
 from triturus_amd import _lib
-from triturus_amd.utils import is_triturus_tf32_enabled
+from triturus_amd.utils import MATRIX_PRECISIONS, matrix_precision
 
 
 _ws_bytes: dict = {}  # (R, I, J, K, variant, splits) -> workspace bytes, as reported by the library
@@ -50,7 +50,9 @@ def lm2exp(
     a = _unit_inner(a)
     b = _unit_inner(b)
     if _precision is None:
-        _precision = "bf16x3" if is_triturus_tf32_enabled() else "fp32"
+        _precision = matrix_precision()
+    elif _precision not in MATRIX_PRECISIONS:
+        raise ValueError(f"unknown matrix precision {_precision!r}")
     if _precision != "fp32":
         with _lib.on_device(a.device):
             status = lib.trt_lm2exp_bf16(

@@ -1,9 +1,15 @@
 """Global flags and seeding, same names as the reference's triturus/utils.py.
 
 ``set_tf32_enabled`` / ``is_triturus_tf32_enabled`` (triturus/utils.py:33-53):
-the flag is recorded, but gfx950 has no TF32/xf32 matrix instruction, so the
-kernels always contract in IEEE fp32 -- strictly tighter than the rtol 5e-4
-the reference tests allow when the flag is on (tests/lm2exp.py:21).
+gfx950 has no TF32/xf32 matrix instruction.  With the flag off the kernels
+contract in IEEE fp32 on the fp32 matrix pipe; with it on they run on the bf16
+matrix pipe with every fp32 operand cut into two bf16 pieces ("bf16x3": three
+MFMAs per product, ~2^-16 relative error per product, fp32 accumulation) --
+several times faster, and tighter than TF32 (2^-11) and than the rtol 5e-4 the
+reference tests allow in that mode (tests/lm2exp.py:21).
+``set_matrix_precision`` (no counterpart in the reference) picks the arithmetic
+explicitly: "fp32", "bf16x3", or "bf16x6" (three pieces, six MFMAs, ~2^-23 per
+product: as accurate as the fp32 pipe and faster); ``None`` follows the flag.
 ``ensure_reproducibility`` (triturus/utils.py:12-30) seeds python, numpy and
 torch and makes the GPU the default device when one is present.
 """
@@ -16,6 +22,8 @@ import numpy as np
 import torch
 
 _TRITURUS_TF32_ENABLED: bool = False
+_MATRIX_PRECISION: str | None = None
+MATRIX_PRECISIONS = ("fp32", "bf16x3", "bf16x6")
 
 
 def ensure_reproducibility(
@@ -45,3 +53,18 @@ def set_tf32_enabled(allow_tf32: bool) -> None:
 
 def is_triturus_tf32_enabled() -> bool:
     return _TRITURUS_TF32_ENABLED
+
+
+def set_matrix_precision(precision: str | None) -> None:
+    """Arithmetic of the lm2exp / lt2exp contractions; None = follow the TF32 flag."""
+    global _MATRIX_PRECISION
+    if precision is not None and precision not in MATRIX_PRECISIONS:
+        raise ValueError(f"unknown matrix precision {precision!r}: expected one of {MATRIX_PRECISIONS} or None")
+    _MATRIX_PRECISION = precision
+
+
+def matrix_precision() -> str:
+    """The arithmetic the next lm2exp / lt2exp call will use."""
+    if _MATRIX_PRECISION is not None:
+        return _MATRIX_PRECISION
+    return "bf16x3" if _TRITURUS_TF32_ENABLED else "fp32"
