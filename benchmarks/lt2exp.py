@@ -12,22 +12,23 @@ from benchmarks.utils import do_bench, eval_gbps, out_dir_from_argv, run_sweep
 from triturus.lt2exp import lt2exp
 from triturus.utils import ensure_reproducibility, set_tf32_enabled
 
-PROVIDERS = ["torch", "triturus", "triturus (unsplit)"]
+PROVIDERS = ["torch", "triturus", "triturus (unsplit)", "triturus (allow_tf32)"]
 
 
 def measure(batch, m, j, k, n, provider):
     ensure_reproducibility()
-    set_tf32_enabled(False)
+    set_tf32_enabled(provider == "triturus (allow_tf32)")
     w = torch.rand(batch, m, j, k)
     a = torch.randn(batch, j, n)
     b = torch.randn(batch, k, n)
     if provider == "torch":
         fn = lambda: torch_lt2exp(w, a, b)
-    elif provider == "triturus":
+    elif provider in ("triturus", "triturus (allow_tf32)"):
         fn = lambda: lt2exp(w, a, b)
     else:
         fn = lambda: lt2exp(w, a, b, mode="unsplit")
     ms, lo, hi = do_bench(fn)
+    set_tf32_enabled(False)
     size = batch * (m * j * k + j * n + k * n)
     return eval_gbps(size, ms), eval_gbps(size, hi), eval_gbps(size, lo)
 

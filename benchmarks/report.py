@@ -18,7 +18,7 @@ re-run with these kernels: same shapes, same input distributions (`rand` weights
 same metrics (GB/s of input bytes for lm2exp / lt2exp; comparisons per second, labelled TFLOPS, for the max
 reductions) and the same protocol (median of event-timed calls, each preceded by a 512 MiB cache flush).
 `torch` is the reference's eager torch recipe on the same GPU (rocBLAS bmm + elementwise kernels); `triturus` is
-this repository.  Only the fp32 lines exist: the TF32 flag does not change these kernels.  Run with
+this repository; `triturus (allow_tf32)` is the same call after `set_tf32_enabled(True)` (split-bf16 matrix path).  Run with
 `python -m benchmarks.lm2exp|lt2exp|max <dir>`, then `python -m benchmarks.report <dir>`.
 """
 

@@ -114,26 +114,34 @@ int trt_lt2exp_variant_count(void);
  * This is the library's counterpart of the reference's reduced-precision mode
  * (ALLOW_TF32 passed to tl.dot, triturus/lt2exp.py:345, flag triturus/utils.py:33-44):
  * gfx950 has no TF32 matrix instruction; two bf16 pieces are more accurate than TF32
- * (2^-11) and several times faster than the fp32 matrix pipe.  Always unsplit; needs no
- * workspace.  variant: 0 = choose by shape, 1..4 pick a tile shape (experiments, tests).
+ * (2^-11) and several times faster than the fp32 matrix pipe.  The bf16 kernels never split
+ * the contraction: with variant 0 a grid too small to be matrix bound (fewer than 192
+ * tiles), and any call in mode SPLIT, is handed to trt_lt2exp_f32, so the call takes
+ * the same mode and workspace (trt_lt2exp_workspace_bytes) as trt_lt2exp_f32.  variant: 0 = choose by shape, 1..4 force a
+ * bf16 tile shape (experiments, tests; no workspace needed).
  */
 #define TRT_PIECES_BF16X3 2
 #define TRT_PIECES_BF16X6 3
 int trt_lt2exp_bf16(const float *w, const float *a, const float *b, float *c,
                     int64_t R, int64_t S, int64_t I, int64_t J, int64_t K,
                     const int64_t sw[3], const int64_t sa[3], const int64_t sb[3],
-                    const int64_t sc[3], int pieces, int variant, void *stream);
+                    const int64_t sc[3], int pieces, int mode, int variant,
+                    void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * trt_lm2exp_f32 on the bf16 matrix pipe, in the same way (ALLOW_TF32 at
  * triturus/lm2exp.py:152 is the reference's counterpart): same tensors, layouts, strides and
- * status codes; pieces as above; never splits the contraction, needs no workspace.
- * variant: 0 = choose by shape, 1..trt_lm2exp_bf16_variant_count() pick a tile shape.
+ * status codes; pieces as above.  With variant 0, grids too small to be matrix bound and
+ * calls that ask for a cut over J (splits > 1) are handed to trt_lm2exp_f32, so the call
+ * takes the same splits and workspace (trt_lm2exp_workspace_bytes(R, I, J, K, 0, splits)).
+ * variant: 0 = choose by shape, 1..trt_lm2exp_bf16_variant_count() force a bf16 tile shape
+ * (no workspace needed).
  */
 int trt_lm2exp_bf16(const float *a, const float *b, float *c,
                     int64_t R, int64_t I, int64_t J, int64_t K,
                     const int64_t sa[3], const int64_t sb[3], const int64_t sc[3],
-                    int pieces, int variant, void *stream);
+                    int pieces, int variant, int splits,
+                    void *workspace, size_t workspace_bytes, void *stream);
 int trt_lm2exp_bf16_variant_count(void);
 
 /*

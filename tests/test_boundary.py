@@ -83,18 +83,25 @@ def test_c_abi_argument_errors_are_statuses():
     big4 = (2, 8, 16, 16, 64, s3(2048, 256, 1), s3(1024, 64, 1), s3(1024, 64, 1), s3(512, 64, 1))
     assert lib.trt_lt2exp_f32(one, one, one, one, *big4, _lib.MODE_SPLIT, 0, null, 0, null) == -3  # split needs a workspace
     # lt2exp on the bf16 matrix pipe: pieces must be 2 or 3, variant 0..4
-    assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 4, 0, null) == -1
-    assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 2, 9, null) == -1
-    assert lib.trt_lt2exp_bf16(null, one, one, one, *args, 2, 0, null) == -1
-    assert lib.trt_lt2exp_bf16(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, 2), ok, ok, ok, 2, 0, null) == -2
-    assert lib.trt_lt2exp_bf16(one, one, one, one, 1 << 31, 1, 1, 1, 1, ok, ok, ok, ok, 3, 0, null) == -4
+    btail = (0, 0, null, 0, null)  # mode, variant, workspace, bytes, stream
+    assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 4, *btail) == -1
+    assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 2, 0, 9, null, 0, null) == -1
+    assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 2, 5, 0, null, 0, null) == -1
+    assert lib.trt_lt2exp_bf16(null, one, one, one, *args, 2, *btail) == -1
+    assert lib.trt_lt2exp_bf16(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, 2), ok, ok, ok, 2, *btail) == -2
+    assert lib.trt_lt2exp_bf16(one, one, one, one, 1 << 31, 1, 1, 1, 1, ok, ok, ok, ok, 3, *btail) == -4
+    # a grid the fp32 path would split is handed to it, and then needs its workspace
+    assert lib.trt_lt2exp_bf16(one, one, one, one, *big4, 2, _lib.MODE_SPLIT, 0, null, 0, null) == -3
     # lm2exp on the bf16 matrix pipe
-    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, ok, ok, 1, 0, null) == -1
-    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, ok, ok, 2, lib.trt_lm2exp_bf16_variant_count() + 1, null) == -1
-    assert lib.trt_lm2exp_bf16(one, null, one, 1, 1, 1, 1, ok, ok, ok, 3, 0, null) == -1
-    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, s3(4, 1, 2), ok, 2, 0, null) == -2
-    assert lib.trt_lm2exp_bf16(one, one, one, 1, 2, 2, 8, ok, ok, s3(16, 4, 1), 2, 0, null) == -2
-    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1 << 30, 1, 1, ok, ok, ok, 2, 0, null) == -4
+    mtail = (0, 0, null, 0, null)  # variant, splits, workspace, bytes, stream
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, ok, ok, 1, *mtail) == -1
+    nv = lib.trt_lm2exp_bf16_variant_count()
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, ok, ok, 2, nv + 1, 0, null, 0, null) == -1
+    assert lib.trt_lm2exp_bf16(one, null, one, 1, 1, 1, 1, ok, ok, ok, 3, *mtail) == -1
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, s3(4, 1, 2), ok, 2, *mtail) == -2
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 2, 2, 8, ok, ok, s3(16, 4, 1), 2, *mtail) == -2
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1 << 30, 1, 1, ok, ok, ok, 2, *mtail) == -4
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1024, 1024, 1024, big, big, big, 2, 0, 4, null, 0, null) == -3
     # max
     assert lib.trt_vmax(null, 5, 0, one, one, one, 1 << 20, null) == -1
     assert lib.trt_vmax(one, 0, 0, one, one, one, 1 << 20, null) == -1

@@ -40,7 +40,7 @@ SIGNATURES = {
     "trt_lm2exp_bf16": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64,
-         POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int, c_int, c_void_p],
+         POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "trt_lm2exp_bf16_variant_count": (c_int, []),
     "trt_lm2exp_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int, c_int]),
@@ -54,7 +54,8 @@ SIGNATURES = {
     "trt_lt2exp_bf16": (
         c_int,
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
-         POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), c_int, c_int, c_void_p],
+         POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
+         c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "trt_lt2exp_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int]),
     "trt_lt2exp_variant_count": (c_int, []),

@@ -302,11 +302,11 @@ extern "C" int trt_lm2exp_bf16_variant_count(void) { return kNumLmBfVariants; }
 
 extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
                                const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], int pieces,
-                               int variant, void *stream) {
+                               int variant, int splits, void *workspace, size_t workspace_bytes, void *stream) {
     if (!a || !b || !c || !sa || !sb || !sc) return TRT_E_INVALID;
     if (R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
-    if (variant < 0 || variant > kNumLmBfVariants) return TRT_E_INVALID;
+    if (variant < 0 || variant > kNumLmBfVariants || splits < 0) return TRT_E_INVALID;
     if (sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
@@ -316,16 +316,24 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     // byte offsets inside one batch slab are 32-bit (buffer addressing)
     if (I * sa[1] + J >= lim || J * sb[1] + K >= lim || I * sc[1] + K >= lim) return TRT_E_RANGE;
 
+    // Tile by grid fill (measured over the reference's benchmark grid): 128 rows when that
+    // leaves >= 1.5 workgroups per CU (j-chunks of 64 for a long contraction, where the fewer
+    // barriers pay; of 32 otherwise, so that three workgroups fit a CU), 64 rows when that
+    // leaves >= 1 per CU.  Smaller grids are latency bound, not matrix bound: there the fp32
+    // path (smaller tiles, contraction cut over J) is as fast or faster and takes the call,
+    // as it does whenever the caller asks for a cut.
     int v;
     if (variant >= 1) {
         v = variant - 1;
     } else {
-        // row tile by grid fill, as for the fp32 kernel; chunks of 32 (more workgroups per CU fit)
         const int64_t ct = ceil_div(K, 128);
-        int rt = 1;
-        if (I > 64 && R * ceil_div(I, 128) * ct >= 384) rt = 4;
-        else if (I > 32 && R * ceil_div(I, 64) * ct >= 384) rt = 2;
-        v = rt == 4 ? 1 : (rt == 2 ? 3 : 5);
+        const int64_t n128 = R * ceil_div(I, 128) * ct, n64 = R * ceil_div(I, 64) * ct;
+        if (splits > 1) v = -1;
+        else if (I > 64 && n128 >= 384) v = (pieces == 2 && J >= 512) ? 0 : 1;
+        else if (I > 32 && n64 >= 256) v = pieces == 2 ? 2 : 3;
+        else v = -1;
+        if (v < 0)
+            return trt_lm2exp_f32(a, b, c, R, I, J, K, sa, sb, sc, 0, splits, workspace, workspace_bytes, stream);
     }
     const LmBfVariant &vr = kLmBfVariants[v];
 

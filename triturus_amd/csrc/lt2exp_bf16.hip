@@ -349,10 +349,12 @@ using namespace trt;
 
 extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, float *c, int64_t R, int64_t S,
                                int64_t I, int64_t J, int64_t K, const int64_t sw[3], const int64_t sa[3],
-                               const int64_t sb[3], const int64_t sc[3], int pieces, int variant, void *stream) {
+                               const int64_t sb[3], const int64_t sc[3], int pieces, int mode, int variant,
+                               void *workspace, size_t workspace_bytes, void *stream) {
     if (!w || !a || !b || !c || !sw || !sa || !sb || !sc) return TRT_E_INVALID;
     if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
+    if (mode != TRT_MODE_AUTO && mode != TRT_MODE_SPLIT && mode != TRT_MODE_UNSPLIT) return TRT_E_INVALID;
     if (variant < 0 || variant > 4) return TRT_E_INVALID;
     if (sw[2] != 1 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
@@ -362,14 +364,23 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
     if (S * sw[1] + I * J >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
 
-    // 32-row tiles for small grids (same reasoning as the fp32 kernel), j-chunks of 64
-    // unless J fits 32
+    // Tile: 64 rows when S allows, j-chunks of 64 unless J fits 32 (measured over the
+    // reference's benchmark grid).  The bf16 kernels never cut the contraction over several
+    // workgroups: a grid of fewer than 192 tiles (256 CUs) is latency bound, not
+    // matrix bound, and is handed to the fp32 path, which may cut it (measured 5-10x faster
+    // there on batch-1 squares, ahead up to ~128 tiles); so is a three-piece call below one
+    // tile per CU, where it does not beat the fp32 pipe it imitates, and any call in mode
+    // SPLIT.
     int rt = S > 32 ? 2 : 1;
-    if (rt == 2 && R * ceil_div(S, 64) * ceil_div(K, 128) < 384) rt = 1;
     int ks = J > 32 ? 4 : 2;
     if (variant >= 1) {  // 1: 64 rows, chunks of 64;  2: 64 rows, 32;  3: 32 rows, 64;  4: 32 rows, 32
         rt = variant <= 2 ? 2 : 1;
         ks = (variant & 1) ? 4 : 2;
+    } else {
+        const int64_t tiles = R * ceil_div(S, 32 * rt) * ceil_div(K, 128);
+        if (mode == TRT_MODE_SPLIT || tiles < (pieces == 3 ? 256 : 192))
+            return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes,
+                                  stream);
     }
 
     Lt2BfArgs args;

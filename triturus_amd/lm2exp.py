@@ -53,29 +53,29 @@ def lm2exp(
         _precision = matrix_precision()
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
-    if _precision != "fp32":
-        with _lib.on_device(a.device):
+    # small grids with a long contraction are cut over J; the partial sums need a workspace
+    fp32_variant = _variant if _precision == "fp32" else 0
+    key = (R, I, J, K, fp32_variant, _splits)
+    ws_bytes = _ws_bytes.get(key)
+    if ws_bytes is None:
+        ws_bytes = _ws_bytes[key] = lib.trt_lm2exp_workspace_bytes(R, I, J, K, fp32_variant, _splits)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+    ws_ptr = ws.data_ptr() if ws_bytes else None
+    with _lib.on_device(a.device):
+        if _precision == "fp32":
+            status = lib.trt_lm2exp_f32(
+                a.data_ptr(), b.data_ptr(), c.data_ptr(),
+                R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
+                _variant, _splits, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
+            )
+        else:
+            # bf16 matrix pipe; the library hands grids that are too small for it back to the
+            # fp32 kernels (which may cut the contraction over J: hence the workspace)
             status = lib.trt_lm2exp_bf16(
                 a.data_ptr(), b.data_ptr(), c.data_ptr(),
                 R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-                _PIECES[_precision], _variant, _lib.raw_stream(a.device),
+                _PIECES[_precision], _variant, _splits, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
             )
-        if status:
-            _lib.check(status, "trt_lm2exp_bf16")
-        return c
-    # small grids with a long contraction are cut over J; the partial sums need a workspace
-    key = (R, I, J, K, _variant, _splits)
-    ws_bytes = _ws_bytes.get(key)
-    if ws_bytes is None:
-        ws_bytes = _ws_bytes[key] = lib.trt_lm2exp_workspace_bytes(R, I, J, K, _variant, _splits)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
-    with _lib.on_device(a.device):
-        status = lib.trt_lm2exp_f32(
-            a.data_ptr(), b.data_ptr(), c.data_ptr(),
-            R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-            _variant, _splits, ws.data_ptr() if ws_bytes else None, ws_bytes,
-            _lib.raw_stream(a.device),
-        )
     if status:
-        _lib.check(status, "trt_lm2exp_f32")
+        _lib.check(status, "trt_lm2exp_f32" if _precision == "fp32" else "trt_lm2exp_bf16")
     return c

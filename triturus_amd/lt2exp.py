@@ -68,29 +68,28 @@ def lt2exp(
         _precision = matrix_precision()
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
-    if _precision != "fp32":
-        with _lib.on_device(a.device):
-            status = lib.trt_lt2exp_bf16(
-                w.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), R, S, I, J, K,
-                _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-                _PIECES[_precision], _variant, _lib.raw_stream(a.device),
-            )
-        if status:
-            _lib.check(status, "trt_lt2exp_bf16")
-        return c
     mode_code = _MODES[mode]
     key = (R, S, I, J, K, mode_code)
     ws_bytes = _ws_bytes.get(key)
     if ws_bytes is None:
         ws_bytes = _ws_bytes[key] = lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, mode_code)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+    ws_ptr = ws.data_ptr() if ws_bytes else None
     with _lib.on_device(a.device):
-        status = lib.trt_lt2exp_f32(
-            w.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), R, S, I, J, K,
-            _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-            mode_code, _variant, ws.data_ptr() if ws_bytes else None, ws_bytes,
-            _lib.raw_stream(a.device),
-        )
+        if _precision == "fp32":
+            status = lib.trt_lt2exp_f32(
+                w.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), R, S, I, J, K,
+                _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
+                mode_code, _variant, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
+            )
+        else:
+            # bf16 matrix pipe; the library hands grids that are too small for it (those the
+            # fp32 path would cut over the contraction) back to the fp32 kernels
+            status = lib.trt_lt2exp_bf16(
+                w.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), R, S, I, J, K,
+                _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
+                _PIECES[_precision], mode_code, _variant, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
+            )
     if status:
-        _lib.check(status, "trt_lt2exp_f32")
+        _lib.check(status, "trt_lt2exp_f32" if _precision == "fp32" else "trt_lt2exp_bf16")
     return c
