@@ -153,7 +153,10 @@ def profile_pass(dev) -> int:
     cfg = W.c5()
     w, a, b = (cfg[k].to(dev) for k in "wab")
     for _ in range(3):
-        lt2exp(w, a, b)
+        lt2exp(w, a, b, _precision="fp32")
+    for prec in ("bf16x3", "bf16x6"):
+        for _ in range(3):
+            lt2exp(w, a, b, _precision=prec)
     torch.cuda.synchronize()
     flat = b.view(-1)
     for _ in range(3):
@@ -165,9 +168,13 @@ def profile_pass(dev) -> int:
     cfg3 = W.c3()
     a3, b3 = cfg3["a"].to(dev), cfg3["b"].to(dev)
     for _ in range(3):
-        lm2exp(a3, b3)
+        lm2exp(a3, b3, _precision="fp32")
+    for prec in ("bf16x3", "bf16x6"):
+        for _ in range(3):
+            lm2exp(a3, b3, _precision=prec)
     torch.cuda.synchronize()
-    log("profile pass done: 3 x (copy 256 MiB, lt2exp large, vmax, matmax x2, lm2exp rectangular)")
+    log("profile pass done: 3 x (copy 256 MiB, lt2exp large [fp32, bf16x3, bf16x6], vmax, matmax x2, "
+        "lm2exp rectangular [fp32, bf16x3, bf16x6])")
     return 0
 
 

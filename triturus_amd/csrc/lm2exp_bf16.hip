@@ -76,10 +76,12 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 
     const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
     if (L >= p.total_wgs) return;
-    int64_t rest = L / p.n_tiles;
-    const int nt = __builtin_amdgcn_readfirstlane((int)(L % p.n_tiles));
-    const int itile = __builtin_amdgcn_readfirstlane((int)(rest % p.i_tiles));
-    const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.i_tiles));
+    // Row tiles of one column panel are neighbours in the launch order: they stream the same
+    // rows of b at the same time, so the panel comes from HBM once and from L2 afterwards.
+    int64_t rest = L / p.i_tiles;
+    const int itile = __builtin_amdgcn_readfirstlane((int)(L % p.i_tiles));
+    const int nt = __builtin_amdgcn_readfirstlane((int)(rest % p.n_tiles));
+    const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.n_tiles));
 
     const int tid = threadIdx.x;
     const int wave = tid / kWave;
