@@ -112,7 +112,7 @@ int trt_lt2exp_variant_count(void);
  *   pieces = 2 (TRT_PIECES_BF16X3): 3 MFMAs per product, relative error ~2^-16 per product
  *   pieces = 3 (TRT_PIECES_BF16X6): 6 MFMAs per product, relative error ~2^-23 per product
  * This is the library's counterpart of the reference's reduced-precision mode
- * (ALLOW_TF32 passed to tl.dot, triturus/lt2exp.py:345, flag triturus/utils.py:33-44):
+ * (ALLOW_TF32 passed to tl.dot, triturus/lt2exp.py:344, flag triturus/utils.py:33-44):
  * gfx950 has no TF32 matrix instruction; two bf16 pieces are more accurate than TF32
  * (2^-11) and several times faster than the fp32 matrix pipe.  The bf16 kernels never split
  * the contraction: with variant 0 a grid too small to be matrix bound (fewer than 192

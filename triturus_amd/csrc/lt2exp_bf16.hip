@@ -2,7 +2,7 @@
 //   c[r,s,k] = log sum_{i,j} w[r,s,i,j] exp(a[r,i,k]) exp(b[r,j,k])
 //
 // The reference has a reduced-precision mode (TF32 operands, triturus/utils.py:33-44,
-// passed to tl.dot at triturus/lt2exp.py:345); gfx950 has no TF32 matrix instruction.
+// passed to tl.dot at triturus/lt2exp.py:344); gfx950 has no TF32 matrix instruction.
 // Its bf16 matrix pipe is 16x faster than the fp32 one, so each fp32 operand is cut
 // into NS bf16 pieces (x = x0 + x1 [+ x2], each the bf16 rounding of what the previous
 // pieces left) and a product is the sum of the piece products that matter:
