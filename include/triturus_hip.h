@@ -61,8 +61,10 @@ const char *trt_error_string(int status);
  * free.  Replaces the `_ker_lm2exp[grid](...)` launch, triturus/lm2exp.py:186-205;
  * arithmetic contract baselines/lm2exp.py:11-14 (column max clamped to
  * +-1e38, an all -inf column gives -inf, never NaN).
- * variant: 0 = choose by shape; 1..trt_lm2exp_variant_count() pick a tile shape
- * (experiments, tests).
+ * variant: 0 = choose by shape; 1..trt_lm2exp_variant_count() pick a tile shape and
+ * how the shift is obtained (experiments, tests); the last one runs two launches -- a
+ * separate pass over b for the column maxima, then the contraction -- and needs
+ * R*K floats of workspace.
  * splits: the contraction over J may be cut over several workgroups whose partial
  * sums are merged by a second kernel in a fixed order (deterministic): 0 = decide
  * by shape (small grids with a long contraction), 1 = never, n = n ways.  The
@@ -164,6 +166,21 @@ size_t trt_matmax_workspace_bytes(int64_t m, int64_t n, int axis, int dtype);
 int trt_vmax(const void *x, int64_t n, int dtype, void *out_val, int64_t *out_idx,
              void *workspace, size_t workspace_bytes, void *stream);
 size_t trt_vmax_workspace_bytes(int64_t n, int dtype);
+
+/*
+ * c = a b for contiguous row-major fp32 matrices, a: m x k, b: k x n, c: m x n, in IEEE fp32
+ * on the fp32 matrix pipe (the lm2exp contraction kernel without shift, exp and log).
+ * Replaces the `_ker_mm[grid](...)` launch, triturus/mm.py:199-213.  Not on the log-space
+ * path: provided so that the reference's module surface is complete.
+ */
+int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n,
+               void *stream);
+
+/*
+ * r = x + y for contiguous vectors of n elements of `dtype` (TRT_F32 ...).  Replaces the
+ * `_ker_vadd[grid](...)` launch, triturus/add.py:45.  Same remark as trt_mm_f32.
+ */
+int trt_vadd(const void *x, const void *y, void *r, int64_t n, int dtype, void *stream);
 
 /*
  * Plain device-to-device copy kernel of nbytes (multiple of 16, 16-byte

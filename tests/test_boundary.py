@@ -110,6 +110,13 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_matmax(one, one, 4, 4, 2, 0, null, 0, null) == -1
     assert lib.trt_matmax(one, one, 0, 4, 0, 0, null, 0, null) == -1
     assert lib.trt_copy_bytes(one, one, 24, null) == -1
+    # mm, vadd
+    assert lib.trt_mm_f32(one, null, one, 2, 2, 2, null) == -1
+    assert lib.trt_mm_f32(one, one, one, 2, 0, 2, null) == -1
+    assert lib.trt_mm_f32(one, one, one, 1 << 30, 2, 2, null) == -4
+    assert lib.trt_vadd(one, one, null, 5, 0, null) == -1
+    assert lib.trt_vadd(one, one, one, 0, 0, null) == -1
+    assert lib.trt_vadd(one, one, one, 5, 7, null) == -1
 
 
 def test_workspace_queries_are_host_only_and_follow_the_mode_rule():
@@ -228,6 +235,8 @@ def test_reference_import_paths_exist():
     from triturus.lt2exp import lt2exp as f2
     from triturus.max import matmax as f3, vamax as f4, vmax as f5
     from triturus.utils import ensure_reproducibility as f6, set_tf32_enabled as f7
+    from triturus.mm import mm as f8
+    from triturus.add import vadd as f9
 
     assert f1 is lm2exp and f2 is lt2exp and (f3, f4, f5) == (matmax, vamax, vmax)
     assert callable(f6) and callable(f7)

@@ -19,7 +19,7 @@ from triturus_amd import _lib, workloads
 pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
-N_VARIANTS = 10
+N_VARIANTS = 11
 N_BF16_VARIANTS = 6
 # Accuracy gates of the split-bf16 paths against the float64 oracle: two pieces (3 MFMAs per
 # product) carry 16 significand bits -- looser than fp32, ten times tighter than the rtol 5e-4
@@ -275,7 +275,7 @@ def test_benchmark_configuration_c3_full_size(dev):
         worst = max(worst, r["worst_err_over_tol"])
     # size-independent properties on the whole output
     assert torch.all(out <= bg.amax(1, keepdim=True) + 1e-3)
-    for variant in (2, 3, 5, 10):  # other tile shapes, and the two-sweep (exact maximum) kernels
+    for variant in (2, 3, 5, 10, 11):  # other tiles, the two-sweep kernels, the two-launch variant
         alt = lm2exp(ag, bg, _variant=variant)
         assert torch.allclose(alt, out, rtol=1e-5, atol=1e-5)
     shifted = lm2exp(ag, bg + 128.0)

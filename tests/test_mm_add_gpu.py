@@ -1,0 +1,72 @@
+"""mm and vadd on the GPU: the reference's own tests (tests/mm.py:8-16, tests/add.py:6-12)
+plus ragged and large shapes.  mm is checked against a float64 product (the oracle for a
+plain matrix product is the product itself in higher precision) and against torch.mm."""
+
+import pytest
+import torch
+
+from triturus.add import vadd
+from triturus.mm import mm
+from triturus.utils import set_tf32_enabled
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("allow_tf32", [False, True])
+def test_mm(dev, allow_tf32):
+    """The reference's test: 150 x 100 x 200, rand inputs, torch.allclose defaults."""
+    set_tf32_enabled(allow_tf32)
+    m, k, n = 150, 100, 200
+    a = torch.rand(m, k, device=dev)
+    b = torch.rand(k, n, device=dev)
+    c = mm(a, b)
+    assert c.shape == (m, n) and c.dtype == torch.float32
+    assert torch.allclose(torch.mm(a, b), c)
+    assert torch.allclose((a.double() @ b.double()).float(), c)
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1), (33, 7, 31), (64, 64, 64), (300, 52, 129), (129, 1000, 257),
+                                   (2048, 512, 1024), (4096, 300, 4096)])
+def test_mm_shapes(dev, shape):
+    m, k, n = shape
+    g = torch.Generator().manual_seed(m + k + n)
+    a = torch.randn(m, k, generator=g).to(dev)
+    b = torch.randn(k, n, generator=g).to(dev)
+    c = mm(a, b)
+    ref = a.double() @ b.double()
+    # fp32 accumulation over k terms of magnitude ~1: error grows like sqrt(k) ulps
+    assert torch.allclose(c.double(), ref, rtol=1e-5, atol=2e-6 * k ** 0.5 + 1e-6)
+    # signs, zeros and exact small integers survive exactly
+    ai = torch.randint(-3, 4, (m, k), generator=g).float().to(dev)
+    bi = torch.randint(-3, 4, (k, n), generator=g).float().to(dev)
+    assert torch.equal(mm(ai, bi), (ai.double() @ bi.double()).float())
+
+
+def test_mm_rejects_what_the_reference_rejects(dev):
+    a = torch.rand(4, 5, device=dev)
+    with pytest.raises(AssertionError):
+        mm(a, torch.rand(4, 5, device=dev))
+    with pytest.raises(AssertionError):
+        mm(a.t(), torch.rand(4, 5, device=dev))
+    with pytest.raises(AssertionError):
+        mm(a.double(), torch.rand(5, 4, device=dev).double())
+
+
+def test_vadd(dev):
+    """The reference's test: n = 2000, rand inputs."""
+    n = 2000
+    x = torch.rand(n, device=dev)
+    y = torch.rand(n, device=dev)
+    assert torch.allclose(x + y, vadd(x, y))
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n", [1, 3, 255, 4097, 1 << 20, (1 << 24) + 5])
+def test_vadd_bit_exact(dev, dtype, n):
+    g = torch.Generator().manual_seed(n)
+    x = torch.randn(n + 1, generator=g).to(dtype).to(dev)
+    y = torch.randn(n + 1, generator=g).to(dtype).to(dev)
+    assert torch.equal(vadd(x[:n], y[:n]), x[:n] + y[:n])
+    # unaligned views take the scalar path
+    assert torch.equal(vadd(x[1:], y[1:]), x[1:] + y[1:])
+    assert torch.equal(vadd(x[:n], y[:n], block_size=64), x[:n] + y[:n])

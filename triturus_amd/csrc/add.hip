@@ -1,0 +1,87 @@
+// Elementwise r = x + y of two contiguous vectors (HBM bound: 3 * sizeof(T) bytes per element).
+// Replaces the `_ker_vadd[grid](...)` launch, triturus/add.py:45.
+
+#include <hip/hip_bf16.h>
+#include <hip/hip_fp16.h>
+
+#include "common.hpp"
+
+namespace trt {
+
+template <typename T>
+struct AddElem;
+template <>
+struct AddElem<float> {
+    static __device__ __forceinline__ float add(float a, float b) { return a + b; }
+};
+template <>
+struct AddElem<double> {
+    static __device__ __forceinline__ double add(double a, double b) { return a + b; }
+};
+template <>
+struct AddElem<__half> {
+    static __device__ __forceinline__ __half add(__half a, __half b) { return __hadd(a, b); }
+};
+template <>
+struct AddElem<__hip_bfloat16> {
+    // one rounding of the exact fp32 sum, as torch does for bf16
+    static __device__ __forceinline__ __hip_bfloat16 add(__hip_bfloat16 a, __hip_bfloat16 b) {
+        return __float2bfloat16(__bfloat162float(a) + __bfloat162float(b));
+    }
+};
+
+// 16 bytes per lane and access; unaligned pointers and the tail take the scalar loop.
+template <typename T>
+__global__ __launch_bounds__(256) void vadd_kernel(const T *__restrict__ x, const T *__restrict__ y,
+                                                   T *__restrict__ r, int64_t n, int aligned) {
+    constexpr int V = 16 / sizeof(T);
+    const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    int64_t done = 0;
+    if (aligned) {
+        const int64_t nv = n / V;
+        const uintx4 *xv = reinterpret_cast<const uintx4 *>(x);
+        const uintx4 *yv = reinterpret_cast<const uintx4 *>(y);
+        uintx4 *rv = reinterpret_cast<uintx4 *>(r);
+        for (int64_t i = tid; i < nv; i += stride) {
+            uintx4 a = xv[i], b = yv[i], c;
+            const T *ap = reinterpret_cast<const T *>(&a);
+            const T *bp = reinterpret_cast<const T *>(&b);
+            T *cp = reinterpret_cast<T *>(&c);
+#pragma unroll
+            for (int e = 0; e < V; ++e) cp[e] = AddElem<T>::add(ap[e], bp[e]);
+            __builtin_nontemporal_store(c, &rv[i]);
+        }
+        done = nv * V;
+    }
+    for (int64_t i = done + tid; i < n; i += stride) r[i] = AddElem<T>::add(x[i], y[i]);
+}
+
+template <typename T>
+static int launch_vadd(const void *x, const void *y, void *r, int64_t n, hipStream_t s) {
+    constexpr int V = 16 / sizeof(T);
+    const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) |
+                           reinterpret_cast<uintptr_t>(r)) & 15) == 0;
+    int64_t blocks = ceil_div(ceil_div(n, V), 256);
+    if (blocks > 256 * 16) blocks = 256 * 16;  // grid-stride beyond 16 workgroups per CU
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(vadd_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const T *>(x),
+                       static_cast<const T *>(y), static_cast<T *>(r), n, aligned ? 1 : 0);
+    return (int)hipGetLastError();
+}
+
+}  // namespace trt
+
+using namespace trt;
+
+extern "C" int trt_vadd(const void *x, const void *y, void *r, int64_t n, int dtype, void *stream) {
+    if (!x || !y || !r || n <= 0) return TRT_E_INVALID;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case TRT_F32: return launch_vadd<float>(x, y, r, n, s);
+        case TRT_F64: return launch_vadd<double>(x, y, r, n, s);
+        case TRT_F16: return launch_vadd<__half>(x, y, r, n, s);
+        case TRT_BF16: return launch_vadd<__hip_bfloat16>(x, y, r, n, s);
+        default: return TRT_E_INVALID;
+    }
+}

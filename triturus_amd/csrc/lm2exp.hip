@@ -46,8 +46,15 @@ struct Lm2Args {
     int64_t total_wgs, padded_wgs;
 };
 
-template <int RT, int CT, int WM, int WN, int NQ, bool VEC, bool ONLINE>
+// How the shift m[n] is obtained (MODE template parameter of the kernel)
+constexpr int kTwoSweep = 0;  // exact column maximum first (sweep 1), then the contraction
+constexpr int kOnline = 1;    // found while sweeping, accumulators rescaled when it moves
+constexpr int kExternal = 2;  // read from p.shift: a separate launch (lm2exp_colmax_kernel) computed it
+constexpr int kPlain = 3;     // no shift, no exp, no log: c = a b (the mm entry point)
+
+template <int RT, int CT, int WM, int WN, int NQ, bool VEC, int MODE>
 __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args p) {
+    constexpr bool ONLINE = MODE == kOnline;
     constexpr int NT = WM * WN * kWave;
     constexpr int TM = 32 * RT * WM;  // rows of I per workgroup
     constexpr int TN = 32 * CT * WN;  // columns of K per workgroup
@@ -183,7 +190,7 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
                     const int j = jc * JC + 8 * q + 4 * h + u;
-                    float raw = -__builtin_inff();
+                    float raw = MODE == kPlain ? 0.f : -__builtin_inff();
                     if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl[ct]];
                     braw[ct][4 * q + u] = raw;
                 }
@@ -219,7 +226,8 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
                 }
             }
 #pragma unroll
-            for (int e = 0; e < NB; ++e) eb[ct][e] = exp_shifted(braw[ct][e] - mref[ct]);
+            for (int e = 0; e < NB; ++e)
+                eb[ct][e] = MODE == kPlain ? braw[ct][e] : exp_shifted(braw[ct][e] - mref[ct]);
         }
     };
 
@@ -231,7 +239,15 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     const int jc1 = (jc0 + p.chunks_per_split < n_jc) ? jc0 + p.chunks_per_split : n_jc;
     const int full_end = jc1 < n_full ? jc1 : n_full;
 
-    if (!ONLINE) {
+    if (MODE == kExternal) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) mref[ct] = p.shift[(int64_t)r * p.K + ncl[ct]];
+    }
+    if (MODE == kPlain) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) mref[ct] = 0.f;
+    }
+    if (MODE == kTwoSweep) {
         // ---- sweep 1: exact column maxima over all J
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
@@ -345,9 +361,49 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
                 const uint32_t trow = 32 * rt + 8 * (v / 4) + (v % 4);  // + 4h in the lane offset
                 if (split_out)  // partial sums are read back by the merge kernel right away
                     buf_store_f32(acc[rt][ct][v], c_rsrc, co, trow * c_row_bytes);
+                else if (MODE == kPlain)
+                    buf_store_f32_stream(acc[rt][ct][v], c_rsrc, co, trow * c_row_bytes);
                 else
                     buf_store_f32_stream(log_plus(acc[rt][ct][v], mref[ct]), c_rsrc, co, trow * c_row_bytes);
             }
+    }
+}
+
+// Clamped column maxima m[r,k] = clamp(max_j b[r,j,k]) for the two-kernel variant (a separate
+// pass over b, then a contraction that reads the shift).  A workgroup owns 256 columns of one
+// batch (a lane 4 adjacent ones); its 4 wavefronts interleave over the rows and combine in LDS.
+__global__ __launch_bounds__(256) void lm2exp_colmax_kernel(const float *__restrict__ b, float *__restrict__ m, int R,
+                                                            int J, int K, int64_t sb0, int64_t sb1) {
+    __shared__ float part[4][256];
+    const int blocks_per_batch = (K + 255) / 256;
+    const int r = blockIdx.x / blocks_per_batch;
+    const int k0 = (blockIdx.x % blocks_per_batch) * 256;
+    const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
+    const float *br = b + (int64_t)r * sb0;
+    float x[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) x[e] = -__builtin_inff();
+    const int kc = k0 + 4 * lane;
+    const bool vec = kc + 3 < K && (sb1 % 4 == 0) && ((reinterpret_cast<uintptr_t>(br) & 15) == 0);
+    for (int j = wave; j < J; j += 4) {
+        const float *row = br + (int64_t)j * sb1;
+        if (vec) {
+            const floatx4 v = *reinterpret_cast<const floatx4 *>(row + kc);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) x[e] = max_nan(x[e], v[e]);
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+                if (kc + e < K) x[e] = max_nan(x[e], row[kc + e]);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) part[wave][4 * lane + e] = x[e];
+    __syncthreads();
+    const int t = threadIdx.x;
+    if (k0 + t < K) {
+        const float y = max_nan(max_nan(part[0][t], part[1][t]), max_nan(part[2][t], part[3][t]));
+        m[(int64_t)r * K + k0 + t] = clamp_shift(y);
     }
 }
 
@@ -377,20 +433,21 @@ __global__ __launch_bounds__(256) void lm2exp_merge_kernel(const float *__restri
 // ------------------------------------------------------------------ host
 struct Lm2Variant {
     int rt, ct, wm, wn, nq;
-    bool online;
+    int mode;
 };
 // variant ids are 1-based in the C ABI (0 = choose by shape)
 static const Lm2Variant kVariants[] = {
-    {4, 1, 1, 4, 4, true},   // 1: 128 x 128 tile, 4 waves each 128 x 32, one sweep (3 waves/SIMD)
-    {4, 1, 1, 8, 4, true},   // 2: 128 x 256 tile, 8 waves each 128 x 32
-    {8, 1, 1, 8, 4, true},   // 3: 256 x 256 tile, 8 waves each 256 x 32
-    {8, 1, 1, 4, 4, true},   // 4: 256 x 128 tile, 4 waves each 256 x 32
-    {8, 1, 1, 8, 4, false},  // 5: as 3, two sweeps (exact column maximum first)
-    {2, 2, 1, 4, 4, true},   // 6: 64 x 256 tile
-    {2, 1, 1, 4, 4, true},   // 7: 64 x 128 tile
-    {1, 1, 1, 4, 4, true},   // 8: 32 x 128 tile
-    {2, 1, 1, 4, 4, false},  // 9: as 7, two sweeps
-    {4, 1, 1, 4, 4, false},  // 10: as 1, two sweeps
+    {4, 1, 1, 4, 4, kOnline},   // 1: 128 x 128 tile, 4 waves each 128 x 32, one sweep (3 waves/SIMD)
+    {4, 1, 1, 8, 4, kOnline},   // 2: 128 x 256 tile, 8 waves each 128 x 32
+    {8, 1, 1, 8, 4, kOnline},   // 3: 256 x 256 tile, 8 waves each 256 x 32
+    {8, 1, 1, 4, 4, kOnline},   // 4: 256 x 128 tile, 4 waves each 256 x 32
+    {8, 1, 1, 8, 4, kTwoSweep},  // 5: as 3, two sweeps (exact column maximum first)
+    {2, 2, 1, 4, 4, kOnline},   // 6: 64 x 256 tile
+    {2, 1, 1, 4, 4, kOnline},   // 7: 64 x 128 tile
+    {1, 1, 1, 4, 4, kOnline},   // 8: 32 x 128 tile
+    {2, 1, 1, 4, 4, kTwoSweep},  // 9: as 7, two sweeps
+    {4, 1, 1, 4, 4, kTwoSweep},  // 10: as 1, two sweeps
+    {4, 1, 1, 4, 4, kExternal},  // 11: as 1, shift from a separate pass over b (two launches)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be opted into per kernel
@@ -408,10 +465,10 @@ constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be op
 //   >= 1.5 tiles of 64 rows per CU         64 x 128   (+2..5 %)
 //   fewer, long contraction (J >= 1280)    the largest tile that leaves >= 128 tiles
 //   fewer, short contraction               32 x 128   (+12..36 %)
-static int find_variant(int rt, int wn, bool online) {
+static int find_variant(int rt, int wn, int mode) {
     for (int v = 0; v < kNumVariants; ++v)
         if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].wm == 1 && kVariants[v].wn == wn &&
-            kVariants[v].nq == 4 && kVariants[v].online == online)
+            kVariants[v].nq == 4 && kVariants[v].mode == mode)
             return v;
     return 0;
 }
@@ -427,7 +484,7 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
         rt = (n64 >= kFill || J >= 1280) ? 2 : 1;
     } else if (n128 >= kFill) {
         if (I * J >= ((int64_t)1 << 20) && K % 256 == 0 && R * ceil_div(I, 128) * (K / 256) >= 512)
-            return find_variant(4, 8, true);
+            return find_variant(4, 8, kOnline);
         rt = 4;
     } else if (n64 >= kFill) {
         rt = 2;
@@ -436,15 +493,15 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     } else {
         rt = 1;
     }
-    return find_variant(rt, 4, true);
+    return find_variant(rt, 4, kOnline);
 }
 
-template <int RT, int CT, int WM, int WN, int NQ, bool VEC, bool ONLINE>
+template <int RT, int CT, int WM, int WN, int NQ, bool VEC, int MODE>
 static int launch_k(const Lm2Args &args, hipStream_t stream) {
     constexpr int TM = 32 * RT * WM;
     constexpr int LDA = 8 * NQ + 4;
     constexpr size_t lds = (size_t)2 * TM * LDA * sizeof(float);
-    auto k = lm2exp_kernel<RT, CT, WM, WN, NQ, VEC, ONLINE>;
+    auto k = lm2exp_kernel<RT, CT, WM, WN, NQ, VEC, MODE>;
     if (lds > kDefaultLdsLimit) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -454,10 +511,10 @@ static int launch_k(const Lm2Args &args, hipStream_t stream) {
     return (int)hipGetLastError();
 }
 
-template <int RT, int CT, int WM, int WN, int NQ, bool ONLINE>
+template <int RT, int CT, int WM, int WN, int NQ, int MODE>
 static int launch_v(const Lm2Args &args, bool vec, hipStream_t stream) {
-    return vec ? launch_k<RT, CT, WM, WN, NQ, true, ONLINE>(args, stream)
-               : launch_k<RT, CT, WM, WN, NQ, false, ONLINE>(args, stream);
+    return vec ? launch_k<RT, CT, WM, WN, NQ, true, MODE>(args, stream)
+               : launch_k<RT, CT, WM, WN, NQ, false, MODE>(args, stream);
 }
 
 struct Lm2Plan {
@@ -478,7 +535,9 @@ static Lm2Plan make_plan(int64_t R, int64_t I, int64_t J, int64_t K, int variant
     const int64_t chunks = ceil_div(J, 8 * vr.nq);
     const int64_t base = R * ceil_div(I, 32 * vr.rt * vr.wm) * ceil_div(K, 32 * vr.ct * vr.wn);
     int64_t splits = 1;
-    if (splits_req == 0)
+    if (vr.mode == kExternal || vr.mode == kPlain)
+        splits = 1;  // these kernels do not write partial sums
+    else if (splits_req == 0)
         // measured: R=16 I=J=K=512 (256 tiles, 16 chunks) is 1.5x slower split, batch-1
         // squares of 512..1536 are 1.2-1.9x faster; the model below reproduces both
         splits = choose_splits(base, chunks, 4 * vr.nq * vr.rt * vr.ct, R * I * K, 2, kMaxSplits, false);
@@ -494,6 +553,7 @@ static Lm2Plan make_plan(int64_t R, int64_t I, int64_t J, int64_t K, int variant
 }
 
 static size_t plan_workspace(const Lm2Plan &pl, int64_t R, int64_t I, int64_t K) {
+    if (kVariants[pl.variant].mode == kExternal) return (size_t)R * K * sizeof(float);  // the shifts
     if (pl.splits <= 1) return 0;
     return ((size_t)pl.splits * R * I * K + (size_t)pl.splits * R * K) * sizeof(float);
 }
@@ -542,7 +602,16 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     args.total_wgs = (int64_t)R * args.i_tiles * args.n_tiles * pl.splits;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
-    if (pl.splits > 1) {
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (vr.mode == kExternal) {
+        // two-kernel variant: a pass over b for the clamped column maxima, then the contraction
+        if (!workspace || workspace_bytes < plan_workspace(pl, R, I, K)) return TRT_E_WORKSPACE;
+        args.shift = static_cast<float *>(workspace);
+        const int64_t blocks = R * ceil_div(K, 256);
+        if (blocks >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+        hipLaunchKernelGGL(lm2exp_colmax_kernel, dim3((unsigned)blocks), dim3(256), 0, s, b, args.shift, (int)R,
+                           (int)J, (int)K, sb[0], sb[1]);
+    } else if (pl.splits > 1) {
         const size_t need = plan_workspace(pl, R, I, K);
         if (!workspace || workspace_bytes < need) return TRT_E_WORKSPACE;
         args.part = static_cast<float *>(workspace);
@@ -550,19 +619,19 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     }
     const bool vec = (J % 4 == 0) && (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
-    hipStream_t s = static_cast<hipStream_t>(stream);
     int st;
     switch (v) {
-        case 0: st = launch_v<4, 1, 1, 4, 4, true>(args, vec, s); break;
-        case 1: st = launch_v<4, 1, 1, 8, 4, true>(args, vec, s); break;
-        case 2: st = launch_v<8, 1, 1, 8, 4, true>(args, vec, s); break;
-        case 3: st = launch_v<8, 1, 1, 4, 4, true>(args, vec, s); break;
-        case 4: st = launch_v<8, 1, 1, 8, 4, false>(args, vec, s); break;
-        case 5: st = launch_v<2, 2, 1, 4, 4, true>(args, vec, s); break;
-        case 6: st = launch_v<2, 1, 1, 4, 4, true>(args, vec, s); break;
-        case 7: st = launch_v<1, 1, 1, 4, 4, true>(args, vec, s); break;
-        case 8: st = launch_v<2, 1, 1, 4, 4, false>(args, vec, s); break;
-        default: st = launch_v<4, 1, 1, 4, 4, false>(args, vec, s); break;
+        case 0: st = launch_v<4, 1, 1, 4, 4, kOnline>(args, vec, s); break;
+        case 1: st = launch_v<4, 1, 1, 8, 4, kOnline>(args, vec, s); break;
+        case 2: st = launch_v<8, 1, 1, 8, 4, kOnline>(args, vec, s); break;
+        case 3: st = launch_v<8, 1, 1, 4, 4, kOnline>(args, vec, s); break;
+        case 4: st = launch_v<8, 1, 1, 8, 4, kTwoSweep>(args, vec, s); break;
+        case 5: st = launch_v<2, 2, 1, 4, 4, kOnline>(args, vec, s); break;
+        case 6: st = launch_v<2, 1, 1, 4, 4, kOnline>(args, vec, s); break;
+        case 7: st = launch_v<1, 1, 1, 4, 4, kOnline>(args, vec, s); break;
+        case 8: st = launch_v<2, 1, 1, 4, 4, kTwoSweep>(args, vec, s); break;
+        case 9: st = launch_v<4, 1, 1, 4, 4, kTwoSweep>(args, vec, s); break;
+        default: st = launch_v<4, 1, 1, 4, 4, kExternal>(args, vec, s); break;
     }
     if (st != 0 || pl.splits <= 1) return st;
     const int64_t total = R * I * K;
@@ -571,4 +640,38 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     hipLaunchKernelGGL(lm2exp_merge_kernel, dim3((unsigned)blocks), dim3(256), 0, s, args.part, args.shift, c,
                        (int)R, (int)I, (int)K, pl.splits, sc[0], sc[1]);
     return (int)hipGetLastError();
+}
+
+// c = a b for row-major fp32 matrices (m x k times k x n): the contraction kernel above without
+// shift, exp and log.  Replaces the `_ker_mm[grid](...)` launch, triturus/mm.py:199-213.
+extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, void *stream) {
+    if (!a || !b || !c) return TRT_E_INVALID;
+    if (m <= 0 || k <= 0 || n <= 0) return TRT_E_INVALID;
+    const int64_t lim = (int64_t)1 << 30;
+    if (m >= lim || k >= lim || n >= lim) return TRT_E_RANGE;
+    if (k * n + n >= lim || m * k + k >= lim || m * n + n >= lim) return TRT_E_RANGE;
+    // row tile by grid fill, as for lm2exp with one batch
+    const int64_t ct = ceil_div(n, 128);
+    int rt = 1;
+    if (m > 64 && ceil_div(m, 128) * ct >= 384) rt = 4;
+    else if (m > 32 && ceil_div(m, 64) * ct >= 256) rt = 2;
+    Lm2Args args;
+    args.a = a; args.b = b; args.c = c;
+    args.part = nullptr; args.shift = nullptr;
+    args.R = 1; args.I = (int)m; args.J = (int)k; args.K = (int)n;
+    args.sa0 = m * k; args.sa1 = k;
+    args.sb0 = k * n; args.sb1 = n;
+    args.sc0 = m * n; args.sc1 = n;
+    args.i_tiles = (int)ceil_div(m, 32 * rt);
+    args.n_tiles = (int)ceil_div(n, 128);
+    args.splits = 1;
+    args.chunks_per_split = (int)ceil_div(k, 32);
+    args.total_wgs = (int64_t)args.i_tiles * args.n_tiles;
+    args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+    const bool vec = (k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (rt == 4) return launch_v<4, 1, 1, 4, 4, kPlain>(args, vec, s);
+    if (rt == 2) return launch_v<2, 1, 1, 4, 4, kPlain>(args, vec, s);
+    return launch_v<1, 1, 1, 4, 4, kPlain>(args, vec, s);
 }
