@@ -9,7 +9,7 @@ import json
 import sys
 from pathlib import Path
 
-ORDER = ["lm2exp", "lt2exp", "vmax", "matmax"]
+ORDER = ["lm2exp", "lt2exp", "vmax", "matmax", "mm", "vadd"]
 
 HEADER = """# Reference benchmark grid on one MI355X
 
@@ -19,7 +19,7 @@ same metrics (GB/s of input bytes for lm2exp / lt2exp; comparisons per second, l
 reductions) and the same protocol (median of event-timed calls, each preceded by a 512 MiB cache flush).
 `torch` is the reference's eager torch recipe on the same GPU (rocBLAS bmm + elementwise kernels); `triturus` is
 this repository; `triturus (allow_tf32)` is the same call after `set_tf32_enabled(True)` (split-bf16 matrix path).  Run with
-`python -m benchmarks.lm2exp|lt2exp|max <dir>`, then `python -m benchmarks.report <dir>`.
+`python -m benchmarks.lm2exp|lt2exp|max|mm <dir>`, then `python -m benchmarks.report <dir>`.
 """
 
 

@@ -242,6 +242,8 @@ def test_capturable_in_a_hip_graph(dev):
         out_t = lt2exp(w, a, b)
         out_t_split = lt2exp(w, a, b, mode="split")
         out_m = lm2exp(a2, b)
+        out_t3 = lt2exp(w, a, b, _precision="bf16x3", _variant=1)
+        out_m6 = lm2exp(a2, b, _precision="bf16x6", _variant=3)
     for rep in range(4):
         a.copy_(torch.randn(2, 16, 256, generator=g))
         b.copy_(torch.randn(2, 32, 256, generator=g) - rep)
@@ -250,6 +252,8 @@ def test_capturable_in_a_hip_graph(dev):
         assert torch.equal(out_t, lt2exp(w, a, b))
         assert torch.equal(out_t_split, lt2exp(w, a, b, mode="split"))
         assert torch.equal(out_m, lm2exp(a2, b))
+        assert torch.equal(out_t3, lt2exp(w, a, b, _precision="bf16x3", _variant=1))
+        assert torch.equal(out_m6, lm2exp(a2, b, _precision="bf16x6", _variant=3))
         torch.cuda.synchronize()
 
 

@@ -30,43 +30,70 @@ struct AddElem<__hip_bfloat16> {
     }
 };
 
-// 16 bytes per lane and access; unaligned pointers and the tail take the scalar loop.
+// A workgroup adds one contiguous block of kAddUnroll * 256 16-byte pieces (no grid-stride
+// loop: measured 6.4 TB/s against 4.7 TB/s for loads spread a whole grid apart), with
+// non-temporal loads and stores -- nothing is reused.  Unaligned pointers and the tail take
+// the scalar kernel.
+constexpr int kAddUnroll = 4;
+
 template <typename T>
 __global__ __launch_bounds__(256) void vadd_kernel(const T *__restrict__ x, const T *__restrict__ y,
-                                                   T *__restrict__ r, int64_t n, int aligned) {
+                                                   T *__restrict__ r, int64_t nv) {
     constexpr int V = 16 / sizeof(T);
-    const int64_t tid = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    int64_t done = 0;
-    if (aligned) {
-        const int64_t nv = n / V;
-        const uintx4 *xv = reinterpret_cast<const uintx4 *>(x);
-        const uintx4 *yv = reinterpret_cast<const uintx4 *>(y);
-        uintx4 *rv = reinterpret_cast<uintx4 *>(r);
-        for (int64_t i = tid; i < nv; i += stride) {
-            uintx4 a = xv[i], b = yv[i], c;
-            const T *ap = reinterpret_cast<const T *>(&a);
-            const T *bp = reinterpret_cast<const T *>(&b);
+    const uintx4 *xv = reinterpret_cast<const uintx4 *>(x);
+    const uintx4 *yv = reinterpret_cast<const uintx4 *>(y);
+    uintx4 *rv = reinterpret_cast<uintx4 *>(r);
+    const int64_t base = (int64_t)blockIdx.x * (kAddUnroll * 256) + threadIdx.x;
+    uintx4 a[kAddUnroll], b[kAddUnroll];
+#pragma unroll
+    for (int u = 0; u < kAddUnroll; ++u) {
+        const int64_t i = base + u * 256;
+        if (i < nv) {
+            a[u] = __builtin_nontemporal_load(&xv[i]);
+            b[u] = __builtin_nontemporal_load(&yv[i]);
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < kAddUnroll; ++u) {
+        const int64_t i = base + u * 256;
+        if (i < nv) {
+            uintx4 c;
+            const T *ap = reinterpret_cast<const T *>(&a[u]);
+            const T *bp = reinterpret_cast<const T *>(&b[u]);
             T *cp = reinterpret_cast<T *>(&c);
 #pragma unroll
             for (int e = 0; e < V; ++e) cp[e] = AddElem<T>::add(ap[e], bp[e]);
             __builtin_nontemporal_store(c, &rv[i]);
         }
-        done = nv * V;
     }
-    for (int64_t i = done + tid; i < n; i += stride) r[i] = AddElem<T>::add(x[i], y[i]);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void vadd_scalar_kernel(const T *__restrict__ x, const T *__restrict__ y,
+                                                          T *__restrict__ r, int64_t begin, int64_t n) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    for (int64_t i = begin + (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += stride)
+        r[i] = AddElem<T>::add(x[i], y[i]);
 }
 
 template <typename T>
 static int launch_vadd(const void *x, const void *y, void *r, int64_t n, hipStream_t s) {
     constexpr int V = 16 / sizeof(T);
+    const T *xp = static_cast<const T *>(x), *yp = static_cast<const T *>(y);
+    T *rp = static_cast<T *>(r);
     const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y) |
                            reinterpret_cast<uintptr_t>(r)) & 15) == 0;
-    int64_t blocks = ceil_div(ceil_div(n, V), 256);
-    if (blocks > 256 * 16) blocks = 256 * 16;  // grid-stride beyond 16 workgroups per CU
-    if (blocks < 1) blocks = 1;
-    hipLaunchKernelGGL(vadd_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, static_cast<const T *>(x),
-                       static_cast<const T *>(y), static_cast<T *>(r), n, aligned ? 1 : 0);
+    const int64_t nv = aligned ? n / V : 0;
+    if (nv > 0) {
+        const int64_t blocks = ceil_div(nv, (int64_t)kAddUnroll * 256);
+        if (blocks >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+        hipLaunchKernelGGL(vadd_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, xp, yp, rp, nv);
+    }
+    if (nv * V < n) {
+        int64_t blocks = ceil_div(n - nv * V, 256);
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(vadd_scalar_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, s, xp, yp, rp, nv * V, n);
+    }
     return (int)hipGetLastError();
 }
 

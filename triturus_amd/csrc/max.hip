@@ -138,25 +138,32 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_stage1(
     const int tid = threadIdx.x;
     if (blockIdx.x == 0 && tid < head) feed(E::up(x[tid]), tid);
 
+    // Workgroups walk the vector in contiguous blocks of kVmaxUnroll * kVmaxThreads 16-byte
+    // pieces (block-cyclic over the grid): measured 6.3 TB/s against 4.7 TB/s for the same
+    // loads spread a whole grid apart.  Indices still increase within a thread.
     const V *xv = reinterpret_cast<const V *>(x + head);
-    const int64_t stride = (int64_t)gridDim.x * kVmaxThreads;
-    int64_t v = (int64_t)blockIdx.x * kVmaxThreads + tid;
-    for (; v + (kVmaxUnroll - 1) * stride < nvec; v += kVmaxUnroll * stride) {
+    constexpr int64_t kBlock = (int64_t)kVmaxUnroll * kVmaxThreads;
+    const int64_t full_blocks = nvec / kBlock;
+    for (int64_t blk = blockIdx.x; blk < full_blocks; blk += gridDim.x) {
+        const int64_t v = blk * kBlock + tid;
         V buf[kVmaxUnroll];
 #pragma unroll
-        for (int u = 0; u < kVmaxUnroll; ++u) buf[u] = xv[v + u * stride];
+        for (int u = 0; u < kVmaxUnroll; ++u) buf[u] = xv[v + u * kVmaxThreads];
 #pragma unroll
         for (int u = 0; u < kVmaxUnroll; ++u) {
-            const int64_t base = head + (v + u * stride) * VN;
+            const int64_t base = head + (v + u * kVmaxThreads) * VN;
 #pragma unroll
             for (int e = 0; e < VN; ++e) feed(E::up(buf[u].e[e]), base + e);
         }
     }
-    for (; v < nvec; v += stride) {
-        V buf = xv[v];
-        const int64_t base = head + v * VN;
+    // the last, partial block goes to the workgroup whose turn it would be
+    if ((int64_t)blockIdx.x == full_blocks % gridDim.x) {
+        for (int64_t v = full_blocks * kBlock + tid; v < nvec; v += kVmaxThreads) {
+            V buf = xv[v];
+            const int64_t base = head + v * VN;
 #pragma unroll
-        for (int e = 0; e < VN; ++e) feed(E::up(buf.e[e]), base + e);
+            for (int e = 0; e < VN; ++e) feed(E::up(buf.e[e]), base + e);
+        }
     }
     const int64_t tail0 = head + nvec * VN;
     if (blockIdx.x == 0 && tail0 + tid < n) feed(E::up(x[tail0 + tid]), tail0 + tid);
@@ -591,20 +598,26 @@ extern "C" int trt_matmax(const void *x, void *y, int64_t m, int64_t n, int axis
 }
 
 // ------------------------------------------------------------ copy kernel
-__global__ __launch_bounds__(256) void copy16_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
-                                                     size_t nvec) {
-    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const size_t stride = (size_t)gridDim.x * 256;
-    for (; i < nvec; i += stride) dst[i] = src[i];
+// One contiguous block of 4 * 256 16-byte pieces per workgroup, non-temporal both ways.
+__global__ __launch_bounds__(256) void copy16_kernel(const trt::uintx4 *__restrict__ src,
+                                                     trt::uintx4 *__restrict__ dst, size_t nvec) {
+    const size_t base = (size_t)blockIdx.x * 1024 + threadIdx.x;
+    trt::uintx4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (base + u * 256 < nvec) v[u] = __builtin_nontemporal_load(&src[base + u * 256]);
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (base + u * 256 < nvec) __builtin_nontemporal_store(v[u], &dst[base + u * 256]);
 }
 
 extern "C" int trt_copy_bytes(const void *src, void *dst, size_t nbytes, void *stream) {
     if (!src || !dst || nbytes == 0 || (nbytes & 15)) return TRT_E_INVALID;
     if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) return TRT_E_LAYOUT;
     const size_t nvec = nbytes / 16;
-    size_t blocks = (nvec + 255) / 256;
-    if (blocks > 8192) blocks = 8192;
+    const size_t blocks = (nvec + 1023) / 1024;
+    if (blocks >= ((size_t)1 << 31)) return TRT_E_RANGE;
     hipLaunchKernelGGL(copy16_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint4 *>(src), static_cast<uint4 *>(dst), nvec);
+                       static_cast<const trt::uintx4 *>(src), static_cast<trt::uintx4 *>(dst), nvec);
     return (int)hipGetLastError();
 }
