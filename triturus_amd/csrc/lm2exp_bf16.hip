@@ -16,14 +16,9 @@
 // exceeds it by more than kBfRescaleMargin -- the scheme of the fp32 kernel (lm2exp.hip).
 // m is clamped to +-1e38 (baselines/lm2exp.py:12): an all -inf column gives -inf, not NaN.
 
-#include "common.hpp"
+#include "bf16_split.hpp"
 
 namespace trt {
-
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef float floatx2 __attribute__((ext_vector_type(2)));
-typedef uint32_t uintx2 __attribute__((ext_vector_type(2)));
 
 constexpr float kBfRescaleMargin = 8.0f;
 
@@ -35,29 +30,6 @@ struct Lm2BfArgs {
     int i_tiles, n_tiles;
     int64_t total_wgs, padded_wgs;
 };
-
-// two fp32 -> one register of two bf16 (round to nearest even), element 0 in the low half
-__device__ __forceinline__ uint32_t lm_pack_bf16(float x0, float x1) {
-    floatx2 v = {x0, x1};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-}
-
-// Cut (x0, x1) into NS bf16 pieces each (out[s] holds piece s of both).  The subtraction is
-// exact.  An infinite x leaves inf - inf = NaN in the later pieces; with KEEP_INF those are
-// set to 0 so that inf stays inf.
-template <int NS, bool KEEP_INF>
-__device__ __forceinline__ void lm_split_pair(float x0, float x1, uint32_t (&out)[NS]) {
-#pragma unroll
-    for (int s = 0; s < NS; ++s) {
-        out[s] = lm_pack_bf16(x0, x1);
-        if (s + 1 < NS) {
-            const float f0 = __builtin_bit_cast(float, out[s] << 16);
-            const float f1 = __builtin_bit_cast(float, out[s] & 0xffff0000u);
-            x0 = (KEEP_INF && __builtin_isinf(f0)) ? 0.f : x0 - f0;
-            x1 = (KEEP_INF && __builtin_isinf(f1)) ? 0.f : x1 - f1;
-        }
-    }
-}
 
 template <int RT, int KS, int NS, bool VEC>
 __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) {
@@ -138,8 +110,8 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
             uint32_t p01[NS], p23[NS];
-            lm_split_pair<NS, false>(stage[sidx][0], stage[sidx][1], p01);
-            lm_split_pair<NS, false>(stage[sidx][2], stage[sidx][3], p23);
+            split_pair<NS, false>(stage[sidx][0], stage[sidx][1], p01);
+            split_pair<NS, false>(stage[sidx][2], stage[sidx][3], p23);
             const int off = (trow + sidx * ROWS_PER_SLOT) * LDA + 4 * tc4;
 #pragma unroll
             for (int sp = 0; sp < NS; ++sp) {
@@ -194,7 +166,7 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
                 uint32_t pk[NS];
-                lm_split_pair<NS, true>(exp_shifted(braw[ks][2 * u] - mref), exp_shifted(braw[ks][2 * u + 1] - mref),
+                split_pair<NS, true>(exp_shifted(braw[ks][2 * u] - mref), exp_shifted(braw[ks][2 * u + 1] - mref),
                                         pk);
 #pragma unroll
                 for (int sp = 0; sp < NS; ++sp) ebp[sp][ks][u] = pk[sp];
