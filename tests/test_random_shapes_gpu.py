@@ -1,0 +1,91 @@
+"""Seeded random shapes, strides and -inf patterns through every arithmetic of lm2exp and
+lt2exp (fp32 matrix pipe, split-bf16 with 2 and 3 pieces), each checked against the float64
+oracle.  Shapes are drawn around the tile boundaries (multiples of 16/32/64/128 +- 1) where
+masking mistakes live; sizes stay small enough for the oracle to finish in milliseconds."""
+
+import random
+
+import pytest
+import torch
+
+from oracle import oracle64
+from triturus.lm2exp import lm2exp
+from triturus.lt2exp import lt2exp
+
+pytestmark = pytest.mark.gpu
+NINF = float("-inf")
+GATES = {"fp32": {}, "bf16x3": {"rtol": 1e-4, "atol": 5e-5}, "bf16x6": {}}
+
+
+def _dim(rng, hi):
+    base = rng.choice([1, 2, 3, 8, 16, 31, 32, 33, 48, 63, 64, 65, 96, 127, 128, 129, 160, 200, 257])
+    return max(1, min(hi, base + rng.choice([-1, 0, 0, 1])))
+
+
+def _view(rng, t):
+    """Random non-contiguous view with the same values: padded rows and/or an offset."""
+    kind = rng.randrange(3)
+    if kind == 0:
+        return t
+    pad = [0, rng.randrange(1, 4)] if kind == 1 else [rng.randrange(1, 3), rng.randrange(0, 3)]
+    big = torch.nn.functional.pad(t, pad + [rng.randrange(0, 2), rng.randrange(0, 2)], value=7.0)
+    sl = [slice(None)] * (t.dim() - 2)
+    r0 = big.shape[-2] - t.shape[-2] - 0
+    lo_r = 0 if big.shape[-2] == t.shape[-2] else rng.randrange(0, big.shape[-2] - t.shape[-2] + 1)
+    v = big[(*sl, slice(lo_r, lo_r + t.shape[-2]), slice(pad[0], pad[0] + t.shape[-1]))]
+    assert v.shape == t.shape and r0 >= 0
+    v.copy_(t)
+    return v
+
+
+def _sprinkle(rng, g, b):
+    p = rng.choice([0.0, 0.02, 0.3])
+    if p:
+        b[torch.rand(b.shape, generator=g) < p] = NINF
+    if rng.random() < 0.5:
+        b[..., rng.randrange(b.shape[-1])] = NINF  # an all -inf column
+    return b
+
+
+@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+def test_lm2exp_random(dev, seed, precision):
+    rng = random.Random(1000 + seed)
+    g = torch.Generator().manual_seed(seed)
+    R, I, J, K = rng.randrange(1, 4), _dim(rng, 200), _dim(rng, 257), _dim(rng, 257)
+    a = torch.rand(R, I, J, generator=g) * rng.choice([1.0, 1e-3, 50.0])
+    if rng.random() < 0.3:
+        a[:, rng.randrange(I)] = 0.0
+    b = _sprinkle(rng, g, torch.randn(R, J, K, generator=g) * rng.choice([1.0, 8.0, 40.0]) + rng.choice([0.0, -60.0, 90.0]))
+    ref = oracle64.lm2exp64(a, b)
+    ag, bg = _view(rng, a.to(dev)), _view(rng, b.to(dev))
+    nvar = 0 if precision == "fp32" else 6
+    variant = rng.randrange(0, nvar + 1)
+    out = lm2exp(ag, bg, _precision=precision, _variant=variant)
+    r = oracle64.compare(out, ref, **GATES[precision])
+    assert r["ok"], (R, I, J, K, variant, r)
+
+
+@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+def test_lt2exp_random(dev, seed, precision):
+    rng = random.Random(2000 + seed)
+    g = torch.Generator().manual_seed(seed)
+    R, S, I, J, K = rng.randrange(1, 3), _dim(rng, 130), _dim(rng, 33), _dim(rng, 70), _dim(rng, 257)
+    w = torch.rand(R, S, I, J, generator=g) * rng.choice([1.0, 1e-4, 30.0])
+    if rng.random() < 0.3:
+        w[:, rng.randrange(S)] = 0.0
+    a = _sprinkle(rng, g, torch.randn(R, I, K, generator=g) * rng.choice([1.0, 10.0]) + rng.choice([0.0, -40.0]))
+    b = _sprinkle(rng, g, torch.randn(R, J, K, generator=g) * rng.choice([1.0, 10.0]) + rng.choice([0.0, 70.0]))
+    ref = oracle64.lt2exp64(w, a, b)
+    ag, bg = _view(rng, a.to(dev)), _view(rng, b.to(dev))
+    wg = w.to(dev)
+    if rng.random() < 0.5:  # padded rows of S: still viewable as R x S x (I*J)
+        big = torch.zeros(R, S + 2, I, J, device=dev)
+        big[:, 1 : S + 1] = wg
+        wg = big[:, 1 : S + 1]
+    mode = rng.choice(["auto", "split", "unsplit"])
+    variant = 0 if precision == "fp32" else rng.randrange(0, 5)
+    out = lt2exp(wg, ag, bg, mode=mode, _precision=precision, _variant=variant)
+    r = oracle64.compare(out, ref, **GATES[precision])
+    assert r["ok"], (R, S, I, J, K, mode, variant, r)
