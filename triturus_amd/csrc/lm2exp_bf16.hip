@@ -127,14 +127,21 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
     const uint32_t b_row_bytes = (uint32_t)p.sb1 * 4u;
     const uint32_t boff = ((uint32_t)(8 * h) * (uint32_t)p.sb1 + (uint32_t)ncl) * 4u;
     auto load_b = [&](int jc) {
-        const bool full = jc * JC + JC <= p.J;  // wave-uniform
+        if (jc * JC + JC <= p.J) {  // wave-uniform: a full chunk needs no masks
 #pragma unroll
-        for (int ks = 0; ks < KS; ++ks)
+            for (int ks = 0; ks < KS; ++ks)
 #pragma unroll
-            for (int e = 0; e < 8; ++e) {
-                const float v = buf_load_f32(b_rsrc, boff, (uint32_t)(jc * JC + 16 * ks + e) * b_row_bytes);
-                braw[ks][e] = (full || jc * JC + 16 * ks + 8 * h + e < p.J) ? v : -__builtin_inff();
-            }
+                for (int e = 0; e < 8; ++e)
+                    braw[ks][e] = buf_load_f32(b_rsrc, boff, (uint32_t)(jc * JC + 16 * ks + e) * b_row_bytes);
+        } else {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float v = buf_load_f32(b_rsrc, boff, (uint32_t)(jc * JC + 16 * ks + e) * b_row_bytes);
+                    braw[ks][e] = (jc * JC + 16 * ks + 8 * h + e < p.J) ? v : -__builtin_inff();
+                }
+        }
     };
     // Maximum of the chunk's column (both lane halves).  A NaN need not survive here:
     // exp(NaN - m) is NaN for any m and poisons the column through the MFMA.
