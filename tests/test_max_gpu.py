@@ -138,6 +138,27 @@ def test_matmax_shapes(dev, shape):
         assert np.array_equal(y.cpu().numpy(), max_ref.matmax_ref(x.numpy(), axis))
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("shape", [(1024, 4096), (1500, 4100), (1025, 8200), (2048, 16384)])
+def test_matmax_long_rows(dev, dtype, shape):
+    """Many rows of at least 16 KiB take the workgroup-per-row kernel along axis 1 (whole
+    blocks, a partial block and a scalar tail, depending on the row length)."""
+    m, n = shape
+    g = torch.Generator().manual_seed(m + n)
+    x = torch.randn(m, n, generator=g).to(dtype)
+    x[3, n - 1] = 50.0          # maximum in the scalar tail
+    x[4, 0] = 60.0
+    x[7, n // 2] = float("nan")
+    x[9, :] = float("-inf")
+    xg = x.to(dev)
+    for axis in (0, 1):
+        _same(matmax(xg, axis), torch.amax(x, axis))
+    # the same rows through a view that is only element-aligned (other kernel path)
+    base = torch.zeros(m * n + 1, dtype=dtype)
+    base[1:] = x.reshape(-1)
+    _same(matmax(base.to(dev)[1:].view(m, n), 1), torch.amax(x, 1))
+
+
 def test_matmax_golden_and_views(dev):
     z = np.load(GOLDEN / "matmax_small.npz")
     x = torch.from_numpy(z["x"]).to(dev)

@@ -374,6 +374,50 @@ __global__ __launch_bounds__(kMatThreads) void rowmax_kernel(
     if (lane == 0) y[row * ldy + split] = E::down(best);
 }
 
+// Row maxima of long rows: one workgroup per row, its 256 lanes walking the row in contiguous
+// blocks of 4 x 256 16-byte pieces (16 KiB).  Contiguous blocks per workgroup stream faster
+// than four wavefronts on four different rows (measured on 16384^2 fp32: 174 us against 189 us).
+template <int DT>
+__global__ __launch_bounds__(kMatThreads) void rowmax_wide_kernel(const typename Elem<DT>::T *__restrict__ x,
+                                                                  int64_t ld, int64_t n,
+                                                                  typename Elem<DT>::T *__restrict__ y) {
+    using E = Elem<DT>;
+    using T = typename E::T;
+    using C = typename E::C;
+    using V = Vec16<T>;
+    constexpr int VN = V::N;
+    const int tid = threadIdx.x;
+    const T *xr = x + (int64_t)blockIdx.x * ld;
+    const V *xv = reinterpret_cast<const V *>(xr);
+    const int64_t nv = n / VN;
+    C best = neg_inf<C>();
+    int64_t v = tid;
+    for (; v + 3 * kMatThreads < nv; v += 4 * kMatThreads) {
+        V b[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) b[u] = xv[v + u * kMatThreads];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int e = 0; e < VN; ++e) best = vmax_nan(best, E::up(b[u].e[e]));
+    }
+    for (; v < nv; v += kMatThreads) {
+        V b0 = xv[v];
+#pragma unroll
+        for (int e = 0; e < VN; ++e) best = vmax_nan(best, E::up(b0.e[e]));
+    }
+    for (int64_t c = nv * VN + tid; c < n; c += kMatThreads) best = vmax_nan(best, E::up(xr[c]));
+    best = wave_max(best);
+    __shared__ C part[kMatWaves];
+    if (lane_id() == 0) part[tid / kWave] = best;
+    __syncthreads();
+    if (tid == 0) {
+#pragma unroll
+        for (int w = 1; w < kMatWaves; ++w) best = vmax_nan(best, part[w]);
+        y[blockIdx.x] = E::down(best);
+    }
+}
+
 // Column maxima (reduction along the strided axis).  Each thread owns CN
 // adjacent columns; the 4 wavefronts of a workgroup interleave over the rows
 // of the workgroup's row chunk and combine through LDS.
@@ -443,6 +487,17 @@ struct MatPlan {
 };
 
 constexpr int64_t kTargetWaves = 4096;
+
+// Rows of at least 16 KiB, enough of them to fill the chip, 16-byte aligned: one workgroup
+// per row (rowmax_wide_kernel), no partial results.  (The same idea for axis 0 -- a
+// workgroup on 4 KiB of each row -- measured no better at 16384^2 and worse at 8192^2.)
+template <int DT>
+static bool rowmax_wide(const void *x, int64_t m, int64_t n) {
+    using T = typename Elem<DT>::T;
+    constexpr int VN = 16 / (int)sizeof(T);
+    return m >= 1024 && n * (int64_t)sizeof(T) >= 16384 && (reinterpret_cast<uintptr_t>(x) & 15) == 0 &&
+           (n % VN) == 0 && m < ((int64_t)1 << 31);
+}
 
 static MatPlan rowmax_plan(int64_t m, int64_t n, int vn) {
     // enough (row, chunk) wavefronts to fill 256 CUs; chunks of >= 2048
@@ -524,7 +579,9 @@ static int matmax_launch(const void *xv, void *yv, int64_t m, int64_t n, int axi
     T *part = static_cast<T *>(ws);
     if (matmax_ws<DT>(m, n, axis) > ws_bytes) return TRT_E_WORKSPACE;
     if (matmax_ws<DT>(m, n, axis) > 0 && ws == nullptr) return TRT_E_WORKSPACE;
-    if (axis == 1) {
+    if (axis == 1 && rowmax_wide<DT>(x, m, n)) {
+        hipLaunchKernelGGL((rowmax_wide_kernel<DT>), dim3((unsigned)m), dim3(kMatThreads), 0, stream, x, n, n, y);
+    } else if (axis == 1) {
         MatPlan p = rowmax_plan(m, n, VN);
         if (p.splits == 1) {
             rowmax_launch<DT>(x, n, m, n, p, y, 1, stream);
