@@ -89,3 +89,32 @@ def test_lt2exp_random(dev, seed, precision):
     out = lt2exp(wg, ag, bg, mode=mode, _precision=precision, _variant=variant)
     r = oracle64.compare(out, ref, **GATES[precision])
     assert r["ok"], (R, S, I, J, K, mode, variant, r)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+def test_results_are_bit_reproducible(dev, precision):
+    """Fixed summation order everywhere (no atomics, merges in split order): the same call on
+    the same inputs gives the same bits, run after run, whatever else the GPU is doing --
+    including the paths that cut the contraction over several workgroups."""
+    g = torch.Generator().manual_seed(99)
+    w = torch.rand(3, 75, 50, 50, generator=g).to(dev)
+    a = torch.randn(3, 50, 100, generator=g).to(dev)
+    b = torch.randn(3, 50, 100, generator=g).to(dev)
+    a2 = torch.rand(2, 96, 700, generator=g).to(dev)
+    b2 = (torch.randn(2, 700, 130, generator=g) * 20).to(dev)
+    big_w = torch.rand(8, 64, 32, 32, generator=g).to(dev)
+    big_a = torch.randn(8, 32, 2048, generator=g).to(dev)
+    big_b = torch.randn(8, 32, 2048, generator=g).to(dev)
+    calls = [
+        lambda: lt2exp(w, a, b, mode="split", _precision=precision),
+        lambda: lt2exp(w, a, b, mode="unsplit", _precision=precision),
+        lambda: lt2exp(big_w, big_a, big_b, _precision=precision),
+        lambda: lm2exp(a2, b2, _precision=precision),
+        lambda: lm2exp(a2, b2, _precision=precision, _splits=5),
+    ]
+    first = [f().clone() for f in calls]
+    noise = torch.randn(4096, 4096, device=dev)
+    for rep in range(3):
+        (noise @ noise).sum()  # unrelated work in between
+        for f, ref in zip(calls, first):
+            assert torch.equal(f(), ref)
