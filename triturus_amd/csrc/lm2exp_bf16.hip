@@ -287,7 +287,7 @@ struct LmBfVariant {
     int rt, ks;
 };
 // variant ids are 1-based in the C ABI (0 = choose by shape)
-static const LmBfVariant kLmBfVariants[] = {{4, 4}, {4, 2}, {2, 4}, {2, 2}, {1, 4}, {1, 2}};
+static const LmBfVariant kLmBfVariants[] = {{4, 4}, {4, 2}, {2, 4}, {2, 2}, {1, 4}, {1, 2}, {8, 1}, {8, 2}};
 constexpr int kNumLmBfVariants = sizeof(kLmBfVariants) / sizeof(kLmBfVariants[0]);
 
 }  // namespace trt
@@ -312,7 +312,9 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     // byte offsets inside one batch slab are 32-bit (buffer addressing)
     if (I * sa[1] + J >= lim || J * sb[1] + K >= lim || I * sc[1] + K >= lim) return TRT_E_RANGE;
 
-    // Tile by grid fill (measured over the reference's benchmark grid): 128 rows when that
+    // Tile by grid fill (measured over the reference's benchmark grid): with two pieces the
+    // kernel is bound by the vector work on the B operand, so 256 rows when that still leaves
+    // two workgroups per CU (6 % at R=64, I=J=256, K=4096); otherwise 128 rows when that
     // leaves >= 1.5 workgroups per CU (j-chunks of 64 for a long contraction, where the fewer
     // barriers pay; of 32 otherwise, so that three workgroups fit a CU), 64 rows when that
     // leaves >= 1 per CU.  Smaller grids are latency bound, not matrix bound: there the fp32
@@ -324,7 +326,9 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     } else {
         const int64_t ct = ceil_div(K, 128);
         const int64_t n128 = R * ceil_div(I, 128) * ct, n64 = R * ceil_div(I, 64) * ct;
+        const int64_t n256 = R * ceil_div(I, 256) * ct;
         if (splits > 1) v = -1;
+        else if (pieces == 2 && I > 128 && n256 >= 512 && J < 512) v = 7;  // 256 rows: each exp feeds 24 MFMAs
         else if (I > 64 && n128 >= 384) v = (pieces == 2 && J >= 512) ? 0 : 1;
         else if (I > 32 && n64 >= 256) v = pieces == 2 ? 2 : 3;
         else v = -1;
@@ -353,6 +357,8 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
         case 2: return launch_lm_bf<2, 4>(args, pieces, vec, s);
         case 3: return launch_lm_bf<2, 2>(args, pieces, vec, s);
         case 4: return launch_lm_bf<1, 4>(args, pieces, vec, s);
-        default: return launch_lm_bf<1, 2>(args, pieces, vec, s);
+        case 5: return launch_lm_bf<1, 2>(args, pieces, vec, s);
+        case 6: return launch_lm_bf<8, 1>(args, pieces, vec, s);
+        default: return launch_lm_bf<8, 2>(args, pieces, vec, s);
     }
 }
