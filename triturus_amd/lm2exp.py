@@ -4,6 +4,11 @@ Same contract as the reference wrapper, triturus/lm2exp.py:167-206:
 a is R x I x J (linear space), b is R x J x K (log space), both fp32 on one
 device; returns a fresh R x I x K tensor, enqueued on the current stream
 without synchronising.
+
+Arithmetic: IEEE fp32 on the fp32 matrix pipe; with the reference's TF32 flag on
+(is_triturus_tf32_enabled(), read at triturus/lm2exp.py:185) the bf16 matrix pipe with operands
+cut into two bf16 pieces, see triturus_amd.utils.  The underscore keywords
+(tile variant, split count, arithmetic) are for tests and experiments.
 """
 
 from __future__ import annotations

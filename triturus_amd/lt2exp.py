@@ -6,6 +6,11 @@ all fp32 on one device; returns a fresh R x S x K tensor.  ``mode`` is
 "auto" | "split" | "unsplit"; anything else raises ValueError.  w must be
 viewable as R x S x (I*J) (``w.view`` raises RuntimeError otherwise, as in the
 reference).
+
+Arithmetic: IEEE fp32 on the fp32 matrix pipe; with the reference's TF32 flag on
+(is_triturus_tf32_enabled(), read at triturus/lt2exp.py:551) the bf16 matrix pipe with operands
+cut into two bf16 pieces, see triturus_amd.utils.  The underscore keywords
+(tile variant, split count, arithmetic) are for tests and experiments.
 """
 
 from __future__ import annotations
