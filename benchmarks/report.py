@@ -23,6 +23,10 @@ this repository; `triturus (allow_tf32)` is the same call after `set_tf32_enable
 """
 
 
+def stem(name: str) -> str:
+    return "".join(c if c.isalnum() else "_" for c in name)
+
+
 def table(sweep: dict) -> str:
     rows = sweep["rows"]
     providers = [k for k in rows[0] if k != "x"]
@@ -36,6 +40,9 @@ def table(sweep: dict) -> str:
         if ratio:
             cells.append(f"{r['triturus'][0] / r['torch'][0]:.2f}")
         lines.append("| " + " | ".join(cells) + " |")
+    plot = Path(__file__).with_name("plots") / (stem(sweep["name"]) + ".png")
+    if plot.exists():
+        lines += ["", f"![{sweep['name']}](plots/{plot.name})"]
     return "\n".join(lines)
 
 
