@@ -118,3 +118,24 @@ def test_results_are_bit_reproducible(dev, precision):
         (noise @ noise).sum()  # unrelated work in between
         for f, ref in zip(calls, first):
             assert torch.equal(f(), ref)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+def test_very_long_column_axis(dev, precision):
+    """K = 2^20 + 3 columns (8193 column tiles, offsets beyond 2^22 elements per row): every
+    column against the float64 oracle."""
+
+    g = torch.Generator().manual_seed(5)
+    K = (1 << 20) + 3
+    a = torch.rand(1, 40, 24, generator=g).to(dev)
+    b = (torch.randn(1, 24, K, generator=g) * 6).to(dev)
+    b[0, :, K - 1] = NINF
+    out = lm2exp(a, b, _precision=precision)
+    ref = oracle64.lm2exp64(a.cpu(), b.cpu())
+    assert oracle64.compare(out, ref, **GATES[precision])["ok"]
+    w = torch.rand(1, 20, 6, 10, generator=g).to(dev)
+    a2 = (torch.randn(1, 6, K, generator=g) * 3).to(dev)
+    b2 = (torch.randn(1, 10, K, generator=g) * 3).to(dev)
+    out = lt2exp(w, a2, b2, _precision=precision)
+    ref = oracle64.lt2exp64(w.cpu(), a2.cpu(), b2.cpu())
+    assert oracle64.compare(out, ref, **GATES[precision])["ok"]
