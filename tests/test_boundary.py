@@ -230,6 +230,15 @@ def test_flags():
     assert torch.equal(x, torch.rand(3))
 
 
+def test_tile_tuning_is_off_by_default():
+    from triturus_amd import autotune
+
+    assert not autotune.is_autotune_enabled()
+    calls = []
+    assert autotune.pick(("k",), (0, 1, 2), calls.append) == 0
+    assert calls == [] and autotune.chosen() == {}
+
+
 def test_reference_import_paths_exist():
     from triturus.lm2exp import lm2exp as f1
     from triturus.lt2exp import lt2exp as f2

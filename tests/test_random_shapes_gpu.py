@@ -139,3 +139,35 @@ def test_very_long_column_axis(dev, precision):
     out = lt2exp(w, a2, b2, _precision=precision)
     ref = oracle64.lt2exp64(w.cpu(), a2.cpu(), b2.cpu())
     assert oracle64.compare(out, ref, **GATES[precision])["ok"]
+
+
+def test_measured_tile_selection(dev):
+    """Opt-in tuning (the reference autotunes per shape key): the first call times the
+    candidate tiles, later calls reuse the choice; results stay within the gate."""
+    from triturus_amd import autotune
+
+    g = torch.Generator().manual_seed(3)
+    a = torch.rand(8, 200, 96, generator=g)
+    b = torch.randn(8, 96, 300, generator=g) * 4
+    w = torch.rand(4, 70, 24, 40, generator=g)
+    a2 = torch.randn(4, 24, 500, generator=g)
+    b2 = torch.randn(4, 40, 500, generator=g)
+    ref_m = oracle64.lm2exp64(a, b)
+    ref_t = oracle64.lt2exp64(w, a2, b2)
+    autotune.clear()
+    autotune.set_autotune(True)
+    try:
+        for precision in ("fp32", "bf16x3"):
+            for _ in range(2):
+                out = lm2exp(a.to(dev), b.to(dev), _precision=precision)
+                assert oracle64.compare(out, ref_m, **GATES[precision])["ok"]
+                out = lt2exp(w.to(dev), a2.to(dev), b2.to(dev), _precision=precision)
+                assert oracle64.compare(out, ref_t, **GATES[precision])["ok"]
+        picked = autotune.chosen()
+        assert ("lm2exp", 8, 200, 96, 300, "fp32") in picked
+        assert ("lt2exp", 4, 70, 24, 40, 500, "auto", "bf16x3") in picked
+        assert all(isinstance(v, int) and v >= 0 for v in picked.values())
+    finally:
+        autotune.set_autotune(False)
+        autotune.clear()
+    assert autotune.pick(("x",), (0, 1), lambda v: None) == 0  # off: the library's rule

@@ -15,7 +15,7 @@ from __future__ import annotations
 
 import torch
 
-from triturus_amd import _lib
+from triturus_amd import _lib, autotune
 from triturus_amd.utils import MATRIX_PRECISIONS, matrix_precision
 
 
@@ -31,6 +31,9 @@ def _unit_inner(t: torch.Tensor) -> torch.Tensor:
 
 
 _PIECES = {"bf16x3": 2, "bf16x6": 3}
+# tile variants worth timing when tuning is on (0 = the library's rule)
+_FP32_CANDIDATES = (0, 1, 2, 7, 8)
+_BF16_CANDIDATES = (0, 1, 2, 3, 4, 8)
 
 
 def lm2exp(
@@ -58,6 +61,12 @@ def lm2exp(
         _precision = matrix_precision()
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
+    if _variant == 0 and _splits == 0 and autotune.is_autotune_enabled():
+        cands = _FP32_CANDIDATES if _precision == "fp32" else _BF16_CANDIDATES
+        _variant = autotune.pick(("lm2exp", R, I, J, K, _precision), cands,
+                                 lambda v: lm2exp(a, b, _variant=v, _splits=-1, _precision=_precision))
+    if _splits < 0:  # tuning launch: the library decides the split for this tile
+        _splits = 0
     # small grids with a long contraction are cut over J; the partial sums need a workspace
     fp32_variant = _variant if _precision == "fp32" else 0
     key = (R, I, J, K, fp32_variant, _splits)

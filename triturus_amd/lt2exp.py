@@ -17,7 +17,7 @@ from __future__ import annotations
 
 import torch
 
-from triturus_amd import _lib
+from triturus_amd import _lib, autotune
 from triturus_amd.lm2exp import _unit_inner
 from triturus_amd.utils import MATRIX_PRECISIONS, matrix_precision
 
@@ -38,11 +38,14 @@ def launches_split(R: int, S: int, I: int, J: int, K: int, mode: str) -> bool:
 
 
 _PIECES = {"bf16x3": 2, "bf16x6": 3}
+# tile variants worth timing when tuning is on (0 = the library's rule)
+_FP32_CANDIDATES = (0, 5, 6, 8)
+_BF16_CANDIDATES = (0, 1, 2, 3, 4)
 
 
 def lt2exp(
     w: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, mode: str = "auto", _variant: int = 0,
-    _precision: str | None = None,
+    _precision: str | None = None, _tuning: bool = False,
 ) -> torch.Tensor:
     assert len(w.shape) == 4
     assert len(a.shape) == len(b.shape) == 3
@@ -73,6 +76,11 @@ def lt2exp(
         _precision = matrix_precision()
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
+    if _variant == 0 and autotune.is_autotune_enabled() and not _tuning:
+        cands = _FP32_CANDIDATES if _precision == "fp32" else _BF16_CANDIDATES
+        _variant = autotune.pick(("lt2exp", R, S, I, J, K, mode, _precision), cands,
+                                 lambda v: lt2exp(w.view(R, S, I, J), a, b, mode=mode, _variant=v,
+                                                  _precision=_precision, _tuning=True))
     mode_code = _MODES[mode]
     key = (R, S, I, J, K, mode_code)
     ws_bytes = _ws_bytes.get(key)
