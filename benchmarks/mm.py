@@ -13,16 +13,17 @@ from triturus.add import vadd
 from triturus.mm import mm
 from triturus.utils import ensure_reproducibility, set_tf32_enabled
 
-PROVIDERS = ["torch", "triturus"]
+PROVIDERS = ["torch", "triturus", "triturus (allow_tf32)"]
 
 
 def measure_mm(n, provider):
     ensure_reproducibility()
-    set_tf32_enabled(False)
+    set_tf32_enabled(provider == "triturus (allow_tf32)")
     a = torch.rand(n, n)
     b = torch.rand(n, n)
     fn = (lambda: torch.mm(a, b)) if provider == "torch" else (lambda: mm(a, b))
     ms, lo, hi = do_bench(fn)
+    set_tf32_enabled(False)
     nflops = n * n * (2 * n - 1)
     return eval_tflops(nflops, ms), eval_tflops(nflops, hi), eval_tflops(nflops, lo)
 
@@ -38,10 +39,10 @@ def measure_vadd(n, provider):
 
 def main():
     out = out_dir_from_argv()
-    run_sweep("mm (allow_tf32=False)", "m=k=n", [48, 128, 192, 512, 768, 2048, 3072, 8192], PROVIDERS, measure_mm,
+    run_sweep("mm", "m=k=n", [48, 128, 192, 512, 768, 2048, 3072, 8192], PROVIDERS, measure_mm,
               unit="TFLOPS", out_dir=out)
     run_sweep("vadd", "n", [32, 48, 128, 192, 512, 768, 2048, 3072, 8192, 12288, 32768, 49152, 1 << 24, 1 << 28],
-              PROVIDERS, measure_vadd, unit="TFLOPS (additions)", out_dir=out)
+              PROVIDERS[:2], measure_vadd, unit="TFLOPS (additions)", out_dir=out)
 
 
 if __name__ == "__main__":

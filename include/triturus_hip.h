@@ -177,6 +177,14 @@ int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, int64_t k, i
                void *stream);
 
 /*
+ * trt_mm_f32 on the bf16 matrix pipe with split operands (pieces as for trt_lt2exp_bf16;
+ * counterpart of ALLOW_TF32 at triturus/mm.py:212).  Grids too small for the bf16 kernels
+ * are handed to trt_mm_f32.
+ */
+int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n,
+                int pieces, void *stream);
+
+/*
  * r = x + y for contiguous vectors of n elements of `dtype` (TRT_F32 ...).  Replaces the
  * `_ker_vadd[grid](...)` launch, triturus/add.py:45.  Same remark as trt_mm_f32.
  */

@@ -114,6 +114,9 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_mm_f32(one, null, one, 2, 2, 2, null) == -1
     assert lib.trt_mm_f32(one, one, one, 2, 0, 2, null) == -1
     assert lib.trt_mm_f32(one, one, one, 1 << 30, 2, 2, null) == -4
+    assert lib.trt_mm_bf16(one, one, one, 2, 2, 2, 4, null) == -1
+    assert lib.trt_mm_bf16(null, one, one, 2, 2, 2, 2, null) == -1
+    assert lib.trt_mm_bf16(one, one, one, 2, 1 << 30, 2, 3, null) == -4
     assert lib.trt_vadd(one, one, null, 5, 0, null) == -1
     assert lib.trt_vadd(one, one, one, 0, 0, null) == -1
     assert lib.trt_vadd(one, one, one, 5, 7, null) == -1

@@ -42,6 +42,28 @@ def test_mm_shapes(dev, shape):
     assert torch.equal(mm(ai, bi), (ai.double() @ bi.double()).float())
 
 
+@pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
+@pytest.mark.parametrize("shape", [(2048, 512, 1024), (4096, 300, 4096), (1500, 1111, 2000), (8192, 64, 4096)])
+def test_mm_on_the_bf16_pipe(dev, precision, shape):
+    """Split-bf16 matrix product against float64: the error of a product is ~2^-16 (two
+    pieces) or ~2^-23 (three) of |a||b|, so the bound scales with sum_k |a_ik| |b_kj|."""
+    m, k, n = shape
+    g = torch.Generator().manual_seed(m + k + n)
+    a = torch.randn(m, k, generator=g).to(dev)
+    b = torch.randn(k, n, generator=g).to(dev)
+    c = mm(a, b, _precision=precision).double()
+    ref = a.double() @ b.double()
+    scale = a.abs().double() @ b.abs().double()
+    eps = 2.0 ** -14 if precision == "bf16x3" else 2.0 ** -21
+    assert torch.all((c - ref).abs() <= eps * scale + 1e-30)
+    if precision == "bf16x6":  # as good as the fp32 pipe
+        e32 = (mm(a, b, _precision="fp32").double() - ref).abs().max()
+        assert (c - ref).abs().max() <= 2 * e32 + 1e-6
+    ai = torch.randint(-3, 4, (m, k), generator=g).float().to(dev)
+    bi = torch.randint(-3, 4, (k, n), generator=g).float().to(dev)
+    assert torch.equal(mm(ai, bi, _precision=precision), (ai.double() @ bi.double()).float())
+
+
 def test_mm_rejects_what_the_reference_rejects(dev):
     a = torch.rand(4, 5, device=dev)
     with pytest.raises(AssertionError):

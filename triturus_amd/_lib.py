@@ -70,6 +70,7 @@ SIGNATURES = {
     ),
     "trt_vmax_workspace_bytes": (c_size_t, [c_int64, c_int]),
     "trt_mm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
+    "trt_mm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "trt_vadd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "trt_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
 }

@@ -32,7 +32,8 @@ struct Lm2BfArgs {
     int64_t total_wgs, padded_wgs;
 };
 
-template <int RT, int KS, int NS, bool VEC>
+// PLAIN: no shift, exp or log -- c = a b, the matrix product of trt_mm_bf16.
+template <int RT, int KS, int NS, bool VEC, bool PLAIN = false>
 __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) {
     constexpr int NT = 256;
     constexpr int TM = 32 * RT;   // rows of I per workgroup
@@ -146,7 +147,7 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 #pragma unroll
                 for (int e = 0; e < 8; ++e) {
                     const float v = buf_load_f32(b_rsrc, boff, (uint32_t)(jc * JC + 16 * ks + e) * b_row_bytes);
-                    braw[ks][e] = (jc * JC + 16 * ks + 8 * h + e < p.J) ? v : -__builtin_inff();
+                    braw[ks][e] = (jc * JC + 16 * ks + 8 * h + e < p.J) ? v : (PLAIN ? 0.f : -__builtin_inff());
                 }
         }
     };
@@ -176,6 +177,18 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
             }
     };
     auto shift_and_exp = [&]() {
+        if (PLAIN) {  // the B operand is b itself
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    uint32_t pk[NS];
+                    split_pair<NS, false>(braw[ks][2 * u], braw[ks][2 * u + 1], pk);
+#pragma unroll
+                    for (int sp = 0; sp < NS; ++sp) ebp[sp][ks][u] = pk[sp];
+                }
+            return;
+        }
         const float cm = chunk_max();
         const bool need = cm > mref + kMargin;
         if (__builtin_amdgcn_ballot_w64(need) != 0) {
@@ -201,7 +214,7 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
     load_tile(0);
     load_b(0);
     store_tile(0);
-    mref = clamp_shift(chunk_max());
+    mref = PLAIN ? 0.f : clamp_shift(chunk_max());
     shift_and_exp();
     __syncthreads();
 
@@ -258,16 +271,16 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4);
-            buf_store_f32_stream(log_plus(acc[rt][v], mref), c_rsrc, co, trow_c * c_row_bytes);
+            buf_store_f32_stream(PLAIN ? acc[rt][v] : log_plus(acc[rt][v], mref), c_rsrc, co, trow_c * c_row_bytes);
         }
 }
 
 constexpr size_t kBfDefaultLdsLimit = 64 * 1024;
 
-template <int RT, int KS, int NS, bool VEC>
+template <int RT, int KS, int NS, bool VEC, bool PLAIN = false>
 static int launch_lm_bf_k(const Lm2BfArgs &args, hipStream_t stream) {
     constexpr size_t lds = (size_t)2 * NS * (32 * RT) * (16 * KS + 8) * sizeof(__bf16);
-    auto k = lm2exp_bf16_kernel<RT, KS, NS, VEC>;
+    auto k = lm2exp_bf16_kernel<RT, KS, NS, VEC, PLAIN>;
     if (lds > kBfDefaultLdsLimit) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -361,4 +374,44 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
         case 6: return launch_lm_bf<8, 1>(args, pieces, vec, s);
         default: return launch_lm_bf<8, 2>(args, pieces, vec, s);
     }
+}
+
+// c = a b for row-major fp32 matrices on the bf16 matrix pipe (operands cut into `pieces`
+// bf16 pieces, fp32 accumulation): the kernel above without shift, exp and log.  Grids too
+// small for it go to trt_mm_f32.  Counterpart of `_ker_mm[grid](..., ALLOW_TF32=True)`,
+// triturus/mm.py:199-213.
+template <int RT, int KS>
+static int launch_mm_bf(const Lm2BfArgs &args, int pieces, bool vec, hipStream_t s) {
+    if (pieces == 2)
+        return vec ? launch_lm_bf_k<RT, KS, 2, true, true>(args, s) : launch_lm_bf_k<RT, KS, 2, false, true>(args, s);
+    return vec ? launch_lm_bf_k<RT, KS, 3, true, true>(args, s) : launch_lm_bf_k<RT, KS, 3, false, true>(args, s);
+}
+
+extern "C" int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, int pieces,
+                           void *stream) {
+    if (!a || !b || !c) return TRT_E_INVALID;
+    if (m <= 0 || k <= 0 || n <= 0) return TRT_E_INVALID;
+    if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
+    const int64_t lim = (int64_t)1 << 30;
+    if (m >= lim || k >= lim || n >= lim) return TRT_E_RANGE;
+    if (k * n + n >= lim || m * k + k >= lim || m * n + n >= lim) return TRT_E_RANGE;
+    const int64_t ct = ceil_div(n, 128);
+    const int64_t n128 = ceil_div(m, 128) * ct, n64 = ceil_div(m, 64) * ct;
+    int rt;
+    if (m > 64 && n128 >= 384) rt = 4;
+    else if (m > 32 && n64 >= 256) rt = 2;
+    else return trt_mm_f32(a, b, c, m, k, n, stream);
+    Lm2BfArgs args;
+    args.a = a; args.b = b; args.c = c;
+    args.R = 1; args.I = (int)m; args.J = (int)k; args.K = (int)n;
+    args.sa0 = m * k; args.sa1 = k;
+    args.sb0 = k * n; args.sb1 = n;
+    args.sc0 = m * n; args.sc1 = n;
+    args.i_tiles = (int)ceil_div(m, 32 * rt);
+    args.n_tiles = (int)ct;
+    args.total_wgs = (int64_t)args.i_tiles * args.n_tiles;
+    args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    const bool vec = (k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    return rt == 4 ? launch_mm_bf<4, 2>(args, pieces, vec, s) : launch_mm_bf<2, 4>(args, pieces, vec, s);
 }

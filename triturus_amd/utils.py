@@ -63,6 +63,11 @@ def set_matrix_precision(precision: str | None) -> None:
     _MATRIX_PRECISION = precision
 
 
+def pinned_matrix_precision() -> str | None:
+    """What set_matrix_precision pinned, or None while the TF32 flag decides."""
+    return _MATRIX_PRECISION
+
+
 def matrix_precision() -> str:
     """The arithmetic the next lm2exp / lt2exp call will use."""
     if _MATRIX_PRECISION is not None:
