@@ -144,9 +144,16 @@ class _NoSwitch:
 _NO_SWITCH = _NoSwitch()
 
 
+try:  # the current device ordinal without torch.cuda's lazy-init checks
+    _get_device = torch._C._cuda_getDevice
+except AttributeError:  # pragma: no cover
+    _get_device = torch.cuda.current_device
+
+
 def on_device(device: torch.device):
     """Context that makes `device` current for the launch; free when it already is."""
-    if device.index is None or device.index == torch.cuda.current_device():
+    idx = device.index
+    if idx is None or idx == _get_device():
         return _NO_SWITCH
     return torch.cuda.device(device)
 
@@ -154,7 +161,7 @@ def on_device(device: torch.device):
 def require_gpu(*tensors: torch.Tensor) -> None:
     """The kernels run on HIP device memory only."""
     for t in tensors:
-        if t.device.type != "cuda":
+        if not t.is_cuda:
             raise RuntimeError(
                 f"triturus_amd runs on the GPU only: got a tensor on '{t.device}'. "
                 "Move the inputs to the HIP device (there is no CPU fallback)."

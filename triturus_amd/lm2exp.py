@@ -25,7 +25,8 @@ _ws_bytes: dict = {}  # (R, I, J, K, variant, splits) -> workspace bytes, as rep
 def _unit_inner(t: torch.Tensor) -> torch.Tensor:
     # The kernels take free batch/row strides but a unit trailing stride (and
     # no negative or zero-broadcast strides); anything else is materialised.
-    if t.stride(-1) == 1 and all(s > 0 for s in t.stride()):
+    st = t.stride()
+    if st[-1] == 1 and min(st) > 0:
         return t
     return t.contiguous()
 
