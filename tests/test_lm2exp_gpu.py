@@ -19,7 +19,7 @@ from triturus_amd import _lib, workloads
 pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
-N_VARIANTS = 11
+N_VARIANTS = 12
 N_BF16_VARIANTS = 8
 # Accuracy gates of the split-bf16 paths against the float64 oracle: two pieces (3 MFMAs per
 # product) carry 16 significand bits -- looser than fp32, ten times tighter than the rtol 5e-4
@@ -154,7 +154,7 @@ def test_neg_inf_columns_zero_rows_and_range(dev):
     assert torch.isfinite(out).all()
 
 
-@pytest.mark.parametrize("variant", [0, 3, 10])
+@pytest.mark.parametrize("variant", [0, 3, 10, 12])
 def test_shift_moves_during_the_sweep(dev, variant):
     """Columns whose maximum keeps growing along J (ascending, step changes of 1e3 and 1e30,
     finite values only in the last rows): the single-sweep kernel must rescale its sums on
@@ -275,7 +275,7 @@ def test_benchmark_configuration_c3_full_size(dev):
         worst = max(worst, r["worst_err_over_tol"])
     # size-independent properties on the whole output
     assert torch.all(out <= bg.amax(1, keepdim=True) + 1e-3)
-    for variant in (2, 3, 5, 10, 11):  # other tiles, the two-sweep kernels, the two-launch variant
+    for variant in (2, 3, 5, 10, 11, 12):  # other tiles, the two-sweep kernels, the two-launch variant
         alt = lm2exp(ag, bg, _variant=variant)
         assert torch.allclose(alt, out, rtol=1e-5, atol=1e-5)
     shifted = lm2exp(ag, bg + 128.0)

@@ -26,7 +26,7 @@ def test_mm(dev, allow_tf32):
 
 
 @pytest.mark.parametrize("shape", [(1, 1, 1), (33, 7, 31), (64, 64, 64), (300, 52, 129), (129, 1000, 257),
-                                   (2048, 512, 1024), (4096, 300, 4096)])
+                                   (2048, 512, 1024), (4096, 300, 4096), (3072, 200, 3072), (285, 70, 16400)])
 def test_mm_shapes(dev, shape):
     m, k, n = shape
     g = torch.Generator().manual_seed(m + k + n)

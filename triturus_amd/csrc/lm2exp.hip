@@ -284,9 +284,9 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     shift_and_exp();
     __syncthreads();
 
-    // Row tiles are taken two at a time so that consecutive MFMAs alternate between
-    // two accumulators while only two A fragments are live.
-    constexpr int RP = RT >= 2 ? 2 : 1;
+    // Row tiles are taken two at a time (all three of a 96-row tile) so that consecutive
+    // MFMAs alternate between accumulators while only two or three A fragments are live.
+    constexpr int RP = RT % 2 == 0 ? 2 : (RT == 3 ? 3 : 1);
     auto mfma_block = [&](const float *tile) {
 #pragma unroll
         for (int q = 0; q < NQ; ++q) {
@@ -448,6 +448,7 @@ static const Lm2Variant kVariants[] = {
     {2, 1, 1, 4, 4, kTwoSweep},  // 9: as 7, two sweeps
     {4, 1, 1, 4, 4, kTwoSweep},  // 10: as 1, two sweeps
     {4, 1, 1, 4, 4, kExternal},  // 11: as 1, shift from a separate pass over b (two launches)
+    {3, 1, 1, 4, 4, kOnline},   // 12: 96 x 128 tile (I = 96, 192, ... without padded rows)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be opted into per kernel
@@ -457,14 +458,12 @@ constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be op
 // registers, 2 per SIMD) although b is then exponentiated once per row tile.
 // Smaller grids want smaller row tiles: a 128-row tile amortises each exp over four
 // MFMAs, but it only pays when there are enough tiles to keep 256 CUs busy with more
-// than one workgroup each.  Rules fitted to a sweep of all variants over the shapes of
-// the reference's benchmark grid (batch-1 squares 128..2048; R=64/384, n=256):
-//   >= 1.5 tiles of 128 rows per CU        128 x 128  (128 x 256 when a[r] outgrows an
-//                                          XCD's L2 and the wide tiles still fill the chip:
-//                                          one LDS copy of the a tile then serves 8 waves)
-//   >= 1.5 tiles of 64 rows per CU         64 x 128   (+2..5 %)
-//   fewer, long contraction (J >= 1280)    the largest tile that leaves >= 128 tiles
-//   fewer, short contraction               32 x 128   (+12..36 %)
+// than one workgroup each.  Rules fitted to sweeps of the variants over the shapes of
+// the reference's benchmark grid (batch-1 squares 128..2048; R=64/384, n=256, m=k=64..1024):
+//   < 1.5 workgroups of 64 rows per CU and a    the largest tile that leaves >= 128 tiles (the
+//   long contraction (J >= 1280)                contraction is then cut over J)
+//   some tile leaves >= 1 workgroup per CU      the one with the least modelled time (pick_tile)
+//   none does                                   32 x 128   (+12..36 %)
 static int find_variant(int rt, int wn, int mode) {
     for (int v = 0; v < kNumVariants; ++v)
         if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].wm == 1 && kVariants[v].wn == wn &&
@@ -473,8 +472,48 @@ static int find_variant(int rt, int wn, int mode) {
     return 0;
 }
 
+// Tile for a grid of R x I rows and K columns among 128 x 128, 96 x 128, 64 x 128 and (wide =
+// true) 128 x 256; returns the rows in units of 32 (4, 3, 2; 8 stands for 128 x 256), or 0 when
+// none of them leaves a workgroup per CU.
+// Modelled time: T = tiles per CU (256 CUs), each costing rt MFMA blocks plus an overhead that
+// does not shrink with the tile (the exp / shift work of the b chunk, loads, barriers: 0.75
+// blocks, less without the exp work), counted in quarter blocks.  A CU holds `res` workgroups at a
+// time (3, four of 64-row tiles, one wide); they share the matrix pipe, so a full round costs
+// the sum of its tiles, but a last round with a single workgroup runs at about 2/3 speed (one
+// wavefront per SIMD hides little latency) and one with two at ~0.8: a tail penalty, fading when
+// T is large (workgroups are dispatched as others finish).  The wide tile costs 6.5 % more per row
+// (measured on large grids) and only ever wins by avoiding such a tail.
+// Fitted at R=384 and R=64, I=J=64..1024, K=256: ranks the tiles as measured in 26 of 28 shapes
+// (both misses within 5 %); I = 96, 160, 192, 288 move to 96 rows (-15..23 %), I = 320 to 64.
+static int pick_tile(int64_t R, int64_t I, int64_t K, int overhead_quarters, bool wide) {
+    const int64_t kFill = 256, kCuCount = 256;  // at least one workgroup per CU
+    int best = 0;
+    int64_t best_cost = 0;
+    auto consider = [&](int id, int64_t n, int64_t c, int res) {
+        if (n < kFill) return;
+        const int64_t T = ceil_div(n, kCuCount);
+        const int64_t rem = T % res;
+        int64_t tail = 0;  // in 1/20 of a tile
+        if (res > 1 && rem == 1) tail = 10;
+        else if (res > 1 && rem == 2) tail = res == 3 ? 4 : 6;
+        else if (res > 1 && rem == 3) tail = 2;
+        if (T > 4) tail = tail * 4 / T;
+        const int64_t cost = T * c * 20 + tail * c;
+        if (best == 0 || cost < best_cost) {
+            best = id;
+            best_cost = cost;
+        }
+    };
+    const int64_t ct = ceil_div(K, 128);
+    for (int rt = 4; rt >= 2; --rt)
+        consider(rt, R * ceil_div(I, 32 * rt) * ct, 4 * rt + overhead_quarters, rt == 2 ? 4 : 3);
+    if (wide && K % 256 == 0)
+        consider(8, R * ceil_div(I, 128) * (K / 256), (2 * (16 + overhead_quarters) * 213) / 200, 1);
+    return best;
+}
+
 static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
-    const int64_t kFill = 384;  // 1.5 workgroups per CU
+    const int64_t kFill = 384;
     const int64_t ct = ceil_div(K, 128);
     const int64_t n128 = R * ceil_div(I, 128) * ct, n64 = R * ceil_div(I, 64) * ct;
     int rt;
@@ -482,14 +521,12 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
         rt = 1;
     } else if (I <= 64) {
         rt = (n64 >= kFill || J >= 1280) ? 2 : 1;
-    } else if (n128 >= kFill) {
-        if (I * J >= ((int64_t)1 << 20) && K % 256 == 0 && R * ceil_div(I, 128) * (K / 256) >= 512)
-            return find_variant(4, 8, kOnline);
-        rt = 4;
-    } else if (n64 >= kFill) {
-        rt = 2;
-    } else if (J >= 1280) {
+    } else if (J >= 1280 && n64 < kFill) {
+        // at most 1.5 workgroups per CU and a long contraction: it will be cut over J, which
+        // fills the chip; take the largest tile that leaves >= 128 tiles
         rt = n128 >= 128 ? 4 : (n64 >= 128 ? 2 : 1);
+    } else if ((rt = pick_tile(R, I, K, 3, true)) != 0) {
+        if (rt == 8) return find_variant(4, 8, kOnline);
     } else {
         rt = 1;
     }
@@ -631,7 +668,8 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         case 7: st = launch_v<1, 1, 1, 4, 4, kOnline>(args, vec, s); break;
         case 8: st = launch_v<2, 1, 1, 4, 4, kTwoSweep>(args, vec, s); break;
         case 9: st = launch_v<4, 1, 1, 4, 4, kTwoSweep>(args, vec, s); break;
-        default: st = launch_v<4, 1, 1, 4, 4, kExternal>(args, vec, s); break;
+        case 10: st = launch_v<4, 1, 1, 4, 4, kExternal>(args, vec, s); break;
+        default: st = launch_v<3, 1, 1, 4, 4, kOnline>(args, vec, s); break;
     }
     if (st != 0 || pl.splits <= 1) return st;
     const int64_t total = R * I * K;
@@ -650,11 +688,11 @@ extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, i
     const int64_t lim = (int64_t)1 << 30;
     if (m >= lim || k >= lim || n >= lim) return TRT_E_RANGE;
     if (k * n + n >= lim || m * k + k >= lim || m * n + n >= lim) return TRT_E_RANGE;
-    // row tile by grid fill, as for lm2exp with one batch
+    // row tile by modelled time as for lm2exp with one batch (the per-tile overhead is smaller
+    // without the exp work), else by grid fill
     const int64_t ct = ceil_div(n, 128);
-    int rt = 1;
-    if (m > 64 && ceil_div(m, 128) * ct >= 384) rt = 4;
-    else if (m > 32 && ceil_div(m, 64) * ct >= 256) rt = 2;
+    int rt = m > 64 ? pick_tile(1, m, n, 1, false) : 0;
+    if (rt == 0) rt = (m > 32 && ceil_div(m, 64) * ct >= 256) ? 2 : 1;
     Lm2Args args;
     args.a = a; args.b = b; args.c = c;
     args.part = nullptr; args.shift = nullptr;
@@ -672,6 +710,7 @@ extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, i
     const bool vec = (k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (rt == 4) return launch_v<4, 1, 1, 4, 4, kPlain>(args, vec, s);
+    if (rt == 3) return launch_v<3, 1, 1, 4, 4, kPlain>(args, vec, s);
     if (rt == 2) return launch_v<2, 1, 1, 4, 4, kPlain>(args, vec, s);
     return launch_v<1, 1, 1, 4, 4, kPlain>(args, vec, s);
 }

@@ -326,12 +326,19 @@ constexpr int kLt2Waves = 4;
 // R=32..128, S=I=J=64, K=256): with fewer than half a workgroup per CU the chip is not full
 // either way and the shorter tile halves each workgroup's chain; up to 1.5 per CU it still
 // wins while the contraction is short (I*J <= 4096).  Long contractions on a filling grid keep
-// the 64-row tile, whose Khatri-Rao multiply is shared by two MFMAs.
+// the 64-row tile, whose Khatri-Rao multiply is shared by two MFMAs (4-6 % per row, measured at
+// S = 64, 192, 256) -- unless S leaves the last 64-row tile at most half full and that padding
+// is more than the 32-row tile costs: S = 96 runs 26-30 % faster on 32-row tiles, S = 160 12 %,
+// S = 224 / 288 7-15 % on a grid that fills the chip (on a small one the 64-row tile with a cut
+// contraction is 14-20 % ahead there).
+// (96- and 128-row tiles were measured too: per 32 rows they cost what the 32-row tile does.)
 static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
     int rt = S > 32 ? 2 : 1;
     if (rt == 2) {
         const int64_t n64 = R * ceil_div(S, 64) * ceil_div(K, 128);
         if (n64 < 128 || (n64 < 384 && I * J <= 4096)) rt = 1;
+        const int64_t last = S % 64;
+        if (last >= 1 && last <= 32 && (S <= 192 || (S <= 384 && n64 >= 512))) rt = 1;
     }
     for (int v = 0; v < kNumVariants; ++v)
         if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == 4) return v;

@@ -351,6 +351,8 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
         if (mode == TRT_MODE_SPLIT || tiles < (pieces == 3 ? 256 : 192))
             return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes,
                                   stream);
+        // S = 65..96: a quarter of two 64-row tiles would be padding (-14 % on 32-row tiles, two pieces)
+        if (pieces == 2 && S > 64 && S <= 96) rt = 1;
     }
 
     Lt2BfArgs args;
