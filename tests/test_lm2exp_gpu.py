@@ -324,6 +324,30 @@ def test_bf16_paths_shift_moves_during_the_sweep(dev, precision, variant):
     assert torch.isfinite(out[0, :, 5]).all() and torch.isfinite(out[0, :, 6]).all()
 
 
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+def test_shift_moves_by_more_than_the_exponent_range(dev, precision):
+    """A term summed just under the rescale margin above the old shift must survive when a later
+    chunk lifts the shift by 88.5: exp(m_old - m_new) alone is below the smallest normal float
+    (e^-87.3), the rescaled sum is not (the term lies at e^-80.6, or e^-56.6 with the wide margin
+    of the two-piece path, of the new shift: inside the range of the two-sweep recipe too).  Same
+    for the merge of a contraction cut over J, whose pieces end with shifts 88.5 apart."""
+    margin = 32.0 if precision == "bf16x3" else 8.0
+    R, I, J, K = 1, 40, 130, 70
+    a = torch.zeros(R, I, J)
+    a[:, :, 5] = 1000.0                      # the only weight: every output is b[5] + log 1000
+    b = torch.full((R, J, K), -50.0)
+    b[:, 0] = 0.0                            # first chunk's maximum, zero weight
+    b[:, 5] = margin - 0.1                   # summed relative to the old shift, almost e^margin
+    b[:, 100] = 88.5                         # a later chunk towers over it, zero weight
+    ag, bg = a.to(dev), b.to(dev)
+    n_variants = N_VARIANTS if precision == "fp32" else N_BF16_VARIANTS
+    for variant in range(0, n_variants + 1):
+        for splits in (0, 1, 3):
+            out = lm2exp(ag, bg, _precision=precision, _variant=variant, _splits=splits)
+            assert torch.isfinite(out).all(), (variant, splits)
+            _check(out, a, b, **PRECISION_GATES.get(precision, {}))
+
+
 @pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
 def test_bf16_paths_strided_nan_and_magnitude(dev, precision):
     g = torch.Generator().manual_seed(5)

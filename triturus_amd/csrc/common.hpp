@@ -127,6 +127,12 @@ constexpr float kLn2 = 0.69314718055994530942f;
 // product into an absolute exponent error of |m| 2^-24, fatal for |m| >~ 1e9.
 __device__ __forceinline__ float exp_shifted(float x) { return __builtin_amdgcn_exp2f(x * kLog2e); }
 
+// Rescaling running sums by exp(d), d <= 0, when the shift moves up: below about e^-87 the factor
+// itself is no longer a normal float (it flushes to zero) although sum * exp(d) may well be one --
+// the sums were taken relative to the old shift and can be as large as e^margin times the weights.
+// When any lane moves by more than this, the factor is applied as two halves, exp(d/2) twice.
+constexpr float kDeepRescale = -80.0f;
+
 // m + log(s) from the hardware log2: log2(0) = -inf gives -inf (m is finite), NaN stays NaN.
 __device__ __forceinline__ float log_plus(float s, float m) {
     return __builtin_fmaf(__builtin_amdgcn_logf(s), kLn2, m);

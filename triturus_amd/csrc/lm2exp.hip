@@ -11,18 +11,18 @@
 // MFMA (q,u) of lane-half h consuming j = 8q + 4h + u of the chunk.
 //
 // The shift m[n].  The result m + log(sum_j a exp(b - m)) does not depend on m,
-// only overflow/underflow do, so m need not be the exact column maximum:
-//   ONLINE = true   one sweep over b.  m starts as the maximum of the first
-//                   chunk of the column; when a later chunk's maximum exceeds
-//                   m by more than kRescaleMargin the accumulators of that
-//                   column are multiplied by exp(m_old - m_new) and m moves
-//                   up.  exp(b - m) therefore never exceeds e^kRescaleMargin,
-//                   and b is read from HBM exactly once.
-//   ONLINE = false  two sweeps, as the reference kernel does
-//                   (triturus/lm2exp.py:125-127): the exact column maximum
-//                   first (wavefront reduction: the two lane halves take
-//                   alternate rows and exchange once), then the contraction.
-// In both, m is clamped to +-1e38 (baselines/lm2exp.py:12) so an all -inf
+// only overflow/underflow do, so m need not be the exact column maximum (MODE):
+//   kOnline    one sweep over b.  m starts as the maximum of the first chunk of the
+//              column; when a later chunk's maximum exceeds m by more than
+//              kRescaleMargin the accumulators of that column are multiplied by
+//              exp(m_old - m_new) and m moves up.  exp(b - m) therefore never exceeds
+//              e^kRescaleMargin, and b is read from HBM exactly once.
+//   kTwoSweep  two sweeps, as the reference kernel does (triturus/lm2exp.py:125-127):
+//              the exact column maximum first (wavefront reduction: the two lane
+//              halves take alternate rows and exchange once), then the contraction.
+//   kExternal  the clamped column maxima come from a separate launch
+//              (lm2exp_colmax_kernel); kPlain: no shift, exp or log at all (mm).
+// m is always clamped to +-1e38 (baselines/lm2exp.py:12) so an all -inf
 // column gives exp(-inf) = 0, log(0) = -inf: -inf out, never NaN.
 //
 // Replaces _ker_lm2exp, triturus/lm2exp.py:63-164.  Ragged contracted-axis
@@ -217,11 +217,19 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
                 const bool need = cm > mref[ct] + kRescaleMargin;
                 if (__builtin_amdgcn_ballot_w64(need) != 0) {
                     const float mnew = need ? clamp_shift(cm) : mref[ct];
-                    const float sc = exp_shifted(mref[ct] - mnew);
+                    const float d = mref[ct] - mnew;  // <= 0; 0 in the lanes that stay
+                    const bool deep = __builtin_amdgcn_ballot_w64(d < kDeepRescale) != 0;  // wave-uniform, rare
+                    const float sc = exp_shifted(deep ? 0.5f * d : d);
 #pragma unroll
                     for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                         for (int v = 0; v < 16; ++v) acc[rt][ct][v] *= sc;
+                    if (deep) {
+#pragma unroll
+                        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                            for (int v = 0; v < 16; ++v) acc[rt][ct][v] *= sc;
+                    }
                     mref[ct] = mnew;
                 }
             }
@@ -425,7 +433,11 @@ __global__ __launch_bounds__(256) void lm2exp_merge_kernel(const float *__restri
         float M = sh[0];
         for (int sp = 1; sp < splits; ++sp) M = max_nan(M, sh[sp * rk]);
         float sum = 0.f;
-        for (int sp = 0; sp < splits; ++sp) sum += part[(int64_t)sp * total + e] * exp_shifted(sh[sp * rk] - M);
+        for (int sp = 0; sp < splits; ++sp) {
+            // exp(m_s - M) in two halves: the factor alone may flush where the product does not
+            const float f = exp_shifted(0.5f * (sh[sp * rk] - M));
+            sum += part[(int64_t)sp * total + e] * f * f;
+        }
         c[(int64_t)r * sc0 + (int64_t)i * sc1 + k] = log_plus(sum, M);
     }
 }

@@ -193,11 +193,19 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
         const bool need = cm > mref + kMargin;
         if (__builtin_amdgcn_ballot_w64(need) != 0) {
             const float mnew = need ? clamp_shift(cm) : mref;
-            const float sc = exp_shifted(mref - mnew);
+            const float d = mref - mnew;  // <= 0; 0 in the lanes that stay
+            const bool deep = __builtin_amdgcn_ballot_w64(d < kDeepRescale) != 0;  // wave-uniform, rare
+            const float sc = exp_shifted(deep ? 0.5f * d : d);
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) acc[rt][v] *= sc;
+            if (deep) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[rt][v] *= sc;
+            }
             mref = mnew;
         }
         // exp(b - m) is infinite only for b = +inf (everything else is at most e^margin above
