@@ -171,3 +171,82 @@ def test_measured_tile_selection(dev):
         autotune.set_autotune(False)
         autotune.clear()
     assert autotune.pick(("x",), (0, 1), lambda v: None) == 0  # off: the library's rule
+
+
+# ---- sparse weights under a wide spread of log-values: the dominant log-value often meets a
+# zero weight, so an output rests on terms far below its column's maximum.  fp32 arithmetic can
+# hold a term only while it stays above 2^-126 of the shift; the check therefore brackets every
+# output between the exact float64 value and the value with all terms more than `cut` below the
+# column maximum dropped (a result may lose those terms, nothing else).
+def _lm_bracket(a, b, cut):
+    a, b = a.double(), b.double()
+    m = torch.clamp(torch.amax(b, dim=1, keepdim=True), -1e38, 1e38)
+    t = b - m
+    e = torch.exp(t)
+    pos = a[a > 0]
+    slack = min(0.0, float(torch.log(pos.min()))) if pos.numel() else 0.0
+    hi = m + torch.log(torch.bmm(a, e))
+    lo = m + torch.log(torch.bmm(a, torch.where(t < -(cut + slack), torch.zeros_like(e), e)))
+    return lo, hi
+
+
+def _lt_bracket(w, a, b, cut):
+    w, a, b = w.double(), a.double(), b.double()
+    R, S, I, J = w.shape
+    K = a.shape[2]
+    ma = torch.clamp(torch.amax(a, dim=1, keepdim=True), -1e38, 1e38)
+    mb = torch.clamp(torch.amax(b, dim=1, keepdim=True), -1e38, 1e38)
+    ta, tb = a - ma, b - mb
+    t = ta.unsqueeze(2) + tb.unsqueeze(1)
+    e = torch.exp(t)
+    pos = w[w > 0]
+    slack = min(0.0, float(torch.log(pos.min()))) if pos.numel() else 0.0
+    drop = (t < -(cut + slack)) | (ta.unsqueeze(2) < -cut) | (tb.unsqueeze(1) < -cut)
+    wf = w.reshape(R, S, I * J)
+    shift = ma + mb
+    hi = shift + torch.log(torch.bmm(wf, e.reshape(R, I * J, K)))
+    lo = shift + torch.log(torch.bmm(wf, torch.where(drop, torch.zeros_like(e), e).reshape(R, I * J, K)))
+    return lo, hi
+
+
+def _inside(x, lo, hi, rtol=1e-4, atol=1e-5):
+    x = x.detach().cpu().double()
+    tol_hi = atol + rtol * torch.nan_to_num(hi.abs(), posinf=0.0)
+    tol_lo = atol + rtol * torch.nan_to_num(lo.abs(), posinf=0.0)
+    fragile = ~((hi - lo).abs() <= tol_hi)  # rests on terms that fp32 may flush or hold as denormals
+    up = x <= hi + tol_hi + torch.where(fragile, 0.75, 0.0)
+    down = (x >= lo - tol_lo) | (lo == NINF)
+    bad = ~(up & down) | torch.isnan(x)
+    return int(bad.sum()), int(fragile.sum())
+
+
+@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+def test_sparse_weights_under_a_wide_spread(dev, seed, precision):
+    rng = random.Random(3000 + seed)
+    g = torch.Generator().manual_seed(3000 + seed)
+    cut = 75.0 if precision == "fp32" else 60.0
+    R, I, J, K = rng.randrange(1, 4), _dim(rng, 200), _dim(rng, 257), _dim(rng, 257)
+    a = torch.rand(R, I, J, generator=g) * rng.choice([1.0, 1e-3, 50.0, 1e20])
+    a[torch.rand(a.shape, generator=g) < 0.8] = 0.0
+    b = torch.randn(R, J, K, generator=g) * rng.choice([40.0, 300.0]) + rng.choice([0.0, 1e4, -1e6])
+    b = _sprinkle(rng, g, b)
+    lo, hi = _lm_bracket(a, b, cut)
+    nvar = 12 if precision == "fp32" else 8
+    variant, splits = rng.randrange(0, nvar + 1), rng.choice([0, 1, 3])
+    out = lm2exp(_view(rng, a.to(dev)), _view(rng, b.to(dev)), _precision=precision, _variant=variant, _splits=splits)
+    bad, _ = _inside(out, lo, hi, **GATES[precision])
+    assert bad == 0, ("lm2exp", R, I, J, K, variant, splits, bad)
+
+    R, S, I, J, K = rng.randrange(1, 3), _dim(rng, 130), _dim(rng, 33), _dim(rng, 70), _dim(rng, 257)
+    w = torch.rand(R, S, I, J, generator=g) * rng.choice([1.0, 1e-4, 1e20])
+    w[torch.rand(w.shape, generator=g) < 0.8] = 0.0
+    a = _sprinkle(rng, g, torch.randn(R, I, K, generator=g) * rng.choice([10.0, 100.0]) + rng.choice([0.0, 1e5]))
+    b = _sprinkle(rng, g, torch.randn(R, J, K, generator=g) * rng.choice([10.0, 100.0]) + rng.choice([0.0, -1e5]))
+    lo, hi = _lt_bracket(w, a, b, cut)
+    mode = rng.choice(["auto", "split", "unsplit"])
+    variant = rng.randrange(0, 9) if precision == "fp32" else rng.randrange(0, 5)
+    out = lt2exp(w.to(dev), _view(rng, a.to(dev)), _view(rng, b.to(dev)), mode=mode, _precision=precision,
+                 _variant=variant)
+    bad, _ = _inside(out, lo, hi, **GATES[precision])
+    assert bad == 0, ("lt2exp", R, S, I, J, K, mode, variant, bad)
