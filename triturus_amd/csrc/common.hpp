@@ -32,25 +32,27 @@ __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) { ret
 
 // Host-side cost model for cutting a contraction over several workgroups ("split").
 // `tiles` output tiles each need `units` steps of `mfmas_per_unit` MFMA instructions per
-// wavefront (64 cycles each on a SIMD).  Unsplit, a tile is one workgroup.  A run takes the
-// longer of (a) one workgroup's dependent chain and (b) all the work spread over the 256
-// CUs, where a CU holding a single workgroup cannot hide its LDS / barrier latencies and
-// reaches ~72 % of the MFMA rate it reaches with three or more.  Split s ways the chain
-// shrinks s-fold and the CUs fill up, but the partial sums make a round trip through memory
-// and a merge kernel is launched.  Returns the split count (1 = do not split) with the
-// smallest estimate; a split must win by 20 %.  The merge constants are pessimistic on
-// purpose (2 TB/s, 5 us): splits the model rates as marginal were losses when measured.
+// wavefront (64 cycles each on a SIMD).  Unsplit, a tile is one workgroup.  A run lasts as long
+// as the busiest of the 256 CUs: it holds q = ceil(workgroups / 256) of them, which share its
+// matrix pipe, so it needs q chains' worth of MFMA time -- at 45 % of the MFMA rate when it
+// holds a single workgroup (one wavefront per SIMD: nothing hides the LDS, barrier and load
+// latencies), 65 % with two, 80 % with three, 90 % from four on.  (Measured: 64 steps of 16
+// MFMAs alone on a CU take 62 us, two workgroups of 128 steps 175 us, 512 workgroups of 32 steps
+// 43 us; counting whole workgroups matters, 288 tiles take twice as long as 256.)  Split s ways
+// the chain shrinks s-fold and the CUs fill up, but the partial sums make a round trip through
+// memory and a merge kernel is launched.  Returns the split count (1 = do not split) with the
+// smallest estimate; a split must win by 20 %.  The merge constants are pessimistic on purpose
+// (2 TB/s, 5 us): splits the model rates as marginal were losses when measured.
 inline int choose_splits(int64_t tiles, int64_t units, int64_t mfmas_per_unit, int64_t out_elems,
                          int min_units_per_split, int max_splits, bool forced) {
-    constexpr double kCyclesPerUs = 2400.0, kCus = 256.0, kLoneEff = 0.72;
+    constexpr double kCyclesPerUs = 2400.0;
+    constexpr int64_t kCuCount = 256;
     const double unit_us = (double)mfmas_per_unit * 64.0 / kCyclesPerUs;
-    const double spread_us = (double)units * unit_us * (double)tiles / kCus;
     auto estimate = [&](int sp) {
-        const double chain_us = (double)ceil_div(units, sp) * unit_us / kLoneEff;
-        const double per_cu = (double)tiles * sp / kCus;  // resident workgroups per CU
-        double eff = kLoneEff;
-        if (per_cu > 1.0) eff += (1.0 - kLoneEff) * (per_cu >= 3.0 ? 1.0 : (per_cu - 1.0) / 2.0);
-        const double body = chain_us > spread_us / eff ? chain_us : spread_us / eff;
+        const double chain_us = (double)ceil_div(units, sp) * unit_us;  // one workgroup at the full MFMA rate
+        const int64_t q = ceil_div(tiles * sp, kCuCount);               // workgroups on the busiest CU
+        const double eff = q >= 4 ? 0.9 : (q == 3 ? 0.8 : (q == 2 ? 0.65 : 0.45));
+        const double body = (double)q * chain_us / eff;
         const double merge_us = sp > 1 ? 5.0 + (double)(sp + 1) * (double)out_elems * 4.0 / 2.0e6 : 0.0;
         return body + merge_us;
     };

@@ -484,20 +484,20 @@ static int find_variant(int rt, int wn, int mode) {
     return 0;
 }
 
-// Tile for a grid of R x I rows and K columns among 128 x 128, 96 x 128, 64 x 128 and (wide =
-// true) 128 x 256; returns the rows in units of 32 (4, 3, 2; 8 stands for 128 x 256), or 0 when
-// none of them leaves a workgroup per CU.
+// Tile for a grid of R x I rows and K columns among 128 x 128, 96 x 128, 64 x 128, 32 x 128 (rows
+// up to 32 * max_rt) and (wide = true) 128 x 256; returns the rows in units of 32 (4, 3, 2, 1; 8
+// stands for 128 x 256), or 0 when none of them leaves a workgroup per CU.
 // Modelled time: T = tiles per CU (256 CUs), each costing rt MFMA blocks plus an overhead that
 // does not shrink with the tile (the exp / shift work of the b chunk, loads, barriers: 0.75
 // blocks, less without the exp work), counted in quarter blocks.  A CU holds `res` workgroups at a
-// time (3, four of 64-row tiles, one wide); they share the matrix pipe, so a full round costs
+// time (3, four of 64-row tiles, six of 32-row tiles, one wide); they share the matrix pipe, so a full round costs
 // the sum of its tiles, but a last round with a single workgroup runs at about 2/3 speed (one
 // wavefront per SIMD hides little latency) and one with two at ~0.8: a tail penalty, fading when
 // T is large (workgroups are dispatched as others finish).  The wide tile costs 6.5 % more per row
 // (measured on large grids) and only ever wins by avoiding such a tail.
 // Fitted at R=384 and R=64, I=J=64..1024, K=256: ranks the tiles as measured in 26 of 28 shapes
 // (both misses within 5 %); I = 96, 160, 192, 288 move to 96 rows (-15..23 %), I = 320 to 64.
-static int pick_tile(int64_t R, int64_t I, int64_t K, int overhead_quarters, bool wide) {
+static int pick_tile(int64_t R, int64_t I, int64_t K, int overhead_quarters, bool wide, int max_rt = 4) {
     const int64_t kFill = 256, kCuCount = 256;  // at least one workgroup per CU
     int best = 0;
     int64_t best_cost = 0;
@@ -517,9 +517,9 @@ static int pick_tile(int64_t R, int64_t I, int64_t K, int overhead_quarters, boo
         }
     };
     const int64_t ct = ceil_div(K, 128);
-    for (int rt = 4; rt >= 2; --rt)
-        consider(rt, R * ceil_div(I, 32 * rt) * ct, 4 * rt + overhead_quarters, rt == 2 ? 4 : 3);
-    if (wide && K % 256 == 0)
+    for (int rt = max_rt; rt >= 1; --rt)
+        consider(rt, R * ceil_div(I, 32 * rt) * ct, 4 * rt + overhead_quarters, rt == 1 ? 6 : (rt == 2 ? 4 : 3));
+    if (wide && max_rt == 4 && K % 256 == 0)
         consider(8, R * ceil_div(I, 128) * (K / 256), (2 * (16 + overhead_quarters) * 213) / 200, 1);
     return best;
 }
@@ -529,7 +529,10 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     const int64_t ct = ceil_div(K, 128);
     const int64_t n128 = R * ceil_div(I, 128) * ct, n64 = R * ceil_div(I, 64) * ct;
     int rt;
-    if (I <= 32) {
+    if (I <= 32 || J <= 32) {
+        // J <= 32 is a single chunk: a workgroup is load, one MFMA block, log and store in
+        // sequence with nothing to overlap inside it, and the call is bound by writing c; many
+        // small workgroups hide the most latency (measured 20-35 % ahead of the 128-row tile)
         rt = 1;
     } else if (I <= 64) {
         rt = (n64 >= kFill || J >= 1280) ? 2 : 1;
@@ -537,7 +540,7 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
         // at most 1.5 workgroups per CU and a long contraction: it will be cut over J, which
         // fills the chip; take the largest tile that leaves >= 128 tiles
         rt = n128 >= 128 ? 4 : (n64 >= 128 ? 2 : 1);
-    } else if ((rt = pick_tile(R, I, K, 3, true)) != 0) {
+    } else if ((rt = pick_tile(R, I, K, 3, true, J <= 64 ? 2 : 4)) != 0) {  // two chunks: 64 rows at most (+2..13 %)
         if (rt == 8) return find_variant(4, 8, kOnline);
     } else {
         rt = 1;

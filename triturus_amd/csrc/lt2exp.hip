@@ -320,25 +320,24 @@ constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLt2Waves = 4;
 
 // Measured on MI355X at R=64, S=I=J=64, K=4096: the narrow wavefront tile (64 x 32,
-// 32 accumulator registers, j-chunks of 32) runs at 87% of the fp32 MFMA peak, the
-// 64 x 64 tiles at 81-85%: occupancy beats operand reuse here.
-// Small grids want the 32-row tile (measured +8..25 % on batch-1 squares of 64..128 and on
-// R=32..128, S=I=J=64, K=256): with fewer than half a workgroup per CU the chip is not full
-// either way and the shorter tile halves each workgroup's chain; up to 1.5 per CU it still
-// wins while the contraction is short (I*J <= 4096).  Long contractions on a filling grid keep
-// the 64-row tile, whose Khatri-Rao multiply is shared by two MFMAs (4-6 % per row, measured at
-// S = 64, 192, 256) -- unless S leaves the last 64-row tile at most half full and that padding
-// is more than the 32-row tile costs: S = 96 runs 26-30 % faster on 32-row tiles, S = 160 12 %,
-// S = 224 / 288 7-15 % on a grid that fills the chip (on a small one the 64-row tile with a cut
-// contraction is 14-20 % ahead there).
-// (96- and 128-row tiles were measured too: per 32 rows they cost what the 32-row tile does.)
+// 32 accumulator registers, j-chunks of 32) runs at 87-89 % of the fp32 MFMA peak, the
+// 64 x 64 tiles at 81-85 %: occupancy beats operand reuse here.
+// Row tile: 32 rows unless the 64-row tile pays.  Its Khatri-Rao multiply is shared by two
+// MFMAs, worth 2-6 % per row on long contractions (I*J >= 4096) when the grid gives every CU
+// a workgroup (measured at S = 64..256 on R = 32..128, and at the large configuration);
+// everywhere else the 32-row tile is as fast or faster -- twice the workgroups hide more
+// latency and balance better (over 288 random shapes: 4-30 % ahead on grids of 1-4 workgroups
+// per CU, 27 % (median) when S leaves the last 64-row tile at most half full, e.g. S = 96,
+// 160, 208).  (96- and 128-row tiles were measured too: per 32 rows they cost what the 32-row
+// tile does.)  Rule checked against the better of the two tiles on those shapes: 0.6 % mean
+// regret, 2 shapes of 288 more than 10 % off.
 static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
-    int rt = S > 32 ? 2 : 1;
-    if (rt == 2) {
-        const int64_t n64 = R * ceil_div(S, 64) * ceil_div(K, 128);
-        if (n64 < 128 || (n64 < 384 && I * J <= 4096)) rt = 1;
+    int rt = 1;
+    if (S > 32) {
         const int64_t last = S % 64;
-        if (last >= 1 && last <= 32 && (S <= 192 || (S <= 384 && n64 >= 512))) rt = 1;
+        const bool same_padding = last == 0 || last > 32;
+        const int64_t n64 = R * ceil_div(S, 64) * ceil_div(K, 128);
+        if (same_padding && I * J >= 4096 && n64 >= 256) rt = 2;
     }
     for (int v = 0; v < kNumVariants; ++v)
         if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == 4) return v;
