@@ -333,28 +333,43 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     // byte offsets inside one batch slab are 32-bit (buffer addressing)
     if (I * sa[1] + J >= lim || J * sb[1] + K >= lim || I * sc[1] + K >= lim) return TRT_E_RANGE;
 
-    // Tile by grid fill (measured over the reference's benchmark grid): with two pieces the
-    // kernel is bound by the vector work on the B operand, so 256 rows when that still leaves
-    // two workgroups per CU (6 % at R=64, I=J=256, K=4096); otherwise 128 rows when that
-    // leaves >= 1.5 workgroups per CU (j-chunks of 64 for a long contraction, where the fewer
-    // barriers pay; of 32 otherwise, so that three workgroups fit a CU), 64 rows when that
-    // leaves >= 1 per CU.  Smaller grids are latency bound, not matrix bound: there the fp32
-    // path (smaller tiles, contraction cut over J) is as fast or faster and takes the call,
-    // as it does whenever the caller asks for a cut.
+    // Tile and hand-over rules, fitted to 223 random shapes (R 1..256, I, J 16..1024, K 64..8192)
+    // timed with every tile and on the fp32 path; against the best of those the rules below lose
+    // 5.4 % (two pieces) / 4.0 % (three) on average, the previous ones 19 / 11 %.
+    //  - Grids of fewer than 128 (three pieces: 192) 32-row tiles are latency bound, not matrix
+    //    bound, and a contraction of at most 16 (32) is bound by writing c: there the fp32 path
+    //    (smaller tiles, contraction cut over J) is as fast or faster and takes the call, as it
+    //    does whenever the caller asks for a cut.
+    //  - j-chunks of 32 (three workgroups fit a CU; chunks of 64 measured 0-17 % behind), except
+    //    with two pieces on 64- and 32-row tiles over a contraction of 512 or more (chunks of 64).
+    //  - Rows: the candidate (128, 64 or 32 rows; at least 1.5, 1, 0 workgroups per CU) with the least
+    //    padded rows x cost per row, the cost being 1.15 for 32 rows, 1 for 64, and for 128 rows
+    //    0.85 (0.95) on a contraction of 256 or more, where each exp then feeds more MFMAs, and
+    //    1.05 on a shorter one.
     int v;
     if (variant >= 1) {
         v = variant - 1;
     } else {
         const int64_t ct = ceil_div(K, 128);
-        const int64_t n128 = R * ceil_div(I, 128) * ct, n64 = R * ceil_div(I, 64) * ct;
-        const int64_t n256 = R * ceil_div(I, 256) * ct;
-        if (splits > 1) v = -1;
-        else if (pieces == 2 && I > 128 && n256 >= 512 && J < 512) v = 7;  // 256 rows: each exp feeds 24 MFMAs
-        else if (I > 64 && n128 >= 384) v = (pieces == 2 && J >= 512) ? 0 : 1;
-        else if (I > 32 && n64 >= 256) v = pieces == 2 ? 2 : 3;
-        else v = -1;
-        if (v < 0)
+        const int64_t n32 = R * ceil_div(I, 32) * ct;
+        if (splits > 1 || n32 < (pieces == 2 ? 128 : 192) || J <= (pieces == 2 ? 16 : 32))
             return trt_lm2exp_f32(a, b, c, R, I, J, K, sa, sb, sc, 0, splits, workspace, workspace_bytes, stream);
+        int best_rt = 1;
+        int64_t best_cost = ceil_div(I, 32) * 115;
+        for (int rt = 2; rt <= 4; rt *= 2) {
+            if (R * ceil_div(I, 32 * rt) * ct < (rt == 4 ? 384 : 256)) continue;  // 1.5 / 1 workgroups per CU
+            const int64_t per_row = rt == 2 ? 100 : (J >= 256 ? (pieces == 2 ? 85 : 95) : 105);
+            const int64_t cost = ceil_div(I, 32 * rt) * rt * per_row;
+            if (cost < best_cost) {
+                best_cost = cost;
+                best_rt = rt;
+            }
+        }
+        v = best_rt == 4 ? 1 : (best_rt == 2 ? 3 : 5);  // {4,2}, {2,2}, {1,2}
+        if (pieces == 2 && best_rt <= 2 && J >= 512) v -= 1;  // {2,4}, {1,4}: fewer barriers pay on a long contraction
+        // two pieces are bound by the vector work on the B operand: 256 rows (each exp feeds 24
+        // MFMAs) when I fills them exactly and two workgroups per CU remain (6-25 % at I = 256, 512)
+        if (pieces == 2 && best_rt == 4 && I % 256 == 0 && J >= 256 && R * (I / 256) * ct >= 512) v = 7;  // {8,2}
     }
     const LmBfVariant &vr = kLmBfVariants[v];
 

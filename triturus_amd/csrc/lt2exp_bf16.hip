@@ -334,25 +334,27 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
     if (S * sw[1] + I * J >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
 
-    // Tile: 64 rows when S allows, j-chunks of 64 unless J fits 32 (measured over the
-    // reference's benchmark grid).  The bf16 kernels never cut the contraction over several
-    // workgroups: a grid of fewer than 192 tiles (256 CUs) is latency bound, not
-    // matrix bound, and is handed to the fp32 path, which may cut it (measured 5-10x faster
-    // there on batch-1 squares, ahead up to ~128 tiles); so is a three-piece call below one
-    // tile per CU, where it does not beat the fp32 pipe it imitates, and any call in mode
-    // SPLIT.
-    int rt = S > 32 ? 2 : 1;
-    int ks = J > 32 ? 4 : 2;
+    // Tile and hand-over rules, fitted to 290 random shapes (R 1..128, S 16..512, I, J 8..128,
+    // K 64..8192) timed with every tile and on the fp32 path; against the best of those the
+    // rules below lose 2.5 % (two pieces) / 1.9 % (three) on average, the previous ones 17 / 14 %.
+    //  - The bf16 kernels never cut the contraction over several workgroups: a grid of fewer
+    //    than 160 32-row tiles -- 256 when the contraction is longer than 4096 -- is latency
+    //    bound, not matrix bound, and goes to the fp32 path, which may cut it;
+    //    so does any call in mode SPLIT.
+    //  - 32 rows per workgroup; 64 when that pads S no further and still leaves two workgroups
+    //    per CU (the pipelined two-row-tile loop then wins 4-11 %).
+    //  - j-chunks of 64, or of 32 when those leave less of the last chunk empty (J = 1..32,
+    //    65..96 modulo 64: 1.15-1.8x), and for J = 33..48 on the 64-row tile.
+    const int64_t ctk = ceil_div(K, 128);
+    const int64_t t32 = R * ceil_div(S, 32) * ctk, t64 = R * ceil_div(S, 64) * ctk;
+    const int64_t s_last = S % 64, j_last = J % 64;
+    int rt = (S > 32 && (s_last == 0 || s_last > 32) && t64 >= 512) ? 2 : 1;
+    int ks = ((j_last >= 1 && j_last <= 32) || (rt == 2 && j_last >= 33 && j_last <= 48)) ? 2 : 4;
     if (variant >= 1) {  // 1: 64 rows, chunks of 64;  2: 64 rows, 32;  3: 32 rows, 64;  4: 32 rows, 32
         rt = variant <= 2 ? 2 : 1;
         ks = (variant & 1) ? 4 : 2;
-    } else {
-        const int64_t tiles = R * ceil_div(S, 32 * rt) * ceil_div(K, 128);
-        if (mode == TRT_MODE_SPLIT || tiles < (pieces == 3 ? 256 : 192))
-            return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes,
-                                  stream);
-        // S = 65..96: a quarter of two 64-row tiles would be padding (-14 % on 32-row tiles, two pieces)
-        if (pieces == 2 && S > 64 && S <= 96) rt = 1;
+    } else if (mode == TRT_MODE_SPLIT || t32 < 160 || (t32 <= 256 && I * J > 4096)) {
+        return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
     }
 
     Lt2BfArgs args;
