@@ -250,3 +250,31 @@ def test_sparse_weights_under_a_wide_spread(dev, seed, precision):
                  _variant=variant)
     bad, _ = _inside(out, lo, hi, **GATES[precision])
     assert bad == 0, ("lt2exp", R, S, I, J, K, mode, variant, bad)
+
+
+def test_concurrent_streams(dev):
+    """The library keeps no state between calls: launches interleaved on two streams (default
+    priority), each with its own split-mode workspace, give the results of the same calls made
+    one after the other."""
+    g = torch.Generator().manual_seed(17)
+    a = torch.rand(2, 96, 700, generator=g).to(dev)
+    b = (torch.randn(2, 700, 130, generator=g) * 20).to(dev)
+    w = torch.rand(3, 75, 50, 50, generator=g).to(dev)
+    x = torch.randn(3, 50, 100, generator=g).to(dev)
+    y = torch.randn(3, 50, 100, generator=g).to(dev)
+    ref_m = lm2exp(a, b, _splits=5)
+    ref_t = lt2exp(w, x, y, mode="split")
+    ref_m6 = lm2exp(a, b, _precision="bf16x6")
+    torch.cuda.synchronize()
+    s1, s2 = torch.cuda.Stream(device=dev), torch.cuda.Stream(device=dev)
+    outs = []
+    for _ in range(20):
+        with torch.cuda.stream(s1):
+            o1 = lm2exp(a, b, _splits=5)
+            o3 = lm2exp(a, b, _precision="bf16x6")
+        with torch.cuda.stream(s2):
+            o2 = lt2exp(w, x, y, mode="split")
+        outs.append((o1, o2, o3))
+    torch.cuda.synchronize()
+    for o1, o2, o3 in outs:
+        assert torch.equal(o1, ref_m) and torch.equal(o2, ref_t) and torch.equal(o3, ref_m6)
