@@ -105,7 +105,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 #pragma unroll
     for (int sidx = 0; sidx < SLOTS; ++sidx)
         woff[sidx] = ((uint32_t)(trow + sidx * ROWS_PER_SLOT) * (uint32_t)p.sw1 + 4u * tc4) * 4u;
-    auto load_tile = [&](int i, int jc) {
+    auto load_tile = [&](int i, int jc) __attribute__((always_inline)) {
         const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
         const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
         if (full) {
@@ -125,7 +125,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
         }
     };
     // split the staged fp32 values and write the pieces to LDS (8 bytes per piece and slot)
-    auto store_tile = [&](int buf) {
+    auto store_tile = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
             uint32_t p01[NS], p23[NS];
@@ -146,7 +146,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 
     // B operand: exp(b[j,n] - mb[n]) of the current j-chunk, split, in MFMA layout
     uintx4 ebp[NS][KS];
-    auto load_eb = [&](int jc) {
+    auto load_eb = [&](int jc) __attribute__((always_inline)) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
             float e[8];
@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 
         // ---- one (i, j-chunk) and row tile: inner = w tile x eb (3 or 6 MFMAs per k-step,
         // starting from zero), then total += ea[i,n] * inner
-        auto mfma_rows = [&](int buf, int rt, floatx16 &inn) {
+        auto mfma_rows = [&](int buf, int rt, floatx16 &inn) __attribute__((always_inline)) {
             bool first = true;
 #pragma unroll
             for (int ks = 0; ks < KS; ++ks) {
@@ -205,7 +205,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
         // The empty asm pins the fmas to this place in the instruction stream: their results
         // are not needed before the next step, and the compiler would otherwise sink them
         // out of the MFMA block they are meant to overlap with.
-        auto scale_add = [&](floatx16 &tot, const floatx16 &inn, float e) {
+        auto scale_add = [&](floatx16 &tot, const floatx16 &inn, float e) __attribute__((always_inline)) {
 #pragma unroll
             for (int v = 0; v < 16; ++v) tot[v] = __builtin_fmaf(inn[v], e, tot[v]);
             asm volatile("" : "+v"(tot));
@@ -250,8 +250,14 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
             scale_add(total[0], inner0, ea);
             scale_add(total[1], inner1, ea);
         } else {
-            floatx16 inner;
-            for (int it = 0; it + 1 < total_iters; ++it) {
+            // One row tile: the same overlap with two result tiles in turn.  While the MFMAs of
+            // this step fill one, the vector ALU adds the other (the previous step's) into the
+            // running sum; steps are taken in pairs so that both live in fixed registers.
+            floatx16 inner_a, inner_b;
+#pragma unroll
+            for (int v = 0; v < 16; ++v) inner_b[v] = 0.f;
+            float ea_old = 0.f;
+            auto step = [&](floatx16 &inner_cur, const floatx16 &inner_old) __attribute__((always_inline)) {
                 int ni = i + 1, njc = jc;
                 if (ni == p.I) {
                     ni = 0;
@@ -260,18 +266,34 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
                 load_tile(ni, njc);
                 ea_raw = buf_load_f32(a_rsrc, aoff, (uint32_t)ni * a_row_bytes);
                 __builtin_amdgcn_sched_barrier(0);
-                mfma_rows(cur, 0, inner);
-                scale_add(total[0], inner, ea);
+                mfma_rows(cur, 0, inner_cur);
+                scale_add(total[0], inner_old, ea_old);
                 store_tile(cur ^ 1);
+                __builtin_amdgcn_sched_barrier(0);
+                ea_old = ea;
                 if (njc != jc) load_eb(njc);
                 ea = exp_shifted(ea_raw - ma);
                 __syncthreads();
                 cur ^= 1;
                 i = ni;
                 jc = njc;
+            };
+            const int steps = total_iters - 1;  // every step but the last prefetches its successor
+            int done = 0;
+            for (; done + 2 <= steps; done += 2) {
+                step(inner_a, inner_b);
+                step(inner_b, inner_a);
             }
-            mfma_rows(cur, 0, inner);
-            scale_add(total[0], inner, ea);
+            if (done < steps) {
+                step(inner_a, inner_b);
+                mfma_rows(cur, 0, inner_b);
+                scale_add(total[0], inner_a, ea_old);
+                scale_add(total[0], inner_b, ea);
+            } else {
+                mfma_rows(cur, 0, inner_a);
+                scale_add(total[0], inner_b, ea_old);
+                scale_add(total[0], inner_a, ea);
+            }
         }
     }
 
