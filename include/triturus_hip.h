@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TRT_ABI_VERSION 3
+#define TRT_ABI_VERSION 4
 
 #define TRT_OK 0
 #define TRT_E_INVALID (-1)   /* null pointer, non-positive size, bad enum   */
@@ -155,6 +155,22 @@ int trt_lm2exp_bf16_variant_count(void);
 int trt_matmax(const void *x, void *y, int64_t m, int64_t n, int axis, int dtype,
                void *workspace, size_t workspace_bytes, void *stream);
 size_t trt_matmax_workspace_bytes(int64_t m, int64_t n, int axis, int dtype);
+
+/*
+ * Batched column maxima m[r,k] = max_j b[r,j,k] of an R x J x K fp32 tensor
+ * (element strides sb, trailing stride 1); m is R x K, contiguous.  A NaN in a
+ * column gives NaN, like torch.amax(b, dim=1).  With clamp != 0 the maxima are
+ * clamped to +-1e38: exactly the shift that the contraction recipes subtract
+ * (baselines/lm2exp.py:11-12, baselines/lt2exp.py:15-19) and that the two-launch
+ * lm2exp variant consumes.  The reference has the 2-D reduction only
+ * (`matmax`, triturus/max.py:125-188); this is its batched form along axis 1.
+ * workspace: trt_colmax_batched_workspace_bytes(R, J, K) bytes (0 unless few
+ * columns stand under a long reduced axis, which is then cut over J).
+ */
+int trt_colmax_batched_f32(const float *b, float *m, int64_t R, int64_t J, int64_t K,
+                           const int64_t sb[3], int clamp, void *workspace, size_t workspace_bytes,
+                           void *stream);
+size_t trt_colmax_batched_workspace_bytes(int64_t R, int64_t J, int64_t K);
 
 /*
  * Max and first-occurrence argmax (int64) of a contiguous vector of n

@@ -120,6 +120,14 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_vadd(one, one, null, 5, 0, null) == -1
     assert lib.trt_vadd(one, one, one, 0, 0, null) == -1
     assert lib.trt_vadd(one, one, one, 5, 7, null) == -1
+    # batched column maxima
+    assert lib.trt_colmax_batched_f32(null, one, 1, 1, 1, ok, 0, null, 0, null) == -1
+    assert lib.trt_colmax_batched_f32(one, one, 1, 0, 1, ok, 0, null, 0, null) == -1
+    assert lib.trt_colmax_batched_f32(one, one, 1, 1, 1, s3(12, 1, 4), 1, null, 0, null) == -2
+    assert lib.trt_colmax_batched_f32(one, one, 1 << 30, 1, 1, ok, 1, null, 0, null) == -4
+    assert lib.trt_colmax_batched_f32(one, one, 1, 4096, 256, ok, 1, null, 0, null) == -3  # cut over J: needs workspace
+    assert lib.trt_colmax_batched_workspace_bytes(64, 64, 4096) == 0
+    assert lib.trt_colmax_batched_workspace_bytes(1, 4096, 256) == 64 * 256 * 4
 
 
 def test_workspace_queries_are_host_only_and_follow_the_mode_rule():
@@ -207,6 +215,13 @@ def test_max_wrapper_validation():
         matmax(x, axis=1, block_size=2)
     with pytest.raises(RuntimeError, match="GPU only"):
         vmax(x[0], block_size=2)
+    from triturus_amd.max import bmatmax
+    with pytest.raises(AssertionError):
+        bmatmax(x)
+    with pytest.raises(AssertionError):
+        bmatmax(torch.zeros(2, 3, 4, dtype=torch.float64))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        bmatmax(torch.zeros(2, 3, 4))
 
 
 def test_flags():

@@ -216,3 +216,46 @@ def test_runs_on_the_current_stream_without_synchronising(dev):
     s.synchronize()
     assert (v.item(), i.item()) == tuple(t.item() for t in torch.max(x, 0))
     _same(y, torch.amax(x.view(1024, 1024), 1))
+
+
+# ---- batched column maxima: the front end of the contraction recipes
+@pytest.mark.parametrize("shape", [(1, 1, 1), (3, 7, 5), (4, 64, 256), (2, 300, 1000), (64, 64, 4096), (5, 33, 257),
+                                   (1, 4096, 300), (2, 1000, 70), (16, 512, 512), (1, 129, 3)])  # the last four are cut over J
+@pytest.mark.parametrize("clamp", [False, True])
+def test_bmatmax(dev, shape, clamp):
+    from triturus_amd.max import bmatmax
+
+    g = torch.Generator().manual_seed(sum(shape))
+    x = torch.randn(*shape, generator=g) * 50
+    x[torch.rand(shape, generator=g) < 0.1] = float("-inf")
+    x[0, :, 0] = float("-inf")                      # an all -inf column
+    if shape[2] > 2:
+        x[0, shape[1] // 2, 2] = float("nan")       # a NaN wins, as in torch.amax
+        x[-1, 0, 1] = float("inf")
+    want = torch.amax(x, dim=1)
+    if clamp:
+        want = torch.clamp(want, -1e38, 1e38)       # baselines/lm2exp.py:12
+    _same(bmatmax(x.to(dev), clamp=clamp), want)
+    # strided input: padded rows and a batch gap
+    big = torch.full((shape[0] * 2, shape[1] + 3, shape[2] + 5), 1e30)
+    v = big[::2, 1 : 1 + shape[1], 2 : 2 + shape[2]]
+    v.copy_(x)
+    bigg = big.to(dev)
+    _same(bmatmax(bigg[::2, 1 : 1 + shape[1], 2 : 2 + shape[2]], clamp=clamp), want)
+
+
+def test_bmatmax_is_the_shift_of_the_contraction(dev):
+    """m = clamp(amax(b, 1)) is what lm2exp subtracts: m + log(a @ exp(b - m)) from it equals lm2exp."""
+    from triturus.lm2exp import lm2exp
+    from triturus_amd.max import bmatmax
+
+    g = torch.Generator().manual_seed(8)
+    a = torch.rand(3, 40, 90, generator=g).to(dev)
+    b = (torch.randn(3, 90, 130, generator=g) * 10).to(dev)
+    b[1, :, 7] = float("-inf")
+    m = bmatmax(b, clamp=True).unsqueeze(1)
+    recipe = m + torch.log(torch.bmm(a, torch.exp(b - m)))
+    out = lm2exp(a, b)
+    assert torch.equal(torch.isneginf(out), torch.isneginf(recipe))
+    fin = torch.isfinite(recipe)
+    assert torch.allclose(out[fin], recipe[fin], rtol=1e-5, atol=1e-5)

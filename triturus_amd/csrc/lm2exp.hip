@@ -377,15 +377,24 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     }
 }
 
-// Clamped column maxima m[r,k] = clamp(max_j b[r,j,k]) for the two-kernel variant (a separate
-// pass over b, then a contraction that reads the shift).  A workgroup owns 256 columns of one
-// batch (a lane 4 adjacent ones); its 4 wavefronts interleave over the rows and combine in LDS.
+// Column maxima m[r,k] = max_j b[r,j,k] (clamped to +-1e38 with CLAMP: the shift of the two-kernel
+// variant; a NaN wins).  A workgroup owns 256 columns of one batch (a lane 4 adjacent ones) and
+// the rows [split * chunk, (split + 1) * chunk); its 4 wavefronts interleave over those rows and
+// combine in LDS.  With splits > 1 the result of a split goes to m + split * R * K and a second
+// launch of this kernel reduces over the splits.
+template <bool CLAMP>
 __global__ __launch_bounds__(256) void lm2exp_colmax_kernel(const float *__restrict__ b, float *__restrict__ m, int R,
-                                                            int J, int K, int64_t sb0, int64_t sb1) {
+                                                            int J, int K, int64_t sb0, int64_t sb1, int chunk,
+                                                            int splits) {
     __shared__ float part[4][256];
     const int blocks_per_batch = (K + 255) / 256;
-    const int r = blockIdx.x / blocks_per_batch;
-    const int k0 = (blockIdx.x % blocks_per_batch) * 256;
+    const int kb = blockIdx.x % blocks_per_batch;
+    const int rs = blockIdx.x / blocks_per_batch;
+    const int r = rs % R;
+    const int split = rs / R;
+    const int k0 = kb * 256;
+    const int j0 = split * chunk;
+    const int j1 = (j0 + chunk < J) ? j0 + chunk : J;
     const int wave = threadIdx.x / kWave, lane = threadIdx.x % kWave;
     const float *br = b + (int64_t)r * sb0;
     float x[4];
@@ -393,7 +402,7 @@ __global__ __launch_bounds__(256) void lm2exp_colmax_kernel(const float *__restr
     for (int e = 0; e < 4; ++e) x[e] = -__builtin_inff();
     const int kc = k0 + 4 * lane;
     const bool vec = kc + 3 < K && (sb1 % 4 == 0) && ((reinterpret_cast<uintptr_t>(br) & 15) == 0);
-    for (int j = wave; j < J; j += 4) {
+    for (int j = j0 + wave; j < j1; j += 4) {
         const float *row = br + (int64_t)j * sb1;
         if (vec) {
             const floatx4 v = *reinterpret_cast<const floatx4 *>(row + kc);
@@ -411,8 +420,18 @@ __global__ __launch_bounds__(256) void lm2exp_colmax_kernel(const float *__restr
     const int t = threadIdx.x;
     if (k0 + t < K) {
         const float y = max_nan(max_nan(part[0][t], part[1][t]), max_nan(part[2][t], part[3][t]));
-        m[(int64_t)r * K + k0 + t] = clamp_shift(y);
+        m[((int64_t)split * R + r) * K + k0 + t] = CLAMP ? clamp_shift(y) : y;
     }
+}
+
+// Rows per split of the batched column maxima: enough workgroups for 256 CUs (>= 1024), at
+// least 64 rows each, at most 64 splits.
+static int colmax_splits(int64_t R, int64_t J, int64_t K) {
+    const int64_t base = R * ceil_div(K, 256);
+    int64_t splits = base >= 1024 ? 1 : ceil_div(1024, base);
+    if (splits > J / 64) splits = J / 64;
+    if (splits > 64) splits = 64;
+    return splits < 1 ? 1 : (int)splits;
 }
 
 // Merge of a split contraction: every split s holds sum_s (relative to its own shift m_s);
@@ -661,8 +680,8 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         args.shift = static_cast<float *>(workspace);
         const int64_t blocks = R * ceil_div(K, 256);
         if (blocks >= ((int64_t)1 << 31)) return TRT_E_RANGE;
-        hipLaunchKernelGGL(lm2exp_colmax_kernel, dim3((unsigned)blocks), dim3(256), 0, s, b, args.shift, (int)R,
-                           (int)J, (int)K, sb[0], sb[1]);
+        hipLaunchKernelGGL(lm2exp_colmax_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, b, args.shift, (int)R,
+                           (int)J, (int)K, sb[0], sb[1], (int)J, 1);
     } else if (pl.splits > 1) {
         const size_t need = plan_workspace(pl, R, I, K);
         if (!workspace || workspace_bytes < need) return TRT_E_WORKSPACE;
@@ -692,6 +711,54 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     if (blocks > 8192) blocks = 8192;
     hipLaunchKernelGGL(lm2exp_merge_kernel, dim3((unsigned)blocks), dim3(256), 0, s, args.part, args.shift, c,
                        (int)R, (int)I, (int)K, pl.splits, sc[0], sc[1]);
+    return (int)hipGetLastError();
+}
+
+// Batched column maxima m[r,k] = max_j b[r,j,k] of an R x J x K fp32 tensor (a NaN wins, as in
+// torch.amax); with `clamp` the result is clamped to +-1e38, which is exactly the shift the
+// contraction kernels subtract (baselines/lm2exp.py:11-12, baselines/lt2exp.py:15-19).  Few
+// columns under a long reduced axis are cut over J (partial maxima in the workspace, then the
+// same kernel over the partials).
+extern "C" size_t trt_colmax_batched_workspace_bytes(int64_t R, int64_t J, int64_t K) {
+    if (R <= 0 || J <= 0 || K <= 0) return 0;
+    const int splits = colmax_splits(R, J, K);
+    return splits > 1 ? (size_t)splits * R * K * sizeof(float) : 0;
+}
+
+extern "C" int trt_colmax_batched_f32(const float *b, float *m, int64_t R, int64_t J, int64_t K,
+                                      const int64_t sb[3], int clamp, void *workspace, size_t workspace_bytes,
+                                      void *stream) {
+    if (!b || !m || !sb) return TRT_E_INVALID;
+    if (R <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
+    if (sb[2] != 1 || sb[0] < 0 || sb[1] < 0) return TRT_E_LAYOUT;
+    const int64_t lim = (int64_t)1 << 30;
+    if (R >= lim || J >= lim || K >= lim) return TRT_E_RANGE;
+    int splits = colmax_splits(R, J, K);
+    const int chunk = (int)ceil_div(J, splits);
+    splits = (int)ceil_div(J, chunk);
+    const int64_t blocks = R * ceil_div(K, 256) * splits;
+    if (blocks >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (splits > 1) {
+        if (!workspace || workspace_bytes < (size_t)splits * R * K * sizeof(float)) return TRT_E_WORKSPACE;
+        float *part = static_cast<float *>(workspace);
+        hipLaunchKernelGGL(lm2exp_colmax_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, b, part, (int)R, (int)J,
+                           (int)K, sb[0], sb[1], chunk, splits);
+        // reduce over the splits: the partials are an R x splits x K tensor with strides (K, R*K, 1)
+        const unsigned blocks2 = (unsigned)(R * ceil_div(K, 256));
+        if (clamp)
+            hipLaunchKernelGGL(lm2exp_colmax_kernel<true>, dim3(blocks2), dim3(256), 0, s, part, m, (int)R, splits, (int)K,
+                               K, R * K, splits, 1);
+        else
+            hipLaunchKernelGGL(lm2exp_colmax_kernel<false>, dim3(blocks2), dim3(256), 0, s, part, m, (int)R, splits,
+                               (int)K, K, R * K, splits, 1);
+    } else if (clamp) {
+        hipLaunchKernelGGL(lm2exp_colmax_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, b, m, (int)R, (int)J,
+                           (int)K, sb[0], sb[1], (int)J, 1);
+    } else {
+        hipLaunchKernelGGL(lm2exp_colmax_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, b, m, (int)R, (int)J,
+                           (int)K, sb[0], sb[1], (int)J, 1);
+    }
     return (int)hipGetLastError();
 }
 

@@ -89,3 +89,39 @@ def matmax(x: torch.Tensor, axis: int = 0, *, block_size: int = 32) -> torch.Ten
     if status:
         _lib.check(status, "trt_matmax")
     return y
+
+
+def bmatmax(x: torch.Tensor, *, clamp: bool = False) -> torch.Tensor:
+    """Batched column maxima: ``torch.amax(x, dim=1)`` of an R x J x K fp32 tensor, R x K.
+
+    The reference reduces 2-D matrices only (``matmax``, triturus/max.py:125-188); this is the
+    batched form along axis 1 that the contraction recipes start with
+    (baselines/lm2exp.py:11, baselines/lt2exp.py:15,18).  With ``clamp`` the maxima are clamped
+    to +-1e38 as there (baselines/lm2exp.py:12): the shift the contraction kernels subtract.
+    """
+    assert len(x.shape) == 3
+    assert x.dtype == torch.float32
+    _lib.require_gpu(x)
+    lib = _lib.load()
+    R, J, K = x.shape
+    if R == 0 or K == 0:
+        return torch.empty((R, K), dtype=x.dtype, device=x.device)
+    if J == 0:
+        raise RuntimeError("max over an empty axis")
+    st = x.stride()
+    if st[-1] != 1 or min(st) <= 0:
+        x = x.contiguous()
+    m = torch.empty((R, K), dtype=x.dtype, device=x.device)
+    key = ("b", R, J, K)
+    ws_bytes = _ws_bytes.get(key)
+    if ws_bytes is None:
+        ws_bytes = _ws_bytes[key] = lib.trt_colmax_batched_workspace_bytes(R, J, K)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=x.device) if ws_bytes else None
+    with _lib.on_device(x.device):
+        status = lib.trt_colmax_batched_f32(
+            x.data_ptr(), m.data_ptr(), R, J, K, _lib.strides3(x), int(bool(clamp)),
+            ws.data_ptr() if ws_bytes else None, ws_bytes, _lib.raw_stream(x.device),
+        )
+    if status:
+        _lib.check(status, "trt_colmax_batched_f32")
+    return m
