@@ -201,7 +201,7 @@ def main() -> int:
     from triturus_amd import workloads as W
     from triturus_amd.lm2exp import lm2exp
     from triturus_amd.lt2exp import lt2exp
-    from triturus_amd.max import matmax, vmax
+    from triturus_amd.max import bmatmax, matmax, vmax
 
     dev = torch.device("cuda", 0)
     torch.cuda.set_device(dev)
@@ -337,6 +337,8 @@ def main() -> int:
         mx = {"bytes": nbytes, "unit": "GB/s", "peak": PEAK_HBM_GBPS}
         for name, fn in (("vmax", lambda: vmax(flat)), ("matmax_axis0", lambda: matmax(mat, 0)),
                          ("matmax_axis1", lambda: matmax(mat, 1)),
+                         ("bmatmax_shift", lambda: bmatmax(x, clamp=True)),  # 64 x 64 x 4096 -> 64 x 4096: the shift m
+                         ("torch_amax_batched", lambda: torch.amax(x, 1)),
                          ("torch_max", lambda: torch.max(flat, 0)), ("torch_amax_axis0", lambda: torch.amax(mat, 0)),
                          ("torch_amax_axis1", lambda: torch.amax(mat, 1))):
             sec = graph_time(fn)
