@@ -145,6 +145,18 @@ def test_lt2exp_reduces_to_lm2exp_on_the_outer_sum():
     _close(oracle64.lt2exp64(w, a, b), oracle64.lm2exp64(w.reshape(R, S, I * J), ab))
 
 
+def test_lt2exp_matches_the_einsum_formulation():
+    """The reference states the recipe a second way, as a three-operand einsum over the shifted
+    exponentials (baselines/lt2exp.py:28-45); in float64 the two agree to rounding."""
+    R, S, I, J, K = 3, 5, 4, 6, 7
+    w, a, b = _rand_lt(12, R, S, I, J, K, p_inf=0.2)
+    w64, a64, b64 = w.double(), a.double(), b.double()
+    ma = torch.clamp(torch.amax(a64, dim=1, keepdim=True), -1e38, 1e38)
+    mb = torch.clamp(torch.amax(b64, dim=1, keepdim=True), -1e38, 1e38)
+    r = torch.einsum("brij,bis,bjs->brs", w64, torch.exp(a64 - ma), torch.exp(b64 - mb))
+    _close(oracle64.lt2exp64(w, a, b), ma + mb + torch.log(r))
+
+
 def test_lt2exp_rank_one_weights_factorise():
     R, S, I, J, K = 2, 4, 3, 5, 6
     _, a, b = _rand_lt(9, R, S, I, J, K)
