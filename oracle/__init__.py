@@ -11,12 +11,15 @@ Modules
                     (log-sum-exp over the contracted axes) that pin them.
     torch_baseline  the same recipes in fp32, op for op: the CPU competitor
                     that the benchmark times on the host cores.
+    oracle_c        the same path restated in plain C (oracle_c.c: scalar loops,
+                    double precision, libm only; built by build_c.py with gcc),
+                    reached through ctypes.  Shares no code with oracle64.
     max_ref         first-occurrence arg-max / max with torch's NaN rule,
                     brute force in NumPy (the reference tests use torch.amax /
                     torch.max, tests/max.py:13,22,32).
 
 Pinning status (see tests/test_oracle.py): every function here is checked
-against an independent formulation -- scipy's logsumexp over the broadcast
+against an independent formulation -- the C restatement against the torch one, scipy's logsumexp over the broadcast
 R x I x J x K (or R x S x I x J x K) tensor, pure-Python ``math.fsum`` loops on
 tiny inputs, and the algebraic special cases (identity a, J = 1, constant b,
 column-shift equivariance, rank-1 w).  No function is "parity unpinned".

@@ -277,3 +277,61 @@ def test_golden_max_oracle():
     x = torch.from_numpy(z["x"])
     assert np.array_equal(torch.amax(x, 0).numpy(), z["axis0"])
     assert np.array_equal(torch.amax(x, 1).numpy(), z["axis1"])
+
+
+# ---- the plain C restatement (oracle/oracle_c.c) against the torch / NumPy oracle: two
+# implementations that share no code (libm scalar loops on one side, ATen on the other)
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1), (2, 5, 7, 6), (3, 17, 33, 20)])
+@pytest.mark.parametrize("p_inf", [0.0, 0.3])
+def test_c_restatement_lm2exp(shape, p_inf):
+    from oracle import oracle_c
+
+    a, b = (t.float() for t in _rand_lm(21, *shape, p_inf=p_inf))  # fp32 values, as the kernels get them
+    b[0, :, 0] = NINF  # an all -inf column: -inf out, never NaN
+    got, want = oracle_c.lm2exp_c(a, b), oracle64.lm2exp64(a, b).numpy()
+    assert np.array_equal(np.isneginf(got), np.isneginf(want)) and not np.isnan(got).any()
+    _close(torch.from_numpy(got), torch.from_numpy(want))
+    _close(torch.from_numpy(got), torch.from_numpy(oracle64.lm2exp_lse(a, b)))
+
+
+@pytest.mark.parametrize("shape", [(1, 1, 1, 1, 1), (2, 3, 4, 5, 6), (2, 9, 7, 3, 17)])
+@pytest.mark.parametrize("p_inf", [0.0, 0.3])
+def test_c_restatement_lt2exp(shape, p_inf):
+    from oracle import oracle_c
+
+    w, a, b = (t.float() for t in _rand_lt(22, *shape, p_inf=p_inf))
+    got, want = oracle_c.lt2exp_c(w, a, b), oracle64.lt2exp64(w, a, b).numpy()
+    assert np.array_equal(np.isneginf(got), np.isneginf(want)) and not np.isnan(got).any()
+    _close(torch.from_numpy(got), torch.from_numpy(want))
+    _close(torch.from_numpy(got), torch.from_numpy(oracle64.lt2exp_lse(w, a, b)))
+
+
+def test_c_restatement_clamp_and_nan():
+    from oracle import oracle_c
+
+    a = torch.tensor([[[1.0, 2.0]]])
+    b = torch.tensor([[[NINF, 3.0, float("nan")], [NINF, 1.0, 0.0]]])
+    got = oracle_c.lm2exp_c(a, b)[0, 0]
+    assert np.isneginf(got[0])                       # all -inf column: the clamp keeps exp(-inf - m) = 0
+    assert abs(got[1] - math.log(math.exp(3.0) + 2 * math.exp(1.0))) < 1e-12
+    assert np.isnan(got[2])                          # a NaN poisons its column, as in the torch recipe
+
+
+def test_c_restatement_max():
+    from oracle import max_ref, oracle_c
+
+    g = torch.Generator().manual_seed(23)
+    x = (torch.randn(37, 53, generator=g) * 3).round()  # many ties
+    for axis in (0, 1):
+        assert np.array_equal(oracle_c.matmax_c(x, axis), torch.amax(x, axis).numpy())
+    flat = x.reshape(-1)
+    assert oracle_c.vmax_c(flat) == max_ref.vmax_ref_fast(flat.numpy())
+    v, i = torch.max(flat, 0)
+    assert oracle_c.vmax_c(flat) == (v.item(), i.item())
+    flat[100] = float("nan")
+    flat[7] = float("nan")
+    v, i = oracle_c.vmax_c(flat)
+    assert math.isnan(v) and i == 7                  # the first NaN
+    y = x.clone()
+    y[3, 4] = float("nan")
+    assert np.isnan(oracle_c.matmax_c(y, 0)[4]) and np.isnan(oracle_c.matmax_c(y, 1)[3])

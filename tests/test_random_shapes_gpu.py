@@ -278,3 +278,19 @@ def test_concurrent_streams(dev):
     torch.cuda.synchronize()
     for o1, o2, o3 in outs:
         assert torch.equal(o1, ref_m) and torch.equal(o2, ref_t) and torch.equal(o3, ref_m6)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+def test_against_the_c_restatement(dev, precision):
+    """The HIP path against the plain C loops (oracle/oracle_c.c), the checker that shares no
+    code with torch: benchmark input distributions at small sizes, -inf included."""
+    from oracle import oracle_c
+    from triturus_amd import workloads
+
+    c2 = workloads.c2(R=2, n=96)
+    out = lm2exp(c2["a"].to(dev), c2["b"].to(dev), _precision=precision)
+    assert oracle64.compare(out, oracle_c.lm2exp_c(c2["a"], c2["b"]), **GATES[precision])["ok"]
+    c4 = workloads.c4(R=2, K=200)
+    for mode in ("unsplit", "split"):
+        out = lt2exp(c4["w"].to(dev), c4["a"].to(dev), c4["b"].to(dev), mode=mode, _precision=precision)
+        assert oracle64.compare(out, oracle_c.lt2exp_c(c4["w"], c4["a"], c4["b"]), **GATES[precision])["ok"]
