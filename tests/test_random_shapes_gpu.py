@@ -59,7 +59,7 @@ def test_lm2exp_random(dev, seed, precision):
     b = _sprinkle(rng, g, torch.randn(R, J, K, generator=g) * rng.choice([1.0, 8.0, 40.0]) + rng.choice([0.0, -60.0, 90.0]))
     ref = oracle64.lm2exp64(a, b)
     ag, bg = _view(rng, a.to(dev)), _view(rng, b.to(dev))
-    nvar = 0 if precision == "fp32" else 8
+    nvar = 0 if precision == "fp32" else 9
     variant = rng.randrange(0, nvar + 1)
     out = lm2exp(ag, bg, _precision=precision, _variant=variant)
     r = oracle64.compare(out, ref, **GATES[precision])
@@ -232,7 +232,7 @@ def test_sparse_weights_under_a_wide_spread(dev, seed, precision):
     b = torch.randn(R, J, K, generator=g) * rng.choice([40.0, 300.0]) + rng.choice([0.0, 1e4, -1e6])
     b = _sprinkle(rng, g, b)
     lo, hi = _lm_bracket(a, b, cut)
-    nvar = 12 if precision == "fp32" else 8
+    nvar = 12 if precision == "fp32" else 9
     variant, splits = rng.randrange(0, nvar + 1), rng.choice([0, 1, 3])
     out = lm2exp(_view(rng, a.to(dev)), _view(rng, b.to(dev)), _precision=precision, _variant=variant, _splits=splits)
     bad, _ = _inside(out, lo, hi, **GATES[precision])

@@ -226,9 +226,9 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
     shift_and_exp();
     __syncthreads();
 
-    // Row tiles are taken two at a time so that consecutive MFMAs alternate between two
-    // accumulators.
-    constexpr int RP = RT >= 2 ? 2 : 1;
+    // Row tiles are taken two at a time (all three of a 96-row tile) so that consecutive MFMAs
+    // alternate between accumulators.
+    constexpr int RP = RT % 2 == 0 ? 2 : (RT == 3 ? 3 : 1);
     auto mfma_block = [&](int buf) {
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
@@ -308,7 +308,7 @@ struct LmBfVariant {
     int rt, ks;
 };
 // variant ids are 1-based in the C ABI (0 = choose by shape)
-static const LmBfVariant kLmBfVariants[] = {{4, 4}, {4, 2}, {2, 4}, {2, 2}, {1, 4}, {1, 2}, {8, 1}, {8, 2}};
+static const LmBfVariant kLmBfVariants[] = {{4, 4}, {4, 2}, {2, 4}, {2, 2}, {1, 4}, {1, 2}, {8, 1}, {8, 2}, {3, 2}};
 constexpr int kNumLmBfVariants = sizeof(kLmBfVariants) / sizeof(kLmBfVariants[0]);
 
 }  // namespace trt
@@ -335,17 +335,18 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
 
     // Tile and hand-over rules, fitted to 223 random shapes (R 1..256, I, J 16..1024, K 64..8192)
     // timed with every tile and on the fp32 path; against the best of those the rules below lose
-    // 5.4 % (two pieces) / 4.0 % (three) on average, the previous ones 19 / 11 %.
+    // 5.6 % (two pieces) / 4.3 % (three) on average, the previous ones 19 / 11 %.
     //  - Grids of fewer than 128 (three pieces: 192) 32-row tiles are latency bound, not matrix
     //    bound, and a contraction of at most 16 (32) is bound by writing c: there the fp32 path
     //    (smaller tiles, contraction cut over J) is as fast or faster and takes the call, as it
     //    does whenever the caller asks for a cut.
     //  - j-chunks of 32 (three workgroups fit a CU; chunks of 64 measured 0-17 % behind), except
     //    with two pieces on 64- and 32-row tiles over a contraction of 512 or more (chunks of 64).
-    //  - Rows: the candidate (128, 64 or 32 rows; at least 1.5, 1, 0 workgroups per CU) with the least
-    //    padded rows x cost per row, the cost being 1.15 for 32 rows, 1 for 64, and for 128 rows
-    //    0.85 (0.95) on a contraction of 256 or more, where each exp then feeds more MFMAs, and
-    //    1.05 on a shorter one.
+    //  - Rows: the candidate (128, 96, 64 or 32 rows; at least 1.5, 1.5, 1, 0 workgroups per CU)
+    //    with the least padded rows x cost per row, the cost being 1.2 for 32 rows, 1 for 64, and on
+    //    a contraction of 256 or more, where each exp feeds more MFMAs, 0.90 (0.93) for 96 and 0.85
+    //    (0.95) for 128 rows; on a shorter one 1 and 1.05.  The 96-row tile (three wavefronts
+    //    per SIMD) takes I = 96, 160, 192, 288 and the like: 10-24 % ahead there.
     int v;
     if (variant >= 1) {
         v = variant - 1;
@@ -355,17 +356,19 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
         if (splits > 1 || n32 < (pieces == 2 ? 128 : 192) || J <= (pieces == 2 ? 16 : 32))
             return trt_lm2exp_f32(a, b, c, R, I, J, K, sa, sb, sc, 0, splits, workspace, workspace_bytes, stream);
         int best_rt = 1;
-        int64_t best_cost = ceil_div(I, 32) * 115;
-        for (int rt = 2; rt <= 4; rt *= 2) {
-            if (R * ceil_div(I, 32 * rt) * ct < (rt == 4 ? 384 : 256)) continue;  // 1.5 / 1 workgroups per CU
-            const int64_t per_row = rt == 2 ? 100 : (J >= 256 ? (pieces == 2 ? 85 : 95) : 105);
+        int64_t best_cost = ceil_div(I, 32) * 120;
+        for (int rt = 2; rt <= 4; ++rt) {
+            if (R * ceil_div(I, 32 * rt) * ct < (rt == 2 ? 256 : 384)) continue;  // 1 / 1.5 workgroups per CU
+            int64_t per_row = 100;
+            if (rt == 3) per_row = J >= 256 ? (pieces == 2 ? 90 : 93) : 100;
+            if (rt == 4) per_row = J >= 256 ? (pieces == 2 ? 85 : 95) : 105;
             const int64_t cost = ceil_div(I, 32 * rt) * rt * per_row;
-            if (cost < best_cost) {
+            if (cost <= best_cost) {  // ties go to the larger tile
                 best_cost = cost;
                 best_rt = rt;
             }
         }
-        v = best_rt == 4 ? 1 : (best_rt == 2 ? 3 : 5);  // {4,2}, {2,2}, {1,2}
+        v = best_rt == 4 ? 1 : (best_rt == 3 ? 8 : (best_rt == 2 ? 3 : 5));  // {4,2}, {3,2}, {2,2}, {1,2}
         if (pieces == 2 && best_rt <= 2 && J >= 512) v -= 1;  // {2,4}, {1,4}: fewer barriers pay on a long contraction
         // two pieces are bound by the vector work on the B operand: 256 rows (each exp feeds 24
         // MFMAs) when I fills them exactly and two workgroups per CU remain (6-25 % at I = 256, 512)
@@ -395,7 +398,8 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
         case 4: return launch_lm_bf<1, 4>(args, pieces, vec, s);
         case 5: return launch_lm_bf<1, 2>(args, pieces, vec, s);
         case 6: return launch_lm_bf<8, 1>(args, pieces, vec, s);
-        default: return launch_lm_bf<8, 2>(args, pieces, vec, s);
+        case 7: return launch_lm_bf<8, 2>(args, pieces, vec, s);
+        default: return launch_lm_bf<3, 2>(args, pieces, vec, s);
     }
 }
 
