@@ -116,11 +116,11 @@ int trt_lt2exp_variant_count(void);
  * This is the library's counterpart of the reference's reduced-precision mode
  * (ALLOW_TF32 passed to tl.dot, triturus/lt2exp.py:344, flag triturus/utils.py:33-44):
  * gfx950 has no TF32 matrix instruction; two bf16 pieces are more accurate than TF32
- * (2^-11) and several times faster than the fp32 matrix pipe.  The bf16 kernels never split
- * the contraction: with variant 0 a grid too small to be matrix bound (fewer than 192
- * tiles), and any call in mode SPLIT, is handed to trt_lt2exp_f32, so the call takes
- * the same mode and workspace (trt_lt2exp_workspace_bytes) as trt_lt2exp_f32.  variant: 0 = choose by shape, 1..4 force a
- * bf16 tile shape (experiments, tests; no workspace needed).
+ * (2^-11) and several times faster than the fp32 matrix pipe.  The call takes the same mode
+ * and workspace (trt_lt2exp_workspace_bytes) as trt_lt2exp_f32: with variant 0 a grid too
+ * small to be matrix bound has its contraction cut over workgroups (as the mode and the
+ * workspace allow) or is handed to trt_lt2exp_f32.  variant: 0 = choose by shape, 1..4
+ * force a bf16 tile shape, 5..8 the same tiles with the contraction cut (experiments, tests).
  */
 #define TRT_PIECES_BF16X3 2
 #define TRT_PIECES_BF16X6 3
@@ -129,6 +129,9 @@ int trt_lt2exp_bf16(const float *w, const float *a, const float *b, float *c,
                     const int64_t sw[3], const int64_t sa[3], const int64_t sb[3],
                     const int64_t sc[3], int pieces, int mode, int variant,
                     void *workspace, size_t workspace_bytes, void *stream);
+/* Workspace for trt_lt2exp_bf16: the larger of this and trt_lt2exp_workspace_bytes. */
+size_t trt_lt2exp_bf16_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K,
+                                       int pieces, int mode);
 
 /*
  * trt_lm2exp_f32 on the bf16 matrix pipe, in the same way (ALLOW_TF32 at

@@ -21,7 +21,7 @@ pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
 N_VARIANTS = 8
-N_BF16_VARIANTS = 4
+N_BF16_VARIANTS = 8  # 1..4 tiles, 5..8 the same tiles with the contraction cut over workgroups
 # Accuracy gates of the split-bf16 paths against the float64 oracle.  Two pieces (3 MFMAs per
 # product) carry 16 significand bits: looser than fp32, ten times tighter than the rtol 5e-4
 # the reference allows its TF32 mode (tests/lt2exp.py:38).  Three pieces (6 MFMAs) carry 24
@@ -272,9 +272,18 @@ def test_bf16_paths_on_ragged_shapes(dev, precision, variant, shape):
     a[torch.rand(a.shape, generator=g) < 0.05] = NINF
     b[:, :, 0] = NINF  # an all -inf column: -inf out, not NaN
     w[:, 0] = 0.0  # a zero row of weights: -inf out
-    out = lt2exp(w.to(dev), a.to(dev), b.to(dev), _precision=precision, _variant=variant)
+    # variants 5..8 cut the contraction as far as the workspace allows: mode "split" sizes it
+    mode = "split" if variant >= 5 else "auto"
+    out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision, _variant=variant)
     r = _check(out, w, a, b, **PRECISION_GATES[precision])
     assert r["n_neg_inf"] > 0
+    if variant >= 5:  # the cut is deterministic: same bits on a second call; and close to the uncut tile
+        again = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision, _variant=variant)
+        assert torch.equal(out, again)
+        uncut = lt2exp(w.to(dev), a.to(dev), b.to(dev), _precision=precision, _variant=variant - 4)
+        fin = torch.isfinite(uncut)
+        assert torch.equal(torch.isfinite(out), fin)
+        assert torch.allclose(out[fin], uncut[fin], rtol=1e-5, atol=1e-5)
 
 
 @pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])

@@ -85,7 +85,7 @@ def test_lt2exp_random(dev, seed, precision):
         big[:, 1 : S + 1] = wg
         wg = big[:, 1 : S + 1]
     mode = rng.choice(["auto", "split", "unsplit"])
-    variant = 0 if precision == "fp32" else rng.randrange(0, 5)
+    variant = 0 if precision == "fp32" else rng.randrange(0, 9)
     out = lt2exp(wg, ag, bg, mode=mode, _precision=precision, _variant=variant)
     r = oracle64.compare(out, ref, **GATES[precision])
     assert r["ok"], (R, S, I, J, K, mode, variant, r)
@@ -245,7 +245,7 @@ def test_sparse_weights_under_a_wide_spread(dev, seed, precision):
     b = _sprinkle(rng, g, torch.randn(R, J, K, generator=g) * rng.choice([10.0, 100.0]) + rng.choice([0.0, -1e5]))
     lo, hi = _lt_bracket(w, a, b, cut)
     mode = rng.choice(["auto", "split", "unsplit"])
-    variant = rng.randrange(0, 9) if precision == "fp32" else rng.randrange(0, 5)
+    variant = rng.randrange(0, 9)
     out = lt2exp(w.to(dev), _view(rng, a.to(dev)), _view(rng, b.to(dev)), mode=mode, _precision=precision,
                  _variant=variant)
     bad, _ = _inside(out, lo, hi, **GATES[precision])

@@ -20,6 +20,7 @@
 // Replaces _ker_lt2exp_unsplit / _ker_lt2exp_split, triturus/lt2exp.py:227-357,365-506.
 
 #include "common.hpp"
+#include "lt2exp_merge.hpp"
 
 namespace trt {
 
@@ -282,25 +283,6 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     }
 }
 
-// c = (ma + mb) + log(sum over splits of the partial sums), in split order.
-__global__ __launch_bounds__(256) void lt2exp_merge_kernel(const float *__restrict__ part,
-                                                           const float *__restrict__ shift, float *__restrict__ c,
-                                                           int R, int S, int K, int splits, int64_t sc0,
-                                                           int64_t sc1) {
-    const int64_t total = (int64_t)R * S * K;
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
-        const int k = (int)(e % K);
-        const int64_t rs = e / K;
-        const int s = (int)(rs % S);
-        const int r = (int)(rs / S);
-        float sum = 0.f;
-        for (int sp = 0; sp < splits; ++sp) sum += part[(int64_t)sp * total + e];
-        const float mm = shift[(int64_t)r * K + k] + shift[((int64_t)R + r) * K + k];
-        c[(int64_t)r * sc0 + (int64_t)s * sc1 + k] = log_plus(sum, mm);
-    }
-}
-
 // ------------------------------------------------------------------ host
 struct Lt2Variant {
     int rt, ct, nq;
@@ -469,12 +451,6 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
                      ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
     launch_variant(v, args, vec, sp.split, s);
-    if (sp.split) {
-        const int64_t total = R * S * K;
-        int64_t blocks = ceil_div(total, 256);
-        if (blocks > 4096) blocks = 4096;
-        hipLaunchKernelGGL(lt2exp_merge_kernel, dim3((unsigned)blocks), dim3(256), 0, s, args.c, args.shift, c,
-                           (int)R, (int)S, (int)K, sp.splits, sc[0], sc[1]);
-    }
+    if (sp.split) launch_lt2exp_merge(args.c, args.shift, c, R, S, K, sp.splits, sc[0], sc[1], s);
     return (int)hipGetLastError();
 }

@@ -24,19 +24,22 @@
 // of a chunk is j = 16 ks + 8 h + e for both operands.
 
 #include "bf16_split.hpp"
+#include "lt2exp_merge.hpp"
 
 namespace trt {
 
 struct Lt2BfArgs {
     const float *w, *a, *b;
-    float *c;
+    float *c;      // output (unsplit) -- or partial sums [splits][R][S][K] (split)
+    float *shift;  // split only: [2][R][K] clamped column maxima
     int R, S, I, J, K;
     int64_t sw0, sw1, sa0, sa1, sb0, sb1, sc0, sc1;
-    int s_tiles, n_tiles;
+    int s_tiles, n_tiles, splits;
+    int iters_per_split;  // (j-chunk, i) iterations per split
     int64_t total_wgs, padded_wgs;
 };
 
-template <int RT, int KS, int NS, bool VEC>
+template <int RT, int KS, int NS, bool VEC, bool SPLIT = false>
 __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) {
     constexpr int NT = 256;
     constexpr int TS = 32 * RT;    // rows of S per workgroup
@@ -54,6 +57,8 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     if (L >= p.total_wgs) return;
     int64_t rest = L / p.n_tiles;
     const int nt = __builtin_amdgcn_readfirstlane((int)(L % p.n_tiles));
+    const int split = SPLIT ? __builtin_amdgcn_readfirstlane((int)(rest % p.splits)) : 0;
+    if (SPLIT) rest /= p.splits;
     const int st = __builtin_amdgcn_readfirstlane((int)(rest % p.s_tiles));
     const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.s_tiles));
 
@@ -83,8 +88,12 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     y = __builtin_fmaxf(y, __shfl_xor(y, 32, kWave));
     const float mb = clamp_shift(y);
 
+    // (j-chunk, i) iterations of this workgroup: all of them, or one split's share
     const int n_jc = (p.J + JC - 1) / JC;
-    const int total_iters = n_jc * p.I;
+    const int it0 = SPLIT ? split * p.iters_per_split : 0;
+    int it1 = SPLIT ? it0 + p.iters_per_split : n_jc * p.I;
+    if (it1 > n_jc * p.I) it1 = n_jc * p.I;
+    const int total_iters = it1 - it0;
 
     floatx16 total[RT];
 #pragma unroll
@@ -168,10 +177,11 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     };
 
     if (total_iters > 0) {
-        int jc = 0, i = 0;
-        load_tile(0, 0);
-        load_eb(0);
-        float ea = exp_shifted(ar[ncl] - ma);
+        int jc = it0 / p.I;
+        int i = it0 - jc * p.I;
+        load_tile(i, jc);
+        load_eb(jc);
+        float ea = exp_shifted(ar[(int64_t)i * p.sa1 + ncl] - ma);
         float ea_raw;
         store_tile(0);
         __syncthreads();
@@ -299,6 +309,22 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 
     // ---- epilogue: register v of lane (h, m) holds row 8*(v/4) + 4*h + v%4, column m
     if (ncol >= p.K) return;
+    if (SPLIT) {
+        // raw partial sums; all splits share ma, mb (they depend on the column only)
+        float *part = p.c + ((int64_t)split * p.R + r) * (int64_t)p.S * p.K;
+        if (split == 0 && st == 0 && h == 0) {
+            p.shift[(int64_t)r * p.K + ncol] = ma;
+            p.shift[((int64_t)p.R + r) * p.K + ncol] = mb;
+        }
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = s0 + 32 * rt + 8 * (v / 4) + 4 * h + (v % 4);
+                if (row < p.S) part[(int64_t)row * p.K + ncol] = total[rt][v];
+            }
+        return;
+    }
     const int crows = p.S - s0;
     const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)s0 * p.sc1,
                                                     (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4));
@@ -315,29 +341,61 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 }
 
 template <int RT, int KS, int NS>
-static void launch_bf(const Lt2BfArgs &args, bool vec, hipStream_t stream) {
-    if (vec)
-        hipLaunchKernelGGL((lt2exp_bf16_kernel<RT, KS, NS, true>), dim3((unsigned)args.padded_wgs), dim3(256), 0,
-                           stream, args);
-    else
-        hipLaunchKernelGGL((lt2exp_bf16_kernel<RT, KS, NS, false>), dim3((unsigned)args.padded_wgs), dim3(256), 0,
-                           stream, args);
+static void launch_bf(const Lt2BfArgs &args, bool vec, bool split, hipStream_t stream) {
+    const dim3 grid((unsigned)args.padded_wgs), block(256);
+    if (vec) {
+        if (split) hipLaunchKernelGGL((lt2exp_bf16_kernel<RT, KS, NS, true, true>), grid, block, 0, stream, args);
+        else hipLaunchKernelGGL((lt2exp_bf16_kernel<RT, KS, NS, true, false>), grid, block, 0, stream, args);
+    } else {
+        if (split) hipLaunchKernelGGL((lt2exp_bf16_kernel<RT, KS, NS, false, true>), grid, block, 0, stream, args);
+        else hipLaunchKernelGGL((lt2exp_bf16_kernel<RT, KS, NS, false, false>), grid, block, 0, stream, args);
+    }
 }
 
 template <int NS>
-static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, hipStream_t stream) {
+static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, bool split, hipStream_t stream) {
     if (rt == 2) {
-        if (ks == 4) launch_bf<2, 4, NS>(args, vec, stream);
-        else launch_bf<2, 2, NS>(args, vec, stream);
+        if (ks == 4) launch_bf<2, 4, NS>(args, vec, split, stream);
+        else launch_bf<2, 2, NS>(args, vec, split, stream);
     } else {
-        if (ks == 4) launch_bf<1, 4, NS>(args, vec, stream);
-        else launch_bf<1, 2, NS>(args, vec, stream);
+        if (ks == 4) launch_bf<1, 4, NS>(args, vec, split, stream);
+        else launch_bf<1, 2, NS>(args, vec, split, stream);
     }
 }
 
 }  // namespace trt
 
 using namespace trt;
+
+// Split count the bf16 path would like for a small grid (32-row tiles): 1 = none.
+static int64_t bf16_small_grid_splits(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int pieces, int mode) {
+    if (mode == TRT_MODE_UNSPLIT) return 1;
+    const int64_t j_last = J % 64;
+    const int ks = (j_last >= 1 && j_last <= 32) ? 2 : 4;
+    const int64_t iters = ceil_div(J, 16 * ks) * I;
+    const int64_t tiles = R * ceil_div(S, 32) * ceil_div(K, 128);
+    if (mode != TRT_MODE_SPLIT && tiles >= 1024) return 1;  // four workgroups per CU: matrix bound as it is
+    // The model counts steps in fp32 MFMAs (64 cycles).  A step of this kernel is ks x 3 (or 6) bf16
+    // MFMAs of 32 cycles, but on a CU that holds one or two workgroups the splitting and scaling
+    // around them is not hidden: measured 0.9 us per step alone on a CU with ks = 4 and two pieces,
+    // which the model reproduces with 5/4 of an fp32 MFMA per bf16 MFMA.
+    return choose_splits(tiles, iters, (int64_t)ks * (pieces == 2 ? 3 : 6) * 5 / 4, R * S * K, 4, 32,
+                         mode == TRT_MODE_SPLIT);
+}
+
+static bool bf16_small_grid(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode) {
+    const int64_t t32 = R * ceil_div(S, 32) * ceil_div(K, 128);
+    return mode == TRT_MODE_SPLIT || t32 < 160 || (t32 <= 256 && I * J > 4096);
+}
+
+// Workspace the bf16 entry wants beyond what trt_lt2exp_workspace_bytes reports for the same
+// call (callers pass the larger of the two): room for its own cut of a small grid.
+extern "C" size_t trt_lt2exp_bf16_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int pieces,
+                                                  int mode) {
+    if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0 || (pieces != 2 && pieces != 3)) return 0;
+    const int64_t splits = bf16_small_grid_splits(R, S, I, J, K, pieces, mode);
+    return splits >= 2 ? ((size_t)splits * R * S * K + (size_t)2 * R * K) * sizeof(float) : 0;
+}
 
 extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, float *c, int64_t R, int64_t S,
                                int64_t I, int64_t J, int64_t K, const int64_t sw[3], const int64_t sa[3],
@@ -347,7 +405,7 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
     if (mode != TRT_MODE_AUTO && mode != TRT_MODE_SPLIT && mode != TRT_MODE_UNSPLIT) return TRT_E_INVALID;
-    if (variant < 0 || variant > 4) return TRT_E_INVALID;
+    if (variant < 0 || variant > 8) return TRT_E_INVALID;
     if (sw[2] != 1 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
@@ -359,10 +417,11 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     // Tile and hand-over rules, fitted to 290 random shapes (R 1..128, S 16..512, I, J 8..128,
     // K 64..8192) timed with every tile and on the fp32 path; against the best of those the
     // rules below lose 2.5 % (two pieces) / 1.9 % (three) on average, the previous ones 17 / 14 %.
-    //  - The bf16 kernels never cut the contraction over several workgroups: a grid of fewer
-    //    than 160 32-row tiles -- 256 when the contraction is longer than 4096 -- is latency
-    //    bound, not matrix bound, and goes to the fp32 path, which may cut it;
-    //    so does any call in mode SPLIT.
+    //  - A grid of fewer than 160 32-row tiles -- 256 when the contraction is longer than 4096 --
+    //    is latency bound, not matrix bound: its contraction is cut over workgroups (32-row tiles,
+    //    as many cuts as the cost model asks for and the workspace holds; 1.5-2.5x ahead of the
+    //    fp32 path on batch-1 squares of 192..512), and when it is not to be cut the call goes to
+    //    the fp32 path.  Mode SPLIT cuts on the bf16 pipe as well.
     //  - 32 rows per workgroup; 64 when that pads S no further and still leaves two workgroups
     //    per CU (the pipelined two-row-tile loop then wins 4-11 %).
     //  - j-chunks of 64, or of 32 when those leave less of the last chunk empty (J = 1..32,
@@ -372,15 +431,61 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     const int64_t s_last = S % 64, j_last = J % 64;
     int rt = (S > 32 && (s_last == 0 || s_last > 32) && t64 >= 512) ? 2 : 1;
     int ks = ((j_last >= 1 && j_last <= 32) || (rt == 2 && j_last >= 33 && j_last <= 48)) ? 2 : 4;
-    if (variant >= 1) {  // 1: 64 rows, chunks of 64;  2: 64 rows, 32;  3: 32 rows, 64;  4: 32 rows, 32
-        rt = variant <= 2 ? 2 : 1;
-        ks = (variant & 1) ? 4 : 2;
-    } else if (mode == TRT_MODE_SPLIT || t32 < 160 || (t32 <= 256 && I * J > 4096)) {
-        return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
+    const int rule_rt = rt, rule_ks = ks;
+    bool split = false, small_grid = false;
+    if (variant >= 1) {
+        // 1: 64 rows, chunks of 64;  2: 64 rows, 32;  3: 32 rows, 64;  4: 32 rows, 32;
+        // 5..8: the same with the contraction cut over workgroups (as far as the workspace allows)
+        const int tile = (variant - 1) % 4 + 1;
+        rt = tile <= 2 ? 2 : 1;
+        ks = (tile & 1) ? 4 : 2;
+        split = variant >= 5;
+    } else {
+        // A grid that is not matrix bound as it is has its contraction cut over workgroups on
+        // 32-row tiles when the cost model asks for it (below); a small grid that is not to be
+        // cut goes to the fp32 path.
+        small_grid = bf16_small_grid(R, S, I, J, K, mode);
+        if (bf16_small_grid_splits(R, S, I, J, K, pieces, mode) >= 2) {
+            split = true;
+            rt = 1;
+            ks = (j_last >= 1 && j_last <= 32) ? 2 : 4;
+        }
     }
+
+    // Cutting the (j-chunk, i) iterations over workgroups: partial sums in the workspace
+    // ([splits][R][S][K], then the two shift planes), merged in split order.
+    int splits = 1, per_split = 0;
+    if (split) {
+        const int64_t iters = ceil_div(J, 16 * ks) * I;
+        const int64_t tiles = R * ceil_div(S, 32 * rt) * ctk;
+        const int64_t out = R * S * K;
+        const int64_t fit = workspace ? ((int64_t)(workspace_bytes / sizeof(float)) - 2 * R * K) / out : 0;
+        int64_t want = variant >= 1
+                           ? choose_splits(tiles, iters, (int64_t)ks * (pieces == 2 ? 3 : 6) * rt / 2, out, 4, 32, true)
+                           : bf16_small_grid_splits(R, S, I, J, K, pieces, mode);
+        if (want > fit) want = fit;
+        if (want >= 2) {
+            per_split = (int)ceil_div(iters, want);
+            splits = (int)ceil_div(iters, per_split);
+        }
+        split = splits >= 2;
+        if (!split && variant == 0) {  // the workspace holds no cut: the uncut tile after all
+            rt = rule_rt;
+            ks = rule_ks;
+        }
+    }
+    if (small_grid && !split)
+        return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
 
     Lt2BfArgs args;
     args.w = w; args.a = a; args.b = b; args.c = c;
+    args.shift = nullptr;
+    args.splits = splits;
+    args.iters_per_split = per_split;
+    if (split) {
+        args.c = static_cast<float *>(workspace);
+        args.shift = args.c + (size_t)splits * R * S * K;
+    }
     args.R = (int)R; args.S = (int)S; args.I = (int)I; args.J = (int)J; args.K = (int)K;
     args.sw0 = sw[0]; args.sw1 = sw[1];
     args.sa0 = sa[0]; args.sa1 = sa[1];
@@ -388,13 +493,14 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     args.sc0 = sc[0]; args.sc1 = sc[1];
     args.s_tiles = (int)ceil_div(S, 32 * rt);
     args.n_tiles = (int)ceil_div(K, 128);
-    args.total_wgs = (int64_t)R * args.s_tiles * args.n_tiles;
+    args.total_wgs = (int64_t)R * args.s_tiles * args.n_tiles * splits;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const bool vec = (J % 4 == 0) && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (pieces == 2) launch_bf_shape<2>(args, rt, ks, vec, s);
-    else launch_bf_shape<3>(args, rt, ks, vec, s);
+    if (pieces == 2) launch_bf_shape<2>(args, rt, ks, vec, split, s);
+    else launch_bf_shape<3>(args, rt, ks, vec, split, s);
+    if (split) launch_lt2exp_merge(args.c, args.shift, c, R, S, K, splits, sc[0], sc[1], s);
     return (int)hipGetLastError();
 }

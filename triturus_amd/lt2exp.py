@@ -21,7 +21,7 @@ from triturus_amd import _lib, autotune
 from triturus_amd.lm2exp import _unit_inner
 from triturus_amd.utils import MATRIX_PRECISIONS, matrix_precision
 
-_ws_bytes: dict = {}  # (R, S, I, J, K, mode) -> workspace bytes, as reported by the library
+_ws_bytes: dict = {}  # (R, S, I, J, K, mode, pieces) -> workspace bytes, as reported by the library
 
 _MODES = {"auto": _lib.MODE_AUTO, "split": _lib.MODE_SPLIT, "unsplit": _lib.MODE_UNSPLIT}
 
@@ -82,10 +82,14 @@ def lt2exp(
                                  lambda v: lt2exp(w.view(R, S, I, J), a, b, mode=mode, _variant=v,
                                                   _precision=_precision, _tuning=True))
     mode_code = _MODES[mode]
-    key = (R, S, I, J, K, mode_code)
+    pieces = _PIECES.get(_precision, 0)
+    key = (R, S, I, J, K, mode_code, pieces)
     ws_bytes = _ws_bytes.get(key)
     if ws_bytes is None:
-        ws_bytes = _ws_bytes[key] = lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, mode_code)
+        ws_bytes = lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, mode_code)
+        if pieces:  # the bf16 entry may cut a small grid itself
+            ws_bytes = max(ws_bytes, lib.trt_lt2exp_bf16_workspace_bytes(R, S, I, J, K, pieces, mode_code))
+        _ws_bytes[key] = ws_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     ws_ptr = ws.data_ptr() if ws_bytes else None
     with _lib.on_device(a.device):
@@ -101,7 +105,7 @@ def lt2exp(
             status = lib.trt_lt2exp_bf16(
                 w.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), R, S, I, J, K,
                 _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-                _PIECES[_precision], mode_code, _variant, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
+                pieces, mode_code, _variant, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
             )
     if status:
         _lib.check(status, "trt_lt2exp_f32" if _precision == "fp32" else "trt_lt2exp_bf16")
