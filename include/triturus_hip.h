@@ -136,17 +136,22 @@ size_t trt_lt2exp_bf16_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t 
 /*
  * trt_lm2exp_f32 on the bf16 matrix pipe, in the same way (ALLOW_TF32 at
  * triturus/lm2exp.py:152 is the reference's counterpart): same tensors, layouts, strides and
- * status codes; pieces as above.  With variant 0, grids too small to be matrix bound and
- * calls that ask for a cut over J (splits > 1) are handed to trt_lm2exp_f32, so the call
- * takes the same splits and workspace (trt_lm2exp_workspace_bytes(R, I, J, K, 0, splits)).
+ * status codes; pieces as above.  splits as for trt_lm2exp_f32: 0 = decide by shape, 1 = never,
+ * > 1 = cut the contraction that many times (capped by its length).  With variant 0, a grid too
+ * small to be matrix bound has its contraction cut over workgroups (as the workspace allows) or
+ * is handed to trt_lm2exp_f32, so the workspace is the larger of
+ * trt_lm2exp_bf16_workspace_bytes(R, I, J, K, pieces, splits) and
+ * trt_lm2exp_workspace_bytes(R, I, J, K, 0, splits).
  * variant: 0 = choose by shape, 1..trt_lm2exp_bf16_variant_count() force a bf16 tile shape
- * (no workspace needed).
+ * (cut only when splits > 1).
  */
 int trt_lm2exp_bf16(const float *a, const float *b, float *c,
                     int64_t R, int64_t I, int64_t J, int64_t K,
                     const int64_t sa[3], const int64_t sb[3], const int64_t sc[3],
                     int pieces, int variant, int splits,
                     void *workspace, size_t workspace_bytes, void *stream);
+size_t trt_lm2exp_bf16_workspace_bytes(int64_t R, int64_t I, int64_t J, int64_t K,
+                                       int pieces, int splits);
 int trt_lm2exp_bf16_variant_count(void);
 
 /*

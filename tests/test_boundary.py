@@ -155,6 +155,13 @@ def test_workspace_queries_are_host_only_and_follow_the_mode_rule():
     assert lib.trt_lm2exp_workspace_bytes(1, 128, 64, 128, 0, 0) == 0  # two chunks: nothing to share
     assert lib.trt_lm2exp_workspace_bytes(16, 512, 512, 512, 0, 0) == 0  # 256 tiles, 16 chunks: not worth a merge
     assert lib.trt_lm2exp_workspace_bytes(2, 100, 256, 50, 0, 4) == 4 * (4 * 2 * 100 * 50 + 4 * 2 * 50)
+    # the bf16 entry's own cut: none on a full grid or when forbidden, sized by the split count
+    assert lib.trt_lm2exp_bf16_workspace_bytes(64, 256, 256, 4096, 2, 0) == 0
+    assert lib.trt_lm2exp_bf16_workspace_bytes(1, 128, 4096, 128, 2, 1) == 0
+    assert lib.trt_lm2exp_bf16_workspace_bytes(1, 128, 4096, 128, 3, 0) > 0
+    assert lib.trt_lm2exp_bf16_workspace_bytes(2, 100, 256, 50, 2, 4) == 4 * (4 * 2 * 100 * 50 + 4 * 2 * 50)
+    assert lib.trt_lm2exp_bf16_workspace_bytes(2, 100, 20, 50, 2, 4) == 4 * (2 * 2 * 100 * 50 + 2 * 2 * 50)
+    assert lib.trt_lm2exp_bf16_workspace_bytes(2, 100, 256, 50, 5, 4) == 0  # pieces must be 2 or 3
     # the reference rule itself, triturus/lt2exp.py:535: at the benchmark configurations it is unsplit
     assert not launches_split(16, 64, 32, 32, 2048, "auto")
     assert not launches_split(64, 64, 64, 64, 4096, "auto")

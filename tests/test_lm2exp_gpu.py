@@ -302,6 +302,30 @@ def test_bf16_paths_on_ragged_shapes(dev, precision, variant, shape):
 
 
 @pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
+@pytest.mark.parametrize("splits", [2, 5, 32])
+@pytest.mark.parametrize("shape", [(3, 37, 141, 70), (1, 64, 64, 64), (2, 130, 300, 257), (2, 33, 7, 31), (1, 96, 1000, 130)])
+def test_bf16_paths_cut_over_the_contraction(dev, precision, splits, shape):
+    """Every bf16 tile with its contraction cut over workgroups (each with its own running
+    shift, merged afterwards): same gates, -inf columns and rows included, and the same
+    result on a second call (the merge adds in a fixed order)."""
+    R, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape) + splits)
+    a = torch.rand(R, I, J, generator=g)
+    b = torch.randn(R, J, K, generator=g) * 6 - 2
+    b[:, : J // 2] += 40.0  # the pieces end with different shifts
+    b[torch.rand(b.shape, generator=g) < 0.05] = NINF
+    b[:, :, 0] = NINF
+    a[:, 0] = 0.0
+    ag, bg = a.to(dev), b.to(dev)
+    for variant in range(0, N_BF16_VARIANTS + 1):
+        out = lm2exp(ag, bg, _precision=precision, _variant=variant, _splits=splits)
+        r = _check(out, a, b, **PRECISION_GATES[precision])
+        assert r["n_neg_inf"] > 0, variant
+        again = lm2exp(ag, bg, _precision=precision, _variant=variant, _splits=splits)
+        assert torch.equal(out, again), variant
+
+
+@pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
 @pytest.mark.parametrize("variant", [0, 1, 4])
 def test_bf16_paths_shift_moves_during_the_sweep(dev, precision, variant):
     """The inputs of test_shift_moves_during_the_sweep: the running shift must move (and the

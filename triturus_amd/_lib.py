@@ -58,6 +58,7 @@ SIGNATURES = {
          c_int, c_int, c_int, c_void_p, c_size_t, c_void_p],
     ),
     "trt_lt2exp_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int]),
+    "trt_lm2exp_bf16_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int, c_int]),
     "trt_lt2exp_bf16_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int]),
     "trt_lt2exp_variant_count": (c_int, []),
     "trt_matmax": (

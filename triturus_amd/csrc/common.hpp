@@ -42,9 +42,12 @@ __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) { ret
 // the chain shrinks s-fold and the CUs fill up, but the partial sums make a round trip through
 // memory and a merge kernel is launched.  Returns the split count (1 = do not split) with the
 // smallest estimate; a split must win by 20 %.  The merge constants are pessimistic on purpose
-// (2 TB/s, 5 us): splits the model rates as marginal were losses when measured.
+// (2 TB/s, 5 us): splits the model rates as marginal were losses when measured.  per_split_us
+// adds a cost per split for callers whose merge is bound by its chain of loads; must_win is the
+// fraction of the uncut estimate a cut has to stay under.
 inline int choose_splits(int64_t tiles, int64_t units, int64_t mfmas_per_unit, int64_t out_elems,
-                         int min_units_per_split, int max_splits, bool forced) {
+                         int min_units_per_split, int max_splits, bool forced, double per_split_us = 0.0,
+                         double must_win = 0.8) {
     constexpr double kCyclesPerUs = 2400.0;
     constexpr int64_t kCuCount = 256;
     const double unit_us = (double)mfmas_per_unit * 64.0 / kCyclesPerUs;
@@ -53,11 +56,12 @@ inline int choose_splits(int64_t tiles, int64_t units, int64_t mfmas_per_unit, i
         const int64_t q = ceil_div(tiles * sp, kCuCount);               // workgroups on the busiest CU
         const double eff = q >= 4 ? 0.9 : (q == 3 ? 0.8 : (q == 2 ? 0.65 : 0.45));
         const double body = (double)q * chain_us / eff;
-        const double merge_us = sp > 1 ? 5.0 + (double)(sp + 1) * (double)out_elems * 4.0 / 2.0e6 : 0.0;
+        const double merge_us =
+            sp > 1 ? 5.0 + (double)sp * per_split_us + (double)(sp + 1) * (double)out_elems * 4.0 / 2.0e6 : 0.0;
         return body + merge_us;
     };
     int best = 1;
-    double best_us = forced ? 1e300 : 0.8 * estimate(1);
+    double best_us = forced ? 1e300 : must_win * estimate(1);
     for (int sp = 2; sp <= max_splits && (int64_t)sp * min_units_per_split <= units; ++sp) {
         const double us = estimate(sp);
         if (us < best_us) {

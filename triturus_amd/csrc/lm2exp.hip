@@ -30,6 +30,7 @@
 // triturus/lm2exp.py:143, which can overflow exp(0 - m); not reproduced).
 
 #include "common.hpp"
+#include "lm2exp_merge.hpp"
 
 namespace trt {
 
@@ -434,33 +435,6 @@ static int colmax_splits(int64_t R, int64_t J, int64_t K) {
     return splits < 1 ? 1 : (int)splits;
 }
 
-// Merge of a split contraction: every split s holds sum_s (relative to its own shift m_s);
-// c = M + log(sum_s sum_s * exp(m_s - M)) with M = max_s m_s, in split order (deterministic).
-__global__ __launch_bounds__(256) void lm2exp_merge_kernel(const float *__restrict__ part,
-                                                           const float *__restrict__ shift, float *__restrict__ c,
-                                                           int R, int I, int K, int splits, int64_t sc0,
-                                                           int64_t sc1) {
-    const int64_t total = (int64_t)R * I * K;
-    const int64_t rk = (int64_t)R * K;
-    const int64_t stride = (int64_t)gridDim.x * 256;
-    for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
-        const int k = (int)(e % K);
-        const int64_t ri = e / K;
-        const int i = (int)(ri % I);
-        const int r = (int)(ri / I);
-        const float *sh = shift + (int64_t)r * K + k;
-        float M = sh[0];
-        for (int sp = 1; sp < splits; ++sp) M = max_nan(M, sh[sp * rk]);
-        float sum = 0.f;
-        for (int sp = 0; sp < splits; ++sp) {
-            // exp(m_s - M) in two halves: the factor alone may flush where the product does not
-            const float f = exp_shifted(0.5f * (sh[sp * rk] - M));
-            sum += part[(int64_t)sp * total + e] * f * f;
-        }
-        c[(int64_t)r * sc0 + (int64_t)i * sc1 + k] = log_plus(sum, M);
-    }
-}
-
 // ------------------------------------------------------------------ host
 struct Lm2Variant {
     int rt, ct, wm, wn, nq;
@@ -706,11 +680,7 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         default: st = launch_v<3, 1, 1, 4, 4, kOnline>(args, vec, s); break;
     }
     if (st != 0 || pl.splits <= 1) return st;
-    const int64_t total = R * I * K;
-    int64_t blocks = ceil_div(total, 256);
-    if (blocks > 8192) blocks = 8192;
-    hipLaunchKernelGGL(lm2exp_merge_kernel, dim3((unsigned)blocks), dim3(256), 0, s, args.part, args.shift, c,
-                       (int)R, (int)I, (int)K, pl.splits, sc[0], sc[1]);
+    launch_lm2exp_merge(args.part, args.shift, c, R, I, K, pl.splits, sc[0], sc[1], s);
     return (int)hipGetLastError();
 }
 

@@ -19,6 +19,7 @@
 #include <type_traits>
 
 #include "bf16_split.hpp"
+#include "lm2exp_merge.hpp"
 
 namespace trt {
 
@@ -26,9 +27,11 @@ namespace trt {
 struct Lm2BfArgs {
     const float *a, *b;
     float *c;
+    float *part;   // splits > 1: [splits][R][I][K] partial sums
+    float *shift;  // splits > 1: [splits][R][K] the shift each partial sum is relative to
     int R, I, J, K;
     int64_t sa0, sa1, sb0, sb1, sc0, sc1;
-    int i_tiles, n_tiles;
+    int i_tiles, n_tiles, splits, chunks_per_split;
     int64_t total_wgs, padded_wgs;
 };
 
@@ -60,6 +63,8 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
     // rows of b at the same time, so the panel comes from HBM once and from L2 afterwards.
     int64_t rest = L / p.i_tiles;
     const int itile = __builtin_amdgcn_readfirstlane((int)(L % p.i_tiles));
+    const int split = __builtin_amdgcn_readfirstlane((int)(rest % p.splits));
+    rest /= p.splits;
     const int nt = __builtin_amdgcn_readfirstlane((int)(rest % p.n_tiles));
     const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.n_tiles));
 
@@ -216,11 +221,14 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
             exp_and_split(std::false_type{});
     };
 
+    // chunks [jc0, jc1) of this workgroup: all of them unless the contraction is cut over J
     const int n_jc = (p.J + JC - 1) / JC;
+    const int jc0 = split * p.chunks_per_split;
+    const int jc1 = (jc0 + p.chunks_per_split < n_jc) ? jc0 + p.chunks_per_split : n_jc;
 
     // ---- prologue: first chunk
-    load_tile(0);
-    load_b(0);
+    load_tile(jc0);
+    load_b(jc0);
     store_tile(0);
     mref = PLAIN ? 0.f : clamp_shift(chunk_max());
     shift_and_exp();
@@ -254,7 +262,7 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
     };
 
     int cur = 0;
-    for (int jc = 0; jc + 1 < n_jc; ++jc) {
+    for (int jc = jc0; jc + 1 < jc1; ++jc) {
         load_tile(jc + 1);
         load_b(jc + 1);
         __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block
@@ -269,6 +277,18 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
     // ---- epilogue: c = m + log(acc); register v of lane (h, m) holds row 8*(v/4) + 4*h +
     // v%4, column m of its 32 x 32 tile.  Rows past I fall outside the buffer extent.
     if (ncol >= p.K) return;
+    if (p.splits > 1) {  // wave-uniform: raw sums and their shift go to the workspace, the merge finishes
+        float *part = p.part + (((int64_t)split * p.R + r) * p.I) * (int64_t)p.K;
+        if (itile == 0 && h == 0) p.shift[((int64_t)split * p.R + r) * p.K + ncol] = mref;
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const int row = i0 + 32 * rt + 8 * (v / 4) + 4 * h + (v % 4);
+                if (row < p.I) part[(int64_t)row * p.K + ncol] = acc[rt][v];
+            }
+        return;
+    }
     const int crows = p.I - i0;
     const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)i0 * p.sc1,
                                                     (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4));
@@ -317,6 +337,44 @@ using namespace trt;
 
 extern "C" int trt_lm2exp_bf16_variant_count(void) { return kNumLmBfVariants; }
 
+// Cut of the contraction for grids that do not fill the chip (batch-1 squares and the like):
+// `splits` workgroups share one 32 x 128 output tile, each sweeping its own range of 32-wide
+// j-chunks with its own running shift; raw sums and shifts go to the workspace and
+// lm2exp_merge_kernel finishes.  Returns 1 when the call is not cut.  requested: 0 = by the
+// cost model, 1 = never, > 1 = that many (capped by the number of chunks).
+static int lm_bf16_cut(int64_t R, int64_t I, int64_t J, int64_t K, int pieces, int requested) {
+    if (requested == 1) return 1;
+    const int64_t n_jc = ceil_div(J, 32);
+    if (n_jc < 2) return 1;
+    int64_t sp;
+    if (requested > 1) {
+        sp = requested > 32 ? 32 : requested;
+        if (sp > n_jc) sp = n_jc;
+    } else {
+        const int64_t tiles = R * ceil_div(I, 32) * ceil_div(K, 128);
+        if (tiles >= 1024) return 1;
+        // Constants fitted to 150 random shapes of fewer than 1500 tiles timed with every cut of
+        // 2..16 on 32- and 64-row tiles: a chunk costs a lone workgroup 0.9 us with two pieces
+        // or three (latency, not MFMAs), 0.3 us per split for the merge of a small output (bound
+        // by its chain of loads), and a cut that the model rates 10 % ahead is taken.  Against
+        // the best measured choice this loses 1.7 %, never cutting 8 % (two pieces) / 5 %.
+        sp = choose_splits(tiles, n_jc, 15, R * I * K, 4, 32, false, 0.3, 0.9);
+    }
+    const int64_t cps = ceil_div(n_jc, sp);
+    return (int)ceil_div(n_jc, cps);  // no split is left without a chunk
+}
+
+extern "C" size_t trt_lm2exp_bf16_workspace_bytes(int64_t R, int64_t I, int64_t J, int64_t K, int pieces,
+                                                  int splits) {
+    if (R <= 0 || I <= 0 || J <= 0 || K <= 0 || splits < 0 || (pieces != 2 && pieces != 3)) return 0;
+    int64_t sp = lm_bf16_cut(R, I, J, K, pieces, splits);
+    if (splits > 1) {  // a forced tile may sweep chunks of 16: room for what any tile would use
+        sp = splits > 32 ? 32 : splits;
+        if (sp > ceil_div(J, 16)) sp = ceil_div(J, 16);
+    }
+    return sp > 1 ? (size_t)sp * (size_t)(R * I * K + R * K) * sizeof(float) : 0;
+}
+
 extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
                                const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], int pieces,
                                int variant, int splits, void *workspace, size_t workspace_bytes, void *stream) {
@@ -336,10 +394,11 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     // Tile and hand-over rules, fitted to 223 random shapes (R 1..256, I, J 16..1024, K 64..8192)
     // timed with every tile and on the fp32 path; against the best of those the rules below lose
     // 5.6 % (two pieces) / 4.3 % (three) on average, the previous ones 19 / 11 %.
-    //  - Grids of fewer than 128 (three pieces: 192) 32-row tiles are latency bound, not matrix
-    //    bound, and a contraction of at most 16 (32) is bound by writing c: there the fp32 path
-    //    (smaller tiles, contraction cut over J) is as fast or faster and takes the call, as it
-    //    does whenever the caller asks for a cut.
+    //  - Grids of fewer than 1024 32-row tiles over a long contraction are cut over J when the
+    //    cost model (lm_bf16_cut) says so, as far as the workspace allows.
+    //  - Uncut grids of fewer than 128 (three pieces: 192) 32-row tiles are latency bound, not
+    //    matrix bound, and a contraction of at most 16 (32) is bound by writing c: there the fp32
+    //    path (smaller tiles, its own cut over J) is as fast or faster and takes the call.
     //  - j-chunks of 32 (three workgroups fit a CU; chunks of 64 measured 0-17 % behind), except
     //    with two pieces on 64- and 32-row tiles over a contraction of 512 or more (chunks of 64).
     //  - Rows: the candidate (128, 96, 64 or 32 rows; at least 1.5, 1.5, 1, 0 workgroups per CU)
@@ -348,12 +407,28 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     //    (0.95) for 128 rows; on a shorter one 1 and 1.05.  The 96-row tile (three wavefronts
     //    per SIMD) takes I = 96, 160, 192, 288 and the like: 10-24 % ahead there.
     int v;
+    int cut = 1;
     if (variant >= 1) {
         v = variant - 1;
+        if (splits > 1) {  // a forced tile with a forced cut (tests and tuning)
+            const int64_t jc = 16 * kLmBfVariants[v].ks;
+            int64_t sp = splits > 32 ? 32 : splits;
+            const int64_t n_jc = ceil_div(J, jc);
+            if (sp > n_jc) sp = n_jc;
+            cut = (int)ceil_div(n_jc, ceil_div(n_jc, sp));
+            const int64_t fit = workspace ? (int64_t)(workspace_bytes / sizeof(float)) / (R * I * K + R * K) : 0;
+            if (cut > 1 && cut > fit) return TRT_E_WORKSPACE;
+        }
     } else {
         const int64_t ct = ceil_div(K, 128);
         const int64_t n32 = R * ceil_div(I, 32) * ct;
-        if (splits > 1 || n32 < (pieces == 2 ? 128 : 192) || J <= (pieces == 2 ? 16 : 32))
+        if (J > (pieces == 2 ? 16 : 32)) {
+            cut = lm_bf16_cut(R, I, J, K, pieces, splits);
+            const int64_t per_split = R * I * K + R * K;
+            const int64_t fit = workspace ? (int64_t)(workspace_bytes / sizeof(float)) / per_split : 0;
+            if (cut > fit) cut = fit >= 2 ? lm_bf16_cut(R, I, J, K, pieces, (int)fit) : 1;
+        }
+        if (cut == 1 && (splits > 1 || n32 < (pieces == 2 ? 128 : 192) || J <= (pieces == 2 ? 16 : 32)))
             return trt_lm2exp_f32(a, b, c, R, I, J, K, sa, sb, sc, 0, splits, workspace, workspace_bytes, stream);
         int best_rt = 1;
         int64_t best_cost = ceil_div(I, 32) * 120;
@@ -373,6 +448,8 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
         // two pieces are bound by the vector work on the B operand: 256 rows (each exp feeds 24
         // MFMAs) when I fills them exactly and two workgroups per CU remain (6-25 % at I = 256, 512)
         if (pieces == 2 && best_rt == 4 && I % 256 == 0 && J >= 256 && R * (I / 256) * ct >= 512) v = 7;  // {8,2}
+        // the cut is made on 32-row tiles, or on 64-row ones where those still number 64
+        if (cut > 1) v = (I > 32 && R * ceil_div(I, 64) * ct >= 64) ? 3 : 5;  // {2,2}, {1,2}
     }
     const LmBfVariant &vr = kLmBfVariants[v];
 
@@ -384,23 +461,32 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     args.sc0 = sc[0]; args.sc1 = sc[1];
     args.i_tiles = (int)ceil_div(I, 32 * vr.rt);
     args.n_tiles = (int)ceil_div(K, 128);
-    args.total_wgs = (int64_t)R * args.i_tiles * args.n_tiles;
+    const int64_t n_jc = ceil_div(J, 16 * vr.ks);
+    args.splits = cut;
+    args.chunks_per_split = (int)ceil_div(n_jc, cut);
+    args.part = cut > 1 ? static_cast<float *>(workspace) : nullptr;
+    args.shift = cut > 1 ? args.part + (int64_t)cut * R * I * K : nullptr;
+    args.total_wgs = (int64_t)R * args.i_tiles * args.n_tiles * cut;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const bool vec = (J % 4 == 0) && (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
+    int status;
     switch (v) {
-        case 0: return launch_lm_bf<4, 4>(args, pieces, vec, s);
-        case 1: return launch_lm_bf<4, 2>(args, pieces, vec, s);
-        case 2: return launch_lm_bf<2, 4>(args, pieces, vec, s);
-        case 3: return launch_lm_bf<2, 2>(args, pieces, vec, s);
-        case 4: return launch_lm_bf<1, 4>(args, pieces, vec, s);
-        case 5: return launch_lm_bf<1, 2>(args, pieces, vec, s);
-        case 6: return launch_lm_bf<8, 1>(args, pieces, vec, s);
-        case 7: return launch_lm_bf<8, 2>(args, pieces, vec, s);
-        default: return launch_lm_bf<3, 2>(args, pieces, vec, s);
+        case 0: status = launch_lm_bf<4, 4>(args, pieces, vec, s); break;
+        case 1: status = launch_lm_bf<4, 2>(args, pieces, vec, s); break;
+        case 2: status = launch_lm_bf<2, 4>(args, pieces, vec, s); break;
+        case 3: status = launch_lm_bf<2, 2>(args, pieces, vec, s); break;
+        case 4: status = launch_lm_bf<1, 4>(args, pieces, vec, s); break;
+        case 5: status = launch_lm_bf<1, 2>(args, pieces, vec, s); break;
+        case 6: status = launch_lm_bf<8, 1>(args, pieces, vec, s); break;
+        case 7: status = launch_lm_bf<8, 2>(args, pieces, vec, s); break;
+        default: status = launch_lm_bf<3, 2>(args, pieces, vec, s); break;
     }
+    if (status != 0 || cut == 1) return status;
+    launch_lm2exp_merge(args.part, args.shift, c, R, I, K, cut, sc[0], sc[1], s);
+    return (int)hipGetLastError();
 }
 
 // c = a b for row-major fp32 matrices on the bf16 matrix pipe (operands cut into `pieces`
@@ -436,6 +522,9 @@ extern "C" int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, 
     args.sc0 = m * n; args.sc1 = n;
     args.i_tiles = (int)ceil_div(m, 32 * rt);
     args.n_tiles = (int)ct;
+    args.part = nullptr; args.shift = nullptr;
+    args.splits = 1;
+    args.chunks_per_split = (int)ceil_div(k, 16);  // at least every chunk
     args.total_wgs = (int64_t)args.i_tiles * args.n_tiles;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
     const bool vec = (k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);

@@ -19,7 +19,7 @@ from triturus_amd import _lib, autotune
 from triturus_amd.utils import MATRIX_PRECISIONS, matrix_precision
 
 
-_ws_bytes: dict = {}  # (R, I, J, K, variant, splits) -> workspace bytes, as reported by the library
+_ws_bytes: dict = {}  # (R, I, J, K, variant, splits, pieces) -> workspace bytes, as reported by the library
 
 
 def _unit_inner(t: torch.Tensor) -> torch.Tensor:
@@ -70,10 +70,14 @@ def lm2exp(
         _splits = 0
     # small grids with a long contraction are cut over J; the partial sums need a workspace
     fp32_variant = _variant if _precision == "fp32" else 0
-    key = (R, I, J, K, fp32_variant, _splits)
+    pieces = 0 if _precision == "fp32" else _PIECES[_precision]
+    key = (R, I, J, K, fp32_variant, _splits, pieces)
     ws_bytes = _ws_bytes.get(key)
     if ws_bytes is None:
-        ws_bytes = _ws_bytes[key] = lib.trt_lm2exp_workspace_bytes(R, I, J, K, fp32_variant, _splits)
+        ws_bytes = lib.trt_lm2exp_workspace_bytes(R, I, J, K, fp32_variant, _splits)
+        if pieces:  # the bf16 entry may cut a small grid itself
+            ws_bytes = max(ws_bytes, lib.trt_lm2exp_bf16_workspace_bytes(R, I, J, K, pieces, _splits))
+        _ws_bytes[key] = ws_bytes
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
     ws_ptr = ws.data_ptr() if ws_bytes else None
     with _lib.on_device(a.device):
@@ -84,8 +88,8 @@ def lm2exp(
                 _variant, _splits, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
             )
         else:
-            # bf16 matrix pipe; the library hands grids that are too small for it back to the
-            # fp32 kernels (which may cut the contraction over J: hence the workspace)
+            # bf16 matrix pipe; a grid too small for it has its contraction cut over J or goes
+            # back to the fp32 kernels (which may cut it as well: hence the workspace)
             status = lib.trt_lm2exp_bf16(
                 a.data_ptr(), b.data_ptr(), c.data_ptr(),
                 R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
