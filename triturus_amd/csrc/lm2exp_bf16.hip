@@ -428,7 +428,11 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
             const int64_t fit = workspace ? (int64_t)(workspace_bytes / sizeof(float)) / per_split : 0;
             if (cut > fit) cut = fit >= 2 ? lm_bf16_cut(R, I, J, K, pieces, (int)fit) : 1;
         }
-        if (cut == 1 && (splits > 1 || n32 < (pieces == 2 ? 128 : 192) || J <= (pieces == 2 ? 16 : 32)))
+        const bool small = n32 < (pieces == 2 ? 128 : 192);
+        // a contraction of 224..416 is too short for a cut here and long enough for the fp32
+        // path to cut it (two launches): one launch of 32-row bf16 tiles is 6-16 % ahead
+        const bool one_launch = small && splits == 0 && J >= 224 && J <= 416;
+        if (cut == 1 && !one_launch && (splits > 1 || small || J <= (pieces == 2 ? 16 : 32)))
             return trt_lm2exp_f32(a, b, c, R, I, J, K, sa, sb, sc, 0, splits, workspace, workspace_bytes, stream);
         int best_rt = 1;
         int64_t best_cost = ceil_div(I, 32) * 120;
