@@ -429,9 +429,11 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
             if (cut > fit) cut = fit >= 2 ? lm_bf16_cut(R, I, J, K, pieces, (int)fit) : 1;
         }
         const bool small = n32 < (pieces == 2 ? 128 : 192);
-        // a contraction of 224..416 is too short for a cut here and long enough for the fp32
-        // path to cut it (two launches): one launch of 32-row bf16 tiles is 6-16 % ahead
-        const bool one_launch = small && splits == 0 && J >= 224 && J <= 416;
+        // where the fp32 path would not cut a contraction of 192..416 either, one launch of
+        // 32-row bf16 tiles is 4-15 % ahead of its one launch; where it would, its cut wins on
+        // operands that come from HBM (by 4-6 us) and loses on cached ones (by 3 us): left to it
+        const bool one_launch = small && splits == 0 && J >= 192 && J <= 416 &&
+                                trt_lm2exp_workspace_bytes(R, I, J, K, 0, 0) == 0;
         if (cut == 1 && !one_launch && (splits > 1 || small || J <= (pieces == 2 ? 16 : 32)))
             return trt_lm2exp_f32(a, b, c, R, I, J, K, sa, sb, sc, 0, splits, workspace, workspace_bytes, stream);
         int best_rt = 1;
