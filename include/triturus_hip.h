@@ -150,6 +150,8 @@ int trt_lm2exp_bf16(const float *a, const float *b, float *c,
                     const int64_t sa[3], const int64_t sb[3], const int64_t sc[3],
                     int pieces, int variant, int splits,
                     void *workspace, size_t workspace_bytes, void *stream);
+/* Workspace for trt_lm2exp_bf16's own cut over J: the larger of this and
+ * trt_lm2exp_workspace_bytes(R, I, J, K, 0, splits) serves every path the call may take. */
 size_t trt_lm2exp_bf16_workspace_bytes(int64_t R, int64_t I, int64_t J, int64_t K,
                                        int pieces, int splits);
 int trt_lm2exp_bf16_variant_count(void);
