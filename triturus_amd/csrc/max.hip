@@ -523,6 +523,11 @@ static MatPlan colmax_plan(int64_t m, int64_t n, int cn) {
     return {splits, rchunk};
 }
 
+// Partial column maxima are combined by the same kernel; more than 128 rows of them (tall,
+// narrow matrices: few column blocks, so many row splits) go through an intermediate level of
+// 64-row pieces instead of one workgroup walking them all.
+static int64_t combine_splits(int64_t rows) { return rows > 128 ? ceil_div(rows, (int64_t)64) : 1; }
+
 template <int DT>
 static bool vec_ok(const void *p, int64_t ld) {
     constexpr int VN = 16 / (int)sizeof(typename Elem<DT>::T);
@@ -563,10 +568,12 @@ static size_t matmax_ws(int64_t m, int64_t n, int axis) {
         MatPlan p = rowmax_plan(m, n, VN);
         return p.splits > 1 ? (size_t)(m * p.splits) * sizeof(T) : 0;
     }
-    // worst case over the vector / scalar column paths
+    // worst case over the vector / scalar column paths, plus the intermediate level
     MatPlan pv = colmax_plan(m, n, VN), ps = colmax_plan(m, n, 1);
     int64_t s = pv.splits > ps.splits ? pv.splits : ps.splits;
-    return s > 1 ? (size_t)(s * n) * sizeof(T) : 0;
+    if (s <= 1) return 0;
+    const int64_t s2 = combine_splits(s);
+    return (size_t)((s + (s2 > 1 ? s2 : 0)) * n) * sizeof(T);
 }
 
 template <int DT>
@@ -597,8 +604,17 @@ static int matmax_launch(const void *xv, void *yv, int64_t m, int64_t n, int axi
             colmax_launch<DT>(x, n, m, n, vec, p, y, n, stream);
         } else {
             colmax_launch<DT>(x, n, m, n, vec, p, part, n, stream);
-            MatPlan p2{1, p.splits};
-            colmax_launch<DT>(part, n, p.splits, n, vec_ok<DT>(part, n), p2, y, n, stream);
+            int64_t rows = p.splits;
+            const int64_t s2 = combine_splits(rows);
+            if (s2 > 1) {  // intermediate level behind the first partials (sized by matmax_ws)
+                MatPlan pc{s2, 64};
+                T *part2 = part + rows * n;
+                colmax_launch<DT>(part, n, rows, n, vec_ok<DT>(part, n), pc, part2, n, stream);
+                part = part2;
+                rows = s2;
+            }
+            MatPlan p2{1, rows};
+            colmax_launch<DT>(part, n, rows, n, vec_ok<DT>(part, n), p2, y, n, stream);
         }
     }
     return (int)hipGetLastError();
