@@ -426,14 +426,16 @@ __global__ __launch_bounds__(256) void lm2exp_colmax_kernel(const float *__restr
 }
 
 // Rows per split of the batched column maxima: enough workgroups for 256 CUs (>= 1024), at
-// least 64 rows each, at most 64 splits.
+// least 64 rows each, at most 1024 splits.  More than 128 partials per column (few columns
+// under a very long axis) are combined in two levels, 64 at a time first.
 static int colmax_splits(int64_t R, int64_t J, int64_t K) {
     const int64_t base = R * ceil_div(K, 256);
     int64_t splits = base >= 1024 ? 1 : ceil_div(1024, base);
     if (splits > J / 64) splits = J / 64;
-    if (splits > 64) splits = 64;
+    if (splits > 1024) splits = 1024;
     return splits < 1 ? 1 : (int)splits;
 }
+static int colmax_mid_splits(int splits) { return splits > 128 ? (splits + 63) / 64 : 1; }
 
 // ------------------------------------------------------------------ host
 struct Lm2Variant {
@@ -692,7 +694,8 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
 extern "C" size_t trt_colmax_batched_workspace_bytes(int64_t R, int64_t J, int64_t K) {
     if (R <= 0 || J <= 0 || K <= 0) return 0;
     const int splits = colmax_splits(R, J, K);
-    return splits > 1 ? (size_t)splits * R * K * sizeof(float) : 0;
+    const int mid = colmax_mid_splits(splits);
+    return splits > 1 ? (size_t)(splits + (mid > 1 ? mid : 0)) * R * K * sizeof(float) : 0;
 }
 
 extern "C" int trt_colmax_batched_f32(const float *b, float *m, int64_t R, int64_t J, int64_t K,
@@ -710,12 +713,21 @@ extern "C" int trt_colmax_batched_f32(const float *b, float *m, int64_t R, int64
     if (blocks >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (splits > 1) {
-        if (!workspace || workspace_bytes < (size_t)splits * R * K * sizeof(float)) return TRT_E_WORKSPACE;
+        const int mid = colmax_mid_splits(splits);
+        if (!workspace || workspace_bytes < (size_t)(splits + (mid > 1 ? mid : 0)) * R * K * sizeof(float))
+            return TRT_E_WORKSPACE;
         float *part = static_cast<float *>(workspace);
         hipLaunchKernelGGL(lm2exp_colmax_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, b, part, (int)R, (int)J,
                            (int)K, sb[0], sb[1], chunk, splits);
         // reduce over the splits: the partials are an R x splits x K tensor with strides (K, R*K, 1)
         const unsigned blocks2 = (unsigned)(R * ceil_div(K, 256));
+        if (mid > 1) {  // 64 partials at a time first
+            float *part2 = part + (int64_t)splits * R * K;
+            hipLaunchKernelGGL(lm2exp_colmax_kernel<false>, dim3(blocks2 * (unsigned)mid), dim3(256), 0, s, part, part2,
+                               (int)R, splits, (int)K, K, R * K, 64, mid);
+            part = part2;
+            splits = mid;
+        }
         if (clamp)
             hipLaunchKernelGGL(lm2exp_colmax_kernel<true>, dim3(blocks2), dim3(256), 0, s, part, m, (int)R, splits, (int)K,
                                K, R * K, splits, 1);
