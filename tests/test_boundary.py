@@ -85,7 +85,7 @@ def test_c_abi_argument_errors_are_statuses():
     # lt2exp on the bf16 matrix pipe: pieces must be 2 or 3, variant 0..4
     btail = (0, 0, null, 0, null)  # mode, variant, workspace, bytes, stream
     assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 4, *btail) == -1
-    assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 2, 0, 9, null, 0, null) == -1
+    assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 2, 0, 17, null, 0, null) == -1
     assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 2, 5, 0, null, 0, null) == -1
     assert lib.trt_lt2exp_bf16(null, one, one, one, *args, 2, *btail) == -1
     assert lib.trt_lt2exp_bf16(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, 2), ok, ok, ok, 2, *btail) == -2

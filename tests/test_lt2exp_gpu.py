@@ -20,8 +20,8 @@ from triturus_amd import _lib, workloads
 pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
-N_VARIANTS = 8
-N_BF16_VARIANTS = 8  # 1..4 tiles, 5..8 the same tiles with the contraction cut over workgroups
+N_VARIANTS = 14
+N_BF16_VARIANTS = 16  # 1..4, 9..12 tiles; 5..8, 13..16 the same tiles with the contraction cut over workgroups
 # Accuracy gates of the split-bf16 paths against the float64 oracle.  Two pieces (3 MFMAs per
 # product) carry 16 significand bits: looser than fp32, ten times tighter than the rtol 5e-4
 # the reference allows its TF32 mode (tests/lt2exp.py:38).  Three pieces (6 MFMAs) carry 24
@@ -68,7 +68,8 @@ def test_golden(dev, name, mode):
 
 @pytest.mark.parametrize("variant", range(1, N_VARIANTS + 1))
 @pytest.mark.parametrize("mode", ["unsplit", "split"])
-@pytest.mark.parametrize("shape", [(2, 35, 9, 13, 45), (1, 70, 20, 33, 300), (2, 16, 5, 72, 64), (1, 33, 3, 3, 31)])
+@pytest.mark.parametrize("shape", [(2, 35, 9, 13, 45), (1, 70, 20, 33, 300), (2, 16, 5, 72, 64), (1, 33, 3, 3, 31),
+                                   (2, 40, 6, 48, 100), (1, 33, 5, 24, 70), (1, 65, 3, 16, 64), (1, 20, 4, 100, 130)])
 def test_every_tile_variant_on_ragged_shapes(dev, variant, mode, shape):
     assert _lib.load().trt_lt2exp_variant_count() == N_VARIANTS
     R, S, I, J, K = shape
@@ -262,7 +263,7 @@ def test_capturable_in_a_hip_graph(dev):
 @pytest.mark.parametrize("variant", range(0, N_BF16_VARIANTS + 1))
 @pytest.mark.parametrize(
     "shape", [(3, 75, 50, 50, 100), (2, 35, 9, 13, 45), (1, 70, 20, 33, 300), (2, 16, 5, 72, 64), (1, 33, 3, 3, 31),
-              (2, 64, 64, 64, 256), (1, 1, 1, 1, 1), (2, 130, 4, 128, 129)])
+              (2, 64, 64, 64, 256), (1, 1, 1, 1, 1), (2, 130, 4, 128, 129), (2, 40, 6, 48, 100), (1, 65, 3, 16, 64)])
 def test_bf16_paths_on_ragged_shapes(dev, precision, variant, shape):
     R, S, I, J, K = shape
     g = torch.Generator().manual_seed(sum(shape) + variant)
@@ -272,12 +273,13 @@ def test_bf16_paths_on_ragged_shapes(dev, precision, variant, shape):
     a[torch.rand(a.shape, generator=g) < 0.05] = NINF
     b[:, :, 0] = NINF  # an all -inf column: -inf out, not NaN
     w[:, 0] = 0.0  # a zero row of weights: -inf out
-    # variants 5..8 cut the contraction as far as the workspace allows: mode "split" sizes it
-    mode = "split" if variant >= 5 else "auto"
+    # variants 5..8 and 13..16 cut the contraction as far as the workspace allows: mode "split" sizes it
+    cut = (variant - 1) % 8 >= 4 if variant else False
+    mode = "split" if cut else "auto"
     out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision, _variant=variant)
     r = _check(out, w, a, b, **PRECISION_GATES[precision])
     assert r["n_neg_inf"] > 0
-    if variant >= 5:  # the cut is deterministic: same bits on a second call; and close to the uncut tile
+    if cut:  # the cut is deterministic: same bits on a second call; and close to the uncut tile
         again = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision, _variant=variant)
         assert torch.equal(out, again)
         uncut = lt2exp(w.to(dev), a.to(dev), b.to(dev), _precision=precision, _variant=variant - 4)

@@ -42,11 +42,17 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     constexpr int JC = 8 * NQ;            // j per chunk
     constexpr int LDW = JC + 4;           // padded LDS row (floats): conflict-free 16-byte reads
     constexpr int F4_PER_ROW = JC / 4;
-    constexpr int SLOTS = TS * F4_PER_ROW / NT;  // float4 tile slots per thread
-    static_assert(TS * F4_PER_ROW % NT == 0, "tile must divide over the threads");
+    constexpr int F4_TILE = TS * F4_PER_ROW;              // 16-byte pieces of a w tile
+    constexpr int SLOTS = (F4_TILE + NT - 1) / NT;        // of which a thread stages this many
+    // REGULAR: a thread keeps its column and steps whole rows from slot to slot; otherwise
+    // (chunks of 24 or 48, or tiles smaller than the workgroup) pieces are dealt out linearly
+    // and the last slot is only partly filled.
+    constexpr bool REGULAR = (NT % F4_PER_ROW == 0) && (F4_TILE % NT == 0);
     constexpr int TN = 32 * CT * NWAVES;
 
-    __shared__ __attribute__((aligned(16))) float wt[2][TS * LDW];
+    // (a thread whose last slot lies past the tile stages into a private 16 bytes behind it:
+    // the steady state carries no predicates)
+    __shared__ __attribute__((aligned(16))) float wt[2][TS * LDW + (REGULAR ? 0 : 4 * NT)];
 
     const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
     if (L >= p.total_wgs) return;
@@ -118,9 +124,23 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     // the last valid row, so rows past S come back as zeros.  Only a ragged j-chunk
     // (J not a multiple of the chunk) or unaligned w takes the masked path.
     floatx4 stage[SLOTS];
-    constexpr int ROWS_PER_SLOT = NT / F4_PER_ROW;
-    const int trow = tid / F4_PER_ROW;  // tile row of this thread's first slot
-    const int tc4 = tid % F4_PER_ROW;
+    int srow[SLOTS], sc4[SLOTS];  // tile row and 16-byte column of each slot
+    int lds_off[SLOTS];           // where the slot goes in the LDS tile (floats)
+    bool sval[SLOTS];
+#pragma unroll
+    for (int sidx = 0; sidx < SLOTS; ++sidx) {
+        if (REGULAR) {
+            srow[sidx] = tid / F4_PER_ROW + sidx * (NT / F4_PER_ROW);
+            sc4[sidx] = tid % F4_PER_ROW;
+            sval[sidx] = true;
+        } else {
+            const int f = tid + sidx * NT;
+            srow[sidx] = f / F4_PER_ROW;
+            sc4[sidx] = f % F4_PER_ROW;
+            sval[sidx] = f < F4_TILE;
+        }
+        lds_off[sidx] = sval[sidx] ? srow[sidx] * LDW + 4 * sc4[sidx] : TS * LDW + 4 * tid;
+    }
     const int wrows = (p.S - s0) < TS ? (p.S - s0) : TS;
     const float *wtile0 = wr + (int64_t)s0 * p.sw1;
     const __amdgpu_buffer_rsrc_t w_rsrc =
@@ -128,21 +148,32 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     uint32_t woff[SLOTS];
 #pragma unroll
     for (int sidx = 0; sidx < SLOTS; ++sidx)
-        woff[sidx] = ((uint32_t)(trow + sidx * ROWS_PER_SLOT) * (uint32_t)p.sw1 + 4u * tc4) * 4u;
+        woff[sidx] = ((uint32_t)srow[sidx] * (uint32_t)p.sw1 + 4u * (uint32_t)sc4[sidx]) * 4u;
+    // (a slot past the tile loads some valid or out-of-extent address: the value is never used)
     auto load_tile = [&](int i, int jc) {
         const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
         if (full) {
             const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) stage[sidx] = buf_load_f32x4(w_rsrc, woff[sidx], soff);
-        } else {
-            const int j = jc * JC + 4 * tc4;
+        } else if (VEC) {
+            // ragged last chunk of aligned rows (J is a multiple of 4): a 16-byte piece is whole
+            // or lies past J, where the next i begins: zeros instead
+            const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) {
-                const int row = trow + sidx * ROWS_PER_SLOT;
+                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                const floatx4 v = buf_load_f32x4(w_rsrc, woff[sidx], soff);
+                stage[sidx] = (jc * JC + 4 * sc4[sidx] < p.J) ? v : zero;
+            }
+        } else {
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx) {
+                const int row = srow[sidx];
+                const int j = jc * JC + 4 * sc4[sidx];
                 const float *src = wtile0 + (int64_t)row * p.sw1 + (int64_t)i * p.J + j;
                 floatx4 v = {0.f, 0.f, 0.f, 0.f};
-                if (row < wrows) {
+                if (sval[sidx] && row < wrows) {
                     if (j + 0 < p.J) v[0] = src[0];
                     if (j + 1 < p.J) v[1] = src[1];
                     if (j + 2 < p.J) v[2] = src[2];
@@ -153,10 +184,8 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
         }
     };
     auto store_tile = [&](int buf) {
-        float *dst = &wt[buf][trow * LDW + 4 * tc4];
 #pragma unroll
-        for (int sidx = 0; sidx < SLOTS; ++sidx)
-            *reinterpret_cast<floatx4 *>(&dst[sidx * ROWS_PER_SLOT * LDW]) = stage[sidx];
+        for (int sidx = 0; sidx < SLOTS; ++sidx) *reinterpret_cast<floatx4 *>(&wt[buf][lds_off[sidx]]) = stage[sidx];
     };
 
     // a rows for the scalar factor exp(a[i,n] - ma[n]): same addressing scheme
@@ -297,6 +326,12 @@ static const Lt2Variant kVariants[] = {
     {2, 1, 4},
     {1, 1, 8},  // 32 x 128 tile
     {1, 1, 4},
+    {1, 1, 2},  // 9..14: j-chunks of 16, 24 and 48 for contractions that chunks of 32 fit badly
+    {1, 1, 3},
+    {1, 1, 6},
+    {2, 1, 2},
+    {2, 1, 3},
+    {2, 1, 6},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLt2Waves = 4;
@@ -321,8 +356,24 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
         const int64_t n64 = R * ceil_div(S, 64) * ceil_div(K, 128);
         if (same_padding && I * J >= 4096 && n64 >= 256) rt = 2;
     }
+    // j-chunk: the one that pads J least.  Per padded j the chunks cost the same within a few
+    // per cent (measured at S = I = 64, K = 4096, R = 64: 15.3 us per j with chunks of 32 or 48,
+    // 15.5-16.5 with 16, 15.5-16.1 with 24), so J = 16, 24, 40, 48, 72 run 1.3-2.2x faster on
+    // chunks that fit than on chunks of 32 (J = 48: 1059 -> 735 us), also because a last chunk
+    // that is only partly filled takes the masked loads.  Ties go to chunks of 32.
+    int nq = 4;
+    int64_t best = ceil_div(J, 32) * 32 * 100;
+    const int cand[3] = {6, 3, 2};
+    const int64_t penalty[3] = {100, 103, 104};
+    for (int c = 0; c < 3; ++c) {
+        const int64_t cost = ceil_div(J, 8 * cand[c]) * 8 * cand[c] * penalty[c];
+        if (cost < best) {
+            best = cost;
+            nq = cand[c];
+        }
+    }
     for (int v = 0; v < kNumVariants; ++v)
-        if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == 4) return v;
+        if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == nq) return v;
     return 0;
 }
 
@@ -352,6 +403,12 @@ static void launch_variant(int v, const Lt2Args &args, bool vec, bool split, hip
         case 4: launch_vs<2, 1, 8>(args, vec, split, stream); break;
         case 5: launch_vs<2, 1, 4>(args, vec, split, stream); break;
         case 6: launch_vs<1, 1, 8>(args, vec, split, stream); break;
+        case 8: launch_vs<1, 1, 2>(args, vec, split, stream); break;
+        case 9: launch_vs<1, 1, 3>(args, vec, split, stream); break;
+        case 10: launch_vs<1, 1, 6>(args, vec, split, stream); break;
+        case 11: launch_vs<2, 1, 2>(args, vec, split, stream); break;
+        case 12: launch_vs<2, 1, 3>(args, vec, split, stream); break;
+        case 13: launch_vs<2, 1, 6>(args, vec, split, stream); break;
         default: launch_vs<1, 1, 4>(args, vec, split, stream); break;
     }
 }

@@ -46,12 +46,17 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     constexpr int JC = 16 * KS;    // j per chunk
     constexpr int LDA = JC + 8;    // padded LDS row in bf16 (16 bytes of padding: conflict-free 16-byte reads)
     constexpr int F4_PER_ROW = JC / 4;
-    constexpr int ROWS_PER_SLOT = NT / F4_PER_ROW;
-    constexpr int SLOTS = TS * F4_PER_ROW / NT;
-    static_assert(TS * F4_PER_ROW % NT == 0, "tile must divide over the threads");
+    constexpr int F4_TILE = TS * F4_PER_ROW;        // 16-byte pieces of a w tile (fp32)
+    constexpr int SLOTS = (F4_TILE + NT - 1) / NT;  // of which a thread stages this many
+    // REGULAR: a thread keeps its column and steps whole rows from slot to slot; otherwise
+    // (chunks of 48, tiles smaller than the workgroup) pieces are dealt out linearly and the
+    // last slot is only partly filled.
+    constexpr bool REGULAR = (NT % F4_PER_ROW == 0) && (F4_TILE % NT == 0);
     constexpr int TN = 128;
 
-    __shared__ __attribute__((aligned(16))) __bf16 wt[2][NS][TS * LDA];
+    // (a thread whose last slot lies past the tile stages into a private 8 bytes behind it: the
+    // steady state carries no predicates)
+    __shared__ __attribute__((aligned(16))) __bf16 wt[2][NS][TS * LDA + (REGULAR ? 0 : 4 * NT)];
 
     const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
     if (L >= p.total_wgs) return;
@@ -104,8 +109,23 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     // ---- w tile staging: a buffer resource whose extent ends at the last valid row (rows
     // past S read as zeros), 32-bit lane offsets, the (i, j-chunk) offset in a scalar.
     floatx4 stage[SLOTS];
-    const int trow = tid / F4_PER_ROW;
-    const int tc4 = tid % F4_PER_ROW;
+    int srow[SLOTS], sc4[SLOTS];  // tile row and 16-byte column of each slot
+    int lds_off[SLOTS];           // where the slot goes in the LDS tile (bf16 elements)
+    bool sval[SLOTS];
+#pragma unroll
+    for (int sidx = 0; sidx < SLOTS; ++sidx) {
+        if (REGULAR) {
+            srow[sidx] = tid / F4_PER_ROW + sidx * (NT / F4_PER_ROW);
+            sc4[sidx] = tid % F4_PER_ROW;
+            sval[sidx] = true;
+        } else {
+            const int f = tid + sidx * NT;
+            srow[sidx] = f / F4_PER_ROW;
+            sc4[sidx] = f % F4_PER_ROW;
+            sval[sidx] = f < F4_TILE;
+        }
+        lds_off[sidx] = sval[sidx] ? srow[sidx] * LDA + 4 * sc4[sidx] : TS * LDA + 4 * tid;
+    }
     const int wrows = (p.S - s0) < TS ? (p.S - s0) : TS;
     const float *wtile0 = wr + (int64_t)s0 * p.sw1;
     const __amdgpu_buffer_rsrc_t w_rsrc =
@@ -113,24 +133,34 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     uint32_t woff[SLOTS];
 #pragma unroll
     for (int sidx = 0; sidx < SLOTS; ++sidx)
-        woff[sidx] = ((uint32_t)(trow + sidx * ROWS_PER_SLOT) * (uint32_t)p.sw1 + 4u * tc4) * 4u;
+        woff[sidx] = ((uint32_t)srow[sidx] * (uint32_t)p.sw1 + 4u * (uint32_t)sc4[sidx]) * 4u;
     auto load_tile = [&](int i, int jc) __attribute__((always_inline)) {
         const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
         const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
         if (full) {
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) stage[sidx] = buf_load_f32x4(w_rsrc, woff[sidx], soff);
+        } else if (VEC) {
+            // ragged last chunk of aligned rows (J is a multiple of 4): a 16-byte piece is whole
+            // or lies past J, where the next i begins: zeros instead
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx) {
+                const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+                const floatx4 v = buf_load_f32x4(w_rsrc, woff[sidx], soff);
+                stage[sidx] = (jc * JC + 4 * sc4[sidx] < p.J) ? v : zero;
+            }
         } else {
             // ragged chunk or unaligned rows: element loads; what lies past J belongs to the
             // next i (or is outside the extent) and is replaced by zero
-            const int j = jc * JC + 4 * tc4;
 #pragma unroll
-            for (int sidx = 0; sidx < SLOTS; ++sidx)
+            for (int sidx = 0; sidx < SLOTS; ++sidx) {
+                const int j = jc * JC + 4 * sc4[sidx];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const float v = buf_load_f32(w_rsrc, woff[sidx] + 4u * e, soff);
                     stage[sidx][e] = (j + e < p.J) ? v : 0.f;
                 }
+            }
         }
     };
     // split the staged fp32 values and write the pieces to LDS (8 bytes per piece and slot)
@@ -140,11 +170,10 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
             uint32_t p01[NS], p23[NS];
             split_pair<NS, false>(stage[sidx][0], stage[sidx][1], p01);
             split_pair<NS, false>(stage[sidx][2], stage[sidx][3], p23);
-            const int off = (trow + sidx * ROWS_PER_SLOT) * LDA + 4 * tc4;
 #pragma unroll
             for (int sp = 0; sp < NS; ++sp) {
                 uintx2 v = {p01[sp], p23[sp]};
-                *reinterpret_cast<uintx2 *>(&wt[buf][sp][off]) = v;
+                *reinterpret_cast<uintx2 *>(&wt[buf][sp][lds_off[sidx]]) = v;
             }
         }
     };
@@ -356,10 +385,14 @@ template <int NS>
 static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, bool split, hipStream_t stream) {
     if (rt == 2) {
         if (ks == 4) launch_bf<2, 4, NS>(args, vec, split, stream);
-        else launch_bf<2, 2, NS>(args, vec, split, stream);
+        else if (ks == 3) launch_bf<2, 3, NS>(args, vec, split, stream);
+        else if (ks == 2) launch_bf<2, 2, NS>(args, vec, split, stream);
+        else launch_bf<2, 1, NS>(args, vec, split, stream);
     } else {
         if (ks == 4) launch_bf<1, 4, NS>(args, vec, split, stream);
-        else launch_bf<1, 2, NS>(args, vec, split, stream);
+        else if (ks == 3) launch_bf<1, 3, NS>(args, vec, split, stream);
+        else if (ks == 2) launch_bf<1, 2, NS>(args, vec, split, stream);
+        else launch_bf<1, 1, NS>(args, vec, split, stream);
     }
 }
 
@@ -367,11 +400,30 @@ static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, boo
 
 using namespace trt;
 
+// j-chunk (in units of 16) that costs least: padded length of the contraction x cost per padded
+// j, measured at S = I = 64, K = 4096, R = 64 with J = 16..144 on 64-row tiles: chunks of 64 cost
+// 5.4 us per j with two pieces (9.2 with three), chunks of 48 2 % (4 %) more, of 32 8 % (4 %)
+// more, of 16 28 % (13 %) more -- and far more on grids that are latency bound (R = 128,
+// S = I = J = 48, K = 256: 85 against 52 us), hence their 35 % (25 %).  Against chunks of 32 or 64
+// alone J = 16 runs 2.6x (1.9x) faster, J = 48 1.7x (1.4x), J = 144 1.2x (1.1x).
+static int bf16_chunk(int64_t J, int pieces) {
+    const int64_t penalty[2][4] = {{135, 108, 102, 100}, {125, 104, 104, 100}};
+    int best_ks = 4;
+    int64_t best = 0;
+    for (int ks = 4; ks >= 1; --ks) {
+        const int64_t cost = ceil_div(J, 16 * ks) * 16 * ks * penalty[pieces == 2 ? 0 : 1][ks - 1];
+        if (ks == 4 || cost < best) {
+            best = cost;
+            best_ks = ks;
+        }
+    }
+    return best_ks;
+}
+
 // Split count the bf16 path would like for a small grid (32-row tiles): 1 = none.
 static int64_t bf16_small_grid_splits(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int pieces, int mode) {
     if (mode == TRT_MODE_UNSPLIT) return 1;
-    const int64_t j_last = J % 64;
-    const int ks = (j_last >= 1 && j_last <= 32) ? 2 : 4;
+    const int ks = bf16_chunk(J, pieces);
     const int64_t iters = ceil_div(J, 16 * ks) * I;
     const int64_t tiles = R * ceil_div(S, 32) * ceil_div(K, 128);
     if (mode != TRT_MODE_SPLIT && tiles >= 1024) return 1;  // four workgroups per CU: matrix bound as it is
@@ -405,7 +457,7 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
     if (mode != TRT_MODE_AUTO && mode != TRT_MODE_SPLIT && mode != TRT_MODE_UNSPLIT) return TRT_E_INVALID;
-    if (variant < 0 || variant > 8) return TRT_E_INVALID;
+    if (variant < 0 || variant > 16) return TRT_E_INVALID;
     if (sw[2] != 1 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
@@ -424,22 +476,24 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     //    the fp32 path.  Mode SPLIT cuts on the bf16 pipe as well.
     //  - 32 rows per workgroup; 64 when that pads S no further and still leaves two workgroups
     //    per CU (the pipelined two-row-tile loop then wins 4-11 %).
-    //  - j-chunks of 64, or of 32 when those leave less of the last chunk empty (J = 1..32,
-    //    65..96 modulo 64: 1.15-1.8x), and for J = 33..48 on the 64-row tile.
+    //  - j-chunks of 64, 48, 32 or 16: the one that pads J least, weighed by its cost per j
+    //    (bf16_chunk).
     const int64_t ctk = ceil_div(K, 128);
     const int64_t t32 = R * ceil_div(S, 32) * ctk, t64 = R * ceil_div(S, 64) * ctk;
-    const int64_t s_last = S % 64, j_last = J % 64;
+    const int64_t s_last = S % 64;
     int rt = (S > 32 && (s_last == 0 || s_last > 32) && t64 >= 512) ? 2 : 1;
-    int ks = ((j_last >= 1 && j_last <= 32) || (rt == 2 && j_last >= 33 && j_last <= 48)) ? 2 : 4;
+    int ks = bf16_chunk(J, pieces);
     const int rule_rt = rt, rule_ks = ks;
     bool split = false, small_grid = false;
     if (variant >= 1) {
         // 1: 64 rows, chunks of 64;  2: 64 rows, 32;  3: 32 rows, 64;  4: 32 rows, 32;
         // 5..8: the same with the contraction cut over workgroups (as far as the workspace allows)
+        // 9..12: chunks of 48 and 16 (64 rows: 9, 10; 32 rows: 11, 12);  13..16: the same, cut
         const int tile = (variant - 1) % 4 + 1;
         rt = tile <= 2 ? 2 : 1;
-        ks = (tile & 1) ? 4 : 2;
-        split = variant >= 5;
+        if (variant <= 8) ks = (tile & 1) ? 4 : 2;
+        else ks = (tile & 1) ? 3 : 1;
+        split = (variant >= 5 && variant <= 8) || variant >= 13;
     } else {
         // A grid that is not matrix bound as it is has its contraction cut over workgroups on
         // 32-row tiles when the cost model asks for it (below); a small grid that is not to be
@@ -448,7 +502,7 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
         if (bf16_small_grid_splits(R, S, I, J, K, pieces, mode) >= 2) {
             split = true;
             rt = 1;
-            ks = (j_last >= 1 && j_last <= 32) ? 2 : 4;
+            ks = bf16_chunk(J, pieces);
         }
     }
 

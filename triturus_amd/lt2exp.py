@@ -39,8 +39,8 @@ def launches_split(R: int, S: int, I: int, J: int, K: int, mode: str) -> bool:
 
 _PIECES = {"bf16x3": 2, "bf16x6": 3}
 # tile variants worth timing when tuning is on (0 = the library's rule)
-_FP32_CANDIDATES = (0, 5, 6, 8)
-_BF16_CANDIDATES = (0, 1, 2, 3, 4)
+_FP32_CANDIDATES = (0, 5, 6, 8, 9, 10, 11, 12, 13, 14)
+_BF16_CANDIDATES = (0, 1, 2, 3, 4, 9, 10, 11, 12)
 
 
 def lt2exp(
