@@ -145,8 +145,20 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         }
     };
     auto load_tile_masked = [&](int jc) {
-        const char *org = reinterpret_cast<const char *>(atile0 + jc * JC);
         const int j = jc * JC + 4 * tc4;
+        if (VEC) {
+            // aligned rows, J a multiple of 4: a 16-byte piece is whole or lies past J (in the
+            // next row, or outside the extent): zeros instead
+            const uint32_t soff = (uint32_t)(jc * JC) * 4u;
+            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx) {
+                const floatx4 v = buf_load_f32x4(a_rsrc, aoff[sidx], soff);
+                stage[sidx] = j < p.J ? v : zero;
+            }
+            return;
+        }
+        const char *org = reinterpret_cast<const char *>(atile0 + jc * JC);
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
             const float *src = reinterpret_cast<const float *>(org + aoff[sidx]);
@@ -183,18 +195,21 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
                 for (int ct = 0; ct < CT; ++ct) braw[ct][4 * q + u] = buf_load_f32(b_rsrc, boff[ct], soff);
             }
     };
+    // ragged last chunk: the same loads (what lies past the extent reads as 0, nothing faults),
+    // rows past J replaced by -inf
     auto load_b_masked = [&](int jc) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct)
+        for (int q = 0; q < NQ; ++q)
 #pragma unroll
-            for (int q = 0; q < NQ; ++q)
+            for (int u = 0; u < 4; ++u) {
+                const uint32_t soff = (uint32_t)(jc * JC + 8 * q + u) * b_row_bytes;  // wave-uniform
+                const int j = jc * JC + 8 * q + 4 * h + u;
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const int j = jc * JC + 8 * q + 4 * h + u;
-                    float raw = MODE == kPlain ? 0.f : -__builtin_inff();
-                    if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl[ct]];
-                    braw[ct][4 * q + u] = raw;
+                for (int ct = 0; ct < CT; ++ct) {
+                    const float raw = buf_load_f32(b_rsrc, boff[ct], soff);
+                    braw[ct][4 * q + u] = j < p.J ? raw : (MODE == kPlain ? 0.f : -__builtin_inff());
                 }
+            }
     };
     // Maximum of the chunk's column.  A NaN need not survive here: exp(NaN - m) is NaN
     // for any m and poisons the whole output column through the MFMA, which is what

@@ -108,6 +108,16 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
         if (full) {
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) stage[sidx] = buf_load_f32x4(a_rsrc, aoff[sidx], soff);
+        } else if (VEC) {
+            // ragged last chunk of aligned rows (J a multiple of 4): a 16-byte piece is whole or
+            // lies past J (in the next row, or outside the extent): zeros instead
+            const int j = jc * JC + 4 * tc4;
+            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int sidx = 0; sidx < SLOTS; ++sidx) {
+                const floatx4 v = buf_load_f32x4(a_rsrc, aoff[sidx], soff);
+                stage[sidx] = j < p.J ? v : zero;
+            }
         } else {
             const int j = jc * JC + 4 * tc4;
 #pragma unroll
