@@ -86,7 +86,9 @@ def test_every_tile_variant_on_ragged_shapes(dev, variant, mode, shape):
 @pytest.mark.parametrize(
     "shape",
     [(1, 1, 1, 1, 1), (2, 1, 3, 1, 5), (1, 3, 1, 4, 1), (1, 65, 2, 2, 257), (3, 8, 64, 4, 40), (1, 8, 4, 64, 40),
-     (1, 129, 17, 65, 33), (1, 4, 300, 3, 16), (1, 4, 3, 300, 16)],
+     (1, 129, 17, 65, 33), (1, 4, 300, 3, 16), (1, 4, 3, 300, 16),
+     # a short j axis under a long i axis runs with the roles of (i, a) and (j, b) exchanged
+     (2, 40, 150, 1, 200), (2, 40, 150, 2, 300), (1, 20, 64, 8, 260), (3, 33, 37, 5, 257), (1, 20, 16, 8, 300)],
 )
 @pytest.mark.parametrize("mode", ["auto", "split"])
 def test_edge_shapes(dev, shape, mode):
@@ -96,6 +98,9 @@ def test_edge_shapes(dev, shape, mode):
     a = 2 * torch.randn(R, I, K, generator=g)
     b = 2 * torch.randn(R, J, K, generator=g)
     _check(lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode), w, a, b)
+    for precision in ("bf16x3", "bf16x6"):
+        _check(lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision), w, a, b,
+               **PRECISION_GATES[precision])
 
 
 def test_empty_inputs(dev):

@@ -449,13 +449,21 @@ static int resolve_variant(int variant, int64_t R, int64_t S, int64_t I, int64_t
 
 extern "C" size_t trt_lt2exp_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode) {
     if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return 0;
-    // the split count depends on the tile shape: size for the largest possible
+    // the split count depends on the tile shape: size for the largest possible; a call with
+    // J = 1 may run with i and j exchanged (trt_lt2exp_f32): room for either
     size_t need = 0;
-    for (int v = 0; v < kNumVariants; ++v) {
-        SplitPlan sp = plan_split(R, S, I, J, K, mode, v);
-        if (!sp.split) continue;
-        size_t b = ((size_t)sp.splits * R * S * K + (size_t)2 * R * K) * sizeof(float);
-        if (b > need) need = b;
+    for (int pass = 0; pass < 2; ++pass) {
+        if (pass == 1) {
+            if (!(J == 1 && I > 1)) break;
+            J = I;
+            I = 1;
+        }
+        for (int v = 0; v < kNumVariants; ++v) {
+            SplitPlan sp = plan_split(R, S, I, J, K, mode, v);
+            if (!sp.split) continue;
+            size_t b = ((size_t)sp.splits * R * S * K + (size_t)2 * R * K) * sizeof(float);
+            if (b > need) need = b;
+        }
     }
     return need;
 }
@@ -476,6 +484,13 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
     // byte offsets inside one batch slab of w, a and c are 32-bit (buffer addressing)
     if (S * sw[1] + I * J >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
+
+    // A single j under several i: the contraction is symmetric in (i, a) and (j, b), and with
+    // J = 1 the same w is an R x S x 1 x I tensor, so the call runs with the roles exchanged
+    // (the kernel walks j in chunks and i one at a time: one chunk of I instead of I chunks of 1).
+    if (J == 1 && I > 1 && variant == 0)
+        return trt_lt2exp_f32(w, b, a, c, R, S, 1, I, K, sw, sb, sa, sc, mode, variant, workspace, workspace_bytes,
+                              stream);
 
     const int v = resolve_variant(variant, R, S, I, J, K);
     const Lt2Variant &vr = kVariants[v];

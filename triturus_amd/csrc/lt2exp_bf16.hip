@@ -445,7 +445,11 @@ static bool bf16_small_grid(int64_t R, int64_t S, int64_t I, int64_t J, int64_t 
 extern "C" size_t trt_lt2exp_bf16_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int pieces,
                                                   int mode) {
     if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0 || (pieces != 2 && pieces != 3)) return 0;
-    const int64_t splits = bf16_small_grid_splits(R, S, I, J, K, pieces, mode);
+    int64_t splits = bf16_small_grid_splits(R, S, I, J, K, pieces, mode);
+    if (J == 1 && I > 1) {  // may run with i and j exchanged (trt_lt2exp_bf16): room for either
+        const int64_t swapped = bf16_small_grid_splits(R, S, 1, I, K, pieces, mode);
+        if (swapped > splits) splits = swapped;
+    }
     return splits >= 2 ? ((size_t)splits * R * S * K + (size_t)2 * R * K) * sizeof(float) : 0;
 }
 
@@ -465,6 +469,11 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
     if (S * sw[1] + I * J >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
+
+    // a single j under several i: run with the roles of (i, a) and (j, b) exchanged (see trt_lt2exp_f32)
+    if (J == 1 && I > 1 && variant == 0)
+        return trt_lt2exp_bf16(w, b, a, c, R, S, 1, I, K, sw, sb, sa, sc, pieces, mode, variant, workspace,
+                               workspace_bytes, stream);
 
     // Tile and hand-over rules, fitted to 290 random shapes (R 1..128, S 16..512, I, J 8..128,
     // K 64..8192) timed with every tile and on the fp32 path; against the best of those the

@@ -43,6 +43,11 @@ _FP32_CANDIDATES = (0, 5, 6, 8, 9, 10, 11, 12, 13, 14)
 _BF16_CANDIDATES = (0, 1, 2, 3, 4, 9, 10, 11, 12)
 
 
+def _padded(n: int) -> int:
+    """Length of a contracted axis of n once padded to whole j-chunks of the size that fits it best."""
+    return min(-(-n // c) * c for c in (16, 24, 32, 48))
+
+
 def lt2exp(
     w: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, mode: str = "auto", _variant: int = 0,
     _precision: str | None = None, _tuning: bool = False,
@@ -69,6 +74,15 @@ def lt2exp(
         return c
     if I * J == 0:
         return c.fill_(float("-inf"))
+    # The kernels walk j in chunks of at least 16 and i one at a time: a short j axis under a
+    # long i axis wastes most of every chunk.  The contraction is symmetric in (i, a) and (j, b),
+    # so such a call runs with the roles exchanged on a transposed copy of w (J = 1 needs no
+    # copy: the library does that exchange itself), when that saves a third of the padded work
+    # and the output is wide enough for the copy not to matter.  Not for forced tiles (tests, tuning).
+    if _variant == 0 and 2 <= J < I and K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I):
+        w = w.view(R, S, I, J).transpose(2, 3).contiguous().view(R, S, I * J)
+        a, b = b, a
+        I, J = J, I
     w = _unit_inner(w)
     a = _unit_inner(a)
     b = _unit_inner(b)
