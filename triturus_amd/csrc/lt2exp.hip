@@ -364,7 +364,7 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
     int nq = 4;
     int64_t best = ceil_div(J, 32) * 32 * 100;
     const int cand[3] = {6, 3, 2};
-    const int64_t penalty[3] = {100, 103, 104};
+    const int64_t penalty[3] = {100, 103, 109};
     for (int c = 0; c < 3; ++c) {
         const int64_t cost = ceil_div(J, 8 * cand[c]) * 8 * cand[c] * penalty[c];
         if (cost < best) {

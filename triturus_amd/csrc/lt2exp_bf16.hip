@@ -406,12 +406,15 @@ using namespace trt;
 // more, of 16 28 % (13 %) more -- and far more on grids that are latency bound (R = 128,
 // S = I = J = 48, K = 256: 85 against 52 us), hence their 35 % (25 %).  Against chunks of 32 or 64
 // alone J = 16 runs 2.6x (1.9x) faster, J = 48 1.7x (1.4x), J = 144 1.2x (1.1x).
+// When J is not a multiple of 4 every chunk takes element loads, which chunks of 16 bear worst
+// (1.9x per padded j over 50 random shapes; 32 and 48 cost 5 % more than 64).
 static int bf16_chunk(int64_t J, int pieces) {
-    const int64_t penalty[2][4] = {{135, 108, 102, 100}, {125, 104, 104, 100}};
+    const int64_t penalty[3][4] = {{135, 108, 102, 100}, {125, 104, 104, 100}, {190, 105, 106, 100}};
+    const int row = J % 4 != 0 ? 2 : (pieces == 2 ? 0 : 1);
     int best_ks = 4;
     int64_t best = 0;
     for (int ks = 4; ks >= 1; --ks) {
-        const int64_t cost = ceil_div(J, 16 * ks) * 16 * ks * penalty[pieces == 2 ? 0 : 1][ks - 1];
+        const int64_t cost = ceil_div(J, 16 * ks) * 16 * ks * penalty[row][ks - 1];
         if (ks == 4 || cost < best) {
             best = cost;
             best_ks = ks;

@@ -79,7 +79,8 @@ def lt2exp(
     # so such a call runs with the roles exchanged on a transposed copy of w (J = 1 needs no
     # copy: the library does that exchange itself), when that saves a third of the padded work
     # and the output is wide enough for the copy not to matter.  Not for forced tiles (tests, tuning).
-    if _variant == 0 and 2 <= J < I and K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I):
+    if (_variant == 0 and 2 <= J < I and K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
+            and 2 * R * S * I * _padded(J) * K >= 4e9):  # worth a copy kernel: some 40 us of padded work
         w = w.view(R, S, I, J).transpose(2, 3).contiguous().view(R, S, I * J)
         a, b = b, a
         I, J = J, I
