@@ -63,10 +63,16 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     constexpr int NB = 4 * NQ;   // b values per lane, column tile and chunk
     constexpr int LDA = JC + 4;  // padded LDS row (floats): conflict-free 16-byte reads
     constexpr int F4_PER_ROW = JC / 4;
-    constexpr int SLOTS = TM * F4_PER_ROW / NT;
-    static_assert(TM * F4_PER_ROW % NT == 0, "tile must divide over the threads");
+    constexpr int F4_TILE = TM * F4_PER_ROW;        // 16-byte pieces of an a tile
+    constexpr int SLOTS = (F4_TILE + NT - 1) / NT;  // of which a thread stages this many
+    // REGULAR: a thread keeps its column and steps whole rows from slot to slot; otherwise
+    // (chunks of 24 or 48, tiles smaller than the workgroup) pieces are dealt out linearly, and
+    // a thread whose last slot lies past the tile stages into a private 16 bytes behind the
+    // buffers, so that the steady state carries no predicates.
+    constexpr bool REGULAR = (NT % F4_PER_ROW == 0) && (F4_TILE % NT == 0);
 
-    extern __shared__ __attribute__((aligned(16))) float at[];  // [2][TM * LDA]
+    constexpr int BUF = TM * LDA + (REGULAR ? 0 : 4 * NT);      // one LDS buffer: the tile, then the private pieces
+    extern __shared__ __attribute__((aligned(16))) float at[];  // [2][BUF]
 
     const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
     if (L >= p.total_wgs) return;
@@ -114,15 +120,26 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     // valid row instead of masked: they only feed accumulator rows that are never
     // stored.  Columns past J (ragged tail chunk only) must be exact zeros.
     floatx4 stage[SLOTS];
-    constexpr int ROWS_PER_SLOT = NT / F4_PER_ROW;
-    const int trow = tid / F4_PER_ROW;  // tile row of this thread's first slot
-    const int tc4 = tid % F4_PER_ROW;
+    int sc4[SLOTS];        // 16-byte column of each slot
+    int lds_off[SLOTS];    // where the slot goes in an LDS buffer (floats)
     uint32_t aoff[SLOTS];  // per-lane byte offsets from the (wave-uniform) tile origin
 #pragma unroll
     for (int sidx = 0; sidx < SLOTS; ++sidx) {
-        int row = i0 + trow + sidx * ROWS_PER_SLOT;
+        int trow;
+        bool inside = true;
+        if (REGULAR) {
+            trow = tid / F4_PER_ROW + sidx * (NT / F4_PER_ROW);
+            sc4[sidx] = tid % F4_PER_ROW;
+        } else {
+            const int f = tid + sidx * NT;
+            trow = f / F4_PER_ROW;
+            sc4[sidx] = f % F4_PER_ROW;
+            inside = f < F4_TILE;
+        }
+        lds_off[sidx] = inside ? trow * LDA + 4 * sc4[sidx] : TM * LDA + 4 * tid;
+        int row = i0 + trow;
         row = row < p.I ? row : p.I - 1;
-        aoff[sidx] = ((uint32_t)(row - i0) * (uint32_t)p.sa1 + 4u * tc4) * 4u;
+        aoff[sidx] = ((uint32_t)(row - i0) * (uint32_t)p.sa1 + 4u * (uint32_t)sc4[sidx]) * 4u;
     }
     const float *atile0 = ar + (int64_t)i0 * p.sa1;
     const int arows = (p.I - i0) < TM ? (p.I - i0) : TM;  // valid rows of this tile
@@ -145,7 +162,6 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         }
     };
     auto load_tile_masked = [&](int jc) {
-        const int j = jc * JC + 4 * tc4;
         if (VEC) {
             // aligned rows, J a multiple of 4: a 16-byte piece is whole or lies past J (in the
             // next row, or outside the extent): zeros instead
@@ -154,13 +170,14 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) {
                 const floatx4 v = buf_load_f32x4(a_rsrc, aoff[sidx], soff);
-                stage[sidx] = j < p.J ? v : zero;
+                stage[sidx] = jc * JC + 4 * sc4[sidx] < p.J ? v : zero;
             }
             return;
         }
         const char *org = reinterpret_cast<const char *>(atile0 + jc * JC);
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
+            const int j = jc * JC + 4 * sc4[sidx];
             const float *src = reinterpret_cast<const float *>(org + aoff[sidx]);
             floatx4 v = {0.f, 0.f, 0.f, 0.f};
             if (j + 0 < p.J) v[0] = src[0];
@@ -171,10 +188,9 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         }
     };
     auto store_tile = [&](int buf) {
-        float *dst = at + buf * (TM * LDA) + trow * LDA + 4 * tc4;
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx)
-            *reinterpret_cast<floatx4 *>(&dst[sidx * ROWS_PER_SLOT * LDA]) = stage[sidx];
+            *reinterpret_cast<floatx4 *>(&at[buf * BUF + lds_off[sidx]]) = stage[sidx];
     };
 
     // ---- b chunk: global -> registers.  Lane (h, m) takes rows 8q + 4h + u.
@@ -341,7 +357,7 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         load_tile_full(jc + 1);
         load_b_full(jc + 1);
         __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block, not sunk into it
-        mfma_block(at + cur * (TM * LDA) + wrow0 * LDA);
+        mfma_block(at + cur * BUF + wrow0 * LDA);
         store_tile(cur ^ 1);
         shift_and_exp();
         __syncthreads();
@@ -351,13 +367,13 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         load_tile_masked(jc + 1);
         load_b_masked(jc + 1);
         __builtin_amdgcn_sched_barrier(0);
-        mfma_block(at + cur * (TM * LDA) + wrow0 * LDA);
+        mfma_block(at + cur * BUF + wrow0 * LDA);
         store_tile(cur ^ 1);
         shift_and_exp();
         __syncthreads();
         cur ^= 1;
     }
-    mfma_block(at + cur * (TM * LDA) + wrow0 * LDA);
+    mfma_block(at + cur * BUF + wrow0 * LDA);
 
     // ---- epilogue: c = m + log(acc).  Register v of lane (h, m) holds row
     // 8*(v/4) + 4*h + v%4, column m of its 32 x 32 tile; the row part of the address
@@ -471,6 +487,12 @@ static const Lm2Variant kVariants[] = {
     {4, 1, 1, 4, 4, kTwoSweep},  // 10: as 1, two sweeps
     {4, 1, 1, 4, 4, kExternal},  // 11: as 1, shift from a separate pass over b (two launches)
     {3, 1, 1, 4, 4, kOnline},   // 12: 96 x 128 tile (I = 96, 192, ... without padded rows)
+    {4, 1, 1, 4, 2, kOnline},   // 13..18: the 128-, 64- and 32-row tiles with j-chunks of 16 and 24
+    {4, 1, 1, 4, 3, kOnline},   //         (chunks of 48 were measured too: 20 more B registers, a
+    {2, 1, 1, 4, 2, kOnline},   //         wavefront less per SIMD on the 128-row tile, 5-60 % slower)
+    {2, 1, 1, 4, 3, kOnline},
+    {1, 1, 1, 4, 2, kOnline},
+    {1, 1, 1, 4, 3, kOnline},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be opted into per kernel
@@ -486,12 +508,30 @@ constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be op
 //   long contraction (J >= 1280)                contraction is then cut over J)
 //   some tile leaves >= 1 workgroup per CU      the one with the least modelled time (pick_tile)
 //   none does                                   32 x 128   (+12..36 %)
-static int find_variant(int rt, int wn, int mode) {
+static int find_variant(int rt, int wn, int mode, int nq = 4) {
     for (int v = 0; v < kNumVariants; ++v)
         if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].wm == 1 && kVariants[v].wn == wn &&
-            kVariants[v].nq == 4 && kVariants[v].mode == mode)
+            kVariants[v].nq == nq && kVariants[v].mode == mode)
             return v;
-    return 0;
+    return nq == 4 ? 0 : find_variant(rt, wn, mode);
+}
+
+// j-chunk of the 128-, 64- and 32-row tiles: 32, or 16 or 24 where those pad J less.  Per padded j
+// they cost 3-4 % more (R=64, I=256, K=4096: J = 256 takes 281 us on chunks of 32, 287 / 297 on
+// 16 / 24), so J = 16, 24, 40, 48, 72, 80, 144, 200 run 17, 8, 15, 13, 16, 12, 9, 6 % faster.
+static int pick_chunk(int64_t J) {
+    int nq = 4;
+    int64_t best = ceil_div(J, 32) * 32 * 100;
+    const int cand[2] = {2, 3};
+    const int64_t penalty[2] = {103, 104};
+    for (int c = 0; c < 2; ++c) {
+        const int64_t cost = ceil_div(J, 8 * cand[c]) * 8 * cand[c] * penalty[c];
+        if (cost < best) {
+            best = cost;
+            nq = cand[c];
+        }
+    }
+    return nq;
 }
 
 // Tile for a grid of R x I rows and K columns among 128 x 128, 96 x 128, 64 x 128, 32 x 128 (rows
@@ -555,14 +595,16 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     } else {
         rt = 1;
     }
-    return find_variant(rt, 4, kOnline);
+    return find_variant(rt, 4, kOnline, pick_chunk(J));  // (the 96-row tile has chunks of 32 only)
 }
 
 template <int RT, int CT, int WM, int WN, int NQ, bool VEC, int MODE>
 static int launch_k(const Lm2Args &args, hipStream_t stream) {
     constexpr int TM = 32 * RT * WM;
     constexpr int LDA = 8 * NQ + 4;
-    constexpr size_t lds = (size_t)2 * TM * LDA * sizeof(float);
+    constexpr int NT = WM * WN * kWave;
+    constexpr bool REGULAR = (NT % (2 * NQ) == 0) && (TM * 2 * NQ % NT == 0);  // as in the kernel
+    constexpr size_t lds = (size_t)2 * (TM * LDA + (REGULAR ? 0 : 4 * NT)) * sizeof(float);
     auto k = lm2exp_kernel<RT, CT, WM, WN, NQ, VEC, MODE>;
     if (lds > kDefaultLdsLimit) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(k),
@@ -694,6 +736,12 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         case 8: st = launch_v<2, 1, 1, 4, 4, kTwoSweep>(args, vec, s); break;
         case 9: st = launch_v<4, 1, 1, 4, 4, kTwoSweep>(args, vec, s); break;
         case 10: st = launch_v<4, 1, 1, 4, 4, kExternal>(args, vec, s); break;
+        case 12: st = launch_v<4, 1, 1, 4, 2, kOnline>(args, vec, s); break;
+        case 13: st = launch_v<4, 1, 1, 4, 3, kOnline>(args, vec, s); break;
+        case 14: st = launch_v<2, 1, 1, 4, 2, kOnline>(args, vec, s); break;
+        case 15: st = launch_v<2, 1, 1, 4, 3, kOnline>(args, vec, s); break;
+        case 16: st = launch_v<1, 1, 1, 4, 2, kOnline>(args, vec, s); break;
+        case 17: st = launch_v<1, 1, 1, 4, 3, kOnline>(args, vec, s); break;
         default: st = launch_v<3, 1, 1, 4, 4, kOnline>(args, vec, s); break;
     }
     if (st != 0 || pl.splits <= 1) return st;
