@@ -44,6 +44,7 @@ struct Lm2Args {
     int R, I, J, K;
     int64_t sa0, sa1, sb0, sb1, sc0, sc1;
     int i_tiles, n_tiles, splits, chunks_per_split;
+    int stream_out;  // rows of c are 16-byte aligned: non-temporal result stores
     int64_t total_wgs, padded_wgs;
 };
 
@@ -402,9 +403,10 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
                 if (split_out)  // partial sums are read back by the merge kernel right away
                     buf_store_f32(acc[rt][ct][v], c_rsrc, co, trow * c_row_bytes);
                 else if (MODE == kPlain)
-                    buf_store_f32_stream(acc[rt][ct][v], c_rsrc, co, trow * c_row_bytes);
+                    buf_store_f32_out(p.stream_out != 0, acc[rt][ct][v], c_rsrc, co, trow * c_row_bytes);
                 else
-                    buf_store_f32_stream(log_plus(acc[rt][ct][v], mref[ct]), c_rsrc, co, trow * c_row_bytes);
+                    buf_store_f32_out(p.stream_out != 0, log_plus(acc[rt][ct][v], mref[ct]), c_rsrc, co,
+                                      trow * c_row_bytes);
             }
     }
 }
@@ -595,11 +597,8 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     } else {
         rt = 1;
     }
-    // (the 96-row tile has chunks of 32 only; with rows of b and c that are not 16-byte aligned
-    // -- K not a multiple of 4 -- the call is bound by partial-line traffic and the smaller
-    // chunks measured 15-30 % slower: R=41, I=2636, J=12: K=2223 328 us on chunks of 32, 421 on
-    // 16; K=2224 256 and 184)
-    return find_variant(rt, 4, kOnline, K % 4 == 0 ? pick_chunk(J) : 4);
+    // (the 96-row tile has chunks of 32 only)
+    return find_variant(rt, 4, kOnline, pick_chunk(J));
 }
 
 template <int RT, int CT, int WM, int WN, int NQ, bool VEC, int MODE>
@@ -709,6 +708,7 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     args.chunks_per_split = pl.chunks_per_split;
     args.total_wgs = (int64_t)R * args.i_tiles * args.n_tiles * pl.splits;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    args.stream_out = rows_16_byte_aligned(c, sc[0], sc[1]);
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (vr.mode == kExternal) {
@@ -837,6 +837,7 @@ extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, i
     args.chunks_per_split = (int)ceil_div(k, 32);
     args.total_wgs = (int64_t)args.i_tiles * args.n_tiles;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    args.stream_out = rows_16_byte_aligned(c, args.sc0, args.sc1);
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const bool vec = (k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);

@@ -32,6 +32,7 @@ struct Lm2BfArgs {
     int R, I, J, K;
     int64_t sa0, sa1, sb0, sb1, sc0, sc1;
     int i_tiles, n_tiles, splits, chunks_per_split;
+    int stream_out;  // rows of c are 16-byte aligned: non-temporal result stores
     int64_t total_wgs, padded_wgs;
 };
 
@@ -309,7 +310,8 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4);
-            buf_store_f32_stream(PLAIN ? acc[rt][v] : log_plus(acc[rt][v], mref), c_rsrc, co, trow_c * c_row_bytes);
+            buf_store_f32_out(p.stream_out != 0, PLAIN ? acc[rt][v] : log_plus(acc[rt][v], mref), c_rsrc, co,
+                              trow_c * c_row_bytes);
         }
 }
 
@@ -484,6 +486,7 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     args.shift = cut > 1 ? args.part + (int64_t)cut * R * I * K : nullptr;
     args.total_wgs = (int64_t)R * args.i_tiles * args.n_tiles * cut;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    args.stream_out = rows_16_byte_aligned(c, sc[0], sc[1]);
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const bool vec = (J % 4 == 0) && (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
@@ -543,6 +546,7 @@ extern "C" int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, 
     args.chunks_per_split = (int)ceil_div(k, 16);  // at least every chunk
     args.total_wgs = (int64_t)args.i_tiles * args.n_tiles;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    args.stream_out = rows_16_byte_aligned(c, args.sc0, args.sc1);
     const bool vec = (k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
     return rt == 4 ? launch_mm_bf<4, 2>(args, pieces, vec, s) : launch_mm_bf<2, 4>(args, pieces, vec, s);

@@ -32,6 +32,7 @@ struct Lt2Args {
     int64_t sw0, sw1, sa0, sa1, sb0, sb1, sc0, sc1;
     int s_tiles, n_tiles, splits;
     int iters_per_split;  // (j-chunk, i) iterations per split
+    int stream_out;       // rows of c are 16-byte aligned: non-temporal result stores
     int64_t total_wgs, padded_wgs;
 };
 
@@ -306,7 +307,8 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
                     const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4);  // + 4h in the lane offset
-                    buf_store_f32_stream(log_plus(acc[rt][ct][v], mm), c_rsrc, co, trow_c * c_row_bytes);
+                    buf_store_f32_out(p.stream_out != 0, log_plus(acc[rt][ct][v], mm), c_rsrc, co,
+                                      trow_c * c_row_bytes);
                 }
         }
     }
@@ -509,6 +511,7 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     args.iters_per_split = sp.iters_per_split;
     args.total_wgs = (int64_t)R * args.s_tiles * args.n_tiles * sp.splits;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    args.stream_out = rows_16_byte_aligned(c, sc[0], sc[1]);
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     args.shift = nullptr;
     args.c = c;

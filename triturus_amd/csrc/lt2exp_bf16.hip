@@ -36,6 +36,7 @@ struct Lt2BfArgs {
     int64_t sw0, sw1, sa0, sa1, sb0, sb1, sc0, sc1;
     int s_tiles, n_tiles, splits;
     int iters_per_split;  // (j-chunk, i) iterations per split
+    int stream_out;       // rows of c are 16-byte aligned: non-temporal result stores
     int64_t total_wgs, padded_wgs;
 };
 
@@ -365,7 +366,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4);
-            buf_store_f32_stream(log_plus(total[rt][v], mm), c_rsrc, co, trow_c * c_row_bytes);
+            buf_store_f32_out(p.stream_out != 0, log_plus(total[rt][v], mm), c_rsrc, co, trow_c * c_row_bytes);
         }
 }
 
@@ -561,6 +562,7 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     args.n_tiles = (int)ceil_div(K, 128);
     args.total_wgs = (int64_t)R * args.s_tiles * args.n_tiles * splits;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
+    args.stream_out = rows_16_byte_aligned(c, sc[0], sc[1]);
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const bool vec = (J % 4 == 0) && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
