@@ -495,6 +495,9 @@ static const Lm2Variant kVariants[] = {
     {2, 1, 1, 4, 3, kOnline},
     {1, 1, 1, 4, 2, kOnline},
     {1, 1, 1, 4, 3, kOnline},
+    {1, 1, 4, 1, 4, kOnline},   // 19: 128 x 32 tile, the 4 waves stacked over rows (outputs of <= 32 columns)
+    {2, 1, 4, 1, 4, kOnline},   // 20: 256 x 32 tile
+    {1, 1, 2, 2, 4, kOnline},   // 21: 64 x 64 tile (outputs of <= 64 columns)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be opted into per kernel
@@ -516,6 +519,14 @@ static int find_variant(int rt, int wn, int mode, int nq = 4) {
             kVariants[v].nq == nq && kVariants[v].mode == mode)
             return v;
     return nq == 4 ? 0 : find_variant(rt, wn, mode);
+}
+
+static int find_variant_shape(int rt, int wm, int wn) {
+    for (int v = 0; v < kNumVariants; ++v)
+        if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].wm == wm && kVariants[v].wn == wn &&
+            kVariants[v].nq == 4 && kVariants[v].mode == kOnline)
+            return v;
+    return 0;
 }
 
 // j-chunk of the 128-, 64- and 32-row tiles: 32, or 16 or 24 where those pad J less.  Per padded j
@@ -577,6 +588,12 @@ static int pick_tile(int64_t R, int64_t I, int64_t K, int overhead_quarters, boo
 }
 
 static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
+    // Outputs of at most 32 (64) columns would leave three (two) of the four wavefronts of a
+    // 128-column tile idle: the wavefronts are stacked over rows instead (128 x 32 and 64 x 64
+    // tiles).  R=31, I=2527, J=2423, K=20: 479 -> 269 us; R=26, I=820, J=2949, K=14: 187 -> 91;
+    // R=96, I=2932, J=135, K=34: 112 -> 81.
+    if (K <= 32 && I > 64) return find_variant_shape(1, 4, 1);
+    if (K <= 64 && I > 32) return find_variant_shape(1, 2, 2);
     const int64_t kFill = 384;
     const int64_t ct = ceil_div(K, 128);
     const int64_t n128 = R * ceil_div(I, 128) * ct, n64 = R * ceil_div(I, 64) * ct;
@@ -746,6 +763,9 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         case 15: st = launch_v<2, 1, 1, 4, 3, kOnline>(args, vec, s); break;
         case 16: st = launch_v<1, 1, 1, 4, 2, kOnline>(args, vec, s); break;
         case 17: st = launch_v<1, 1, 1, 4, 3, kOnline>(args, vec, s); break;
+        case 18: st = launch_v<1, 1, 4, 1, 4, kOnline>(args, vec, s); break;
+        case 19: st = launch_v<2, 1, 4, 1, 4, kOnline>(args, vec, s); break;
+        case 20: st = launch_v<1, 1, 2, 2, 4, kOnline>(args, vec, s); break;
         default: st = launch_v<3, 1, 1, 4, 4, kOnline>(args, vec, s); break;
     }
     if (st != 0 || pl.splits <= 1) return st;

@@ -446,7 +446,9 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
         // operands that come from HBM (by 4-6 us) and loses on cached ones (by 3 us): left to it
         const bool one_launch = small && splits == 0 && J >= 192 && J <= 416 &&
                                 trt_lm2exp_workspace_bytes(R, I, J, K, 0, 0) == 0;
-        if (cut == 1 && !one_launch && (splits > 1 || small || J <= (pieces == 2 ? 16 : 32)))
+        // outputs of at most 32 columns: the fp32 path has a tile with its wavefronts stacked over rows
+        const bool narrow = K <= 32 && I > 64;
+        if (narrow || (cut == 1 && !one_launch && (splits > 1 || small || J <= (pieces == 2 ? 16 : 32))))
             return trt_lm2exp_f32(a, b, c, R, I, J, K, sa, sb, sc, 0, splits, workspace, workspace_bytes, stream);
         int best_rt = 1;
         int64_t best_cost = ceil_div(I, 32) * 120;

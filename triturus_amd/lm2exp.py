@@ -33,7 +33,7 @@ def _unit_inner(t: torch.Tensor) -> torch.Tensor:
 
 _PIECES = {"bf16x3": 2, "bf16x6": 3}
 # tile variants worth timing when tuning is on (0 = the library's rule)
-_FP32_CANDIDATES = (0, 1, 2, 7, 8, 12, 13, 14, 15, 16, 17, 18)
+_FP32_CANDIDATES = (0, 1, 2, 7, 8, 12, 13, 14, 15, 16, 17, 18, 19, 21)
 _BF16_CANDIDATES = (0, 1, 2, 3, 4, 8, 9)
 
 
