@@ -247,7 +247,7 @@ def test_sparse_weights_under_a_wide_spread(dev, seed, precision):
     mode = rng.choice(["auto", "split", "unsplit"])
     variant = rng.randrange(0, 9)
     if precision == "fp32" and rng.random() < 0.4:  # the tiles with j-chunks of 16, 24 and 48
-        variant = rng.randrange(9, 15)
+        variant = rng.randrange(9, 17)
     out = lt2exp(w.to(dev), _view(rng, a.to(dev)), _view(rng, b.to(dev)), mode=mode, _precision=precision,
                  _variant=variant)
     bad, _ = _inside(out, lo, hi, **GATES[precision])

@@ -36,10 +36,13 @@ struct Lt2Args {
     int64_t total_wgs, padded_wgs;
 };
 
-template <int RT, int CT, int NQ, int NWAVES, bool VEC, bool SPLIT>
+// WM: wavefronts stacked over rows (1: all NWAVES side by side over columns; 2 or 4 for narrow
+// outputs, so that K <= 64 or 32 does not leave most of them idle).
+template <int RT, int CT, int NQ, int NWAVES, bool VEC, bool SPLIT, int WM = 1>
 __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args p) {
     constexpr int NT = NWAVES * kWave;
-    constexpr int TS = 32 * RT;           // rows of S per workgroup
+    constexpr int WN = NWAVES / WM;
+    constexpr int TS = 32 * RT * WM;      // rows of S per workgroup
     constexpr int JC = 8 * NQ;            // j per chunk
     constexpr int LDW = JC + 4;           // padded LDS row (floats): conflict-free 16-byte reads
     constexpr int F4_PER_ROW = JC / 4;
@@ -49,7 +52,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     // (chunks of 24 or 48, or tiles smaller than the workgroup) pieces are dealt out linearly
     // and the last slot is only partly filled.
     constexpr bool REGULAR = (NT % F4_PER_ROW == 0) && (F4_TILE % NT == 0);
-    constexpr int TN = 32 * CT * NWAVES;
+    constexpr int TN = 32 * CT * WN;
 
     // (a thread whose last slot lies past the tile stages into a private 16 bytes behind it:
     // the steady state carries no predicates)
@@ -73,7 +76,9 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     const int h = lane / 32;
     const int m = lane % 32;
     const int s0 = st * TS;
-    const int n0 = nt * TN + wave * 32 * CT;
+    const int wm = wave % WM;
+    const int n0 = nt * TN + (wave / WM) * 32 * CT;
+    const int wrow0 = wm * 32 * RT;  // first tile row of this wavefront
 
     int ncol[CT], ncl[CT];
 #pragma unroll
@@ -258,7 +263,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 #pragma unroll
             for (int ct = 0; ct < CT; ++ct) ea_raw[ct] = buf_load_f32(a_rsrc, aoff[ct], (uint32_t)ni * a_row_bytes);
             __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block, not sunk into it
-            mfma_block(wt[cur]);
+            mfma_block(wt[cur] + wrow0 * LDW);
             store_tile(cur ^ 1);
             if (njc != jc) load_eb(njc);
 #pragma unroll
@@ -268,7 +273,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
             i = ni;
             jc = njc;
         }
-        mfma_block(wt[cur]);
+        mfma_block(wt[cur] + wrow0 * LDW);
     }
 
     // ---- epilogue.  D layout of 32x32x2: register v of lane (h, m) holds
@@ -279,7 +284,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
             if (ncol[ct] >= p.K) continue;
-            if (split == 0 && st == 0 && h == 0) {
+            if (split == 0 && st == 0 && wm == 0 && h == 0) {
                 p.shift[(int64_t)r * p.K + ncol[ct]] = ma[ct];
                 p.shift[((int64_t)p.R + r) * p.K + ncol[ct]] = mb[ct];
             }
@@ -287,15 +292,16 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
             for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
                 for (int v = 0; v < 16; ++v) {
-                    const int row = s0 + 32 * rt + 8 * (v / 4) + 4 * h + (v % 4);
+                    const int row = s0 + wrow0 + 32 * rt + 8 * (v / 4) + 4 * h + (v % 4);
                     if (row < p.S) part[(int64_t)row * p.K + ncol[ct]] = acc[rt][ct][v];
                 }
         }
     } else {
         // Rows past S fall outside the buffer extent and are dropped by the hardware.
-        const int crows = p.S - s0;
-        const __amdgpu_buffer_rsrc_t c_rsrc = make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)s0 * p.sc1,
-                                                        (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4));
+        const int crows = p.S - (s0 + wrow0);  // valid rows below this wavefront's first row
+        const __amdgpu_buffer_rsrc_t c_rsrc =
+            make_rsrc(p.c + (int64_t)r * p.sc0 + (int64_t)(s0 + wrow0) * p.sc1,
+                      crows > 0 ? (uint32_t)(((int64_t)(crows - 1) * p.sc1 + p.K) * 4) : 0u);
         const uint32_t c_row_bytes = (uint32_t)p.sc1 * 4u;
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) {
@@ -317,6 +323,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 // ------------------------------------------------------------------ host
 struct Lt2Variant {
     int rt, ct, nq;
+    int wm = 1;  // wavefronts stacked over rows
 };
 // variant ids (1-based in the C ABI; 0 = choose by shape)
 static const Lt2Variant kVariants[] = {
@@ -334,6 +341,8 @@ static const Lt2Variant kVariants[] = {
     {2, 1, 2},
     {2, 1, 3},
     {2, 1, 6},
+    {1, 1, 4, 4},  // 15: 128 x 32 tile, the 4 wavefronts stacked over rows (outputs of <= 32 columns)
+    {1, 1, 4, 2},  // 16: 64 x 64 tile (outputs of <= 64 columns)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLt2Waves = 4;
@@ -351,6 +360,13 @@ constexpr int kLt2Waves = 4;
 // tile does.)  Rule checked against the better of the two tiles on those shapes: 0.6 % mean
 // regret, 2 shapes of 288 more than 10 % off.
 static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
+    // Outputs of at most 32 (64) columns would leave three (two) of the four wavefronts idle:
+    // they are stacked over rows instead (128 x 32 and 64 x 64 tiles).
+    if ((K <= 32 && S > 64) || (K <= 64 && S > 32)) {
+        const int wm = (K <= 32 && S > 64) ? 4 : 2;
+        for (int v = 0; v < kNumVariants; ++v)
+            if (kVariants[v].wm == wm) return v;
+    }
     int rt = 1;
     if (S > 32) {
         const int64_t last = S % 64;
@@ -375,24 +391,24 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
         }
     }
     for (int v = 0; v < kNumVariants; ++v)
-        if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == nq) return v;
+        if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == nq && kVariants[v].wm == 1) return v;
     return 0;
 }
 
-template <int RT, int CT, int NQ, bool VEC, bool SPLIT>
+template <int RT, int CT, int NQ, bool VEC, bool SPLIT, int WM>
 static void launch_one(const Lt2Args &args, hipStream_t stream) {
-    hipLaunchKernelGGL((lt2exp_kernel<RT, CT, NQ, kLt2Waves, VEC, SPLIT>), dim3((unsigned)args.padded_wgs),
+    hipLaunchKernelGGL((lt2exp_kernel<RT, CT, NQ, kLt2Waves, VEC, SPLIT, WM>), dim3((unsigned)args.padded_wgs),
                        dim3(kLt2Waves * kWave), 0, stream, args);
 }
 
-template <int RT, int CT, int NQ>
+template <int RT, int CT, int NQ, int WM = 1>
 static void launch_vs(const Lt2Args &args, bool vec, bool split, hipStream_t stream) {
     if (vec) {
-        if (split) launch_one<RT, CT, NQ, true, true>(args, stream);
-        else launch_one<RT, CT, NQ, true, false>(args, stream);
+        if (split) launch_one<RT, CT, NQ, true, true, WM>(args, stream);
+        else launch_one<RT, CT, NQ, true, false, WM>(args, stream);
     } else {
-        if (split) launch_one<RT, CT, NQ, false, true>(args, stream);
-        else launch_one<RT, CT, NQ, false, false>(args, stream);
+        if (split) launch_one<RT, CT, NQ, false, true, WM>(args, stream);
+        else launch_one<RT, CT, NQ, false, false, WM>(args, stream);
     }
 }
 
@@ -411,6 +427,8 @@ static void launch_variant(int v, const Lt2Args &args, bool vec, bool split, hip
         case 11: launch_vs<2, 1, 2>(args, vec, split, stream); break;
         case 12: launch_vs<2, 1, 3>(args, vec, split, stream); break;
         case 13: launch_vs<2, 1, 6>(args, vec, split, stream); break;
+        case 14: launch_vs<1, 1, 4, 4>(args, vec, split, stream); break;
+        case 15: launch_vs<1, 1, 4, 2>(args, vec, split, stream); break;
         default: launch_vs<1, 1, 4>(args, vec, split, stream); break;
     }
 }
@@ -429,7 +447,7 @@ static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t 
     const Lt2Variant &v = kVariants[variant];
     const int64_t iters = ceil_div(J, 8 * v.nq) * I;
     if (mode == TRT_MODE_UNSPLIT) return {false, 1, (int)iters};
-    const int64_t base = R * ceil_div(S, 32 * v.rt) * ceil_div(K, 32 * v.ct * kLt2Waves);
+    const int64_t base = R * ceil_div(S, 32 * v.rt * v.wm) * ceil_div(K, 32 * v.ct * (kLt2Waves / v.wm));
     int64_t splits = choose_splits(base, iters, 4 * v.nq * v.rt * v.ct, R * S * K, 4, 32, mode == TRT_MODE_SPLIT);
     if (splits <= 1) return {false, 1, (int)iters};
     const int64_t per = ceil_div(iters, splits);
@@ -505,8 +523,8 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     args.sa0 = sa[0]; args.sa1 = sa[1];
     args.sb0 = sb[0]; args.sb1 = sb[1];
     args.sc0 = sc[0]; args.sc1 = sc[1];
-    args.s_tiles = (int)ceil_div(S, 32 * vr.rt);
-    args.n_tiles = (int)ceil_div(K, 32 * vr.ct * kLt2Waves);
+    args.s_tiles = (int)ceil_div(S, 32 * vr.rt * vr.wm);
+    args.n_tiles = (int)ceil_div(K, 32 * vr.ct * (kLt2Waves / vr.wm));
     args.splits = sp.splits;
     args.iters_per_split = sp.iters_per_split;
     args.total_wgs = (int64_t)R * args.s_tiles * args.n_tiles * sp.splits;
