@@ -164,14 +164,15 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     };
     auto load_tile_masked = [&](int jc) {
         if (VEC) {
-            // aligned rows, J a multiple of 4: a 16-byte piece is whole or lies past J (in the
-            // next row, or outside the extent): zeros instead
+            // aligned rows: what a 16-byte piece holds past J (row padding, the next row, or
+            // nothing: outside the extent) is replaced by zeros
             const uint32_t soff = (uint32_t)(jc * JC) * 4u;
-            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) {
                 const floatx4 v = buf_load_f32x4(a_rsrc, aoff[sidx], soff);
-                stage[sidx] = jc * JC + 4 * sc4[sidx] < p.J ? v : zero;
+                const int j = jc * JC + 4 * sc4[sidx];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) stage[sidx][e] = j + e < p.J ? v[e] : 0.f;
             }
             return;
         }
@@ -742,7 +743,9 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         args.part = static_cast<float *>(workspace);
         args.shift = args.part + (size_t)pl.splits * R * I * K;
     }
-    const bool vec = (J % 4 == 0) && (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
+    // (rows of a that start 16-byte aligned: J itself need not be a multiple of 4 when the row
+    // stride is -- a padded copy -- since the piece that straddles J is masked by element)
+    const bool vec = (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     int st;
     switch (v) {

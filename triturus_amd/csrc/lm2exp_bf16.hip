@@ -110,14 +110,14 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) stage[sidx] = buf_load_f32x4(a_rsrc, aoff[sidx], soff);
         } else if (VEC) {
-            // ragged last chunk of aligned rows (J a multiple of 4): a 16-byte piece is whole or
-            // lies past J (in the next row, or outside the extent): zeros instead
+            // ragged last chunk of aligned rows: what a 16-byte piece holds past J (row padding, the
+            // next row, or nothing: outside the extent) is replaced by zeros
             const int j = jc * JC + 4 * tc4;
-            const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) {
                 const floatx4 v = buf_load_f32x4(a_rsrc, aoff[sidx], soff);
-                stage[sidx] = j < p.J ? v : zero;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) stage[sidx][e] = j + e < p.J ? v[e] : 0.f;
             }
         } else {
             const int j = jc * JC + 4 * tc4;
@@ -490,7 +490,9 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
     args.stream_out = rows_16_byte_aligned(c, sc[0], sc[1]);
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
-    const bool vec = (J % 4 == 0) && (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
+    // (J itself need not be a multiple of 4 when the row stride is: the piece that straddles J
+    // is masked by element)
+    const bool vec = (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
     int status;

@@ -66,6 +66,12 @@ def lm2exp(
         cands = _FP32_CANDIDATES if _precision == "fp32" else _BF16_CANDIDATES
         _variant = autotune.pick(("lm2exp", R, I, J, K, _precision), cands,
                                  lambda v: lm2exp(a, b, _variant=v, _splits=-1, _precision=_precision))
+    # Rows of a are read 16 bytes at a time when they start aligned; with J not a multiple of 4 a
+    # contiguous a does not qualify and the kernels fall back to element loads (10-50 % slower).
+    # A call with enough work per element of a (the copy costs ~3 ps per element, the element loads
+    # ~15 % of 20 fs x K) runs on a copy of a whose rows are padded to a multiple of 4.
+    if J % 4 != 0 and J > 4 and K >= 2048 and 2 * R * I * J * K >= 2e9:
+        a = torch.nn.functional.pad(a, (0, (-J) % 4))[..., :J]
     if _splits < 0:  # tuning launch: the library decides the split for this tile
         _splits = 0
     # small grids with a long contraction are cut over J; the partial sums need a workspace
