@@ -123,6 +123,33 @@ def test_small_grid_long_contraction_splits_by_itself(dev):
     assert torch.allclose(torch_baseline.lm2exp_fp32(a, b), out.cpu())  # the reference's bar
 
 
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+@pytest.mark.parametrize("shape", [(3, 37, 41, 70), (2, 130, 129, 257), (1, 64, 7, 64), (2, 33, 301, 31), (24, 150, 99, 200)])
+def test_padded_rows_of_a(dev, precision, shape, monkeypatch):
+    """J not a multiple of 4: the wrapper pads the rows of a (thresholds lowered so that small
+    inputs take that path) and the kernels read them 16 bytes at a time, masking what lies past J."""
+    import triturus_amd.lm2exp as mod
+
+    monkeypatch.setattr(mod, "_PAD_MIN_K", 1)
+    monkeypatch.setattr(mod, "_PAD_MIN_FLOPS", 0.0)
+    R, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(R, I, J, generator=g)
+    a[:, 0] = 0.0
+    b = torch.randn(R, J, K, generator=g) * 6 - 2
+    b[torch.rand(b.shape, generator=g) < 0.05] = NINF
+    b[:, :, 0] = NINF
+    for splits in (0, 1, 3):
+        out = lm2exp(a.to(dev), b.to(dev), _precision=precision, _splits=splits)
+        r = _check(out, a, b, **PRECISION_GATES.get(precision, {}))
+        assert r["n_neg_inf"] > 0
+    # a caller's own padded rows (a view of a wider tensor) qualify as well
+    wide = torch.full((R, I, J + (-J) % 4 + 4), float("nan"))
+    wide[..., :J] = a
+    out = lm2exp(wide.to(dev)[..., :J], b.to(dev), _precision=precision)
+    _check(out, a, b, **PRECISION_GATES.get(precision, {}))
+
+
 def test_empty_inputs(dev):
     assert lm2exp(torch.rand(0, 3, 4, device=dev), torch.rand(0, 4, 5, device=dev)).shape == (0, 3, 5)
     assert lm2exp(torch.rand(2, 0, 4, device=dev), torch.rand(2, 4, 5, device=dev)).shape == (2, 0, 5)

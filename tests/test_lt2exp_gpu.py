@@ -103,6 +103,31 @@ def test_edge_shapes(dev, shape, mode):
                **PRECISION_GATES[precision])
 
 
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+@pytest.mark.parametrize("shape", [(2, 40, 150, 2, 300), (1, 20, 64, 8, 260), (2, 33, 21, 7, 257), (2, 35, 9, 13, 45),
+                                   (1, 70, 20, 33, 300), (2, 16, 5, 50, 64)])
+def test_reshaping_front_ends(dev, precision, shape, monkeypatch):
+    """The wrapper's two front ends -- roles of (i, a) and (j, b) exchanged on a transposed copy
+    of w for a short j axis, and w / b padded to a multiple of 4 in J -- with their work
+    thresholds lowered so that small inputs take them: same results, -inf and zero weights included."""
+    import triturus_amd.lt2exp as mod
+
+    monkeypatch.setattr(mod, "_RESHAPE_MIN_FLOPS", 0.0)
+    monkeypatch.setattr(mod, "_PAD_MIN_K", 1)
+    R, S, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    w = torch.rand(R, S, I, J, generator=g)
+    w[:, 0] = 0.0
+    a = -3 + 2 * torch.randn(R, I, K, generator=g)
+    b = -3 + 2 * torch.randn(R, J, K, generator=g)
+    a[torch.rand(a.shape, generator=g) < 0.1] = NINF
+    b[:, :, 0] = NINF
+    for mode in ("auto", "split", "unsplit"):
+        out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision)
+        r = _check(out, w, a, b, **PRECISION_GATES.get(precision, {}))
+        assert r["n_neg_inf"] > 0
+
+
 def test_empty_inputs(dev):
     def z(*shape):
         return torch.rand(*shape, device=dev)

@@ -32,6 +32,10 @@ def _unit_inner(t: torch.Tensor) -> torch.Tensor:
 
 
 _PIECES = {"bf16x3": 2, "bf16x6": 3}
+# from this output width and this much work on, rows of a that are not a multiple of 4 long are
+# padded (tests lower the thresholds to reach that path on small inputs)
+_PAD_MIN_K = 2048
+_PAD_MIN_FLOPS = 2e9
 # tile variants worth timing when tuning is on (0 = the library's rule)
 _FP32_CANDIDATES = (0, 1, 2, 7, 8, 12, 13, 14, 15, 16, 17, 18, 19, 21)
 _BF16_CANDIDATES = (0, 1, 2, 3, 4, 8, 9)
@@ -70,7 +74,7 @@ def lm2exp(
     # contiguous a does not qualify and the kernels fall back to element loads (10-50 % slower).
     # A call with enough work per element of a (the copy costs ~3 ps per element, the element loads
     # ~15 % of 20 fs x K) runs on a copy of a whose rows are padded to a multiple of 4.
-    if J % 4 != 0 and J > 4 and K >= 2048 and 2 * R * I * J * K >= 2e9:
+    if J % 4 != 0 and J > 4 and K >= _PAD_MIN_K and 2 * R * I * J * K >= _PAD_MIN_FLOPS:
         a = torch.nn.functional.pad(a, (0, (-J) % 4))[..., :J]
     if _splits < 0:  # tuning launch: the library decides the split for this tile
         _splits = 0

@@ -43,6 +43,13 @@ _FP32_CANDIDATES = (0, 5, 6, 8, 9, 10, 11, 12, 13, 14)
 _BF16_CANDIDATES = (0, 1, 2, 3, 4, 9, 10, 11, 12)
 
 
+# Thresholds of the two reshaping front ends below (tests lower them to reach those paths on
+# small inputs): padded work that repays a copy kernel, and the output width from which padding
+# J to a multiple of 4 pays.
+_RESHAPE_MIN_FLOPS = 4e9
+_PAD_MIN_K = 1024
+
+
 def _padded(n: int) -> int:
     """Length of a contracted axis of n once padded to whole j-chunks of the size that fits it best."""
     return min(-(-n // c) * c for c in (16, 24, 32, 48))
@@ -80,7 +87,7 @@ def lt2exp(
     # copy: the library does that exchange itself), when that saves a third of the padded work
     # and the output is wide enough for the copy not to matter.  Not for forced tiles (tests, tuning).
     if (_variant == 0 and 2 <= J < I and K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
-            and 2 * R * S * I * _padded(J) * K >= 4e9):  # worth a copy kernel: some 40 us of padded work
+            and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS):  # worth a copy kernel: some 40 us of work
         w = w.view(R, S, I, J).transpose(2, 3).contiguous().view(R, S, I * J)
         a, b = b, a
         I, J = J, I
@@ -88,7 +95,8 @@ def lt2exp(
     # starts aligned); otherwise the kernels fall back to element loads, 15-60 % slower.  A call
     # with enough work runs on copies padded to the next multiple of 4 instead: zeros in w, -inf
     # rows in b (terms of weight 0: the result is the same).
-    if _variant == 0 and J % 4 != 0 and J > 4 and K >= 1024 and 2 * R * S * I * _padded(J) * K >= 4e9:
+    if (_variant == 0 and J % 4 != 0 and J > 4 and K >= _PAD_MIN_K
+            and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS):
         J4 = J + (-J) % 4
         w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
         b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
