@@ -362,8 +362,11 @@ constexpr int kLt2Waves = 4;
 static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
     // Outputs of at most 32 (64) columns would leave three (two) of the four wavefronts idle:
     // they are stacked over rows instead (128 x 32 and 64 x 64 tiles).
-    if ((K <= 32 && S > 64) || (K <= 64 && S > 32)) {
-        const int wm = (K <= 32 && S > 64) ? 4 : 2;
+    // (No lower bound on the number of tiles as lm2exp has: tried, 1.4-2x slower on grids of 64
+    // narrow tiles -- a tile's chain of I x J steps is long enough to keep its CU busy.)
+    const bool tall = K <= 32 && S > 64;
+    if (tall || (K <= 64 && S > 32)) {
+        const int wm = tall ? 4 : 2;
         for (int v = 0; v < kNumVariants; ++v)
             if (kVariants[v].wm == wm) return v;
     }
