@@ -19,7 +19,7 @@ from triturus_amd import _lib, workloads
 pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
-N_VARIANTS = 21
+N_VARIANTS = 23
 N_BF16_VARIANTS = 9
 # Accuracy gates of the split-bf16 paths against the float64 oracle: two pieces (3 MFMAs per
 # product) carry 16 significand bits -- looser than fp32, ten times tighter than the rtol 5e-4

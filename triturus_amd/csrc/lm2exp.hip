@@ -499,6 +499,8 @@ static const Lm2Variant kVariants[] = {
     {1, 1, 4, 1, 4, kOnline},   // 19: 128 x 32 tile, the 4 waves stacked over rows (outputs of <= 32 columns)
     {2, 1, 4, 1, 4, kOnline},   // 20: 256 x 32 tile
     {1, 1, 2, 2, 4, kOnline},   // 21: 64 x 64 tile (outputs of <= 64 columns)
+    {3, 1, 1, 4, 2, kOnline},   // 22, 23: the 96-row tile with j-chunks of 16 and 24
+    {3, 1, 1, 4, 3, kOnline},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be opted into per kernel
@@ -619,7 +621,6 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     } else {
         rt = 1;
     }
-    // (the 96-row tile has chunks of 32 only)
     return find_variant(rt, 4, kOnline, pick_chunk(J));
 }
 
@@ -773,6 +774,8 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         case 18: st = launch_v<1, 1, 4, 1, 4, kOnline>(args, vec, s); break;
         case 19: st = launch_v<2, 1, 4, 1, 4, kOnline>(args, vec, s); break;
         case 20: st = launch_v<1, 1, 2, 2, 4, kOnline>(args, vec, s); break;
+        case 21: st = launch_v<3, 1, 1, 4, 2, kOnline>(args, vec, s); break;
+        case 22: st = launch_v<3, 1, 1, 4, 3, kOnline>(args, vec, s); break;
         default: st = launch_v<3, 1, 1, 4, 4, kOnline>(args, vec, s); break;
     }
     if (st != 0 || pl.splits <= 1) return st;

@@ -37,7 +37,7 @@ _PIECES = {"bf16x3": 2, "bf16x6": 3}
 _PAD_MIN_K = 2048
 _PAD_MIN_FLOPS = 2e9
 # tile variants worth timing when tuning is on (0 = the library's rule)
-_FP32_CANDIDATES = (0, 1, 2, 7, 8, 12, 13, 14, 15, 16, 17, 18, 19, 21)
+_FP32_CANDIDATES = (0, 1, 2, 7, 8, 12, 13, 14, 15, 16, 17, 18, 19, 21, 22, 23)
 _BF16_CANDIDATES = (0, 1, 2, 3, 4, 8, 9)
 
 
