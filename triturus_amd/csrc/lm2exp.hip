@@ -535,7 +535,11 @@ static int find_variant_shape(int rt, int wm, int wn) {
 // j-chunk of the 128-, 64- and 32-row tiles: 32, or 16 or 24 where those pad J less.  Per padded j
 // they cost 3-4 % more (R=64, I=256, K=4096: J = 256 takes 281 us on chunks of 32, 287 / 297 on
 // 16 / 24), so J = 16, 24, 40, 48, 72, 80, 144, 200 run 17, 8, 15, 13, 16, 12, 9, 6 % faster.
+// (Not when J is not a multiple of 4: rows of a are then read by element unless the caller padded
+// them, and the smaller chunks, whose tiles leave part of the workgroup without a piece to stage,
+// bear that worst: R=2, I=87, J=482, K=2925 runs 47 % slower on chunks of 16.)
 static int pick_chunk(int64_t J) {
+    if (J % 4 != 0) return 4;
     int nq = 4;
     int64_t best = ceil_div(J, 32) * 32 * 100;
     const int cand[2] = {2, 3};
