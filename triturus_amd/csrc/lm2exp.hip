@@ -146,7 +146,24 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     const int arows = (p.I - i0) < TM ? (p.I - i0) : TM;  // valid rows of this tile
     const __amdgpu_buffer_rsrc_t a_rsrc =
         make_rsrc(atile0, (uint32_t)(((int64_t)(arows - 1) * p.sa1 + p.J) * 4));
+    // element-wise staging of the unaligned build (chunks that divide the workgroup evenly):
+    // single floats, consecutive lanes on consecutive columns (coalesced), a thread's floats
+    // NT / JC rows apart (scalar offsets); rows past I lie outside the extent and read as zeros
+    constexpr bool ELEM = !VEC && (NT % JC == 0) && ((TM * JC) % NT == 0) && (TM * JC / NT <= 4 * SLOTS);
+    constexpr int NE = ELEM ? TM * JC / NT : 1;  // floats per thread
+    const int ecol = tid % JC;
+    const uint32_t ebase = ((uint32_t)(tid / JC) * (uint32_t)p.sa1 + (uint32_t)ecol) * 4u;
+    auto load_tile_elem = [&](int jc) {
+        const uint32_t soff = (uint32_t)(jc * JC) * 4u;
+        const bool inside = jc * JC + ecol < p.J;
+#pragma unroll
+        for (int e = 0; e < NE; ++e) {
+            const float v = buf_load_f32(a_rsrc, ebase, soff + (uint32_t)(e * (NT / JC)) * (uint32_t)p.sa1 * 4u);
+            stage[e / 4][e % 4] = inside ? v : 0.f;
+        }
+    };
     auto load_tile_full = [&](int jc) {
+        if (ELEM) return load_tile_elem(jc);
         const uint32_t soff = (uint32_t)(jc * JC) * 4u;  // wave-uniform
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
@@ -176,6 +193,7 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
             }
             return;
         }
+        if (ELEM) return load_tile_elem(jc);
         const char *org = reinterpret_cast<const char *>(atile0 + jc * JC);
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
@@ -190,6 +208,11 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
         }
     };
     auto store_tile = [&](int buf) {
+        if (ELEM) {
+#pragma unroll
+            for (int e = 0; e < NE; ++e) at[buf * BUF + (tid / JC + e * (NT / JC)) * LDA + ecol] = stage[e / 4][e % 4];
+            return;
+        }
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx)
             *reinterpret_cast<floatx4 *>(&at[buf * BUF + lds_off[sidx]]) = stage[sidx];

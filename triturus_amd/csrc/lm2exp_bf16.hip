@@ -103,6 +103,11 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
     const int arows = (p.I - i0) < TM ? (p.I - i0) : TM;
     const __amdgpu_buffer_rsrc_t a_rsrc =
         make_rsrc(atile0, (uint32_t)(((int64_t)(arows - 1) * p.sa1 + p.J) * 4));
+    // pair-wise staging of the unaligned build (chunks that divide the workgroup evenly)
+    constexpr bool ELEM = !VEC && (NT % (JC / 2) == 0) && ((TM * JC / 2) % NT == 0) && (TM * JC / 2 / NT <= 2 * SLOTS);
+    constexpr int NP = ELEM ? TM * JC / 2 / NT : 1;  // column pairs per thread
+    const int ecp = tid % (JC / 2);
+    const uint32_t ebase = ((uint32_t)(tid / (JC / 2)) * (uint32_t)p.sa1 + 2u * (uint32_t)ecp) * 4u;
     auto load_tile = [&](int jc) {
         const uint32_t soff = (uint32_t)(jc * JC) * 4u;  // wave-uniform
         const bool full = VEC && (jc * JC + JC <= p.J);
@@ -119,6 +124,19 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 #pragma unroll
                 for (int e = 0; e < 4; ++e) stage[sidx][e] = j + e < p.J ? v[e] : 0.f;
             }
+        } else if (ELEM) {
+            // rows that are not 16-byte aligned: a thread takes pairs of adjacent columns (one
+            // register of two bf16 per piece afterwards), consecutive lanes consecutive pairs, its
+            // pairs NT / (JC / 2) rows apart (scalar offsets); rows past I lie outside the extent
+            // and read as zeros, as do columns past J
+            const bool in0 = jc * JC + 2 * ecp < p.J, in1 = jc * JC + 2 * ecp + 1 < p.J;
+#pragma unroll
+            for (int e = 0; e < NP; ++e) {
+                const uint32_t so = soff + (uint32_t)(e * (2 * NT / JC)) * (uint32_t)p.sa1 * 4u;
+                const float v0 = buf_load_f32(a_rsrc, ebase, so), v1 = buf_load_f32(a_rsrc, ebase + 4u, so);
+                stage[e / 2][2 * (e % 2)] = in0 ? v0 : 0.f;
+                stage[e / 2][2 * (e % 2) + 1] = in1 ? v1 : 0.f;
+            }
         } else {
             const int j = jc * JC + 4 * tc4;
 #pragma unroll
@@ -131,6 +149,17 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
         }
     };
     auto store_tile = [&](int buf) {
+        if (ELEM) {
+#pragma unroll
+            for (int e = 0; e < NP; ++e) {
+                uint32_t pk[NS];
+                split_pair<NS, false>(stage[e / 2][2 * (e % 2)], stage[e / 2][2 * (e % 2) + 1], pk);
+                const int off = (tid / (JC / 2) + e * (2 * NT / JC)) * LDA + 2 * ecp;
+#pragma unroll
+                for (int sp = 0; sp < NS; ++sp) *reinterpret_cast<uint32_t *>(tile_ptr(buf, sp) + off) = pk[sp];
+            }
+            return;
+        }
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
             uint32_t p01[NS], p23[NS];

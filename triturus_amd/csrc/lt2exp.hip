@@ -155,6 +155,11 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 #pragma unroll
     for (int sidx = 0; sidx < SLOTS; ++sidx)
         woff[sidx] = ((uint32_t)srow[sidx] * (uint32_t)p.sw1 + 4u * (uint32_t)sc4[sidx]) * 4u;
+    // element-wise staging of the unaligned build (chunks that divide the workgroup evenly)
+    constexpr bool ELEM = !VEC && (NT % JC == 0) && ((TS * JC) % NT == 0) && (TS * JC / NT <= 4 * SLOTS);
+    constexpr int NE = ELEM ? TS * JC / NT : 1;  // floats per thread
+    const int ecol = tid % JC;
+    const uint32_t ebase = ((uint32_t)(tid / JC) * (uint32_t)p.sw1 + (uint32_t)ecol) * 4u;
     // (a slot past the tile loads some valid or out-of-extent address: the value is never used)
     auto load_tile = [&](int i, int jc) {
         const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
@@ -171,6 +176,16 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                 const floatx4 v = buf_load_f32x4(w_rsrc, woff[sidx], soff);
                 stage[sidx] = (jc * JC + 4 * sc4[sidx] < p.J) ? v : zero;
+            }
+        } else if (ELEM) {
+            // rows that are not 16-byte aligned: single floats, consecutive lanes on consecutive
+            // columns (coalesced), a thread's floats NT / JC rows apart (scalar offsets)
+            const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
+            const bool inside = jc * JC + ecol < p.J;
+#pragma unroll
+            for (int e = 0; e < NE; ++e) {
+                const float v = buf_load_f32(w_rsrc, ebase, soff + (uint32_t)(e * (NT / JC)) * (uint32_t)p.sw1 * 4u);
+                stage[e / 4][e % 4] = inside ? v : 0.f;
             }
         } else {
 #pragma unroll
@@ -190,6 +205,11 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
         }
     };
     auto store_tile = [&](int buf) {
+        if (ELEM) {
+#pragma unroll
+            for (int e = 0; e < NE; ++e) wt[buf][(tid / JC + e * (NT / JC)) * LDW + ecol] = stage[e / 4][e % 4];
+            return;
+        }
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) *reinterpret_cast<floatx4 *>(&wt[buf][lds_off[sidx]]) = stage[sidx];
     };
@@ -387,6 +407,9 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
     const int cand[3] = {6, 3, 2};
     const int64_t penalty[3] = {100, 103, 109};
     for (int c = 0; c < 3; ++c) {
+        // rows of w that are not 16-byte aligned (J not a multiple of 4) are staged float by
+        // float, coalesced only for chunks that divide the workgroup evenly: 16 and 32
+        if (J % 4 != 0 && cand[c] != 2) continue;
         const int64_t cost = ceil_div(J, 8 * cand[c]) * 8 * cand[c] * penalty[c];
         if (cost < best) {
             best = cost;

@@ -135,6 +135,11 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 #pragma unroll
     for (int sidx = 0; sidx < SLOTS; ++sidx)
         woff[sidx] = ((uint32_t)srow[sidx] * (uint32_t)p.sw1 + 4u * (uint32_t)sc4[sidx]) * 4u;
+    // pair-wise staging of the unaligned build (chunks that divide the workgroup evenly)
+    constexpr bool ELEM = !VEC && (NT % (JC / 2) == 0) && ((TS * JC / 2) % NT == 0) && (TS * JC / 2 / NT <= 2 * SLOTS);
+    constexpr int NP = ELEM ? TS * JC / 2 / NT : 1;  // column pairs per thread
+    const int ecp = tid % (JC / 2);
+    const uint32_t ebase = ((uint32_t)(tid / (JC / 2)) * (uint32_t)p.sw1 + 2u * (uint32_t)ecp) * 4u;
     auto load_tile = [&](int i, int jc) __attribute__((always_inline)) {
         const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
         const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
@@ -149,6 +154,18 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                 const floatx4 v = buf_load_f32x4(w_rsrc, woff[sidx], soff);
                 stage[sidx] = (jc * JC + 4 * sc4[sidx] < p.J) ? v : zero;
+            }
+        } else if (ELEM) {
+            // rows that are not 16-byte aligned: a thread takes pairs of adjacent columns (one
+            // register of two bf16 per piece afterwards), consecutive lanes consecutive pairs, its
+            // pairs NT / (JC / 2) rows apart (scalar offsets); what lies past J reads as zero
+            const bool in0 = jc * JC + 2 * ecp < p.J, in1 = jc * JC + 2 * ecp + 1 < p.J;
+#pragma unroll
+            for (int e = 0; e < NP; ++e) {
+                const uint32_t so = soff + (uint32_t)(e * (2 * NT / JC)) * (uint32_t)p.sw1 * 4u;
+                const float v0 = buf_load_f32(w_rsrc, ebase, so), v1 = buf_load_f32(w_rsrc, ebase + 4u, so);
+                stage[e / 2][2 * (e % 2)] = in0 ? v0 : 0.f;
+                stage[e / 2][2 * (e % 2) + 1] = in1 ? v1 : 0.f;
             }
         } else {
             // ragged chunk or unaligned rows: element loads; what lies past J belongs to the
@@ -166,6 +183,17 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     };
     // split the staged fp32 values and write the pieces to LDS (8 bytes per piece and slot)
     auto store_tile = [&](int buf) __attribute__((always_inline)) {
+        if (ELEM) {
+#pragma unroll
+            for (int e = 0; e < NP; ++e) {
+                uint32_t pk[NS];
+                split_pair<NS, false>(stage[e / 2][2 * (e % 2)], stage[e / 2][2 * (e % 2) + 1], pk);
+                const int off = (tid / (JC / 2) + e * (2 * NT / JC)) * LDA + 2 * ecp;
+#pragma unroll
+                for (int sp = 0; sp < NS; ++sp) *reinterpret_cast<uint32_t *>(&wt[buf][sp][off]) = pk[sp];
+            }
+            return;
+        }
 #pragma unroll
         for (int sidx = 0; sidx < SLOTS; ++sidx) {
             uint32_t p01[NS], p23[NS];
@@ -410,7 +438,7 @@ using namespace trt;
 // When J is not a multiple of 4 every chunk takes element loads, which chunks of 16 bear worst
 // (1.9x per padded j over 50 random shapes; 32 and 48 cost 5 % more than 64).
 static int bf16_chunk(int64_t J, int pieces) {
-    const int64_t penalty[3][4] = {{135, 108, 102, 100}, {125, 104, 104, 100}, {190, 105, 106, 100}};
+    const int64_t penalty[3][4] = {{135, 108, 102, 100}, {125, 104, 104, 100}, {150, 105, 130, 100}};
     const int row = J % 4 != 0 ? 2 : (pieces == 2 ? 0 : 1);
     int best_ks = 4;
     int64_t best = 0;
