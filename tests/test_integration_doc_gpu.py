@@ -1,4 +1,5 @@
-"""The reference-side binding shown in INTEGRATION.md is executed as written: the first python
+"""The reference-side binding shown in the integration guide at the repository root is executed as
+written: the first python
 block (the lm2exp stub) and the second (the lt2exp fragment) must run against the built library
 and reproduce the package's own results."""
 
