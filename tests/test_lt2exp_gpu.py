@@ -20,7 +20,7 @@ from triturus_amd import _lib, workloads
 pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
-N_VARIANTS = 16
+N_VARIANTS = 18
 N_BF16_VARIANTS = 16  # 1..4, 9..12 tiles; 5..8, 13..16 the same tiles with the contraction cut over workgroups
 # Accuracy gates of the split-bf16 paths against the float64 oracle.  Two pieces (3 MFMAs per
 # product) carry 16 significand bits: looser than fp32, ten times tighter than the rtol 5e-4
@@ -69,7 +69,9 @@ def test_golden(dev, name, mode):
 @pytest.mark.parametrize("variant", range(1, N_VARIANTS + 1))
 @pytest.mark.parametrize("mode", ["unsplit", "split"])
 @pytest.mark.parametrize("shape", [(2, 35, 9, 13, 45), (1, 70, 20, 33, 300), (2, 16, 5, 72, 64), (1, 33, 3, 3, 31),
-                                   (2, 40, 6, 48, 100), (1, 33, 5, 24, 70), (1, 65, 3, 16, 64), (1, 20, 4, 100, 130)])
+                                   (2, 40, 6, 48, 100), (1, 33, 5, 24, 70), (1, 65, 3, 16, 64), (1, 20, 4, 100, 130),
+                                   # short rows of w that pack into chunks of 16 (variants 17, 18; last chunk ragged)
+                                   (2, 70, 37, 8, 150), (2, 40, 50, 2, 100), (1, 33, 9, 4, 70), (1, 65, 64, 4, 40)])
 def test_every_tile_variant_on_ragged_shapes(dev, variant, mode, shape):
     assert _lib.load().trt_lt2exp_variant_count() == N_VARIANTS
     R, S, I, J, K = shape
@@ -88,7 +90,9 @@ def test_every_tile_variant_on_ragged_shapes(dev, variant, mode, shape):
     [(1, 1, 1, 1, 1), (2, 1, 3, 1, 5), (1, 3, 1, 4, 1), (1, 65, 2, 2, 257), (3, 8, 64, 4, 40), (1, 8, 4, 64, 40),
      (1, 129, 17, 65, 33), (1, 4, 300, 3, 16), (1, 4, 3, 300, 16),
      # a short j axis under a long i axis runs with the roles of (i, a) and (j, b) exchanged
-     (2, 40, 150, 1, 200), (2, 40, 150, 2, 300), (1, 20, 64, 8, 260), (3, 33, 37, 5, 257), (1, 20, 16, 8, 300)],
+     (2, 40, 150, 1, 200), (2, 40, 150, 2, 300), (1, 20, 64, 8, 260), (3, 33, 37, 5, 257), (1, 20, 16, 8, 300),
+     # short rows that pack (J = 2, 4, 8 with I*J a multiple of 4), and one that does not (I*J = 6)
+     (2, 100, 193, 8, 145), (1, 40, 77, 4, 130), (2, 70, 22, 2, 99), (1, 8, 3, 2, 40), (1, 8, 4, 8, 40)],
 )
 @pytest.mark.parametrize("mode", ["auto", "split"])
 def test_edge_shapes(dev, shape, mode):

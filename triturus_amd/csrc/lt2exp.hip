@@ -38,8 +38,13 @@ struct Lt2Args {
 
 // WM: wavefronts stacked over rows (1: all NWAVES side by side over columns; 2 or 4 for narrow
 // outputs, so that K <= 64 or 32 does not leave most of them idle).
-template <int RT, int CT, int NQ, int NWAVES, bool VEC, bool SPLIT, int WM = 1>
+// PJ: packed short rows.  With J = 2, 4 or 8 a chunk of 16 values of j would be mostly padding;
+// w is contiguous over (i, j), so the kernel walks that flat axis in chunks of 16 instead: a chunk
+// holds 16 / PJ values of i, and MFMA slot f = 8q + 4h + u of it multiplies exp a[i0 + f / PJ]
+// by exp b[f % PJ] (the factors of b are the same in every chunk).
+template <int RT, int CT, int NQ, int NWAVES, bool VEC, bool SPLIT, int WM = 1, int PJ = 0>
 __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args p) {
+    static_assert(PJ == 0 || (VEC && NQ == 2 && (PJ == 2 || PJ == 4 || PJ == 8)), "packed rows: chunks of 16");
     constexpr int NT = NWAVES * kWave;
     constexpr int WN = NWAVES / WM;
     constexpr int TS = 32 * RT * WM;      // rows of S per workgroup
@@ -109,8 +114,9 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
         mb[ct] = clamp_shift(y);
     }
 
-    const int n_jc = (p.J + JC - 1) / JC;
-    const int total_iters = n_jc * p.I;
+    const int n_jc = PJ ? 1 : (p.J + JC - 1) / JC;
+    const int n_i = PJ ? (p.I * p.J + JC - 1) / JC : p.I;  // steps per j-chunk (packed: flat chunks over (i, j))
+    const int total_iters = n_jc * n_i;
     int it = split * p.iters_per_split;
     int it_end = it + p.iters_per_split;
     if (it_end > total_iters) it_end = total_iters;
@@ -162,20 +168,23 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     const uint32_t ebase = ((uint32_t)(tid / JC) * (uint32_t)p.sw1 + (uint32_t)ecol) * 4u;
     // (a slot past the tile loads some valid or out-of-extent address: the value is never used)
     auto load_tile = [&](int i, int jc) {
-        const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
+        // floats of the chunk that belong to this step (packed: of the flat (i, j) axis)
+        const int left = PJ ? p.I * p.J - i * JC : p.J - jc * JC;
+        const int step = PJ ? JC : p.J;
+        const bool full = VEC && left >= JC;  // wave-uniform
         if (full) {
-            const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
+            const uint32_t soff = (uint32_t)(i * step + jc * JC) * 4u;
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) stage[sidx] = buf_load_f32x4(w_rsrc, woff[sidx], soff);
         } else if (VEC) {
             // ragged last chunk of aligned rows (J is a multiple of 4): a 16-byte piece is whole
             // or lies past J, where the next i begins: zeros instead
-            const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
+            const uint32_t soff = (uint32_t)(i * step + jc * JC) * 4u;
 #pragma unroll
             for (int sidx = 0; sidx < SLOTS; ++sidx) {
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                 const floatx4 v = buf_load_f32x4(w_rsrc, woff[sidx], soff);
-                stage[sidx] = (jc * JC + 4 * sc4[sidx] < p.J) ? v : zero;
+                stage[sidx] = (4 * sc4[sidx] < left) ? v : zero;
             }
         } else if (ELEM) {
             // rows that are not 16-byte aligned: single floats, consecutive lanes on consecutive
@@ -229,22 +238,53 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
             for (int q = 0; q < NQ; ++q)
 #pragma unroll
                 for (int u = 0; u < 4; ++u) {
-                    const int j = jc * JC + 8 * q + 4 * h + u;
+                    const int j = PJ ? (8 * q + 4 * h + u) % (PJ ? PJ : 1) : jc * JC + 8 * q + 4 * h + u;
                     float raw = -__builtin_inff();
                     if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl[ct]];
                     eb[ct][4 * q + u] = exp_shifted(raw - mb[ct]);
                 }
     };
 
-    float ea[CT], ea_raw[CT];
+    // Factors of a per step: one (row i); packed, one per value of i in the chunk that this
+    // lane's slots meet: slot f = 8q + 4h + u lies in row f / PJ of the chunk.
+    constexpr int EA_N = PJ == 0 ? 1 : (PJ == 2 ? 2 * NQ : NQ);
+    constexpr int RPC = PJ ? JC / PJ : 1;  // rows of a per step
+    float ea[CT][EA_N], ea_raw[CT][EA_N];
+    int erow[EA_N];
+#pragma unroll
+    for (int e = 0; e < EA_N; ++e) erow[e] = PJ == 8 ? e : (PJ == 4 ? 2 * e + h : (PJ == 2 ? 4 * (e / 2) + 2 * h + e % 2 : 0));
+    // (packed: the last chunk may reach past row I - 1: the address is clamped, the factor zero)
+    auto load_ea = [&](int i) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int e = 0; e < EA_N; ++e) {
+                if (PJ) {
+                    int row = i * RPC + erow[e];
+                    row = row < p.I ? row : p.I - 1;
+                    ea_raw[ct][e] = buf_load_f32(a_rsrc, aoff[ct] + (uint32_t)row * a_row_bytes, 0u);
+                } else {
+                    ea_raw[ct][e] = buf_load_f32(a_rsrc, aoff[ct], (uint32_t)i * a_row_bytes);
+                }
+            }
+    };
+    auto finish_ea = [&](int i) {
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+            for (int e = 0; e < EA_N; ++e) {
+                const float x = exp_shifted(ea_raw[ct][e] - ma[ct]);
+                ea[ct][e] = (PJ == 0 || i * RPC + erow[e] < p.I) ? x : 0.f;
+            }
+    };
 
     if (it < it_end) {
-        int jc = it / p.I;
-        int i = it - jc * p.I;
+        int jc = it / n_i;
+        int i = it - jc * n_i;
         load_tile(i, jc);
         load_eb(jc);
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) ea[ct] = exp_shifted(ar[(int64_t)i * p.sa1 + ncl[ct]] - ma[ct]);
+        load_ea(i);
+        finish_ea(i);
         store_tile(0);
         __syncthreads();
 
@@ -260,7 +300,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
                 for (int u = 0; u < 4; ++u) {
 #pragma unroll
                     for (int ct = 0; ct < CT; ++ct) {
-                        const float bop = ea[ct] * eb[ct][4 * q + u];
+                        const float bop = ea[ct][PJ == 2 ? 2 * q + u / 2 : (PJ ? q : 0)] * eb[ct][4 * q + u];
 #pragma unroll
                         for (int rt = 0; rt < RT; ++rt)
                             acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[rt][u], bop, acc[rt][ct], 0, 0, 0);
@@ -275,19 +315,17 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
         int cur = 0;
         for (; it + 1 < it_end; ++it) {
             int ni = i + 1, njc = jc;
-            if (ni == p.I) {
+            if (ni == n_i) {
                 ni = 0;
                 njc = jc + 1;
             }
             load_tile(ni, njc);
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) ea_raw[ct] = buf_load_f32(a_rsrc, aoff[ct], (uint32_t)ni * a_row_bytes);
+            load_ea(ni);
             __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block, not sunk into it
             mfma_block(wt[cur] + wrow0 * LDW);
             store_tile(cur ^ 1);
             if (njc != jc) load_eb(njc);
-#pragma unroll
-            for (int ct = 0; ct < CT; ++ct) ea[ct] = exp_shifted(ea_raw[ct] - ma[ct]);
+            finish_ea(ni);
             __syncthreads();
             cur ^= 1;
             i = ni;
@@ -343,7 +381,8 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 // ------------------------------------------------------------------ host
 struct Lt2Variant {
     int rt, ct, nq;
-    int wm = 1;  // wavefronts stacked over rows
+    int wm = 1;     // wavefronts stacked over rows
+    bool pack = false;  // J = 2, 4 or 8: chunks of 16 over the flat (i, j) axis
 };
 // variant ids (1-based in the C ABI; 0 = choose by shape)
 static const Lt2Variant kVariants[] = {
@@ -363,6 +402,8 @@ static const Lt2Variant kVariants[] = {
     {2, 1, 6},
     {1, 1, 4, 4},  // 15: 128 x 32 tile, the 4 wavefronts stacked over rows (outputs of <= 32 columns)
     {1, 1, 4, 2},  // 16: 64 x 64 tile (outputs of <= 64 columns)
+    {1, 1, 2, 1, true},  // 17, 18: short rows of w packed into chunks of 16 (other shapes: as 9 and 12)
+    {2, 1, 2, 1, true},
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLt2Waves = 4;
@@ -379,6 +420,20 @@ constexpr int kLt2Waves = 4;
 // 160, 208).  (96- and 128-row tiles were measured too: per 32 rows they cost what the 32-row
 // tile does.)  Rule checked against the better of the two tiles on those shapes: 0.6 % mean
 // regret, 2 shapes of 288 more than 10 % off.
+// Short rows that pack: whole rows per chunk of 16, 16-byte pieces that do not straddle the end
+// of the flat axis, and more than one chunk.
+static bool packs(int64_t I, int64_t J) {
+    return (J == 2 || J == 4 || J == 8) && (I * J) % 4 == 0 && I * J >= 32;
+}
+
+static int find_lt2_variant(int rt, int nq, bool pack) {
+    for (int v = 0; v < kNumVariants; ++v)
+        if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == nq && kVariants[v].wm == 1 &&
+            kVariants[v].pack == pack)
+            return v;
+    return 0;
+}
+
 static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
     // Outputs of at most 32 (64) columns would leave three (two) of the four wavefronts idle:
     // they are stacked over rows instead (128 x 32 and 64 x 64 tiles).
@@ -396,12 +451,17 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
         const bool same_padding = last == 0 || last > 32;
         const int64_t n64 = R * ceil_div(S, 64) * ceil_div(K, 128);
         if (same_padding && I * J >= 4096 && n64 >= 256) rt = 2;
+        // packed rows spend more vector instructions per step (a factor of a per row of the chunk):
+        // sharing them between two MFMAs pays from half a wave of workgroups on, whatever the
+        // length of the contraction (measured: 6-13 % at 128..2048 tiles, 15 % behind at 20)
+        if (same_padding && packs(I, J) && n64 >= 128) rt = 2;
     }
     // j-chunk: the one that pads J least.  Per padded j the chunks cost the same within a few
     // per cent (measured at S = I = 64, K = 4096, R = 64: 15.3 us per j with chunks of 32 or 48,
     // 15.5-16.5 with 16, 15.5-16.1 with 24), so J = 16, 24, 40, 48, 72 run 1.3-2.2x faster on
     // chunks that fit than on chunks of 32 (J = 48: 1059 -> 735 us), also because a last chunk
     // that is only partly filled takes the masked loads.  Ties go to chunks of 32.
+    if (packs(I, J)) return find_lt2_variant(rt, 2, true);
     int nq = 4;
     int64_t best = ceil_div(J, 32) * 32 * 100;
     const int cand[3] = {6, 3, 2};
@@ -416,9 +476,7 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
             nq = cand[c];
         }
     }
-    for (int v = 0; v < kNumVariants; ++v)
-        if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == nq && kVariants[v].wm == 1) return v;
-    return 0;
+    return find_lt2_variant(rt, nq, false);
 }
 
 template <int RT, int CT, int NQ, bool VEC, bool SPLIT, int WM>
@@ -438,7 +496,29 @@ static void launch_vs(const Lt2Args &args, bool vec, bool split, hipStream_t str
     }
 }
 
+template <int RT, int PJ>
+static void launch_packed_pj(const Lt2Args &args, bool split, hipStream_t stream) {
+    if (split)
+        hipLaunchKernelGGL((lt2exp_kernel<RT, 1, 2, kLt2Waves, true, true, 1, PJ>), dim3((unsigned)args.padded_wgs),
+                           dim3(kLt2Waves * kWave), 0, stream, args);
+    else
+        hipLaunchKernelGGL((lt2exp_kernel<RT, 1, 2, kLt2Waves, true, false, 1, PJ>), dim3((unsigned)args.padded_wgs),
+                           dim3(kLt2Waves * kWave), 0, stream, args);
+}
+
+template <int RT>
+static void launch_packed(const Lt2Args &args, bool split, hipStream_t stream) {
+    if (args.J == 8) launch_packed_pj<RT, 8>(args, split, stream);
+    else if (args.J == 4) launch_packed_pj<RT, 4>(args, split, stream);
+    else launch_packed_pj<RT, 2>(args, split, stream);
+}
+
 static void launch_variant(int v, const Lt2Args &args, bool vec, bool split, hipStream_t stream) {
+    if (kVariants[v].pack) {
+        if (kVariants[v].rt == 2) launch_packed<2>(args, split, stream);
+        else launch_packed<1>(args, split, stream);
+        return;
+    }
     switch (v) {
         case 0: launch_vs<2, 2, 8>(args, vec, split, stream); break;
         case 1: launch_vs<2, 2, 4>(args, vec, split, stream); break;
@@ -471,7 +551,7 @@ struct SplitPlan {
 // iterations, is 1.4x slower split; R=32 S=I=J=48..256 K=256 is 1.3-2.8x faster).
 static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode, int variant) {
     const Lt2Variant &v = kVariants[variant];
-    const int64_t iters = ceil_div(J, 8 * v.nq) * I;
+    const int64_t iters = v.pack ? ceil_div(I * J, 8 * v.nq) : ceil_div(J, 8 * v.nq) * I;
     if (mode == TRT_MODE_UNSPLIT) return {false, 1, (int)iters};
     const int64_t base = R * ceil_div(S, 32 * v.rt * v.wm) * ceil_div(K, 32 * v.ct * (kLt2Waves / v.wm));
     int64_t splits = choose_splits(base, iters, 4 * v.nq * v.rt * v.ct, R * S * K, 4, 32, mode == TRT_MODE_SPLIT);
@@ -538,7 +618,10 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
         return trt_lt2exp_f32(w, b, a, c, R, S, 1, I, K, sw, sb, sa, sc, mode, variant, workspace, workspace_bytes,
                               stream);
 
-    const int v = resolve_variant(variant, R, S, I, J, K);
+    int v = resolve_variant(variant, R, S, I, J, K);
+    const bool w_aligned = (sw[0] % 4 == 0) && (sw[1] % 4 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
+    // packed rows need 16-byte loads along the flat (i, j) axis; any other call runs the same tile unpacked
+    if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
     const Lt2Variant &vr = kVariants[v];
     const SplitPlan sp = plan_split(R, S, I, J, K, mode, v);
 
@@ -566,8 +649,7 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
         args.shift = args.c + (size_t)sp.splits * R * S * K;
     }
     // 16-byte loads of w need aligned rows
-    const bool vec = (J % 4 == 0) && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) &&
-                     ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
+    const bool vec = (J % 4 == 0) && w_aligned;
     hipStream_t s = static_cast<hipStream_t>(stream);
     launch_variant(v, args, vec, sp.split, s);
     if (sp.split) launch_lt2exp_merge(args.c, args.shift, c, R, S, K, sp.splits, sc[0], sc[1], s);

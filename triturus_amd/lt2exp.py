@@ -39,7 +39,7 @@ def launches_split(R: int, S: int, I: int, J: int, K: int, mode: str) -> bool:
 
 _PIECES = {"bf16x3": 2, "bf16x6": 3}
 # tile variants worth timing when tuning is on (0 = the library's rule)
-_FP32_CANDIDATES = (0, 5, 6, 8, 9, 10, 11, 12, 13, 14)
+_FP32_CANDIDATES = (0, 5, 6, 8, 9, 10, 11, 12, 13, 14, 17, 18)
 _BF16_CANDIDATES = (0, 1, 2, 3, 4, 9, 10, 11, 12)
 
 
@@ -53,6 +53,11 @@ _PAD_MIN_K = 1024
 def _padded(n: int) -> int:
     """Length of a contracted axis of n once padded to whole j-chunks of the size that fits it best."""
     return min(-(-n // c) * c for c in (16, 24, 32, 48))
+
+
+def _packs(I: int, J: int) -> bool:
+    """Rows of w short enough for the fp32 kernel to walk (i, j) as one flat axis (no padding of j)."""
+    return J in (2, 4, 8) and (I * J) % 4 == 0 and I * J >= 32
 
 
 def lt2exp(
@@ -85,8 +90,13 @@ def lt2exp(
     # long i axis wastes most of every chunk.  The contraction is symmetric in (i, a) and (j, b),
     # so such a call runs with the roles exchanged on a transposed copy of w (J = 1 needs no
     # copy: the library does that exchange itself), when that saves a third of the padded work
-    # and the output is wide enough for the copy not to matter.  Not for forced tiles (tests, tuning).
-    if (_variant == 0 and 2 <= J < I and K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
+    # and the output is wide enough for the copy not to matter.  Not for forced tiles (tests, tuning),
+    # nor where the fp32 kernel packs the short rows itself.
+    if _precision is None:
+        _precision = matrix_precision()
+    elif _precision not in MATRIX_PRECISIONS:
+        raise ValueError(f"unknown matrix precision {_precision!r}")
+    if (_variant == 0 and 2 <= J < I and not (_precision == "fp32" and _packs(I, J)) and K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
             and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS):  # worth a copy kernel: some 40 us of work
         w = w.view(R, S, I, J).transpose(2, 3).contiguous().view(R, S, I * J)
         a, b = b, a
@@ -104,10 +114,6 @@ def lt2exp(
     w = _unit_inner(w)
     a = _unit_inner(a)
     b = _unit_inner(b)
-    if _precision is None:
-        _precision = matrix_precision()
-    elif _precision not in MATRIX_PRECISIONS:
-        raise ValueError(f"unknown matrix precision {_precision!r}")
     if _variant == 0 and autotune.is_autotune_enabled() and not _tuning:
         cands = _FP32_CANDIDATES if _precision == "fp32" else _BF16_CANDIDATES
         _variant = autotune.pick(("lt2exp", R, S, I, J, K, mode, _precision), cands,
