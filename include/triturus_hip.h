@@ -97,6 +97,11 @@ int trt_lm2exp_variant_count(void);
  * the contracted (i,j) range over several workgroups and merges the partial
  * sums deterministically; it needs a workspace of
  * trt_lt2exp_workspace_bytes(...) bytes (UNSPLIT needs none: pass NULL, 0).
+ * variant: 0 = choose by shape; 1..trt_lt2exp_variant_count() force a tile shape
+ * and j-chunk (tests, tuning).  With J = 1 and variant 0 the call runs with the
+ * roles of (i, a) and (j, b) exchanged; with J = 2, 4 or 8, I*J a multiple of 4
+ * and 16-byte aligned rows of w (base, sw[0], sw[1]) the kernel walks (i, j) as
+ * one flat axis, so short rows cost no padding.
  */
 int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c,
                    int64_t R, int64_t S, int64_t I, int64_t J, int64_t K,
