@@ -507,6 +507,14 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
         return trt_lt2exp_bf16(w, b, a, c, R, S, 1, I, K, sw, sb, sa, sc, pieces, mode, variant, workspace,
                                workspace_bytes, stream);
 
+    // Rows of w of 2 or 4 values fill an eighth or a quarter of this kernel's smallest j-chunk;
+    // the fp32 kernel walks such rows packed, without padding (measured 1.4-2.5x ahead on
+    // R=64 S=64 I=64..128 K=200, R=20 S=200 I=300 K=128; rows of 8: level with two pieces,
+    // 5-20 % ahead of three).  Same conditions as trt_lt2exp_f32 applies.
+    if (variant == 0 && (J == 2 || J == 4 || (J == 8 && pieces == 3)) && (I * J) % 4 == 0 && I * J >= 32 &&
+        sw[0] % 4 == 0 && sw[1] % 4 == 0 && (reinterpret_cast<uintptr_t>(w) & 15) == 0)
+        return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
+
     // Tile and hand-over rules, fitted to 290 random shapes (R 1..128, S 16..512, I, J 8..128,
     // K 64..8192) timed with every tile and on the fp32 path; against the best of those the
     // rules below lose 2.5 % (two pieces) / 1.9 % (three) on average, the previous ones 17 / 14 %.
