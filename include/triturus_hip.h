@@ -124,7 +124,8 @@ int trt_lt2exp_variant_count(void);
  * (2^-11) and several times faster than the fp32 matrix pipe.  The call takes the same mode
  * and workspace (trt_lt2exp_workspace_bytes) as trt_lt2exp_f32: with variant 0 a grid too
  * small to be matrix bound has its contraction cut over workgroups (as the mode and the
- * workspace allow) or is handed to trt_lt2exp_f32.  variant: 0 = choose by shape, 1..4 and
+ * workspace allow) or is handed to trt_lt2exp_f32, and so are rows of w of 2 or 4 values
+ * (8 with three pieces) that the fp32 kernel packs.  variant: 0 = choose by shape, 1..4 and
  * 9..12 force a bf16 tile shape, 5..8 and 13..16 the same tiles with the contraction cut
  * (experiments, tests).
  */
