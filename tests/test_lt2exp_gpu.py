@@ -109,15 +109,18 @@ def test_edge_shapes(dev, shape, mode):
 
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
 @pytest.mark.parametrize("shape", [(2, 40, 150, 2, 300), (1, 20, 64, 8, 260), (2, 33, 21, 7, 257), (2, 35, 9, 13, 45),
-                                   (1, 70, 20, 33, 300), (2, 16, 5, 50, 64)])
+                                   (1, 70, 20, 33, 300), (2, 16, 5, 50, 64), (2, 40, 30, 3, 100), (1, 70, 9, 5, 64),
+                                   (2, 33, 11, 6, 130)])
 def test_reshaping_front_ends(dev, precision, shape, monkeypatch):
     """The wrapper's two front ends -- roles of (i, a) and (j, b) exchanged on a transposed copy
-    of w for a short j axis, and w / b padded to a multiple of 4 in J -- with their work
+    of w for a short j axis, and w / b padded to a multiple of 4 in J (for aligned rows, or for
+    short rows that then pack) -- with their work
     thresholds lowered so that small inputs take them: same results, -inf and zero weights included."""
     import triturus_amd.lt2exp as mod
 
     monkeypatch.setattr(mod, "_RESHAPE_MIN_FLOPS", 0.0)
     monkeypatch.setattr(mod, "_PAD_MIN_K", 1)
+    monkeypatch.setattr(mod, "_PACK_PAD_MIN_FLOPS", 0.0)
     R, S, I, J, K = shape
     g = torch.Generator().manual_seed(sum(shape))
     w = torch.rand(R, S, I, J, generator=g)

@@ -48,6 +48,7 @@ _BF16_CANDIDATES = (0, 1, 2, 3, 4, 9, 10, 11, 12)
 # J to a multiple of 4 pays.
 _RESHAPE_MIN_FLOPS = 4e9
 _PAD_MIN_K = 1024
+_PACK_PAD_MIN_FLOPS = 2e10  # padded work from which rows of 3, 5, 6, 7 are worth padding to 4 or 8 (fp32)
 
 
 def _padded(n: int) -> int:
@@ -96,7 +97,8 @@ def lt2exp(
         _precision = matrix_precision()
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
-    if (_variant == 0 and 2 <= J < I and not (_precision == "fp32" and _packs(I, J)) and K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
+    packed = _precision == "fp32" and _packs(I, J)
+    if (_variant == 0 and 2 <= J < I and not packed and K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
             and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS):  # worth a copy kernel: some 40 us of work
         w = w.view(R, S, I, J).transpose(2, 3).contiguous().view(R, S, I * J)
         a, b = b, a
@@ -108,6 +110,15 @@ def lt2exp(
     if (_variant == 0 and J % 4 != 0 and J > 4 and K >= _PAD_MIN_K
             and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS):
         J4 = J + (-J) % 4
+        w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
+        b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
+        J = J4
+    # Rows of 3, 5, 6 or 7 fill a fifth to a half of a j-chunk; padded to 4 or 8 the fp32 kernel
+    # packs them (measured R=86 S=482 I=193 K=145: J = 3 574 -> 244 us, J = 5..7 576-594 -> 453-480;
+    # at a tenth of that work the copies cost more than they save).
+    if (_variant == 0 and _precision == "fp32" and J in (3, 5, 6, 7) and I * (4 if J == 3 else 8) >= 32
+            and 2 * R * S * I * 16 * K >= _PACK_PAD_MIN_FLOPS):
+        J4 = 4 if J == 3 else 8
         w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
         b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
         J = J4
