@@ -37,7 +37,7 @@ PEAK_BF16_MFMA_TFLOPS = 2516.6  # 16x the fp32 matrix rate
 # each over `bench.py --profile-pass`), scaled by what the same counters read for
 # trt_copy_bytes of 256 MiB (factors 2.000 and 1.000 to KiB); the summary of those runs is
 # profiles/lt2exp_lm2exp_max_counters.md.  A constant, not a live measurement.
-MEASURED_TRAFFIC_BYTES = {"lt2exp_c5": 453.0e6, "lm2exp_c3": 681.8e6}
+MEASURED_TRAFFIC_BYTES = {"lt2exp_c5": 452.9e6, "lm2exp_c3": 682.4e6}
 
 
 def log(*a):

@@ -171,7 +171,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
         // floats of the chunk that belong to this step (packed: of the flat (i, j) axis)
         const int left = PJ ? p.I * p.J - i * JC : p.J - jc * JC;
         const int step = PJ ? JC : p.J;
-        const bool full = VEC && left >= JC;  // wave-uniform
+        const bool full = VEC && (PJ ? left >= JC : jc * JC + JC <= p.J);  // wave-uniform
         if (full) {
             const uint32_t soff = (uint32_t)(i * step + jc * JC) * 4u;
 #pragma unroll
@@ -184,7 +184,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
             for (int sidx = 0; sidx < SLOTS; ++sidx) {
                 const floatx4 zero = {0.f, 0.f, 0.f, 0.f};
                 const floatx4 v = buf_load_f32x4(w_rsrc, woff[sidx], soff);
-                stage[sidx] = (4 * sc4[sidx] < left) ? v : zero;
+                stage[sidx] = (PJ ? 4 * sc4[sidx] < left : jc * JC + 4 * sc4[sidx] < p.J) ? v : zero;
             }
         } else if (ELEM) {
             // rows that are not 16-byte aligned: single floats, consecutive lanes on consecutive
