@@ -82,6 +82,12 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, s3(1, 1, 2), ok, 0, 0, null, 0, null) == -2
     big4 = (2, 8, 16, 16, 64, s3(2048, 256, 1), s3(1024, 64, 1), s3(1024, 64, 1), s3(512, 64, 1))
     assert lib.trt_lt2exp_f32(one, one, one, one, *big4, _lib.MODE_SPLIT, 0, null, 0, null) == -3  # split needs a workspace
+    assert lib.trt_lt2exp_f32(one, one, one, one, *args, 0, lib.trt_lt2exp_variant_count() + 1, null, 0, null) == -1
+    # short rows of w (J = 8) walked packed: a forced split still asks for its workspace
+    packed = (2, 64, 256, 8, 64, s3(64 * 2048, 2048, 1), s3(256 * 64, 64, 1), s3(8 * 64, 64, 1), s3(64 * 64, 64, 1))
+    assert lib.trt_lt2exp_workspace_bytes(2, 64, 256, 8, 64, _lib.MODE_SPLIT) > 0
+    assert lib.trt_lt2exp_f32(one, one, one, one, *packed, _lib.MODE_SPLIT, 0, null, 0, null) == -3
+    assert lib.trt_lt2exp_bf16(one, one, one, one, *packed, 3, _lib.MODE_SPLIT, 0, null, 0, null) == -3  # handed to fp32
     # lt2exp on the bf16 matrix pipe: pieces must be 2 or 3, variant 0..4
     btail = (0, 0, null, 0, null)  # mode, variant, workspace, bytes, stream
     assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 4, *btail) == -1
@@ -285,3 +291,14 @@ def test_product_never_imports_the_oracle():
             if f.suffix in {".py", ".hip", ".hpp", ".h"}:
                 text = f.read_text()
                 assert "oracle" not in text.replace("the oracle the reference tests use", ""), f
+
+
+def test_short_row_rule_of_the_lt2exp_wrapper():
+    """Rows of w that the fp32 kernel packs: 2, 4 or 8 values, a whole number of 16-byte pieces in
+    all, more than one chunk of 16."""
+    from triturus_amd.lt2exp import _packs
+
+    assert _packs(193, 8) and _packs(64, 4) and _packs(50, 2)
+    assert not _packs(3, 2)        # 6 floats: not a multiple of 4
+    assert not _packs(2, 8)        # a single chunk
+    assert not _packs(64, 16) and not _packs(64, 3) and not _packs(64, 1)
