@@ -439,8 +439,10 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
     // they are stacked over rows instead (128 x 32 and 64 x 64 tiles).
     // (No lower bound on the number of tiles as lm2exp has: tried, 1.4-2x slower on grids of 64
     // narrow tiles -- a tile's chain of I x J steps is long enough to keep its CU busy.)
+    // (Not for short rows that pack: padding such rows to a chunk of 32 costs more than the idle
+    // wavefronts -- the packed 128-column tile is 1.1-5x ahead at K = 16..64, J = 2, 4, 8.)
     const bool tall = K <= 32 && S > 64;
-    if (tall || (K <= 64 && S > 32)) {
+    if (!packs(I, J) && (tall || (K <= 64 && S > 32))) {
         const int wm = tall ? 4 : 2;
         for (int v = 0; v < kNumVariants; ++v)
             if (kVariants[v].wm == wm) return v;
@@ -453,8 +455,9 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
         if (same_padding && I * J >= 4096 && n64 >= 256) rt = 2;
         // packed rows spend more vector instructions per step (a factor of a per row of the chunk):
         // sharing them between two MFMAs pays from half a wave of workgroups on, whatever the
-        // length of the contraction (measured: 6-13 % at 128..2048 tiles, 15 % behind at 20)
-        if (same_padding && packs(I, J) && n64 >= 128) rt = 2;
+        // length of the contraction (measured: 6-13 % at 256..2048 tiles, level at 192, from 4 %
+        // ahead to 20 % behind at 128, 15 % behind at 20)
+        if (same_padding && packs(I, J) && n64 >= 192) rt = 2;
     }
     // j-chunk: the one that pads J least.  Per padded j the chunks cost the same within a few
     // per cent (measured at S = I = 64, K = 4096, R = 64: 15.3 us per j with chunks of 32 or 48,
