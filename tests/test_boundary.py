@@ -261,6 +261,48 @@ def test_flags():
     assert torch.equal(x, torch.rand(3))
 
 
+def test_flags_write_the_torch_settings_the_reference_writes():
+    """triturus/utils.py:26-30,33-48: the flag functions also set torch's own matmul precision,
+    its two allow_tf32 backends, and (with determinism) cudnn benchmarking, the BLAS workspace
+    variable and the dynamo recompile limit."""
+    import os
+
+    from triturus.utils import is_torch_tf32_enabled as shim_fn
+    from triturus_amd.utils import is_torch_tf32_enabled
+
+    assert shim_fn is is_torch_tf32_enabled
+    before = (torch.get_float32_matmul_precision(), torch.backends.cuda.matmul.allow_tf32,
+              torch.backends.cudnn.allow_tf32, torch.backends.cudnn.benchmark,
+              torch.are_deterministic_algorithms_enabled(), torch.is_deterministic_algorithms_warn_only_enabled(),
+              os.environ.get("CUBLAS_WORKSPACE_CONFIG"))
+    try:
+        set_tf32_enabled(True)
+        assert torch.get_float32_matmul_precision() == "high"
+        assert torch.backends.cuda.matmul.allow_tf32 is True and torch.backends.cudnn.allow_tf32 is True
+        assert is_torch_tf32_enabled() is True and is_triturus_tf32_enabled()
+        set_tf32_enabled(False)
+        assert torch.get_float32_matmul_precision() == "highest"
+        assert torch.backends.cuda.matmul.allow_tf32 is False and torch.backends.cudnn.allow_tf32 is False
+        assert is_torch_tf32_enabled() is False and not is_triturus_tf32_enabled()
+        torch.backends.cudnn.benchmark = True
+        ensure_reproducibility(seed=3, determinism=True, device="cpu")
+        assert torch.are_deterministic_algorithms_enabled()
+        assert torch.backends.cudnn.benchmark is False
+        assert os.environ["CUBLAS_WORKSPACE_CONFIG"] == ":16:8"
+        assert torch._dynamo.config.recompile_limit == 64
+    finally:
+        torch.set_float32_matmul_precision(before[0])
+        torch.backends.cuda.matmul.allow_tf32 = before[1]
+        torch.backends.cudnn.allow_tf32 = before[2]
+        torch.backends.cudnn.benchmark = before[3]
+        torch.use_deterministic_algorithms(before[4], warn_only=before[5])
+        if before[6] is None:
+            os.environ.pop("CUBLAS_WORKSPACE_CONFIG", None)
+        else:
+            os.environ["CUBLAS_WORKSPACE_CONFIG"] = before[6]
+        set_tf32_enabled(False)
+
+
 def test_tile_tuning_is_off_by_default():
     from triturus_amd import autotune
 

@@ -12,10 +12,16 @@ explicitly: "fp32", "bf16x3", or "bf16x6" (three pieces, six MFMAs, ~2^-23 per
 product: as accurate as the fp32 pipe and faster); ``None`` follows the flag.
 ``ensure_reproducibility`` (triturus/utils.py:12-30) seeds python, numpy and
 torch and makes the GPU the default device when one is present.
+Both functions also write the same torch-side settings as the reference
+(float32 matmul precision and the two ``allow_tf32`` backends; cudnn
+benchmarking, the BLAS workspace variable and the dynamo recompile limit), so
+that torch code run beside these kernels -- the "torch" line of a benchmark --
+computes under the same settings as it does beside the reference.
 """
 
 from __future__ import annotations
 
+import os
 import random
 
 import numpy as np
@@ -44,11 +50,32 @@ def ensure_reproducibility(
         # every kernel of this library is deterministic (fixed summation order,
         # no atomics); the flag only concerns torch's own ops
         torch.use_deterministic_algorithms(True, warn_only=True)
+        torch.backends.cudnn.benchmark = False
+        os.environ["CUBLAS_WORKSPACE_CONFIG"] = ":16:8"
+    try:  # triturus/utils.py:30
+        torch._dynamo.config.recompile_limit = 64
+    except Exception:  # a torch build without dynamo: nothing to configure
+        pass
 
 
 def set_tf32_enabled(allow_tf32: bool) -> None:
+    """triturus/utils.py:33-44: the library's own flag and torch's matmul settings together."""
     global _TRITURUS_TF32_ENABLED
-    _TRITURUS_TF32_ENABLED = bool(allow_tf32)
+    if allow_tf32:
+        torch.set_float32_matmul_precision("high")
+        torch.backends.cuda.matmul.allow_tf32 = True
+        torch.backends.cudnn.allow_tf32 = True
+        _TRITURUS_TF32_ENABLED = True
+    else:
+        torch.set_float32_matmul_precision("highest")
+        torch.backends.cuda.matmul.allow_tf32 = False
+        torch.backends.cudnn.allow_tf32 = False
+        _TRITURUS_TF32_ENABLED = False
+
+
+def is_torch_tf32_enabled() -> bool:
+    """triturus/utils.py:47-48."""
+    return bool(torch.backends.cuda.matmul.allow_tf32 and torch.backends.cudnn.allow_tf32)
 
 
 def is_triturus_tf32_enabled() -> bool:
