@@ -115,6 +115,11 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_vmax(one, 1 << 20, 0, one, one, null, 0, null) == -3
     assert lib.trt_matmax(one, one, 4, 4, 2, 0, null, 0, null) == -1
     assert lib.trt_matmax(one, one, 0, 4, 0, 0, null, 0, null) == -1
+    # more workgroups than a 32-bit grid holds: refused, not truncated (2^34 rows along axis 1 are
+    # 2^32 workgroups of 4 rows; 2^40 fp16 columns along axis 0 are 2^31 workgroups of 512 columns)
+    assert lib.trt_matmax(one, one, 1 << 34, 1, 1, _lib.TRT_F16, null, 0, null) == -4
+    assert lib.trt_matmax(one, one, 1 << 33, 2, 1, _lib.TRT_F16, null, 0, null) == -4
+    assert lib.trt_matmax(one, one, 1, 1 << 40, 0, _lib.TRT_F16, null, 0, null) == -4
     assert lib.trt_copy_bytes(one, one, 24, null) == -1
     # mm, vadd
     assert lib.trt_mm_f32(one, null, one, 2, 2, 2, null) == -1

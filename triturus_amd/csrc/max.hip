@@ -620,6 +620,26 @@ static int matmax_launch(const void *xv, void *yv, int64_t m, int64_t n, int axi
     return (int)hipGetLastError();
 }
 
+// Largest workgroup count among the launches of a matmax call (same plans as matmax_launch).
+static int64_t matmax_max_blocks(int64_t m, int64_t n, int axis, int dtype) {
+    const int vn = 16 / (int)elem_size(dtype);
+    if (axis == 1) {
+        // one workgroup per row (long rows), or one per 4 rows and column chunk
+        const int64_t wide = m;
+        const int64_t split = rowmax_plan(m, n, vn).splits * ceil_div(m, (int64_t)kMatWaves);
+        return wide > split ? wide : split;
+    }
+    int64_t most = 0;
+    for (int cn = 1; cn <= vn; cn += vn - 1 > 0 ? vn - 1 : 1) {  // the scalar and the vector column paths
+        const int64_t colblocks = ceil_div(n, (int64_t)kWave * cn);
+        const int64_t splits = colmax_plan(m, n, cn).splits;
+        const int64_t s2 = combine_splits(splits);
+        const int64_t blocks = colblocks * (splits > s2 ? splits : s2);
+        if (blocks > most) most = blocks;
+    }
+    return most;
+}
+
 }  // namespace trt
 
 using namespace trt;
@@ -659,8 +679,9 @@ extern "C" int trt_matmax(const void *x, void *y, int64_t m, int64_t n, int axis
     if (!x || !y || m <= 0 || n <= 0 || (axis != 0 && axis != 1) || !elem_size(dtype))
         return TRT_E_INVALID;
     if ((reinterpret_cast<uintptr_t>(x) % elem_size(dtype)) != 0) return TRT_E_LAYOUT;
-    // grid sizes below are computed in 32 bits
     if (m > (int64_t)1 << 40 || n > (int64_t)1 << 40) return TRT_E_RANGE;
+    // workgroup ids are 32-bit: every launch of the call must stay below 2^31 workgroups
+    if (matmax_max_blocks(m, n, axis, dtype) >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
         case TRT_F32: return matmax_launch<TRT_F32>(x, y, m, n, axis, workspace, workspace_bytes, s);

@@ -23,11 +23,15 @@ _ws_bytes: dict = {}  # (R, I, J, K, variant, splits, pieces) -> workspace bytes
 
 
 def _unit_inner(t: torch.Tensor) -> torch.Tensor:
-    # The kernels take free batch/row strides but a unit trailing stride (and
-    # no negative or zero-broadcast strides); anything else is materialised.
+    # The kernels take any non-negative batch and row strides (zero included: an expanded
+    # operand is read in place) but want a unit trailing stride; only a tensor without one is
+    # materialised.  (A trailing axis of one element has no stride to speak of: reshaping it
+    # gives it the unit stride without a copy.)
     st = t.stride()
-    if st[-1] == 1 and min(st) > 0:
+    if st[-1] == 1 and min(st) >= 0:
         return t
+    if t.shape[-1] == 1 and min(st[:-1]) >= 0:
+        return t.as_strided(t.shape, (*st[:-1], 1), t.storage_offset())
     return t.contiguous()
 
 

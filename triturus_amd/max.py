@@ -109,7 +109,7 @@ def bmatmax(x: torch.Tensor, *, clamp: bool = False) -> torch.Tensor:
     if J == 0:
         raise RuntimeError("max over an empty axis")
     st = x.stride()
-    if st[-1] != 1 or min(st) <= 0:
+    if st[-1] != 1 or min(st) < 0:  # zero strides (an expanded operand) are read in place
         x = x.contiguous()
     m = torch.empty((R, K), dtype=x.dtype, device=x.device)
     key = ("b", R, J, K)
