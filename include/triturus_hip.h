@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TRT_ABI_VERSION 5
+#define TRT_ABI_VERSION 6
 
 #define TRT_OK 0
 #define TRT_E_INVALID (-1)   /* null pointer, non-positive size, bad enum   */
@@ -56,15 +56,16 @@ const char *trt_error_string(int status);
 /*
  * c[r,i,k] = log sum_j a[r,i,j] * exp(b[r,j,k])            (fp32)
  * a: R x I x J linear-space, b: R x J x K log-space, c: R x I x K.
- * sa/sb/sc: element strides of the three axes.  The trailing stride of each
- * tensor must be 1 (TRT_E_LAYOUT otherwise); the two leading strides are
- * free.  Replaces the `_ker_lm2exp[grid](...)` launch, triturus/lm2exp.py:186-205;
- * arithmetic contract baselines/lm2exp.py:11-14 (column max clamped to
- * +-1e38, an all -inf column gives -inf, never NaN).
- * variant: 0 = choose by shape; 1..trt_lm2exp_variant_count() pick a tile shape and
- * how the shift is obtained (experiments, tests); the last one runs two launches -- a
- * separate pass over b for the column maxima, then the contraction -- and needs
- * R*K floats of workspace.
+ * sa/sb/sc: element strides of the three axes, all non-negative (zero: an
+ * expanded operand).  a may have any strides, as the reference forwards them to its
+ * kernel (triturus/lm2exp.py:190-198): a transposed or column-strided a is read in
+ * place.  The trailing stride of b and c must be 1 (TRT_E_LAYOUT otherwise); their two
+ * leading strides are free.  Replaces the `_ker_lm2exp[grid](...)` launch,
+ * triturus/lm2exp.py:186-205; arithmetic contract baselines/lm2exp.py:11-14 (column
+ * max clamped to +-1e38, an all -inf column gives -inf, never NaN).
+ * variant: 0 = choose by shape; 1..trt_lm2exp_variant_count() force a tile shape and
+ * kernel (experiments, tests); a forced variant that is not one of the paired-wavefront
+ * tiles (the last five) needs sa[2] == 1.
  * splits: the contraction over J may be cut over several workgroups whose partial
  * sums are merged by a second kernel in a fixed order (deterministic): 0 = decide
  * by shape (small grids with a long contraction), 1 = never, n = n ways.  The

@@ -68,7 +68,11 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_lm2exp_f32(one, one, one, 0, 1, 1, 1, ok, ok, ok, *tail) == -1
     assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, ok, 99, 0, null, 0, null) == -1
     assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, ok, 0, -1, null, 0, null) == -1
-    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, s3(12, 1, 4), ok, ok, *tail) == -2
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, s3(12, 1, 4), ok, *tail) == -2  # b, c: unit trailing stride
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, s3(12, 1, 4), *tail) == -2
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, s3(12, 4, -1), ok, ok, *tail) == -2
+    # a may have any non-negative strides, except under a forced tile that reads rows 16 bytes at a time
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, s3(12, 1, 4), ok, ok, 1, 0, null, 0, null) == -2
     assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, s3(-12, 4, 1), ok, *tail) == -2
     assert lib.trt_lm2exp_f32(one, one, one, 1 << 31, 1, 1, 1, ok, ok, ok, *tail) == -4
     assert lib.trt_lm2exp_f32(one, one, one, 1, 2, 2, 8, ok, ok, s3(16, 4, 1), *tail) == -2  # overlapping output rows

@@ -20,7 +20,7 @@ from triturus_amd import _lib, workloads
 pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
-N_VARIANTS = 18
+N_VARIANTS = 14
 N_BF16_VARIANTS = 16  # 1..4, 9..12 tiles; 5..8, 13..16 the same tiles with the contraction cut over workgroups
 # Accuracy gates of the split-bf16 paths against the float64 oracle.  Two pieces (3 MFMAs per
 # product) carry 16 significand bits: looser than fp32, ten times tighter than the rtol 5e-4
@@ -70,7 +70,7 @@ def test_golden(dev, name, mode):
 @pytest.mark.parametrize("mode", ["unsplit", "split"])
 @pytest.mark.parametrize("shape", [(2, 35, 9, 13, 45), (1, 70, 20, 33, 300), (2, 16, 5, 72, 64), (1, 33, 3, 3, 31),
                                    (2, 40, 6, 48, 100), (1, 33, 5, 24, 70), (1, 65, 3, 16, 64), (1, 20, 4, 100, 130),
-                                   # short rows of w that pack into chunks of 16 (variants 17, 18; last chunk ragged)
+                                   # short rows of w that pack into chunks of 16 (variants 13, 14; last chunk ragged)
                                    (2, 70, 37, 8, 150), (2, 40, 50, 2, 100), (1, 33, 9, 4, 70), (1, 65, 64, 4, 40)])
 def test_every_tile_variant_on_ragged_shapes(dev, variant, mode, shape):
     assert _lib.load().trt_lt2exp_variant_count() == N_VARIANTS
@@ -253,7 +253,7 @@ def test_benchmark_configuration_c5_full_size(dev):
         assert torch.allclose(out[sl], via, rtol=1e-5, atol=1e-4)
         del ab, via
     assert torch.allclose(lt2exp(wg, ag + 64.0, bg - 32.0), out + 32.0, rtol=1e-5, atol=1e-3)
-    for variant in (2, 5):
+    for variant in (1, 3):
         assert torch.allclose(lt2exp(wg, ag, bg, _variant=variant), out, rtol=1e-5, atol=1e-5)
     assert torch.allclose(lt2exp(wg, ag, bg, mode="split"), out, rtol=1e-5, atol=1e-5)
 

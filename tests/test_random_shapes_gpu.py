@@ -232,7 +232,7 @@ def test_sparse_weights_under_a_wide_spread(dev, seed, precision):
     b = torch.randn(R, J, K, generator=g) * rng.choice([40.0, 300.0]) + rng.choice([0.0, 1e4, -1e6])
     b = _sprinkle(rng, g, b)
     lo, hi = _lm_bracket(a, b, cut)
-    nvar = 12 if precision == "fp32" else 9
+    nvar = 20 if precision == "fp32" else 9
     variant, splits = rng.randrange(0, nvar + 1), rng.choice([0, 1, 3])
     out = lm2exp(_view(rng, a.to(dev)), _view(rng, b.to(dev)), _precision=precision, _variant=variant, _splits=splits)
     bad, _ = _inside(out, lo, hi, **GATES[precision])

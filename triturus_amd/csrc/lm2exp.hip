@@ -10,18 +10,15 @@
 // The contraction runs on v_mfma_f32_32x32x2_f32 (IEEE fp32 in, fp32 accumulate),
 // MFMA (q,u) of lane-half h consuming j = 8q + 4h + u of the chunk.
 //
-// The shift m[n].  The result m + log(sum_j a exp(b - m)) does not depend on m,
-// only overflow/underflow do, so m need not be the exact column maximum (MODE):
-//   kOnline    one sweep over b.  m starts as the maximum of the first chunk of the
-//              column; when a later chunk's maximum exceeds m by more than
-//              kRescaleMargin the accumulators of that column are multiplied by
-//              exp(m_old - m_new) and m moves up.  exp(b - m) therefore never exceeds
-//              e^kRescaleMargin, and b is read from HBM exactly once.
-//   kTwoSweep  two sweeps, as the reference kernel does (triturus/lm2exp.py:125-127):
-//              the exact column maximum first (wavefront reduction: the two lane
-//              halves take alternate rows and exchange once), then the contraction.
-//   kExternal  the clamped column maxima come from a separate launch
-//              (lm2exp_colmax_kernel); kPlain: no shift, exp or log at all (mm).
+// The shift m[n].  The result m + log(sum_j a exp(b - m)) does not depend on m, only
+// overflow/underflow do, so m need not be the exact column maximum.  This kernel makes one
+// sweep over b: m starts as the maximum of the first chunk of the column; when a later chunk's
+// maximum exceeds m by more than kRescaleMargin the accumulators of that column are multiplied
+// by exp(m_old - m_new) and m moves up.  exp(b - m) therefore never exceeds e^kRescaleMargin, and
+// b is read from HBM exactly once.  (The reference kernel sweeps b twice, exact column maximum
+// first, triturus/lm2exp.py:125-127; so does the paired-wavefront kernel of lm2exp_pair.hpp,
+// which the host prefers where the panel of b stays in cache.)  MODE kPlain: no shift, exp or
+// log at all (the mm entry point).
 // m is always clamped to +-1e38 (baselines/lm2exp.py:12) so an all -inf
 // column gives exp(-inf) = 0, log(0) = -inf: -inf out, never NaN.
 //
@@ -43,16 +40,22 @@ struct Lm2Args {
     float *shift;  // splits > 1: [splits][R][K] the shift each partial sum is relative to
     int R, I, J, K;
     int64_t sa0, sa1, sb0, sb1, sc0, sc1;
+    int64_t sa2;  // trailing stride of a (1 for every kernel but the paired-wavefront one)
     int i_tiles, n_tiles, splits, chunks_per_split;
     int stream_out;  // rows of c are 16-byte aligned: non-temporal result stores
     int64_t total_wgs, padded_wgs;
 };
 
 // How the shift m[n] is obtained (MODE template parameter of the kernel)
-constexpr int kTwoSweep = 0;  // exact column maximum first (sweep 1), then the contraction
 constexpr int kOnline = 1;    // found while sweeping, accumulators rescaled when it moves
-constexpr int kExternal = 2;  // read from p.shift: a separate launch (lm2exp_colmax_kernel) computed it
 constexpr int kPlain = 3;     // no shift, no exp, no log: c = a b (the mm entry point)
+constexpr int kPair = 4;      // lm2exp_pair_kernel: exact column maximum first, exp shared by two wavefronts
+
+}  // namespace trt
+
+#include "lm2exp_pair.hpp"
+
+namespace trt {
 
 template <int RT, int CT, int WM, int WN, int NQ, bool VEC, int MODE>
 __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args p) {
@@ -304,35 +307,10 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     const int jc1 = (jc0 + p.chunks_per_split < n_jc) ? jc0 + p.chunks_per_split : n_jc;
     const int full_end = jc1 < n_full ? jc1 : n_full;
 
-    if (MODE == kExternal) {
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) mref[ct] = p.shift[(int64_t)r * p.K + ncl[ct]];
-    }
     if (MODE == kPlain) {
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) mref[ct] = 0.f;
     }
-    if (MODE == kTwoSweep) {
-        // ---- sweep 1: exact column maxima over all J
-#pragma unroll
-        for (int ct = 0; ct < CT; ++ct) {
-            float x[8];
-#pragma unroll
-            for (int e = 0; e < 8; ++e) x[e] = -__builtin_inff();
-            int j = h;
-            for (; j + 14 < p.J; j += 16) {
-                const float *bp = br + (int64_t)j * p.sb1 + ncl[ct];
-#pragma unroll
-                for (int e = 0; e < 8; ++e) x[e] = max_nan(x[e], bp[(int64_t)(2 * e) * p.sb1]);
-            }
-            for (; j < p.J; j += 2) x[0] = max_nan(x[0], br[(int64_t)j * p.sb1 + ncl[ct]]);
-            float y = max_nan(max_nan(max_nan(x[0], x[1]), max_nan(x[2], x[3])),
-                              max_nan(max_nan(x[4], x[5]), max_nan(x[6], x[7])));
-            y = max_nan(y, __shfl_xor(y, 32, kWave));
-            mref[ct] = clamp_shift(y);
-        }
-    }
-
     // ---- prologue: first chunk
     if (jc0 < n_full) {
         load_tile_full(jc0);
@@ -501,36 +479,35 @@ struct Lm2Variant {
 };
 // variant ids are 1-based in the C ABI (0 = choose by shape)
 static const Lm2Variant kVariants[] = {
-    {4, 1, 1, 4, 4, kOnline},   // 1: 128 x 128 tile, 4 waves each 128 x 32, one sweep (3 waves/SIMD)
+    {4, 1, 1, 4, 4, kOnline},   // 1: 128 x 128 tile, 4 waves each 128 x 32 (3 waves/SIMD)
     {4, 1, 1, 8, 4, kOnline},   // 2: 128 x 256 tile, 8 waves each 128 x 32
-    {8, 1, 1, 8, 4, kOnline},   // 3: 256 x 256 tile, 8 waves each 256 x 32
-    {8, 1, 1, 4, 4, kOnline},   // 4: 256 x 128 tile, 4 waves each 256 x 32
-    {8, 1, 1, 8, 4, kTwoSweep},  // 5: as 3, two sweeps (exact column maximum first)
-    {2, 2, 1, 4, 4, kOnline},   // 6: 64 x 256 tile
-    {2, 1, 1, 4, 4, kOnline},   // 7: 64 x 128 tile
-    {1, 1, 1, 4, 4, kOnline},   // 8: 32 x 128 tile
-    {2, 1, 1, 4, 4, kTwoSweep},  // 9: as 7, two sweeps
-    {4, 1, 1, 4, 4, kTwoSweep},  // 10: as 1, two sweeps
-    {4, 1, 1, 4, 4, kExternal},  // 11: as 1, shift from a separate pass over b (two launches)
-    {3, 1, 1, 4, 4, kOnline},   // 12: 96 x 128 tile (I = 96, 192, ... without padded rows)
-    {4, 1, 1, 4, 2, kOnline},   // 13..18: the 128-, 64- and 32-row tiles with j-chunks of 16 and 24
-    {4, 1, 1, 4, 3, kOnline},   //         (chunks of 48 were measured too: 20 more B registers, a
-    {2, 1, 1, 4, 2, kOnline},   //         wavefront less per SIMD on the 128-row tile, 5-60 % slower)
+    {2, 1, 1, 4, 4, kOnline},   // 3: 64 x 128 tile
+    {1, 1, 1, 4, 4, kOnline},   // 4: 32 x 128 tile
+    {3, 1, 1, 4, 4, kOnline},   // 5: 96 x 128 tile (I = 96, 192, ... without padded rows)
+    {4, 1, 1, 4, 2, kOnline},   // 6..11: the 128-, 64- and 32-row tiles with j-chunks of 16 and 24
+    {4, 1, 1, 4, 3, kOnline},   //        (chunks of 48 were measured too: 20 more B registers, a
+    {2, 1, 1, 4, 2, kOnline},   //        wavefront less per SIMD on the 128-row tile, 5-60 % slower)
     {2, 1, 1, 4, 3, kOnline},
     {1, 1, 1, 4, 2, kOnline},
     {1, 1, 1, 4, 3, kOnline},
-    {1, 1, 4, 1, 4, kOnline},   // 19: 128 x 32 tile, the 4 waves stacked over rows (outputs of <= 32 columns)
-    {2, 1, 4, 1, 4, kOnline},   // 20: 256 x 32 tile
-    {1, 1, 2, 2, 4, kOnline},   // 21: 64 x 64 tile (outputs of <= 64 columns)
-    {3, 1, 1, 4, 2, kOnline},   // 22, 23: the 96-row tile with j-chunks of 16 and 24
+    {1, 1, 4, 1, 4, kOnline},   // 12: 128 x 32 tile, the 4 waves stacked over rows (outputs of <= 32 columns)
+    {1, 1, 2, 2, 4, kOnline},   // 13: 64 x 64 tile (outputs of <= 64 columns)
+    {3, 1, 1, 4, 2, kOnline},   // 14, 15: the 96-row tile with j-chunks of 16 and 24
     {3, 1, 1, 4, 3, kOnline},
+    {4, 1, 2, 4, 2, kPair},     // 16: 256 x 128 tile of 2 x 4 wavefronts, exact shift first, exp shared by a pair
+    {2, 1, 2, 4, 2, kPair},     // 17: 128 x 128
+    {2, 1, 2, 2, 2, kPair},     // 18: 128 x 64 tile of 2 x 2 wavefronts
+    {1, 1, 2, 2, 2, kPair},     // 19: 64 x 64
+    {3, 1, 2, 2, 2, kPair},     // 20: 192 x 64
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr size_t kDefaultLdsLimit = 64 * 1024;  // larger dynamic LDS must be opted into per kernel
 
 // Measured on MI355X at R=64, I=J=256, K=4096: the 128-row tiles (64 accumulator
-// registers, 3-4 wavefronts per SIMD) beat the 256-row tiles (128 accumulator
-// registers, 2 per SIMD) although b is then exponentiated once per row tile.
+// registers, 3-4 wavefronts per SIMD) beat 256-row tiles of the same kernel (128 accumulator
+// registers, 2 per SIMD) although b is then exponentiated once per row tile; so did they beat
+// a two-sweep build (exact maximum first: 0.35-0.37 ms against 0.29-0.31 ms) and a two-launch
+// build (column maxima by a separate kernel: 0.33 ms).  None of those is kept.
 // Smaller grids want smaller row tiles: a 128-row tile amortises each exp over four
 // MFMAs, but it only pays when there are enough tiles to keep 256 CUs busy with more
 // than one workgroup each.  Rules fitted to sweeps of the variants over the shapes of
@@ -552,6 +529,12 @@ static int find_variant_shape(int rt, int wm, int wn) {
         if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].wm == wm && kVariants[v].wn == wn &&
             kVariants[v].nq == 4 && kVariants[v].mode == kOnline)
             return v;
+    return 0;
+}
+
+static int find_pair_variant(int rt, int wn = 2) {
+    for (int v = 0; v < kNumVariants; ++v)
+        if (kVariants[v].mode == kPair && kVariants[v].rt == rt && kVariants[v].wn == wn) return v;
     return 0;
 }
 
@@ -674,6 +657,27 @@ static int launch_v(const Lm2Args &args, bool vec, hipStream_t stream) {
                : launch_k<RT, CT, WM, WN, NQ, false, MODE>(args, stream);
 }
 
+template <int RT, int WN, int NQ, int LOADA>
+static int launch_pair_k(const Lm2Args &args, hipStream_t stream) {
+    constexpr int TM = 64 * RT;
+    constexpr size_t lds = (size_t)(2 * (2 * NQ) * (TM * 4) + 2 * 2 * WN * 64 * 2 * NQ) * sizeof(float);
+    static_assert(lds <= kDefaultLdsLimit, "the paired-wavefront tiles fit the default dynamic LDS limit");
+    hipLaunchKernelGGL((lm2exp_pair_kernel<RT, WN, NQ, LOADA>), dim3((unsigned)args.padded_wgs), dim3(128 * WN), lds,
+                       stream, args);
+    return (int)hipGetLastError();
+}
+
+// loada: how the a tile is read (kLoadVec, kLoadByCol, kLoadByRow); lanes along i need a tile
+// height that divides the workgroup, which 192 rows do not: such a call reads by column.
+template <int RT, int WN>
+static int launch_pair(const Lm2Args &args, int loada, hipStream_t stream) {
+    if (loada == kLoadVec) return launch_pair_k<RT, WN, 2, kLoadVec>(args, stream);
+    if constexpr (RT != 3) {
+        if (loada == kLoadByRow) return launch_pair_k<RT, WN, 2, kLoadByRow>(args, stream);
+    }
+    return launch_pair_k<RT, WN, 2, kLoadByCol>(args, stream);
+}
+
 struct Lm2Plan {
     int variant;           // index into kVariants
     int splits;            // workgroups sharing one output tile
@@ -692,8 +696,8 @@ static Lm2Plan make_plan(int64_t R, int64_t I, int64_t J, int64_t K, int variant
     const int64_t chunks = ceil_div(J, 8 * vr.nq);
     const int64_t base = R * ceil_div(I, 32 * vr.rt * vr.wm) * ceil_div(K, 32 * vr.ct * vr.wn);
     int64_t splits = 1;
-    if (vr.mode == kExternal || vr.mode == kPlain)
-        splits = 1;  // these kernels do not write partial sums
+    if (vr.mode == kPlain)
+        splits = 1;  // this build does not write partial sums
     else if (splits_req == 0)
         // measured: R=16 I=J=K=512 (256 tiles, 16 chunks) is 1.5x slower split, batch-1
         // squares of 512..1536 are 1.2-1.9x faster; the model below reproduces both
@@ -710,7 +714,6 @@ static Lm2Plan make_plan(int64_t R, int64_t I, int64_t J, int64_t K, int variant
 }
 
 static size_t plan_workspace(const Lm2Plan &pl, int64_t R, int64_t I, int64_t K) {
-    if (kVariants[pl.variant].mode == kExternal) return (size_t)R * K * sizeof(float);  // the shifts
     if (pl.splits <= 1) return 0;
     return ((size_t)pl.splits * R * I * K + (size_t)pl.splits * R * K) * sizeof(float);
 }
@@ -733,16 +736,33 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     if (!a || !b || !c || !sa || !sb || !sc) return TRT_E_INVALID;
     if (R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (variant < 0 || variant > kNumVariants || splits < 0) return TRT_E_INVALID;
-    if (sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
+    if (sb[2] != 1 || sc[2] != 1 || sa[2] < 0) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     if (sc[1] < K || sc[0] < 0) return TRT_E_LAYOUT;  // output rows must not overlap (stores rely on it)
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || I >= lim || J >= lim || K >= lim) return TRT_E_RANGE;
     // byte offsets inside one batch slab of a, b and c are 32-bit (buffer addressing)
-    if (J * sb[1] + K >= lim || I * sa[1] + J >= lim || I * sc[1] + K >= lim || I * K >= lim) return TRT_E_RANGE;
+    if (J * sb[1] + K >= lim || I * sa[1] + J * sa[2] >= lim || I * sc[1] + K >= lim || I * K >= lim)
+        return TRT_E_RANGE;
 
-    const Lm2Plan pl = make_plan(R, I, J, K, variant, splits);
+    Lm2Plan pl = make_plan(R, I, J, K, variant, splits);
+    // a trailing stride of a other than 1 (a transposed or strided view): only the
+    // paired-wavefront kernel reads such a tile; a call that would take another kernel takes
+    // the paired tile of the same height instead, cut over J no further than the caller's
+    // workspace (sized without knowledge of the strides) holds
+    if (sa[2] != 1 && kVariants[pl.variant].mode != kPair) {
+        if (variant >= 1) return TRT_E_LAYOUT;
+        const bool narrow = K <= 64;
+        const int64_t big_tiles = R * ceil_div(I, 256) * ceil_div(K, 128);
+        const int pv = narrow ? find_pair_variant(I > 64 ? 2 : 1, 2)
+                       : I > 128 && big_tiles >= 256 ? find_pair_variant(4, 4)
+                       : I > 64 ? find_pair_variant(2, 4)
+                                : find_pair_variant(1, 2);
+        pl = make_plan(R, I, J, K, 1 + pv, splits);
+        while (pl.splits > 1 && (!workspace || plan_workspace(pl, R, I, K) > workspace_bytes))
+            pl = make_plan(R, I, J, K, 1 + pv, pl.splits - 1);
+    }
     const int v = pl.variant;
     const Lm2Variant &vr = kVariants[v];
     Lm2Args args;
@@ -752,6 +772,7 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     args.sa0 = sa[0]; args.sa1 = sa[1];
     args.sb0 = sb[0]; args.sb1 = sb[1];
     args.sc0 = sc[0]; args.sc1 = sc[1];
+    args.sa2 = sa[2];
     args.i_tiles = (int)ceil_div(I, 32 * vr.rt * vr.wm);
     args.n_tiles = (int)ceil_div(K, 32 * vr.ct * vr.wn);
     args.splits = pl.splits;
@@ -761,15 +782,7 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     args.stream_out = rows_16_byte_aligned(c, sc[0], sc[1]);
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (vr.mode == kExternal) {
-        // two-kernel variant: a pass over b for the clamped column maxima, then the contraction
-        if (!workspace || workspace_bytes < plan_workspace(pl, R, I, K)) return TRT_E_WORKSPACE;
-        args.shift = static_cast<float *>(workspace);
-        const int64_t blocks = R * ceil_div(K, 256);
-        if (blocks >= ((int64_t)1 << 31)) return TRT_E_RANGE;
-        hipLaunchKernelGGL(lm2exp_colmax_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, b, args.shift, (int)R,
-                           (int)J, (int)K, sb[0], sb[1], (int)J, 1);
-    } else if (pl.splits > 1) {
+    if (pl.splits > 1) {
         const size_t need = plan_workspace(pl, R, I, K);
         if (!workspace || workspace_bytes < need) return TRT_E_WORKSPACE;
         args.part = static_cast<float *>(workspace);
@@ -780,29 +793,36 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     const bool vec = (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     int st;
+    if (vr.mode == kPair) {
+        const int loada = (vec && sa[2] == 1) ? kLoadVec : ((sa[2] != 1 && sa[1] < sa[2]) ? kLoadByRow : kLoadByCol);
+        if (vr.wn == 4) {
+            st = vr.rt == 4 ? launch_pair<4, 4>(args, loada, s) : launch_pair<2, 4>(args, loada, s);
+        } else {
+            switch (vr.rt) {
+                case 3: st = launch_pair<3, 2>(args, loada, s); break;
+                case 2: st = launch_pair<2, 2>(args, loada, s); break;
+                default: st = launch_pair<1, 2>(args, loada, s); break;
+            }
+        }
+        if (st != 0 || pl.splits <= 1) return st;
+        launch_lm2exp_merge(args.part, args.shift, c, R, I, K, pl.splits, sc[0], sc[1], s, true);
+        return (int)hipGetLastError();
+    }
     switch (v) {
         case 0: st = launch_v<4, 1, 1, 4, 4, kOnline>(args, vec, s); break;
         case 1: st = launch_v<4, 1, 1, 8, 4, kOnline>(args, vec, s); break;
-        case 2: st = launch_v<8, 1, 1, 8, 4, kOnline>(args, vec, s); break;
-        case 3: st = launch_v<8, 1, 1, 4, 4, kOnline>(args, vec, s); break;
-        case 4: st = launch_v<8, 1, 1, 8, 4, kTwoSweep>(args, vec, s); break;
-        case 5: st = launch_v<2, 2, 1, 4, 4, kOnline>(args, vec, s); break;
-        case 6: st = launch_v<2, 1, 1, 4, 4, kOnline>(args, vec, s); break;
-        case 7: st = launch_v<1, 1, 1, 4, 4, kOnline>(args, vec, s); break;
-        case 8: st = launch_v<2, 1, 1, 4, 4, kTwoSweep>(args, vec, s); break;
-        case 9: st = launch_v<4, 1, 1, 4, 4, kTwoSweep>(args, vec, s); break;
-        case 10: st = launch_v<4, 1, 1, 4, 4, kExternal>(args, vec, s); break;
-        case 12: st = launch_v<4, 1, 1, 4, 2, kOnline>(args, vec, s); break;
-        case 13: st = launch_v<4, 1, 1, 4, 3, kOnline>(args, vec, s); break;
-        case 14: st = launch_v<2, 1, 1, 4, 2, kOnline>(args, vec, s); break;
-        case 15: st = launch_v<2, 1, 1, 4, 3, kOnline>(args, vec, s); break;
-        case 16: st = launch_v<1, 1, 1, 4, 2, kOnline>(args, vec, s); break;
-        case 17: st = launch_v<1, 1, 1, 4, 3, kOnline>(args, vec, s); break;
-        case 18: st = launch_v<1, 1, 4, 1, 4, kOnline>(args, vec, s); break;
-        case 19: st = launch_v<2, 1, 4, 1, 4, kOnline>(args, vec, s); break;
-        case 20: st = launch_v<1, 1, 2, 2, 4, kOnline>(args, vec, s); break;
-        case 21: st = launch_v<3, 1, 1, 4, 2, kOnline>(args, vec, s); break;
-        case 22: st = launch_v<3, 1, 1, 4, 3, kOnline>(args, vec, s); break;
+        case 2: st = launch_v<2, 1, 1, 4, 4, kOnline>(args, vec, s); break;
+        case 3: st = launch_v<1, 1, 1, 4, 4, kOnline>(args, vec, s); break;
+        case 5: st = launch_v<4, 1, 1, 4, 2, kOnline>(args, vec, s); break;
+        case 6: st = launch_v<4, 1, 1, 4, 3, kOnline>(args, vec, s); break;
+        case 7: st = launch_v<2, 1, 1, 4, 2, kOnline>(args, vec, s); break;
+        case 8: st = launch_v<2, 1, 1, 4, 3, kOnline>(args, vec, s); break;
+        case 9: st = launch_v<1, 1, 1, 4, 2, kOnline>(args, vec, s); break;
+        case 10: st = launch_v<1, 1, 1, 4, 3, kOnline>(args, vec, s); break;
+        case 11: st = launch_v<1, 1, 4, 1, 4, kOnline>(args, vec, s); break;
+        case 12: st = launch_v<1, 1, 2, 2, 4, kOnline>(args, vec, s); break;
+        case 13: st = launch_v<3, 1, 1, 4, 2, kOnline>(args, vec, s); break;
+        case 14: st = launch_v<3, 1, 1, 4, 3, kOnline>(args, vec, s); break;
         default: st = launch_v<3, 1, 1, 4, 4, kOnline>(args, vec, s); break;
     }
     if (st != 0 || pl.splits <= 1) return st;
@@ -888,6 +908,7 @@ extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, i
     args.sa0 = m * k; args.sa1 = k;
     args.sb0 = k * n; args.sb1 = n;
     args.sc0 = m * n; args.sc1 = n;
+    args.sa2 = 1;
     args.i_tiles = (int)ceil_div(m, 32 * rt);
     args.n_tiles = (int)ceil_div(n, 128);
     args.splits = 1;
@@ -903,3 +924,4 @@ extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, i
     if (rt == 2) return launch_v<2, 1, 1, 4, 4, kPlain>(args, vec, s);
     return launch_v<1, 1, 1, 4, 4, kPlain>(args, vec, s);
 }
+

@@ -41,7 +41,7 @@ _PIECES = {"bf16x3": 2, "bf16x6": 3}
 _PAD_MIN_K = 2048
 _PAD_MIN_FLOPS = 2e9
 # tile variants worth timing when tuning is on (0 = the library's rule)
-_FP32_CANDIDATES = (0, 1, 2, 7, 8, 12, 13, 14, 15, 16, 17, 18, 19, 21, 22, 23)
+_FP32_CANDIDATES = (0, 1, 2, 3, 4, 5, 6, 7, 8, 9, 10, 11, 12, 13, 14, 15, 16, 17)
 _BF16_CANDIDATES = (0, 1, 2, 3, 4, 8, 9)
 
 
@@ -64,13 +64,17 @@ def lm2exp(
     if J == 0:
         # empty contraction: log(0)
         return c.fill_(float("-inf"))
-    a = _unit_inner(a)
-    b = _unit_inner(b)
     if _precision is None:
         _precision = matrix_precision()
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
-    if _variant == 0 and _splits == 0 and autotune.is_autotune_enabled():
+    # a goes to the fp32 kernels with whatever non-negative strides it has (a transposed or
+    # strided view is read in place, as the reference does: triturus/lm2exp.py:190-198); the
+    # bf16 kernels and every kernel's b want a unit trailing stride
+    if _precision != "fp32" or min(a.stride()) < 0:
+        a = _unit_inner(a)
+    b = _unit_inner(b)
+    if _variant == 0 and _splits == 0 and a.stride(2) == 1 and autotune.is_autotune_enabled():
         cands = _FP32_CANDIDATES if _precision == "fp32" else _BF16_CANDIDATES
         _variant = autotune.pick(("lm2exp", R, I, J, K, _precision), cands,
                                  lambda v: lm2exp(a, b, _variant=v, _splits=-1, _precision=_precision))
@@ -78,7 +82,7 @@ def lm2exp(
     # contiguous a does not qualify and the kernels fall back to element loads (10-50 % slower).
     # A call with enough work per element of a (the copy costs ~3 ps per element, the element loads
     # ~15 % of 20 fs x K) runs on a copy of a whose rows are padded to a multiple of 4.
-    if J % 4 != 0 and J > 4 and K >= _PAD_MIN_K and 2 * R * I * J * K >= _PAD_MIN_FLOPS:
+    if J % 4 != 0 and J > 4 and a.stride(2) == 1 and K >= _PAD_MIN_K and 2 * R * I * J * K >= _PAD_MIN_FLOPS:
         a = torch.nn.functional.pad(a, (0, (-J) % 4))[..., :J]
     if _splits < 0:  # tuning launch: the library decides the split for this tile
         _splits = 0

@@ -39,7 +39,7 @@ def launches_split(R: int, S: int, I: int, J: int, K: int, mode: str) -> bool:
 
 _PIECES = {"bf16x3": 2, "bf16x6": 3}
 # tile variants worth timing when tuning is on (0 = the library's rule)
-_FP32_CANDIDATES = (0, 5, 6, 8, 9, 10, 11, 12, 13, 14, 17, 18)
+_FP32_CANDIDATES = (0, 1, 2, 4, 5, 6, 7, 8, 9, 10, 13, 14)
 _BF16_CANDIDATES = (0, 1, 2, 3, 4, 9, 10, 11, 12)
 
 
