@@ -272,6 +272,8 @@ def test_views_of_a_are_read_in_place(dev, shape):
         "every other column": wide.to(dev)[:, :, 1::2],
         "batch first in memory": a.permute(1, 2, 0).contiguous().to(dev).permute(2, 0, 1),
     }
+    if R == 1:
+        del views["batch first in memory"]  # the trailing stride is the batch size
     for name, ag in views.items():
         assert ag.stride(2) != 1 and torch.equal(ag.cpu(), a), name
         lm2exp(ag, bg)  # first call: library load, workspace query cache

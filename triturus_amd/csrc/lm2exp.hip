@@ -805,7 +805,7 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
             }
         }
         if (st != 0 || pl.splits <= 1) return st;
-        launch_lm2exp_merge(args.part, args.shift, c, R, I, K, pl.splits, sc[0], sc[1], s, true);
+        launch_lm2exp_merge(args.part, args.shift, c, R, I, K, pl.splits, sc[0], sc[1], s);
         return (int)hipGetLastError();
     }
     switch (v) {

@@ -2,15 +2,12 @@
 // its own shift m_s (the shift is found while sweeping, so the pieces end with different ones);
 //   c = M + log(sum_s part_s * exp(m_s - M)),  M = max_s m_s,
 // added in split order: deterministic.  Shared by the fp32 and the bf16 kernels.
-// LOG2: the shifts are integers n_s in units of log 2 (the paired-wavefront kernel): the sums
-// are relative to 2^n_s exactly, so c = ln2 (N + log2(sum_s part_s * 2^(n_s - N))), N = max_s n_s.
 #pragma once
 
 #include "common.hpp"
 
 namespace trt {
 
-template <bool LOG2>
 static __global__ __launch_bounds__(256) void lm2exp_merge_kernel(const float *__restrict__ part,
                                                                   const float *__restrict__ shift,
                                                                   float *__restrict__ c, int R, int I, int K,
@@ -29,26 +26,20 @@ static __global__ __launch_bounds__(256) void lm2exp_merge_kernel(const float *_
         float sum = 0.f;
         for (int sp = 0; sp < splits; ++sp) {
             // exp(m_s - M) in two halves: the factor alone may flush where the product does not
-            const float d = 0.5f * (sh[sp * rk] - M);
-            const float f = LOG2 ? __builtin_amdgcn_exp2f(d) : exp_shifted(d);
+            const float f = exp_shifted(0.5f * (sh[sp * rk] - M));
             sum += part[(int64_t)sp * total + e] * f * f;
         }
-        c[(int64_t)r * sc0 + (int64_t)i * sc1 + k] = log_plus(sum, LOG2 ? M * kLn2 : M);
+        c[(int64_t)r * sc0 + (int64_t)i * sc1 + k] = log_plus(sum, M);
     }
 }
 
 // part: [splits][R][I][K] partial sums; shift: [splits][R][K] their shifts.
 static inline void launch_lm2exp_merge(const float *part, const float *shift, float *c, int64_t R, int64_t I,
-                                       int64_t K, int splits, int64_t sc0, int64_t sc1, hipStream_t stream,
-                                       bool log2_shifts = false) {
+                                       int64_t K, int splits, int64_t sc0, int64_t sc1, hipStream_t stream) {
     int64_t blocks = ceil_div(R * I * K, 256);
     if (blocks > 8192) blocks = 8192;
-    if (log2_shifts)
-        hipLaunchKernelGGL(lm2exp_merge_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, stream, part, shift, c,
-                           (int)R, (int)I, (int)K, splits, sc0, sc1);
-    else
-        hipLaunchKernelGGL(lm2exp_merge_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, stream, part, shift, c,
-                           (int)R, (int)I, (int)K, splits, sc0, sc1);
+    hipLaunchKernelGGL(lm2exp_merge_kernel, dim3((unsigned)blocks), dim3(256), 0, stream, part, shift, c, (int)R,
+                       (int)I, (int)K, splits, sc0, sc1);
 }
 
 }  // namespace trt

@@ -11,10 +11,6 @@
 //     triturus/lm2exp.py:125-127): the main loop carries no running maximum, no branch and no
 //     rescaling of accumulators.  The panel (J x 32*WN columns) is read again by the main loop
 //     while it is still in cache, which is why the host picks this kernel for moderate J only;
-//   * the shift is applied in the base-2 domain as an integer: with n = rint(m log2(e)),
-//     exp(b - m') = 2^(b log2(e) - n) is one fma and one v_exp_f32 per element, and the result
-//     is ln2 * (log2(acc) + n).  Any shift gives the same result as long as the epilogue adds back
-//     exactly what was subtracted, and an integer n is subtracted exactly by the fma;
 //   * the two wavefronts that share a column panel (wm = 0, 1) each evaluate half of every
 //     chunk of exp(b - m') and hand it to the other through LDS, so an exp is taken once per
 //     workgroup and element: a quarter of a vector instruction per MFMA with 256-row tiles;
@@ -108,7 +104,7 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
     // ---- column maxima of rows [jbeg, jend): the four (wm, h) classes take every fourth row.
     // (Called after the loads of the first chunks have been issued, so that the trips to memory
     // a workgroup starts with overlap.)
-    float nsh = 0.f;  // the shift in units of log 2, an integer
+    float msh = 0.f;  // the shift: the clamped column maximum
     auto find_shift = [&]() {
         const uint32_t poff = ((uint32_t)h * (uint32_t)p.sb1 + (uint32_t)ncl) * 4u;
         float x0 = -__builtin_inff(), x1 = x0;
@@ -144,7 +140,7 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
         if (h == 0) mxs[(wn * 2 + wm) * 32 + m] = x0;
         __syncthreads();
         const float mx = max3_raw(mxs[(wn * 2) * 32 + m], mxs[(wn * 2 + 1) * 32 + m], x0);
-        nsh = __builtin_rintf(clamp_shift(mx) * kLog2e);
+        msh = clamp_shift(mx);
     };
 
     floatx16 acc[RT];
@@ -249,7 +245,7 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
                 raw[4 * qq + u] = (!masked || row + 4 * h < p.J) ? v : -__builtin_inff();
             }
     };
-    auto exp_one = [&](float raw) { return __builtin_amdgcn_exp2f(__builtin_fmaf(raw, kLog2e, -nsh)); };
+    auto exp_one = [&](float raw) { return exp_shifted(raw - msh); };
     float *xmine = xb + (wave * NH) * 256 + lane * 4;
     const float *xpartner = xb + ((wave ^ 1) * NH) * 256 + lane * 4;
     auto publish = [&](const float (&e)[NB], int buf) {
@@ -376,10 +372,10 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
         ++t;
     }
 
-    // ---- epilogue: c = ln2 (log2(acc) + n).  Register v of lane (h, m) holds row
+    // ---- epilogue: c = m + log(acc).  Register v of lane (h, m) holds row
     // 8 (v / 4) + 4h + v % 4, column m of its 32 x 32 tile.  Rows past I fall outside the
     // buffer extent and are dropped by the hardware.  With a cut contraction the raw sums and
-    // their shift n go to the workspace instead.
+    // their shift go to the workspace instead.
     const bool split_out = p.splits > 1;  // wave-uniform
     const int crows = p.I - (i0 + wrow0);
     float *obase = split_out ? p.part + (((int64_t)split * p.R + r) * p.I + (i0 + wrow0)) * (int64_t)p.K
@@ -390,8 +386,7 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
     const uint32_t c_row_bytes = orow * 4u;
     if (ncol < p.K) {
         const uint32_t co = ((uint32_t)(4 * h) * orow + (uint32_t)ncol) * 4u;
-        if (split_out && itile == 0 && wm == 0 && h == 0) p.shift[((int64_t)split * p.R + r) * p.K + ncol] = nsh;
-        const float nl = nsh * kLn2;
+        if (split_out && itile == 0 && wm == 0 && h == 0) p.shift[((int64_t)split * p.R + r) * p.K + ncol] = msh;
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
@@ -400,7 +395,7 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
                 if (split_out)  // partial sums are read back by the merge kernel right away
                     buf_store_f32(acc[rt][v], c_rsrc, co, trow * c_row_bytes);
                 else
-                    buf_store_f32_out(p.stream_out != 0, log_plus(acc[rt][v], nl), c_rsrc, co, trow * c_row_bytes);
+                    buf_store_f32_out(p.stream_out != 0, log_plus(acc[rt][v], msh), c_rsrc, co, trow * c_row_bytes);
             }
     }
 }
