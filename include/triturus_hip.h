@@ -34,6 +34,7 @@ extern "C" {
 #define TRT_E_LAYOUT (-2)    /* stride pattern the kernels do not handle    */
 #define TRT_E_WORKSPACE (-3) /* workspace missing or smaller than required  */
 #define TRT_E_RANGE (-4)     /* a size exceeds what the index math supports */
+#define TRT_E_SCRATCH (-5)   /* the call needs more than the library's static scratch holds */
 
 /* Element types of the max reductions (triturus/max.py:37,98,178 accept any
  * floating dtype). */
@@ -112,6 +113,27 @@ int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c,
 size_t trt_lt2exp_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t J,
                                   int64_t K, int mode);
 int trt_lt2exp_variant_count(void);
+
+#define TRT_STATIC_SCRATCH_BYTES ((size_t)16 << 20)
+/*
+ * trt_lt2exp_f32 without a workspace argument, for callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  No counterpart in the reference (whose wrapper allocates its lock and output
+ * with torch, triturus/lt2exp.py:544-562).  The split-mode workspace (partial sums and
+ * shifts) lives in a device array inside the library of TRT_STATIC_SCRATCH_BYTES bytes
+ * (16 MiB; every GPU the library runs on holds its copy until the process ends).  The call
+ * allocates and frees nothing.  A shape whose split mode may need more than that
+ * (trt_lt2exp_workspace_bytes(R, S, I, J, K, mode) > TRT_STATIC_SCRATCH_BYTES) is refused
+ * with TRT_E_SCRATCH and nothing is enqueued; TRT_MODE_UNSPLIT needs no scratch at all.  The
+ * first call on a device looks up the address of that device's copy of the array (make it
+ * outside graph capture).  All calls on one GPU share the array: calls that overlap in time
+ * (two streams, two threads) race; calls enqueued on one stream do not.  Nothing in the array
+ * has to be cleared between calls.  Results are bit-identical to trt_lt2exp_f32.
+ */
+int trt_lt2exp_f32_static(const float *w, const float *a, const float *b, float *c,
+                          int64_t R, int64_t S, int64_t I, int64_t J, int64_t K,
+                          const int64_t sw[3], const int64_t sa[3], const int64_t sb[3],
+                          const int64_t sc[3], int mode, int variant, void *stream);
 
 /*
  * The same contraction as trt_lt2exp_f32 (fp32 tensors in and out, same layouts, strides

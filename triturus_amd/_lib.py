@@ -18,6 +18,8 @@ ABI_VERSION = 6
 
 TRT_F32, TRT_F64, TRT_F16, TRT_BF16 = 0, 1, 2, 3
 MODE_AUTO, MODE_SPLIT, MODE_UNSPLIT = 0, 1, 2
+STATIC_SCRATCH_BYTES = 16 << 20  # TRT_STATIC_SCRATCH_BYTES
+E_SCRATCH = -5
 
 DTYPE_CODES = {
     torch.float32: TRT_F32,
@@ -50,6 +52,12 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
          POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
          c_int, c_int, c_void_p, c_size_t, c_void_p],
+    ),
+    "trt_lt2exp_f32_static": (
+        c_int,
+        [c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int64, c_int64,
+         POINTER(c_int64), POINTER(c_int64), POINTER(c_int64), POINTER(c_int64),
+         c_int, c_int, c_void_p],
     ),
     "trt_lt2exp_bf16": (
         c_int,

@@ -22,6 +22,8 @@
 #include "common.hpp"
 #include "lt2exp_merge.hpp"
 
+#include <mutex>
+
 namespace trt {
 
 struct Lt2Args {
@@ -651,4 +653,57 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     launch_variant(v, args, vec, sp.split, s);
     if (sp.split) launch_lt2exp_merge(args.c, args.shift, c, R, S, K, sp.splits, sc[0], sc[1], s);
     return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------
+// trt_lt2exp_f32_static: the same call for callers that cannot allocate (code under HIP graph
+// capture, tight serving loops, harnesses that forbid hipMalloc).  The split-mode workspace --
+// partial sums of every split and the two shift vectors -- lives in a file-scope device array
+// of kStaticScratchBytes instead of a caller's buffer.  Host code never passes the array's name
+// to a kernel (it is a host-side stand-in, not a device address): at the first call on a device
+// the address of that device's copy is looked up with hipGetSymbolAddress and kept, and the
+// kernels take it as the workspace argument exactly as they take a caller's buffer.  Every
+// element of the workspace that the merge kernel reads is written by the contraction kernel of
+// the same call first, so nothing has to be cleared between calls; calls that overlap on one
+// GPU share the array and race.
+namespace trt {
+constexpr size_t kStaticScratchBytes = TRT_STATIC_SCRATCH_BYTES;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static void *g_scratch_ptr[kMaxDevices];  // per device: address of that device's copy of `scratch`
+static std::mutex g_scratch_mutex;
+
+// Address of the current device's copy of the static scratch array (set-up on first use).
+static int static_scratch(void **ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return TRT_E_RANGE;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return (int)e;
+        if (!p) return TRT_E_INVALID;
+        g_scratch_ptr[dev] = p;
+    }
+    *ptr = g_scratch_ptr[dev];
+    return 0;
+}
+}  // namespace trt
+
+extern "C" int trt_lt2exp_f32_static(const float *w, const float *a, const float *b, float *c, int64_t R, int64_t S,
+                                     int64_t I, int64_t J, int64_t K, const int64_t sw[3], const int64_t sa[3],
+                                     const int64_t sb[3], const int64_t sc[3], int mode, int variant, void *stream) {
+    if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
+    // what the call may need at most (any tile the shape rule can pick): beyond the array, refuse
+    const size_t need = trt_lt2exp_workspace_bytes(R, S, I, J, K, mode);
+    if (need > trt::kStaticScratchBytes) return TRT_E_SCRATCH;
+    void *ws = nullptr;
+    if (need > 0) {
+        const int st = trt::static_scratch(&ws);
+        if (st != 0) return st;
+    }
+    return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, variant, ws,
+                          need > 0 ? trt::kStaticScratchBytes : 0, stream);
 }
