@@ -17,27 +17,29 @@ from scipy.special import logsumexp
 CLAMP = 1e38  # baselines/lm2exp.py:12
 
 
-def _f64(t) -> torch.Tensor:
-    return torch.as_tensor(t).detach().to("cpu", torch.float64)
+def _f64(t, device="cpu") -> torch.Tensor:
+    return torch.as_tensor(t).detach().to(device, torch.float64)
 
 
-def lm2exp64(a, b) -> torch.Tensor:
-    """c[r,i,k] = log sum_j a[r,i,j] exp b[r,j,k]; recipe of baselines/lm2exp.py:11-14."""
-    a, b = _f64(a), _f64(b)
+def lm2exp64(a, b, *, device="cpu") -> torch.Tensor:
+    """c[r,i,k] = log sum_j a[r,i,j] exp b[r,j,k]; recipe of baselines/lm2exp.py:11-14.
+    ``device``: where torch evaluates it (the CPU; or the GPU, whose float64 ATen / BLAS
+    routines share nothing with the kernels under test, for full-size inputs)."""
+    a, b = _f64(a, device), _f64(b, device)
     m = torch.amax(b, dim=1, keepdim=True)
     m = torch.clamp(m, -CLAMP, CLAMP)
     r = torch.bmm(a, torch.exp(b - m))
     return m + torch.log(r)
 
 
-def lt2exp64(w, a, b, *, batch_chunk: int = 1) -> torch.Tensor:
+def lt2exp64(w, a, b, *, batch_chunk: int = 1, device="cpu") -> torch.Tensor:
     """c[r,s,k] = log sum_ij w[r,s,i,j] exp a[r,i,k] exp b[r,j,k]; recipe of
     baselines/lt2exp.py:15-25, evaluated ``batch_chunk`` batches at a time so the
-    R x (I*J) x K intermediate stays small."""
-    w, a, b = _f64(w), _f64(a), _f64(b)
+    R x (I*J) x K intermediate stays small.  ``device`` as for lm2exp64."""
+    w, a, b = _f64(w, device), _f64(a, device), _f64(b, device)
     R, S, I, J = w.shape
     K = a.shape[2]
-    out = torch.empty((R, S, K), dtype=torch.float64)
+    out = torch.empty((R, S, K), dtype=torch.float64, device=device)
     for r0 in range(0, R, batch_chunk):
         sl = slice(r0, min(R, r0 + batch_chunk))
         ma = torch.clamp(torch.amax(a[sl], dim=1, keepdim=True), -CLAMP, CLAMP)

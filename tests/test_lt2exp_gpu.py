@@ -233,18 +233,38 @@ def test_benchmark_configuration_c4(dev):
     assert torch.allclose(torch_baseline.lt2exp_fp32(w, a, b), out.cpu(), rtol=1e-5, atol=1e-5)
 
 
+def _all_batches_against_float64_on_the_gpu(out, wg, ag, bg, **gate):
+    """Every batch of a full-size result against the float64 recipe evaluated by torch on the GPU
+    (ATen / BLAS float64 routines: nothing of this library), 8 batches at a time."""
+    worst = 0.0
+    for r0 in range(0, wg.shape[0], 8):
+        sl = slice(r0, r0 + 8)
+        ref = oracle64.lt2exp64(wg[sl], ag[sl], bg[sl], device=wg.device)
+        res = oracle64.compare(out[sl], ref, **gate)
+        assert res["ok"], (r0, res)
+        worst = max(worst, res["worst_err_over_tol"])
+    return worst
+
+
 def test_benchmark_configuration_c5_full_size(dev):
-    """R=64, S=I=J=64, K=4096: float64 oracle on 8 of the 64 batches, the lm2exp
-    identity and shift equivariance on the whole output."""
+    """R=64, S=I=J=64, K=4096: all 64 batches against the float64 recipe (evaluated by torch on the
+    GPU; 8 of them also on the CPU), then the lm2exp identity and shift equivariance on the
+    whole output."""
     cfg = workloads.c5()
     w, a, b = cfg["w"], cfg["a"], cfg["b"]
     wg, ag, bg = w.to(dev), a.to(dev), b.to(dev)
     out = lt2exp(wg, ag, bg)
     torch.cuda.synchronize()
     assert out.shape == (64, 64, 4096) and torch.isfinite(out).all()
+    _all_batches_against_float64_on_the_gpu(out, wg, ag, bg)
     for r in (0, 9, 18, 27, 36, 45, 54, 63):
         res = oracle64.compare(out[r:r + 1], oracle64.lt2exp64(w[r:r + 1], a[r:r + 1], b[r:r + 1]))
         assert res["ok"], (r, res)
+    # and the reference's own bar against its fp32 recipe, evaluated by torch on the GPU
+    # (tests/lt2exp.py:23-40: allclose defaults would be rtol 1e-5; the values here are ~ -50)
+    for r0 in range(0, 64, 4):
+        sl = slice(r0, r0 + 4)
+        assert torch.allclose(torch_baseline.lt2exp_fp32(wg[sl], ag[sl], bg[sl]), out[sl], rtol=1e-5, atol=1e-5)
     # the same contraction through the other kernel, 16 batches at a time (1 GiB intermediate each)
     for r0 in range(0, 64, 16):
         sl = slice(r0, r0 + 16)
@@ -254,8 +274,12 @@ def test_benchmark_configuration_c5_full_size(dev):
         del ab, via
     assert torch.allclose(lt2exp(wg, ag + 64.0, bg - 32.0), out + 32.0, rtol=1e-5, atol=1e-3)
     for variant in (1, 3):
-        assert torch.allclose(lt2exp(wg, ag, bg, _variant=variant), out, rtol=1e-5, atol=1e-5)
-    assert torch.allclose(lt2exp(wg, ag, bg, mode="split"), out, rtol=1e-5, atol=1e-5)
+        alt = lt2exp(wg, ag, bg, _variant=variant)
+        _all_batches_against_float64_on_the_gpu(alt, wg, ag, bg)
+        assert torch.allclose(alt, out, rtol=1e-5, atol=1e-5)
+    split = lt2exp(wg, ag, bg, mode="split")
+    _all_batches_against_float64_on_the_gpu(split, wg, ag, bg)
+    assert torch.allclose(split, out, rtol=1e-5, atol=1e-5)
 
 
 def test_capturable_in_a_hip_graph(dev):
@@ -367,13 +391,14 @@ def test_bf16x6_is_as_accurate_as_the_fp32_kernel(dev):
 
 @pytest.mark.parametrize("precision", ["bf16x3", "bf16x6"])
 def test_bf16_paths_c5_full_size(dev, precision):
-    """Full-size check through properties that need no oracle: shifting a column of a or b
-    by t shifts the output column by t, scaling a row of w by 2^k adds k*log(2) exactly up
-    to rounding, and a sample of batches is compared with the float64 oracle."""
+    """All 64 batches against the float64 recipe (torch on the GPU; three of them on the CPU as
+    well), and properties that need no oracle: shifting a column of a or b by t shifts the
+    output column by t, scaling a row of w by 2^k adds k*log(2) exactly up to rounding."""
     c = workloads.c5()
     w, a, b = (c[k].to(dev) for k in "wab")
     out = lt2exp(w, a, b, _precision=precision)
     gate = PRECISION_GATES[precision]
+    _all_batches_against_float64_on_the_gpu(out, w, a, b, **gate)
     for r in (0, 37, 63):
         ref = oracle64.lt2exp64(c["w"][r : r + 1], c["a"][r : r + 1], c["b"][r : r + 1])
         res = oracle64.compare(out[r : r + 1], ref, **gate)
