@@ -4,7 +4,8 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W]
 
 A step is one ``lt2exp`` call on the large configuration (R=64, S=I=J=64, K=4096,
-fp32, seeded synthetic inputs already resident in HBM).  W untimed steps, then
+fp32, seeded synthetic inputs already resident in HBM).  An untimed pre-conditioning
+phase of the same call (250 ms, reported as ``prewarm_ms``), W untimed steps, then
 exactly K steps bracketed by ``torch.cuda.synchronize()``; rank 0 prints ONE
 JSON line on stdout (progress goes to stderr).  The same line carries
 
@@ -33,19 +34,47 @@ PEAK_FP32_MFMA_TFLOPS = 157.3  # 256 CU x 4 SIMD x 64 flop/clk x 2.4 GHz
 PEAK_HBM_GBPS = 8000.0
 PEAK_BF16_MFMA_TFLOPS = 2516.6  # 16x the fp32 matrix rate
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, then WRITE_SIZE, one run
-# each over `bench.py --profile-pass`), scaled by what the same counters read for
-# trt_copy_bytes of 256 MiB (factors 2.000 and 1.000 to KiB); the summary of those runs is
-# profiles/lt2exp_lm2exp_max_counters.md.  A constant, not a live measurement.
-MEASURED_TRAFFIC_BYTES = {"lt2exp_c5": 452.9e6, "lm2exp_c3": 682.4e6}
+# HBM bytes per launch come from the committed counter summary (rocprofv3 --pmc FETCH_SIZE, then
+# WRITE_SIZE, one run each over `bench.py --profile-pass`, scaled by what the same counters read for
+# trt_copy_bytes of 256 MiB): the row of the kernel that this run times, looked up by the name
+# the library reports for the call.  No row for that kernel: the bench stops and says so.
+COUNTER_SUMMARY = os.path.join(os.path.dirname(os.path.abspath(__file__)), "profiles",
+                               "lt2exp_lm2exp_max_counters.md")
+PREWARM_MS = 250.0  # untimed launches of the same call before the warm-up steps (clock / power settle)
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
+def measured_traffic_bytes(kernel: str) -> float:
+    """HBM bytes per launch of `kernel` from the 'total MB' column of the counter summary."""
+    with open(COUNTER_SUMMARY) as f:
+        rows = [ln for ln in f if ln.startswith("| `")]
+    for ln in rows:
+        cells = [c.strip() for c in ln.strip().strip("|").split("|")]
+        if cells[0].strip("`") == kernel and len(cells) >= 7:
+            return float(cells[5]) * 1e6
+    raise SystemExit(
+        f"bench.py: {COUNTER_SUMMARY} has no HBM-traffic row for the kernel this run times, `{kernel}`: "
+        "regenerate the counter summary (the commands are in that file) before quoting a roofline")
+
+
 def timed_region(fn, steps: int, warmup: int):
-    """(wall seconds, HIP-event seconds) over exactly `steps` calls."""
+    """Times exactly `steps` calls: {wall_s, event_s} over the whole region (HIP events recorded on
+    the launch stream) and the median / q10 / q90 of per-call HIP-event times from a second pass of
+    the same length.  Before the warm-up steps the call is repeated, untimed, for PREWARM_MS so
+    that a short region does not measure the clock and power transient left by what ran before."""
+    fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    n_pre = 0
+    while (time.perf_counter() - t0) * 1e3 < PREWARM_MS:
+        for _ in range(8):
+            fn()
+        torch.cuda.synchronize()
+        n_pre += 8
+    prewarm_ms = (time.perf_counter() - t0) * 1e3
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -58,7 +87,17 @@ def timed_region(fn, steps: int, warmup: int):
     stop.record()
     torch.cuda.synchronize()
     wall = time.perf_counter() - t0
-    return wall, start.elapsed_time(stop) * 1e-3
+    ev = start.elapsed_time(stop) * 1e-3
+    marks = [torch.cuda.Event(enable_timing=True) for _ in range(steps + 1)]
+    marks[0].record()
+    for i in range(steps):
+        fn()
+        marks[i + 1].record()
+    torch.cuda.synchronize()
+    per = sorted(marks[i].elapsed_time(marks[i + 1]) for i in range(steps))
+    q = lambda f: per[min(len(per) - 1, int(f * len(per)))]
+    return {"wall_s": wall, "event_s": ev, "median_ms": q(0.5), "q10_ms": q(0.1), "q90_ms": q(0.9),
+            "prewarm_ms": round(prewarm_ms, 1), "prewarm_calls": n_pre}
 
 
 def do_bench(fn, *, warmup_ms=150.0, rep_ms=1000.0, flush_bytes=512 << 20):
@@ -198,6 +237,7 @@ def main() -> int:
         log("bench.py: no HIP device visible")
         return 3
 
+    from triturus_amd import _lib
     from triturus_amd import workloads as W
     from triturus_amd.lm2exp import lm2exp
     from triturus_amd.lt2exp import lt2exp
@@ -216,7 +256,9 @@ def main() -> int:
     w, a, b = (cfg[k].to(dev) for k in "wab")
     flops = W.lt2exp_flops(R, S, I, J, K)
     step = lambda: lt2exp(w, a, b, _precision="fp32")
-    wall, ev = timed_region(step, args.steps, args.warmup)
+    kernel = _lib.kernel_name("lt2exp", R, S, I, J, K, _lib.MODE_AUTO, 0, 1)
+    tr = timed_region(step, args.steps, args.warmup)
+    wall, ev = tr["wall_s"], tr["event_s"]
     ms_per_step = wall / args.steps * 1e3
     value = flops * args.steps / wall / 1e9
     achieved = flops / (ev / args.steps) / 1e12
@@ -243,9 +285,13 @@ def main() -> int:
             "peak": PEAK_FP32_MFMA_TFLOPS,
             "unit": "TFLOP/s",
             "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4),
-            "traffic": MEASURED_TRAFFIC_BYTES["lt2exp_c5"],
-            "kernel": "lt2exp_kernel<RT=2,CT=1,NQ=4,NWAVES=4,VEC,unsplit>",
+            "traffic": measured_traffic_bytes(kernel),
+            "kernel": kernel,
+            "launch_ms": {"mean": round(ev / args.steps * 1e3, 5), "median": round(tr["median_ms"], 5),
+                          "q10": round(tr["q10_ms"], 5), "q90": round(tr["q90_ms"], 5)},
+            "frac_at_median": round(flops / (tr["median_ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4),
         },
+        "prewarm_ms": tr["prewarm_ms"],
     }
 
     from oracle import torch_baseline  # CPU competitor lines only; never on the GPU path
@@ -273,8 +319,7 @@ def main() -> int:
         out = {}
         for prec, mfmas in (("bf16x3", 3), ("bf16x6", 6)):
             fn = lambda: fn_of_precision(prec)
-            _, evp = timed_region(fn, args.steps, args.warmup)
-            t = evp / args.steps
+            t = timed_region(fn, args.steps, args.warmup)["event_s"] / args.steps
             out[prec] = {
                 "ms": round(t * 1e3, 5),
                 "equivalent_TFLOPs": round(flops_alg / t / 1e12, 2),
@@ -299,7 +344,9 @@ def main() -> int:
         a3, b3 = cfg3["a"].to(dev), cfg3["b"].to(dev)
         fl3 = W.lm2exp_flops(R2, I2, J2, K2)
         step3 = lambda: lm2exp(a3, b3, _precision="fp32")
-        wall3, ev3 = timed_region(step3, args.steps, args.warmup)
+        kernel3 = _lib.kernel_name("lm2exp", R2, I2, J2, K2, 0, 0, 1)
+        tr3 = timed_region(step3, args.steps, args.warmup)
+        wall3, ev3 = tr3["wall_s"], tr3["event_s"]
         ach3 = fl3 / (ev3 / args.steps) / 1e12
         lm = {
             "workload": "lm2exp R=64 I=256 J=256 K=4096 (b ~ N(-50,20), 5% -inf)",
@@ -309,7 +356,11 @@ def main() -> int:
             "algorithmic_bytes": W.lm2exp_bytes(R2, I2, J2, K2),
             "roofline": {"bound": "mfma", "achieved": round(ach3, 2), "peak": PEAK_FP32_MFMA_TFLOPS,
                          "unit": "TFLOP/s", "frac": round(ach3 / PEAK_FP32_MFMA_TFLOPS, 4),
-                         "traffic": MEASURED_TRAFFIC_BYTES["lm2exp_c3"]},
+                         "traffic": measured_traffic_bytes(kernel3), "kernel": kernel3,
+                         "launch_ms": {"mean": round(ev3 / args.steps * 1e3, 5), "median": round(tr3["median_ms"], 5),
+                                       "q10": round(tr3["q10_ms"], 5), "q90": round(tr3["q90_ms"], 5)},
+                         "frac_at_median": round(fl3 / (tr3["median_ms"] * 1e-3) / 1e12 / PEAK_FP32_MFMA_TFLOPS, 4)},
+            "prewarm_ms": tr3["prewarm_ms"],
             "do_bench": do_bench(step3),
         }
         log(f"lm2exp rect: {ev3 / args.steps * 1e3:.4f} ms/launch, {ach3:.1f} TFLOP/s = "
@@ -329,6 +380,23 @@ def main() -> int:
         lm["split_bf16"] = sb3
         result["lm2exp"] = lm
         del a3, b3
+
+        # ------------------------------------ lm2exp, smallest configuration: bound by the host
+        c1 = W.c1()
+        a1, b1 = c1["a"].to(dev), c1["b"].to(dev)
+        for _ in range(200):
+            lm2exp(a1, b1)
+        torch.cuda.synchronize()
+        n1 = 2000
+        t0 = time.perf_counter()
+        for _ in range(n1):
+            lm2exp(a1, b1)
+        torch.cuda.synchronize()
+        eager_us = (time.perf_counter() - t0) / n1 * 1e6
+        result["c1"] = {"workload": "lm2exp R=4 I=J=K=64", "eager_us_per_call": round(eager_us, 2),
+                        "hip_graph_us_per_call": round(graph_time(lambda: lm2exp(a1, b1)) * 1e6, 2)}
+        log(f"lm2exp smallest configuration: {eager_us:.2f} us per eager call through the Python wrapper, "
+            f"{result['c1']['hip_graph_us_per_call']:.2f} us inside a HIP graph")
 
         # ------------------------------------------------ max reductions (HBM bound)
         x = cfg["b"].to(dev)  # 64 x 64 x 4096

@@ -247,6 +247,19 @@ int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, int64_t k, 
 int trt_vadd(const void *x, const void *y, void *r, int64_t n, int dtype, void *stream);
 
 /*
+ * Name of the contraction kernel that a trt_lt2exp_f32 / trt_lm2exp_f32 call with these sizes
+ * and choices launches, written to buf as a profiler prints it (e.g.
+ * "trt::lt2exp_kernel<2, 1, 4, 4, true, false, 1, 0>").  Host only.  w_aligned / a_vec: the
+ * operand's base and leading strides are multiples of 16 bytes (and a has a unit trailing
+ * stride).  No counterpart in the reference: benchmarks use it to find their kernel in
+ * profiler output.
+ */
+int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode,
+                           int variant, int w_aligned, char *buf, size_t buf_bytes);
+int trt_lm2exp_kernel_name(int64_t R, int64_t I, int64_t J, int64_t K, int variant, int splits,
+                           int a_vec, char *buf, size_t buf_bytes);
+
+/*
  * Plain device-to-device copy kernel of nbytes (multiple of 16, 16-byte
  * aligned pointers).  No counterpart in the reference: it is the known-size
  * kernel that hardware byte counters are calibrated against.

@@ -88,6 +88,8 @@ SIGNATURES = {
     "trt_mm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "trt_vadd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "trt_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "trt_lt2exp_kernel_name": (c_int, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_char_p, c_size_t]),
+    "trt_lm2exp_kernel_name": (c_int, [c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_char_p, c_size_t]),
 }
 
 _lock = threading.Lock()
@@ -126,8 +128,29 @@ def check(status: int, what: str) -> None:
         raise RuntimeError(f"{what} failed with status {status}: {text.decode() if text else '?'}")
 
 
+def kernel_name(op: str, *args: int) -> str:
+    """Profiler name of the contraction kernel a call launches (trt_lt2exp_kernel_name / trt_lm2exp_kernel_name)."""
+    buf = ctypes.create_string_buffer(160)
+    check(getattr(load(), f"trt_{op}_kernel_name")(*args, buf, len(buf)), f"trt_{op}_kernel_name")
+    return buf.value.decode()
+
+
+_stride_arrays: dict = {}  # stride tuple -> ctypes array (read-only to the library, so shareable)
+
+
 def strides3(t: torch.Tensor):
-    return _I64x3(*t.stride())
+    return stride_array(t.stride())
+
+
+def stride_array(st: tuple):
+    """ctypes int64[3] of an element-stride tuple, cached: building one costs as much as a dict lookup
+    saves on the small calls that are bound by the host."""
+    arr = _stride_arrays.get(st)
+    if arr is None:
+        if len(_stride_arrays) > 4096:
+            _stride_arrays.clear()
+        arr = _stride_arrays[st] = _I64x3(*st)
+    return arr
 
 
 def current_stream(device: torch.device) -> c_void_p:
@@ -171,6 +194,7 @@ def on_device(device: torch.device):
     if idx is None or idx == _get_device():
         return _NO_SWITCH
     return torch.cuda.device(device)
+
 
 
 def require_gpu(*tensors: torch.Tensor) -> None:

@@ -29,6 +29,8 @@
 #include "common.hpp"
 #include "lm2exp_merge.hpp"
 
+#include <cstdio>
+
 namespace trt {
 
 constexpr float kRescaleMargin = 8.0f;
@@ -828,6 +830,25 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     if (st != 0 || pl.splits <= 1) return st;
     launch_lm2exp_merge(args.part, args.shift, c, R, I, K, pl.splits, sc[0], sc[1], s);
     return (int)hipGetLastError();
+}
+
+// Name of the contraction kernel a trt_lm2exp_f32 call with these arguments launches, as a
+// profiler prints it (host only; a_vec: a has a unit trailing stride and base and leading
+// strides that are multiples of 16 bytes).  Benchmarks use it to look their kernel up in
+// profiler output.
+extern "C" int trt_lm2exp_kernel_name(int64_t R, int64_t I, int64_t J, int64_t K, int variant, int splits, int a_vec,
+                                      char *buf, size_t buf_bytes) {
+    if (!buf || buf_bytes == 0 || R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
+    if (variant < 0 || variant > kNumVariants || splits < 0) return TRT_E_INVALID;
+    const Lm2Variant &vr = kVariants[make_plan(R, I, J, K, variant, splits).variant];
+    int n;
+    if (vr.mode == kPair)
+        n = snprintf(buf, buf_bytes, "trt::lm2exp_pair_kernel<%d, %d, %d, %d>", vr.rt, vr.wn, vr.nq,
+                     a_vec ? kLoadVec : kLoadByCol);
+    else
+        n = snprintf(buf, buf_bytes, "trt::lm2exp_kernel<%d, %d, %d, %d, %d, %s, %d>", vr.rt, vr.ct, vr.wm, vr.wn, vr.nq,
+                     a_vec ? "true" : "false", vr.mode);
+    return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
 }
 
 // Batched column maxima m[r,k] = max_j b[r,j,k] of an R x J x K fp32 tensor (a NaN wins, as in

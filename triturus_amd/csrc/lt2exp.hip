@@ -22,6 +22,7 @@
 #include "common.hpp"
 #include "lt2exp_merge.hpp"
 
+#include <cstdio>
 #include <mutex>
 
 namespace trt {
@@ -653,6 +654,28 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     launch_variant(v, args, vec, sp.split, s);
     if (sp.split) launch_lt2exp_merge(args.c, args.shift, c, R, S, K, sp.splits, sc[0], sc[1], s);
     return (int)hipGetLastError();
+}
+
+// Name of the contraction kernel a trt_lt2exp_f32 call with these arguments launches, as a
+// profiler prints it (host only; w_aligned: base and both leading strides of w are multiples
+// of 16 bytes).  Benchmarks use it to look their kernel up in profiler output.
+extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode, int variant,
+                                      int w_aligned, char *buf, size_t buf_bytes) {
+    if (!buf || buf_bytes == 0 || R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
+    if (variant < 0 || variant > kNumVariants) return TRT_E_INVALID;
+    if (J == 1 && I > 1 && variant == 0) {  // runs with the roles of i and j exchanged
+        J = I;
+        I = 1;
+    }
+    int v = resolve_variant(variant, R, S, I, J, K);
+    if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
+    const Lt2Variant &vr = kVariants[v];
+    const SplitPlan sp = plan_split(R, S, I, J, K, mode, v);
+    const bool vec = vr.pack || ((J % 4 == 0) && w_aligned);
+    const int n = snprintf(buf, buf_bytes, "trt::lt2exp_kernel<%d, %d, %d, %d, %s, %s, %d, %d>", vr.rt, vr.ct,
+                           vr.pack ? 2 : vr.nq, kLt2Waves, vec ? "true" : "false", sp.split ? "true" : "false", vr.wm,
+                           vr.pack ? (int)J : 0);
+    return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
 }
 
 // ---------------------------------------------------------------------------------------------

@@ -48,18 +48,21 @@ _BF16_CANDIDATES = (0, 1, 2, 3, 4, 8, 9)
 def lm2exp(
     a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0, _splits: int = 0, _precision: str | None = None
 ) -> torch.Tensor:
-    assert len(a.shape) == len(b.shape) == 3
-    assert a.shape[0] == b.shape[0]
-    assert a.shape[2] == b.shape[1]
+    ash, bsh = a.shape, b.shape
+    assert len(ash) == len(bsh) == 3
+    assert ash[0] == bsh[0]
+    assert ash[2] == bsh[1]
     assert a.dtype == b.dtype == torch.float32
-    assert a.device == b.device
-    _lib.require_gpu(a, b)
-    lib = _lib.load()
+    dev = a.device
+    assert dev == b.device
+    if not a.is_cuda:
+        _lib.require_gpu(a, b)
+    lib = _lib._lib or _lib.load()
 
-    R, I, J = a.shape
-    K = b.shape[2]
-    c = torch.empty((R, I, K), dtype=a.dtype, device=a.device)
-    if c.numel() == 0:
+    R, I, J = ash
+    K = bsh[2]
+    c = a.new_empty((R, I, K))
+    if R * I * K == 0:
         return c
     if J == 0:
         # empty contraction: log(0)
@@ -68,27 +71,33 @@ def lm2exp(
         _precision = matrix_precision()
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
+    fp32 = _precision == "fp32"
     # a goes to the fp32 kernels with whatever non-negative strides it has (a transposed or
     # strided view is read in place, as the reference does: triturus/lm2exp.py:190-198); the
     # bf16 kernels and every kernel's b want a unit trailing stride
-    if _precision != "fp32" or min(a.stride()) < 0:
+    sa, sb = a.stride(), b.stride()
+    if (not fp32 and sa[2] != 1) or min(sa) < 0:
         a = _unit_inner(a)
-    b = _unit_inner(b)
-    if _variant == 0 and _splits == 0 and a.stride(2) == 1 and autotune.is_autotune_enabled():
-        cands = _FP32_CANDIDATES if _precision == "fp32" else _BF16_CANDIDATES
+        sa = a.stride()
+    if sb[2] != 1 or min(sb) < 0:
+        b = _unit_inner(b)
+        sb = b.stride()
+    if _variant == 0 and _splits == 0 and sa[2] == 1 and autotune.is_autotune_enabled():
+        cands = _FP32_CANDIDATES if fp32 else _BF16_CANDIDATES
         _variant = autotune.pick(("lm2exp", R, I, J, K, _precision), cands,
                                  lambda v: lm2exp(a, b, _variant=v, _splits=-1, _precision=_precision))
     # Rows of a are read 16 bytes at a time when they start aligned; with J not a multiple of 4 a
     # contiguous a does not qualify and the kernels fall back to element loads (10-50 % slower).
     # A call with enough work per element of a (the copy costs ~3 ps per element, the element loads
     # ~15 % of 20 fs x K) runs on a copy of a whose rows are padded to a multiple of 4.
-    if J % 4 != 0 and J > 4 and a.stride(2) == 1 and K >= _PAD_MIN_K and 2 * R * I * J * K >= _PAD_MIN_FLOPS:
+    if J % 4 != 0 and J > 4 and sa[2] == 1 and K >= _PAD_MIN_K and 2 * R * I * J * K >= _PAD_MIN_FLOPS:
         a = torch.nn.functional.pad(a, (0, (-J) % 4))[..., :J]
+        sa = a.stride()
     if _splits < 0:  # tuning launch: the library decides the split for this tile
         _splits = 0
     # small grids with a long contraction are cut over J; the partial sums need a workspace
-    fp32_variant = _variant if _precision == "fp32" else 0
-    pieces = 0 if _precision == "fp32" else _PIECES[_precision]
+    fp32_variant = _variant if fp32 else 0
+    pieces = 0 if fp32 else _PIECES[_precision]
     key = (R, I, J, K, fp32_variant, _splits, pieces)
     ws_bytes = _ws_bytes.get(key)
     if ws_bytes is None:
@@ -96,23 +105,27 @@ def lm2exp(
         if pieces:  # the bf16 entry may cut a small grid itself
             ws_bytes = max(ws_bytes, lib.trt_lm2exp_bf16_workspace_bytes(R, I, J, K, pieces, _splits))
         _ws_bytes[key] = ws_bytes
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
-    ws_ptr = ws.data_ptr() if ws_bytes else None
-    with _lib.on_device(a.device):
-        if _precision == "fp32":
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+        ws_ptr = ws.data_ptr()
+    else:
+        ws_ptr = None
+    stride_array = _lib.stride_array
+    with _lib.on_device(dev):
+        if fp32:
             status = lib.trt_lm2exp_f32(
                 a.data_ptr(), b.data_ptr(), c.data_ptr(),
-                R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-                _variant, _splits, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
+                R, I, J, K, stride_array(sa), stride_array(sb), stride_array((I * K, K, 1)),
+                _variant, _splits, ws_ptr, ws_bytes, _lib.raw_stream(dev),
             )
         else:
             # bf16 matrix pipe; a grid too small for it has its contraction cut over J or goes
             # back to the fp32 kernels (which may cut it as well: hence the workspace)
             status = lib.trt_lm2exp_bf16(
                 a.data_ptr(), b.data_ptr(), c.data_ptr(),
-                R, I, J, K, _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-                _PIECES[_precision], _variant, _splits, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
+                R, I, J, K, stride_array(sa), stride_array(sb), stride_array((I * K, K, 1)),
+                pieces, _variant, _splits, ws_ptr, ws_bytes, _lib.raw_stream(dev),
             )
     if status:
-        _lib.check(status, "trt_lm2exp_f32" if _precision == "fp32" else "trt_lm2exp_bf16")
+        _lib.check(status, "trt_lm2exp_f32" if fp32 else "trt_lm2exp_bf16")
     return c

@@ -65,25 +65,29 @@ def lt2exp(
     w: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, mode: str = "auto", _variant: int = 0,
     _precision: str | None = None, _tuning: bool = False,
 ) -> torch.Tensor:
-    assert len(w.shape) == 4
-    assert len(a.shape) == len(b.shape) == 3
-    assert w.shape[0] == a.shape[0] == b.shape[0]
-    assert w.shape[2] == a.shape[1]
-    assert w.shape[3] == b.shape[1]
-    assert a.shape[2] == b.shape[2]
+    wsh, ash, bsh = w.shape, a.shape, b.shape
+    assert len(wsh) == 4
+    assert len(ash) == len(bsh) == 3
+    assert wsh[0] == ash[0] == bsh[0]
+    assert wsh[2] == ash[1]
+    assert wsh[3] == bsh[1]
+    assert ash[2] == bsh[2]
     assert w.dtype == a.dtype == b.dtype == torch.float32
     assert w.device == a.device == b.device
-    R, S, I, J = w.shape
-    K = a.shape[2]
-    launches_split(R, S, I, J, K, mode)  # validates mode
-    _lib.require_gpu(w, a, b)
-    lib = _lib.load()
+    R, S, I, J = wsh
+    K = ash[2]
+    mode_code = _MODES.get(mode)
+    if mode_code is None:
+        launches_split(R, S, I, J, K, mode)  # raises the reference's ValueError
+    if not w.is_cuda:
+        _lib.require_gpu(w, a, b)
+    lib = _lib._lib or _lib.load()
 
-    c = torch.empty((R, S, K), dtype=a.dtype, device=a.device)
+    c = a.new_empty((R, S, K))
     # the reference flattens with w.view(batch, m, -1) (triturus/lt2exp.py:549); naming the
     # size keeps the same RuntimeError for non-viewable w and also accepts empty tensors
     w = w.view(R, S, I * J)
-    if c.numel() == 0:
+    if R * S * K == 0:
         return c
     if I * J == 0:
         return c.fill_(float("-inf"))
@@ -122,15 +126,21 @@ def lt2exp(
         w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
         b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
         J = J4
-    w = _unit_inner(w)
-    a = _unit_inner(a)
-    b = _unit_inner(b)
+    sw, sa, sb = w.stride(), a.stride(), b.stride()
+    if sw[2] != 1 or min(sw) < 0:
+        w = _unit_inner(w)
+        sw = w.stride()
+    if sa[2] != 1 or min(sa) < 0:
+        a = _unit_inner(a)
+        sa = a.stride()
+    if sb[2] != 1 or min(sb) < 0:
+        b = _unit_inner(b)
+        sb = b.stride()
     if _variant == 0 and autotune.is_autotune_enabled() and not _tuning:
         cands = _FP32_CANDIDATES if _precision == "fp32" else _BF16_CANDIDATES
         _variant = autotune.pick(("lt2exp", R, S, I, J, K, mode, _precision), cands,
                                  lambda v: lt2exp(w.view(R, S, I, J), a, b, mode=mode, _variant=v,
                                                   _precision=_precision, _tuning=True))
-    mode_code = _MODES[mode]
     pieces = _PIECES.get(_precision, 0)
     key = (R, S, I, J, K, mode_code, pieces)
     ws_bytes = _ws_bytes.get(key)
@@ -139,23 +149,28 @@ def lt2exp(
         if pieces:  # the bf16 entry may cut a small grid itself
             ws_bytes = max(ws_bytes, lib.trt_lt2exp_bf16_workspace_bytes(R, S, I, J, K, pieces, mode_code))
         _ws_bytes[key] = ws_bytes
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
-    ws_ptr = ws.data_ptr() if ws_bytes else None
-    with _lib.on_device(a.device):
-        if _precision == "fp32":
+    if ws_bytes:
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device)
+        ws_ptr = ws.data_ptr()
+    else:
+        ws_ptr = None
+    dev = a.device
+    stride_array = _lib.stride_array
+    with _lib.on_device(dev):
+        if pieces == 0:
             status = lib.trt_lt2exp_f32(
                 w.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), R, S, I, J, K,
-                _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-                mode_code, _variant, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
+                stride_array(sw), stride_array(sa), stride_array(sb), stride_array((S * K, K, 1)),
+                mode_code, _variant, ws_ptr, ws_bytes, _lib.raw_stream(dev),
             )
         else:
             # bf16 matrix pipe; the library hands grids that are too small for it (those the
             # fp32 path would cut over the contraction) back to the fp32 kernels
             status = lib.trt_lt2exp_bf16(
                 w.data_ptr(), a.data_ptr(), b.data_ptr(), c.data_ptr(), R, S, I, J, K,
-                _lib.strides3(w), _lib.strides3(a), _lib.strides3(b), _lib.strides3(c),
-                pieces, mode_code, _variant, ws_ptr, ws_bytes, _lib.raw_stream(a.device),
+                stride_array(sw), stride_array(sa), stride_array(sb), stride_array((S * K, K, 1)),
+                pieces, mode_code, _variant, ws_ptr, ws_bytes, _lib.raw_stream(dev),
             )
     if status:
-        _lib.check(status, "trt_lt2exp_f32" if _precision == "fp32" else "trt_lt2exp_bf16")
+        _lib.check(status, "trt_lt2exp_f32" if pieces == 0 else "trt_lt2exp_bf16")
     return c
