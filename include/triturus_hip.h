@@ -187,6 +187,16 @@ size_t trt_lm2exp_bf16_workspace_bytes(int64_t R, int64_t I, int64_t J, int64_t 
 int trt_lm2exp_bf16_variant_count(void);
 
 /*
+ * Workspaces of the max reductions (trt_matmax, trt_vmax) start with arrival counters: the
+ * workgroup that finishes last combines the partial results of all of them, so a reduction is
+ * one launch.  The first TRT_MAX_TICKET_BYTES of such a workspace must be ZERO before the first
+ * call that uses it (one hipMemset when it is allocated); every call leaves them zero, so a
+ * workspace can be reused from call to call -- by one stream at a time: calls that overlap in
+ * time need workspaces of their own.
+ */
+#define TRT_MAX_TICKET_BYTES 65536
+
+/*
  * Max of a contiguous m x n row-major matrix along axis 0 (y has n entries)
  * or axis 1 (y has m entries).  NaN propagates as in torch.amax.  Replaces the
  * multi-launch `_ker_matmax` tree, triturus/max.py:190-225.  workspace:

@@ -56,6 +56,10 @@ __device__ __forceinline__ double neg_inf<double>() { return -__builtin_inf(); }
 
 constexpr int64_t kNoIdx = INT64_MAX;
 
+// max that ignores a NaN operand (both NaN: NaN), one instruction without canonicalisation moves
+__device__ __forceinline__ float max_ignoring_nan(float a, float b) { return max3_raw(a, b, b); }
+__device__ __forceinline__ double max_ignoring_nan(double a, double b) { return __builtin_fmax(a, b); }
+
 template <typename C>
 __device__ __forceinline__ C vmax_nan(C a, C b) {
     return (a > b || a != a) ? a : b;
@@ -71,33 +75,78 @@ __device__ __forceinline__ bool prefer(C v, int64_t i, C bv, int64_t bi) {
     return strictly || (same && i < bi);
 }
 
-template <typename C>
-__device__ __forceinline__ C shfl_xor_c(C v, int off) { return __shfl_xor(v, off, kWave); }
-
-__device__ __forceinline__ int64_t shfl_xor_i64(int64_t v, int off) {
-    int lo = __shfl_xor((int)(uint32_t)(uint64_t)v, off, kWave);
-    int hi = __shfl_xor((int)(uint32_t)((uint64_t)v >> 32), off, kWave);
-    return (int64_t)(((uint64_t)(uint32_t)hi << 32) | (uint64_t)(uint32_t)lo);
+// ---- wavefront reductions on the data-parallel-primitive path: six register moves between
+// lanes (within quads, within rows of 16, then row to row) instead of six round trips through
+// the LDS permute unit; the result is complete in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_move(float v) {
+    const int x = __builtin_bit_cast(int, v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(x, x, CTRL, ROW_MASK, 0xf, false));
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ double dpp_move(double v) {
+    const uint64_t x = __builtin_bit_cast(uint64_t, v);
+    const int lo = (int)(uint32_t)x, hi = (int)(uint32_t)(x >> 32);
+    const uint32_t l2 = (uint32_t)__builtin_amdgcn_update_dpp(lo, lo, CTRL, ROW_MASK, 0xf, false);
+    const uint32_t h2 = (uint32_t)__builtin_amdgcn_update_dpp(hi, hi, CTRL, ROW_MASK, 0xf, false);
+    return __builtin_bit_cast(double, ((uint64_t)h2 << 32) | l2);
+}
+__device__ __forceinline__ float read_lane(float v, int lane) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), lane));
+}
+__device__ __forceinline__ double read_lane(double v, int lane) {
+    const uint64_t x = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)x, lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(x >> 32), lane);
+    return __builtin_bit_cast(double, ((uint64_t)hi << 32) | lo);
 }
 
+// Maximum over the wavefront (a NaN wins), the same value in every lane.
 template <typename C>
 __device__ __forceinline__ C wave_max(C v) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) v = vmax_nan(v, shfl_xor_c(v, off));
-    return v;
+    v = vmax_nan(v, dpp_move<0xb1, 0xf>(v));   // quad_perm [1,0,3,2]
+    v = vmax_nan(v, dpp_move<0x4e, 0xf>(v));   // quad_perm [2,3,0,1]
+    v = vmax_nan(v, dpp_move<0x114, 0xf>(v));  // row_shr 4
+    v = vmax_nan(v, dpp_move<0x118, 0xf>(v));  // row_shr 8
+    v = vmax_nan(v, dpp_move<0x142, 0xa>(v));  // row_bcast 15 into rows 1 and 3
+    v = vmax_nan(v, dpp_move<0x143, 0xc>(v));  // row_bcast 31 into rows 2 and 3
+    return read_lane(v, 63);
 }
 
+__device__ __forceinline__ int64_t read_lane(int64_t v, int lane) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(uint64_t)v, lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)((uint64_t)v >> 32), lane);
+    return (int64_t)(((uint64_t)hi << 32) | lo);
+}
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ int64_t min_with_moved(int64_t v) {
+    const int lo = (int)(uint32_t)(uint64_t)v, hi = (int)(uint32_t)((uint64_t)v >> 32);
+    const uint32_t l2 = (uint32_t)__builtin_amdgcn_update_dpp(lo, lo, CTRL, ROW_MASK, 0xf, false);
+    const uint32_t h2 = (uint32_t)__builtin_amdgcn_update_dpp(hi, hi, CTRL, ROW_MASK, 0xf, false);
+    const int64_t o = (int64_t)(((uint64_t)h2 << 32) | l2);
+    return o < v ? o : v;
+}
+
+// (Maximum, lowest index among the lanes that hold it) over the wavefront, in every lane: the
+// value by wave_max, then the smallest index of the lanes that hold it by the same six moves
+// (a fixed cost whether one lane holds the maximum or all of them do).
 template <typename C>
 __device__ __forceinline__ void wave_argmax(C &v, int64_t &i) {
-#pragma unroll
-    for (int off = kWave / 2; off > 0; off >>= 1) {
-        C ov = shfl_xor_c(v, off);
-        int64_t oi = shfl_xor_i64(i, off);
-        if (prefer(ov, oi, v, i)) {
-            v = ov;
-            i = oi;
-        }
-    }
+    const C m = wave_max(v);
+    const bool mine = (v == m) || (v != v && m != m);
+    int64_t j = mine ? i : kNoIdx;
+    j = min_with_moved<0xb1, 0xf>(j);
+    j = min_with_moved<0x4e, 0xf>(j);
+    j = min_with_moved<0x114, 0xf>(j);
+    j = min_with_moved<0x118, 0xf>(j);
+    j = min_with_moved<0x142, 0xa>(j);
+    j = min_with_moved<0x143, 0xc>(j);
+    const int64_t best = read_lane(j, 63);
+    // the value as the winning lane holds it (-0.0 and +0.0 compare equal: the bits of the
+    // element at the reported index are what torch.max returns)
+    const uint64_t winner = __builtin_amdgcn_ballot_w64(mine && i == best);
+    v = read_lane(v, __builtin_ctzll(winner ? winner : 1));
+    i = best;
 }
 
 // 16-byte vector of T
@@ -109,41 +158,78 @@ struct alignas(16) Vec16 {
 
 // ------------------------------------------------------------------- vmax
 constexpr int kVmaxThreads = 256;
-constexpr int kVmaxMaxBlocks = 2048;
-constexpr int kVmaxUnroll = 4;
+constexpr int kVmaxMaxBlocks = 512;  // two workgroups per compute unit; each walks several blocks
+constexpr int kVmaxUnroll = 8;
+constexpr int kVmaxGroup = 32;  // workgroups that draw from one arrival counter
 
-// FINAL: the launch has a single workgroup, which writes the result itself (short vectors
-// take one launch instead of two).
+// Arrival counters ("tickets") at the head of a max workspace: a launch whose workgroups leave
+// partial results takes one ticket per workgroup; the workgroup that draws the last one
+// combines the partials and puts the counter back to zero.  The counters must be zero before
+// the first call that uses a workspace and every call leaves them zero, so one launch does the
+// work of two and the library still keeps no state of its own.
+constexpr size_t kTicketBytes = TRT_MAX_TICKET_BYTES;
+// Counters that different groups of workgroups draw from sit 256 bytes apart: device-scope atomics on
+// one memory line are served one after the other (measured ~10 ns each), on different lines side by side.
+constexpr int kTicketStride = 256 / (int)sizeof(unsigned);
+constexpr int kMaxTickets = (int)(kTicketBytes / 256);
+static_assert(kVmaxMaxBlocks / kVmaxGroup < kMaxTickets, "one counter per group and one for the groups");
+
+// The partials of the other workgroups were written on other compute units (and other dies,
+// each with its own L2), so partials and tickets are device-scope atomic accesses, which go
+// past the caches that are not coherent across the device.  A device-scope FENCE would do as
+// well but writes back and invalidates whole caches, once per workgroup: measured 120 us
+// instead of 12 us on a 64 MiB vector.  Between its partial stores and its ticket a wavefront
+// waits for the stores to be acknowledged (a workgroup-scope release: a wait, no cache action).
+__device__ __forceinline__ unsigned take_ticket(unsigned *ticket) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    return __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Max and first-occurrence argmax in one launch.  Every 16-byte piece costs a couple of vector
+// instructions: the maximum of its elements (NaN ignored), one unordered test per pair of elements
+// to notice NaNs, and a compare-and-select of (value, piece number) -- the position inside the
+// piece is worked out once, at the end, by reading the winning piece again.  A wavefront that has
+// seen a NaN repeats its share element by element with the exact rule (a NaN wins, first one
+// reported), which costs nothing on inputs without NaN.
+// FINAL: the launch has a single workgroup, which writes the result itself.
 template <int DT, bool WITH_IDX, bool FINAL>
-__global__ __launch_bounds__(kVmaxThreads) void vmax_stage1(
+__global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     const typename Elem<DT>::T *__restrict__ x, int64_t n, int64_t head, int64_t nvec,
-    typename Elem<DT>::C *__restrict__ pval, int64_t *__restrict__ pidx,
+    typename Elem<DT>::C *pval, int64_t *pidx, unsigned *ticket,
     typename Elem<DT>::T *__restrict__ out_val, int64_t *__restrict__ out_idx) {
     using E = Elem<DT>;
     using T = typename E::T;
     using C = typename E::C;
     using V = Vec16<T>;
     constexpr int VN = V::N;
-
-    C best = neg_inf<C>();
-    int64_t bidx = kNoIdx;
-    auto feed = [&](C c, int64_t i) {
-        // indices arrive in increasing order within a thread: strict compare
-        // keeps the first occurrence.
-        const bool take = (c > best) || (c != c && best == best);
-        best = take ? c : best;
-        if (WITH_IDX) bidx = take ? i : bidx;
-    };
-
     const int tid = threadIdx.x;
-    if (blockIdx.x == 0 && tid < head) feed(E::up(x[tid]), tid);
-
-    // Workgroups walk the vector in contiguous blocks of kVmaxUnroll * kVmaxThreads 16-byte
-    // pieces (block-cyclic over the grid): measured 6.3 TB/s against 4.7 TB/s for the same
-    // loads spread a whole grid apart.  Indices still increase within a thread.
     const V *xv = reinterpret_cast<const V *>(x + head);
     constexpr int64_t kBlock = (int64_t)kVmaxUnroll * kVmaxThreads;
     const int64_t full_blocks = nvec / kBlock;
+
+    // ---- fast sweep: best piece maximum and the number of the piece (in this thread's
+    // visiting order) that first reached it
+    C bv = neg_inf<C>();
+    unsigned bk = 0xffffffffu;  // no piece yet
+    V bpiece;                   // the piece itself: its elements decide the position at the end
+#pragma unroll
+    for (int e = 0; e < VN; ++e) bpiece.e[e] = T();
+    bool saw_nan = false;
+    auto piece_max = [&](const V &b, C &m, bool &un) {
+        C c[VN];
+#pragma unroll
+        for (int e = 0; e < VN; ++e) c[e] = E::up(b.e[e]);
+        m = c[0];
+#pragma unroll
+        for (int e = 1; e < VN; ++e) m = max_ignoring_nan(m, c[e]);
+#pragma unroll
+        for (int e = 0; e + 1 < VN; e += 2) un |= __builtin_isunordered(c[e], c[e + 1]);
+    };
+    // Workgroups walk the vector in contiguous blocks of kVmaxUnroll * kVmaxThreads 16-byte
+    // pieces (block-cyclic over the grid): measured 6.3 TB/s against 4.7 TB/s for the same
+    // loads spread a whole grid apart.  Piece numbers increase with the index within a thread.
+    unsigned k = 0;
     for (int64_t blk = blockIdx.x; blk < full_blocks; blk += gridDim.x) {
         const int64_t v = blk * kBlock + tid;
         V buf[kVmaxUnroll];
@@ -151,107 +237,179 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_stage1(
         for (int u = 0; u < kVmaxUnroll; ++u) buf[u] = xv[v + u * kVmaxThreads];
 #pragma unroll
         for (int u = 0; u < kVmaxUnroll; ++u) {
-            const int64_t base = head + (v + u * kVmaxThreads) * VN;
+            C m;
+            piece_max(buf[u], m, saw_nan);
+            const bool take = m > bv;
+            bv = take ? m : bv;
+            if (WITH_IDX) {
+                bk = take ? k + u : bk;
 #pragma unroll
-            for (int e = 0; e < VN; ++e) feed(E::up(buf[u].e[e]), base + e);
+                for (int e = 0; e < VN; ++e) bpiece.e[e] = take ? buf[u].e[e] : bpiece.e[e];
+            }
         }
+        k += kVmaxUnroll;
     }
+    const unsigned in_full = k;  // pieces of whole blocks come first in the visiting order
     // the last, partial block goes to the workgroup whose turn it would be
-    if ((int64_t)blockIdx.x == full_blocks % gridDim.x) {
+    const bool has_tail_block = (int64_t)blockIdx.x == full_blocks % gridDim.x;
+    if (has_tail_block) {
         for (int64_t v = full_blocks * kBlock + tid; v < nvec; v += kVmaxThreads) {
-            V buf = xv[v];
-            const int64_t base = head + v * VN;
+            C m;
+            const V b = xv[v];
+            piece_max(b, m, saw_nan);
+            const bool take = m > bv;
+            bv = take ? m : bv;
+            if (WITH_IDX) {
+                bk = take ? k : bk;
 #pragma unroll
-            for (int e = 0; e < VN; ++e) feed(E::up(buf.e[e]), base + e);
+                for (int e = 0; e < VN; ++e) bpiece.e[e] = take ? b.e[e] : bpiece.e[e];
+            }
+            ++k;
         }
     }
+    // piece number -> absolute piece index (the inverse of the two loops above)
+    auto piece_index = [&](unsigned kk) -> int64_t {
+        if (kk < in_full)
+            return ((int64_t)blockIdx.x + (int64_t)(kk / kVmaxUnroll) * gridDim.x) * kBlock + tid +
+                   (int64_t)(kk % kVmaxUnroll) * kVmaxThreads;
+        return full_blocks * kBlock + tid + (int64_t)(kk - in_full) * kVmaxThreads;
+    };
+
+    C best = neg_inf<C>();
+    int64_t bidx = kNoIdx;
+    auto feed = [&](C c, int64_t i) {  // exact rule, any order
+        if (prefer(c, i, best, bidx)) {
+            best = c;
+            bidx = i;
+        }
+    };
+    if (__builtin_amdgcn_ballot_w64(saw_nan) != 0) {
+        // ---- a NaN somewhere in this wavefront's share: element by element, exact rule
+        for (int64_t blk = blockIdx.x; blk < full_blocks; blk += gridDim.x)
+            for (int u = 0; u < kVmaxUnroll; ++u) {
+                const int64_t v = blk * kBlock + tid + u * kVmaxThreads;
+                const V b = xv[v];
+#pragma unroll
+                for (int e = 0; e < VN; ++e) feed(E::up(b.e[e]), head + v * VN + e);
+            }
+        if (has_tail_block)
+            for (int64_t v = full_blocks * kBlock + tid; v < nvec; v += kVmaxThreads) {
+                const V b = xv[v];
+#pragma unroll
+                for (int e = 0; e < VN; ++e) feed(E::up(b.e[e]), head + v * VN + e);
+            }
+    } else if (bk != 0xffffffffu || !WITH_IDX) {
+        // ---- the winning piece: its first element equal to the maximum (the element's own
+        // bits are reported: -0.0 and +0.0 compare equal)
+        best = bv;
+        if (WITH_IDX) {
+            const int64_t v = piece_index(bk);
+#pragma unroll
+            for (int e = VN - 1; e >= 0; --e) {
+                const C c = E::up(bpiece.e[e]);
+                if (c == bv) {
+                    best = c;
+                    bidx = head + v * VN + e;
+                }
+            }
+        }
+    }
+    // elements before the first and after the last whole 16-byte piece
+    if (blockIdx.x == 0 && tid < head) feed(E::up(x[tid]), tid);
     const int64_t tail0 = head + nvec * VN;
     if (blockIdx.x == 0 && tail0 + tid < n) feed(E::up(x[tail0 + tid]), tail0 + tid);
 
     __shared__ C sval[kVmaxThreads / kWave];
     __shared__ int64_t sidx[kVmaxThreads / kWave];
-    if (WITH_IDX) {
-        wave_argmax(best, bidx);
-    } else {
-        best = wave_max(best);
-    }
-    const int wave = tid / kWave;
-    if (lane_id() == 0) {
-        sval[wave] = best;
-        sidx[wave] = bidx;
-    }
-    __syncthreads();
-    if (tid == 0) {
-        for (int w = 1; w < kVmaxThreads / kWave; ++w) {
-            if (WITH_IDX) {
-                if (prefer(sval[w], sidx[w], best, bidx)) {
-                    best = sval[w];
-                    bidx = sidx[w];
-                }
-            } else {
-                best = vmax_nan(best, sval[w]);
-            }
-        }
-        if (FINAL) {
-            *out_val = E::down(best);
-            // every element is -inf: the first one is the answer, as in torch.max
-            if (WITH_IDX) *out_idx = (bidx == kNoIdx) ? 0 : bidx;
-        } else {
-            pval[blockIdx.x] = best;
-            if (WITH_IDX) pidx[blockIdx.x] = bidx;
-        }
-    }
-}
-
-template <int DT, bool WITH_IDX>
-__global__ __launch_bounds__(kVmaxThreads) void vmax_stage2(
-    const typename Elem<DT>::C *__restrict__ pval, const int64_t *__restrict__ pidx, int nparts,
-    typename Elem<DT>::T *__restrict__ out_val, int64_t *__restrict__ out_idx) {
-    using E = Elem<DT>;
-    using C = typename E::C;
-    C best = neg_inf<C>();
-    int64_t bidx = kNoIdx;
-    const int tid = threadIdx.x;
-    for (int p = tid; p < nparts; p += kVmaxThreads) {
-        C v = pval[p];
+    __shared__ bool last_block;
+    auto wave_reduce = [&]() {
         if (WITH_IDX) {
-            int64_t i = pidx[p];
-            if (prefer(v, i, best, bidx)) {
-                best = v;
-                bidx = i;
-            }
+            wave_argmax(best, bidx);
         } else {
-            best = vmax_nan(best, v);
+            best = wave_max(best);
         }
+    };
+    auto block_reduce = [&]() {  // result in thread 0
+        wave_reduce();
+        if (lane_id() == 0) {
+            sval[tid / kWave] = best;
+            sidx[tid / kWave] = bidx;
+        }
+        __syncthreads();
+        if (tid == 0) {
+            for (int w = 1; w < kVmaxThreads / kWave; ++w) {
+                if (WITH_IDX) {
+                    if (prefer(sval[w], sidx[w], best, bidx)) {
+                        best = sval[w];
+                        bidx = sidx[w];
+                    }
+                } else {
+                    best = vmax_nan(best, sval[w]);
+                }
+            }
+        }
+    };
+    auto write_result = [&]() {
+        *out_val = E::down(best);
+        // every element is -inf: the first one is the answer, as in torch.max
+        if (WITH_IDX) *out_idx = (bidx == kNoIdx) ? 0 : bidx;
+    };
+    block_reduce();
+    if (FINAL) {
+        if (tid == 0) write_result();
+        return;
     }
-    __shared__ C sval[kVmaxThreads / kWave];
-    __shared__ int64_t sidx[kVmaxThreads / kWave];
-    if (WITH_IDX) {
-        wave_argmax(best, bidx);
-    } else {
-        best = wave_max(best);
-    }
-    const int wave = tid / kWave;
-    if (lane_id() == 0) {
-        sval[wave] = best;
-        sidx[wave] = bidx;
+    // ---- "the last to arrive combines", counted at two levels: the last workgroup of a group of
+    // kVmaxGroup draws from the counter of the groups, and the last of those combines all the
+    // partials.  (One counter for all workgroups would serialise a burst of device-scope atomics
+    // at the end of the sweep; combining group by group would add a round trip of partials.)
+    const int nblocks = (int)gridDim.x;
+    const int group = blockIdx.x / kVmaxGroup;
+    const int ngroups = (nblocks + kVmaxGroup - 1) / kVmaxGroup;
+    const int gfirst = group * kVmaxGroup;
+    const int gsize = nblocks - gfirst < kVmaxGroup ? nblocks - gfirst : kVmaxGroup;
+    unsigned *tick1 = ticket + group * kTicketStride;
+    unsigned *tick2 = ticket + (kMaxTickets - 1) * kTicketStride;
+    if (tid == 0) {
+        __hip_atomic_store(&pval[blockIdx.x], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (WITH_IDX) __hip_atomic_store(&pidx[blockIdx.x], bidx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        bool last = take_ticket(tick1) == (unsigned)gsize - 1;
+        if (last) {
+            last = take_ticket(tick2) == (unsigned)ngroups - 1;
+            __hip_atomic_store(tick1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next call
+        }
+        last_block = last;
     }
     __syncthreads();
-    if (tid == 0) {
-        for (int w = 1; w < kVmaxThreads / kWave; ++w) {
-            if (WITH_IDX) {
-                if (prefer(sval[w], sidx[w], best, bidx)) {
-                    best = sval[w];
-                    bidx = sidx[w];
-                }
-            } else {
-                best = vmax_nan(best, sval[w]);
-            }
+    if (!last_block) return;
+    best = neg_inf<C>();
+    bidx = kNoIdx;
+    // every partial is asked for before the first is looked at: one round trip, not one per partial
+    constexpr int kPer = (kVmaxMaxBlocks + kVmaxThreads - 1) / kVmaxThreads;
+    C pc[kPer];
+    int64_t pi[kPer];
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+        const int i = tid + u * kVmaxThreads;
+        pc[u] = neg_inf<C>();
+        pi[u] = kNoIdx;
+        if (i < nblocks) {
+            pc[u] = __hip_atomic_load(&pval[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (WITH_IDX) pi[u] = __hip_atomic_load(&pidx[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        *out_val = E::down(best);
-        // Every element is -inf (nothing compared greater than the initial
-        // value): the first element is the answer, as in torch.max.
-        if (WITH_IDX) *out_idx = (bidx == kNoIdx) ? 0 : bidx;
+    }
+#pragma unroll
+    for (int u = 0; u < kPer; ++u) {
+        if (WITH_IDX) {
+            feed(pc[u], pi[u]);
+        } else {
+            best = vmax_nan(best, pc[u]);
+        }
+    }
+    block_reduce();
+    if (tid == 0) {
+        write_result();
+        __hip_atomic_store(tick2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
 }
 
@@ -272,14 +430,14 @@ static size_t elem_size(int dtype) {
     }
 }
 
-// workspace layout: [kVmaxMaxBlocks x 8-byte value slots][kVmaxMaxBlocks x int64]; vectors
-// short enough for one workgroup need none
+// workspace layout: [tickets][kVmaxMaxBlocks x 8-byte value slots][kVmaxMaxBlocks x int64];
+// vectors short enough for one workgroup need none
 static bool vmax_single_block(int64_t n, int dtype) {
     const int64_t vn = 16 / (int64_t)elem_size(dtype);
     return n <= (int64_t)kVmaxThreads * kVmaxUnroll * vn * 2;
 }
 static size_t vmax_ws_bytes(int64_t n, int dtype) {
-    return vmax_single_block(n, dtype) ? 0 : (size_t)kVmaxMaxBlocks * 16;
+    return vmax_single_block(n, dtype) ? 0 : kTicketBytes + (size_t)kVmaxMaxBlocks * 16;
 }
 
 template <int DT>
@@ -298,27 +456,23 @@ static int vmax_launch(const void *x, int64_t n, void *out_val, int64_t *out_idx
     T *ov = static_cast<T *>(out_val);
     if (vmax_single_block(n, DT)) {
         if (out_idx)
-            hipLaunchKernelGGL((vmax_stage1<DT, true, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                               nvec, (C *)nullptr, (int64_t *)nullptr, ov, out_idx);
+            hipLaunchKernelGGL((vmax_kernel<DT, true, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
+                               nvec, (C *)nullptr, (int64_t *)nullptr, (unsigned *)nullptr, ov, out_idx);
         else
-            hipLaunchKernelGGL((vmax_stage1<DT, false, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                               nvec, (C *)nullptr, (int64_t *)nullptr, ov, out_idx);
+            hipLaunchKernelGGL((vmax_kernel<DT, false, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
+                               nvec, (C *)nullptr, (int64_t *)nullptr, (unsigned *)nullptr, ov, out_idx);
         return (int)hipGetLastError();
     }
     const int blocks = vmax_blocks(nvec);
-    C *pval = static_cast<C *>(ws);
-    int64_t *pidx = reinterpret_cast<int64_t *>(static_cast<char *>(ws) + (size_t)kVmaxMaxBlocks * 8);
-    if (out_idx) {
-        hipLaunchKernelGGL((vmax_stage1<DT, true, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n,
-                           head, nvec, pval, pidx, ov, out_idx);
-        hipLaunchKernelGGL((vmax_stage2<DT, true>), dim3(1), dim3(kVmaxThreads), 0, stream, pval, pidx,
-                           blocks, ov, out_idx);
-    } else {
-        hipLaunchKernelGGL((vmax_stage1<DT, false, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n,
-                           head, nvec, pval, pidx, ov, out_idx);
-        hipLaunchKernelGGL((vmax_stage2<DT, false>), dim3(1), dim3(kVmaxThreads), 0, stream, pval, pidx,
-                           blocks, ov, out_idx);
-    }
+    unsigned *ticket = static_cast<unsigned *>(ws);
+    C *pval = reinterpret_cast<C *>(static_cast<char *>(ws) + kTicketBytes);
+    int64_t *pidx = reinterpret_cast<int64_t *>(static_cast<char *>(ws) + kTicketBytes + (size_t)kVmaxMaxBlocks * 8);
+    if (out_idx)
+        hipLaunchKernelGGL((vmax_kernel<DT, true, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n, head,
+                           nvec, pval, pidx, ticket, ov, out_idx);
+    else
+        hipLaunchKernelGGL((vmax_kernel<DT, false, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n, head,
+                           nvec, pval, pidx, ticket, ov, out_idx);
     return (int)hipGetLastError();
 }
 
@@ -421,6 +575,10 @@ __global__ __launch_bounds__(kMatThreads) void rowmax_wide_kernel(const typename
 // Column maxima (reduction along the strided axis).  Each thread owns CN
 // adjacent columns; the 4 wavefronts of a workgroup interleave over the rows
 // of the workgroup's row chunk and combine through LDS.
+// (Combining the row splits in the same launch -- the workgroup of a column block that finishes
+// last reduces the partials, arrival counters in the workspace -- was built and measured: 18.6 us
+// at best on a 4096 x 4096 matrix against 18.2 us for the two launches below; the device-scope
+// round trips of the hand-over cost what the second launch costs.  Not kept.)
 template <int DT, bool VEC>
 __global__ __launch_bounds__(kMatThreads) void colmax_kernel(
     const typename Elem<DT>::T *__restrict__ x, int64_t ld, int64_t m, int64_t n, int64_t rchunk,
@@ -560,20 +718,21 @@ static void colmax_launch(const typename Elem<DT>::T *x, int64_t ld, int64_t m, 
                            x, ld, m, n, p.chunk, colblocks, y, ldy);
 }
 
+// workspace: [tickets][partials]
 template <int DT>
 static size_t matmax_ws(int64_t m, int64_t n, int axis) {
     using T = typename Elem<DT>::T;
     constexpr int VN = 16 / (int)sizeof(T);
     if (axis == 1) {
         MatPlan p = rowmax_plan(m, n, VN);
-        return p.splits > 1 ? (size_t)(m * p.splits) * sizeof(T) : 0;
+        return p.splits > 1 ? kTicketBytes + (size_t)(m * p.splits) * sizeof(T) : 0;
     }
     // worst case over the vector / scalar column paths, plus the intermediate level
     MatPlan pv = colmax_plan(m, n, VN), ps = colmax_plan(m, n, 1);
     int64_t s = pv.splits > ps.splits ? pv.splits : ps.splits;
     if (s <= 1) return 0;
     const int64_t s2 = combine_splits(s);
-    return (size_t)((s + (s2 > 1 ? s2 : 0)) * n) * sizeof(T);
+    return kTicketBytes + (size_t)((s + (s2 > 1 ? s2 : 0)) * n) * sizeof(T);
 }
 
 template <int DT>
@@ -583,7 +742,7 @@ static int matmax_launch(const void *xv, void *yv, int64_t m, int64_t n, int axi
     constexpr int VN = 16 / (int)sizeof(T);
     const T *x = static_cast<const T *>(xv);
     T *y = static_cast<T *>(yv);
-    T *part = static_cast<T *>(ws);
+    T *part = reinterpret_cast<T *>(static_cast<char *>(ws) + kTicketBytes);
     if (matmax_ws<DT>(m, n, axis) > ws_bytes) return TRT_E_WORKSPACE;
     if (matmax_ws<DT>(m, n, axis) > 0 && ws == nullptr) return TRT_E_WORKSPACE;
     if (axis == 1 && rowmax_wide<DT>(x, m, n)) {

@@ -15,6 +15,20 @@ import torch
 from triturus_amd import _lib
 
 _ws_bytes: dict = {}  # (op, shape..., dtype code) -> workspace bytes, as reported by the library
+# (device index, raw stream) -> workspace of the reductions launched on that stream.  The library
+# wants the arrival counters at the head of a max workspace zero before the first use and leaves
+# them zero (one launch per reduction: the workgroup that finishes last combines the partial
+# results), so the workspace is allocated once per stream, zero-filled, and kept: calls on one
+# stream run one after the other, calls on different streams never share one.
+_workspaces: dict = {}
+
+
+def _workspace(dev: torch.device, nbytes: int):
+    key = (dev.index, _lib.raw_stream(dev))
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = _workspaces[key] = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=dev)
+    return ws
 
 
 def _dtype_code(x: torch.Tensor) -> int:
@@ -38,7 +52,7 @@ def _vmax_impl(x: torch.Tensor, with_index: bool):
     ws_bytes = _ws_bytes.get(key)
     if ws_bytes is None:
         ws_bytes = _ws_bytes[key] = lib.trt_vmax_workspace_bytes(n, code)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    ws = _workspace(dev, ws_bytes) if ws_bytes else None
     with _lib.on_device(dev):
         status = lib.trt_vmax(
             x.data_ptr(), n, code, val.data_ptr(), idx.data_ptr() if with_index else None,
@@ -80,7 +94,7 @@ def matmax(x: torch.Tensor, axis: int = 0, *, block_size: int = 32) -> torch.Ten
     ws_bytes = _ws_bytes.get(key)
     if ws_bytes is None:
         ws_bytes = _ws_bytes[key] = lib.trt_matmax_workspace_bytes(m, n, axis, code)
-    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev) if ws_bytes else None
+    ws = _workspace(dev, ws_bytes) if ws_bytes else None
     with _lib.on_device(dev):
         status = lib.trt_matmax(
             x.data_ptr(), y.data_ptr(), m, n, axis, code,
