@@ -185,6 +185,14 @@ __device__ __forceinline__ unsigned take_ticket(unsigned *ticket) {
     __builtin_amdgcn_s_waitcnt(0);
     return __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// The same for a whole wavefront that has stored: lane 0 draws, the others wait with it.
+__device__ __forceinline__ unsigned take_ticket_wave(unsigned *ticket) {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_s_waitcnt(0);
+    unsigned t = 0;
+    if (lane_id() == 0) t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return t;
+}
 
 // Max and first-occurrence argmax in one launch.  Every 16-byte piece costs a couple of vector
 // instructions: the maximum of its elements (NaN ignored), one unordered test per pair of elements
@@ -572,13 +580,20 @@ __global__ __launch_bounds__(kMatThreads) void rowmax_wide_kernel(const typename
     }
 }
 
+// Workgroups go to the 8 dies (each with an L2 of its own) round-robin, and rows a power of two
+// apart map to the same few channels of a die's L2.  A column reduction therefore hands each
+// die whole row splits -- all column blocks of them -- and not one column block of every split:
+// measured 14.6 us against 18.2 us on a 4096 x 4096 fp32 matrix.
+constexpr int kDies = 8;
+__device__ __forceinline__ int64_t die_major(int64_t block, int64_t total) {
+    return (total % kDies == 0) ? (block % kDies) * (total / kDies) + block / kDies : block;
+}
+
 // Column maxima (reduction along the strided axis).  Each thread owns CN
 // adjacent columns; the 4 wavefronts of a workgroup interleave over the rows
 // of the workgroup's row chunk and combine through LDS.
-// (Combining the row splits in the same launch -- the workgroup of a column block that finishes
-// last reduces the partials, arrival counters in the workspace -- was built and measured: 18.6 us
-// at best on a 4096 x 4096 matrix against 18.2 us for the two launches below; the device-scope
-// round trips of the hand-over cost what the second launch costs.  Not kept.)
+// Row splits leave partial rows that further launches of this kernel combine; matrices that
+// colmax_fused_kernel covers take that one-launch path instead.
 template <int DT, bool VEC>
 __global__ __launch_bounds__(kMatThreads) void colmax_kernel(
     const typename Elem<DT>::T *__restrict__ x, int64_t ld, int64_t m, int64_t n, int64_t rchunk,
@@ -590,8 +605,9 @@ __global__ __launch_bounds__(kMatThreads) void colmax_kernel(
     constexpr int CN = VEC ? V::N : 1;
     const int wave = threadIdx.x / kWave;
     const int lane = lane_id();
-    const int64_t cb = blockIdx.x % colblocks;
-    const int64_t split = blockIdx.x / colblocks;
+    const int64_t logical = die_major(blockIdx.x, gridDim.x);
+    const int64_t cb = logical % colblocks;
+    const int64_t split = logical / colblocks;
     const int64_t col = (cb * kWave + lane) * CN;
     const int64_t r0 = split * rchunk;
     const int64_t r1 = (r0 + rchunk < m) ? r0 + rchunk : m;
@@ -639,6 +655,111 @@ __global__ __launch_bounds__(kMatThreads) void colmax_kernel(
     }
 }
 
+// Column maxima in one launch, for 16-byte-aligned matrices whose row splits number at most
+// kColFusedSplits: as colmax_kernel, then the workgroup of a column block that finishes last
+// combines the block's partial rows (device-scope 8-byte accesses, see take_ticket) and writes y.
+constexpr int kColFusedSplits = 32;
+constexpr int kColFusedUnroll = 8;  // 16-byte loads in flight per lane
+template <int DT>
+__global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
+    const typename Elem<DT>::T *__restrict__ x, int64_t ld, int64_t m, int64_t n, int64_t rchunk,
+    int colblocks, int splits, unsigned long long *part, unsigned *ticket, typename Elem<DT>::T *__restrict__ y) {
+    using E = Elem<DT>;
+    using T = typename E::T;
+    using C = typename E::C;
+    using V = Vec16<T>;
+    constexpr int CN = V::N;
+    const int wave = threadIdx.x / kWave;
+    const int lane = lane_id();
+    const int logical = (int)die_major(blockIdx.x, gridDim.x);
+    const int cb = logical % colblocks;
+    const int split = logical / colblocks;
+    const int64_t col = ((int64_t)cb * kWave + lane) * CN;
+    const int64_t r0 = split * rchunk;
+    const int64_t r1 = (r0 + rchunk < m) ? r0 + rchunk : m;
+    C best[CN];
+#pragma unroll
+    for (int e = 0; e < CN; ++e) best[e] = neg_inf<C>();
+    if (col < n) {
+        const T *xc = x + col;
+        int64_t r = r0 + wave;
+        for (; r + (kColFusedUnroll - 1) * kMatWaves < r1; r += kColFusedUnroll * kMatWaves) {
+            V b[kColFusedUnroll];
+#pragma unroll
+            for (int u = 0; u < kColFusedUnroll; ++u) b[u] = *reinterpret_cast<const V *>(xc + (r + u * kMatWaves) * ld);
+#pragma unroll
+            for (int u = 0; u < kColFusedUnroll; ++u)
+#pragma unroll
+                for (int e = 0; e < CN; ++e) best[e] = vmax_nan(best[e], E::up(b[u].e[e]));
+        }
+        for (; r < r1; r += kMatWaves) {
+            V b0 = *reinterpret_cast<const V *>(xc + r * ld);
+#pragma unroll
+            for (int e = 0; e < CN; ++e) best[e] = vmax_nan(best[e], E::up(b0.e[e]));
+        }
+    }
+    __shared__ C sm[kMatWaves][kWave * CN];
+    __shared__ bool last_block;
+    auto across_waves = [&]() {  // wave 0 ends up with the maxima of the workgroup
+#pragma unroll
+        for (int e = 0; e < CN; ++e) sm[wave][lane * CN + e] = best[e];
+        __syncthreads();
+        if (wave == 0) {
+#pragma unroll
+            for (int e = 0; e < CN; ++e)
+                for (int w = 1; w < kMatWaves; ++w) best[e] = vmax_nan(best[e], sm[w][lane * CN + e]);
+        }
+    };
+    across_waves();
+    // a partial row: 16 bytes per lane of wave 0, as two 8-byte words
+    const int64_t words_per_row = (int64_t)colblocks * kWave * 2;
+    unsigned long long *prow = part + (int64_t)cb * kWave * 2 + lane * 2;
+    if (wave == 0) {
+        union { V v; unsigned long long w[2]; } u;
+#pragma unroll
+        for (int e = 0; e < CN; ++e) u.v.e[e] = E::down(best[e]);
+        __hip_atomic_store(&prow[split * words_per_row], u.w[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        __hip_atomic_store(&prow[split * words_per_row + 1], u.w[1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned t = take_ticket_wave(ticket + cb * kTicketStride);
+        if (lane == 0) last_block = t == (unsigned)splits - 1;
+    }
+    __syncthreads();
+    if (!last_block) return;
+    constexpr int kPer = kColFusedSplits / kMatWaves;
+    unsigned long long w0[kPer], w1[kPer];
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+        const int sp = wave + q * kMatWaves;
+        if (sp < splits) {
+            w0[q] = __hip_atomic_load(&prow[sp * words_per_row], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            w1[q] = __hip_atomic_load(&prow[sp * words_per_row + 1], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+    }
+#pragma unroll
+    for (int e = 0; e < CN; ++e) best[e] = neg_inf<C>();
+#pragma unroll
+    for (int q = 0; q < kPer; ++q) {
+        const int sp = wave + q * kMatWaves;
+        if (sp < splits) {
+            union { V v; unsigned long long w[2]; } u;
+            u.w[0] = w0[q];
+            u.w[1] = w1[q];
+#pragma unroll
+            for (int e = 0; e < CN; ++e) best[e] = vmax_nan(best[e], E::up(u.v.e[e]));
+        }
+    }
+    __syncthreads();  // sm is reused
+    across_waves();
+    if (wave == 0) {
+        if (col < n) {
+#pragma unroll
+            for (int e = 0; e < CN; ++e)
+                if (col + e < n) y[col + e] = E::down(best[e]);
+        }
+        if (lane == 0) __hip_atomic_store(ticket + cb * kTicketStride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+}
+
 struct MatPlan {
     int64_t splits;  // partial results per output element (1: written straight to y)
     int64_t chunk;   // reduced-axis elements per partial
@@ -679,6 +800,20 @@ static MatPlan colmax_plan(int64_t m, int64_t n, int cn) {
     int64_t rchunk = ceil_div(m, splits);
     splits = ceil_div(m, rchunk);
     return {splits, rchunk};
+}
+
+// One-launch column maxima (colmax_fused_kernel): two workgroups per compute unit when the
+// matrix allows, every split at least 32 rows, at most kColFusedSplits splits and one arrival
+// counter per column block.  splits < 2: not applicable.
+static MatPlan colmax_fused_plan(int64_t m, int64_t n, int vn) {
+    const int64_t colblocks = ceil_div(n, (int64_t)kWave * vn);
+    if (colblocks > kMaxTickets) return {1, m};
+    int64_t splits = ceil_div((int64_t)512, colblocks);
+    if (splits > kColFusedSplits) splits = kColFusedSplits;
+    if (splits > m / 32) splits = m / 32;
+    if (splits < 2) return {1, m};
+    const int64_t rchunk = ceil_div(m, splits);
+    return {ceil_div(m, rchunk), rchunk};
 }
 
 // Partial column maxima are combined by the same kernel; more than 128 rows of them (tall,
@@ -728,11 +863,16 @@ static size_t matmax_ws(int64_t m, int64_t n, int axis) {
         return p.splits > 1 ? kTicketBytes + (size_t)(m * p.splits) * sizeof(T) : 0;
     }
     // worst case over the vector / scalar column paths, plus the intermediate level
-    MatPlan pv = colmax_plan(m, n, VN), ps = colmax_plan(m, n, 1);
+    MatPlan pv = colmax_plan(m, n, VN), ps = colmax_plan(m, n, 1), pf = colmax_fused_plan(m, n, VN);
+    const size_t fused = pf.splits > 1 ? (size_t)(pf.splits * ceil_div(n, (int64_t)kWave * VN)) * kWave * 16 : 0;
     int64_t s = pv.splits > ps.splits ? pv.splits : ps.splits;
-    if (s <= 1) return 0;
-    const int64_t s2 = combine_splits(s);
-    return kTicketBytes + (size_t)((s + (s2 > 1 ? s2 : 0)) * n) * sizeof(T);
+    size_t tree = 0;
+    if (s > 1) {
+        const int64_t s2 = combine_splits(s);
+        tree = (size_t)((s + (s2 > 1 ? s2 : 0)) * n) * sizeof(T);
+    }
+    const size_t most = fused > tree ? fused : tree;
+    return most ? kTicketBytes + most : 0;
 }
 
 template <int DT>
@@ -759,7 +899,13 @@ static int matmax_launch(const void *xv, void *yv, int64_t m, int64_t n, int axi
     } else {
         const bool vec = vec_ok<DT>(x, n);
         MatPlan p = colmax_plan(m, n, vec ? VN : 1);
-        if (p.splits == 1) {
+        const MatPlan pf = colmax_fused_plan(m, n, VN);
+        if (vec && pf.splits > 1) {
+            const int colblocks = (int)ceil_div(n, (int64_t)kWave * VN);
+            hipLaunchKernelGGL((colmax_fused_kernel<DT>), dim3((unsigned)(colblocks * pf.splits)), dim3(kMatThreads), 0,
+                               stream, x, n, m, n, pf.chunk, colblocks, (int)pf.splits,
+                               reinterpret_cast<unsigned long long *>(part), static_cast<unsigned *>(ws), y);
+        } else if (p.splits == 1) {
             colmax_launch<DT>(x, n, m, n, vec, p, y, n, stream);
         } else {
             colmax_launch<DT>(x, n, m, n, vec, p, part, n, stream);
