@@ -87,8 +87,10 @@ int trt_lm2exp_variant_count(void);
  * c[r,s,k] = log sum_{i,j} w[r,s,i,j] * exp(a[r,i,k]) * exp(b[r,j,k])   (fp32)
  * w: R x S x (I*J) linear-space (the reference flattens the two trailing axes
  * with w.view(batch, m, -1), triturus/lt2exp.py:549, so sw has 3 entries),
- * a: R x I x K, b: R x J x K log-space, c: R x S x K.  Trailing strides must
- * be 1.  Replaces the `_ker_lt2exp_unsplit[grid](...)` launch,
+ * a: R x I x K, b: R x J x K log-space, c: R x S x K.  Trailing strides of a, b
+ * and c must be 1; w takes any non-negative strides (a flat axis with another
+ * stride than 1 -- a sliced view -- is read in place, element by element; the
+ * reference's kernels take the stride too, triturus/lt2exp.py:577-579).  Replaces the `_ker_lt2exp_unsplit[grid](...)` launch,
  * triturus/lt2exp.py:601-629, and the `_ker_lt2exp_split[grid](...)` launch,
  * triturus/lt2exp.py:564-597; arithmetic contract baselines/lt2exp.py:15-25.
  * mode: TRT_MODE_*.  AUTO decides like the reference does -- by the size of the
@@ -136,8 +138,8 @@ int trt_lt2exp_f32_static(const float *w, const float *a, const float *b, float 
                           const int64_t sc[3], int mode, int variant, void *stream);
 
 /*
- * The same contraction as trt_lt2exp_f32 (fp32 tensors in and out, same layouts, strides
- * and status codes) on the bf16 matrix pipe: every fp32 operand is cut into `pieces` bf16
+ * The same contraction as trt_lt2exp_f32 (fp32 tensors in and out, same layouts and status
+ * codes; every trailing stride, that of w included, must be 1) on the bf16 matrix pipe: every fp32 operand is cut into `pieces` bf16
  * pieces and a product is the sum of the piece products that matter, accumulated in fp32.
  *   pieces = 2 (TRT_PIECES_BF16X3): 3 MFMAs per product, relative error ~2^-16 per product
  *   pieces = 3 (TRT_PIECES_BF16X6): 6 MFMAs per product, relative error ~2^-23 per product

@@ -84,6 +84,8 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_lt2exp_f32(one, null, one, one, *args, 0, 0, null, 0, null) == -1
     assert lib.trt_lt2exp_f32(one, one, one, one, *args, 7, 0, null, 0, null) == -1
     assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, s3(1, 1, 2), ok, 0, 0, null, 0, null) == -2
+    assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, -1), ok, ok, ok, 0, 0, null, 0, null) == -2
+    assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, ok, s3(1, 1, 2), 0, 0, null, 0, null) == -2
     big4 = (2, 8, 16, 16, 64, s3(2048, 256, 1), s3(1024, 64, 1), s3(1024, 64, 1), s3(512, 64, 1))
     assert lib.trt_lt2exp_f32(one, one, one, one, *big4, _lib.MODE_SPLIT, 0, null, 0, null) == -3  # split needs a workspace
     assert lib.trt_lt2exp_f32(one, one, one, one, *args, 0, lib.trt_lt2exp_variant_count() + 1, null, 0, null) == -1

@@ -206,6 +206,49 @@ def test_strided_inputs(dev):
     _check(out, w, at.transpose(1, 2), b)
 
 
+@pytest.mark.parametrize("shape", [(2, 70, 12, 20, 130), (3, 33, 7, 5, 64), (1, 200, 4, 8, 40), (2, 64, 40, 1, 256),
+                                   (2, 48, 3, 200, 96)])
+@pytest.mark.parametrize("mode", ["unsplit", "split"])
+def test_views_of_w_are_read_in_place(dev, shape, mode):
+    """The reference hands the strides of the flattened w to its kernel (triturus/lt2exp.py:577-579,
+    :612-614): a w whose (i, j) axes are jointly viewable but not dense -- every other element of
+    a wider tensor -- or expanded over the batch must give the oracle's result without a copy
+    (the call may allocate its output and, in split mode, its workspace, and nothing else)."""
+    R, S, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    w = torch.rand(R, S, I, J, generator=g)
+    w[torch.rand(w.shape, generator=g) < 0.2] = 0.0
+    a = 3 * torch.randn(R, I, K, generator=g)
+    b = -2 + 3 * torch.randn(R, J, K, generator=g)
+    ref = oracle64.lt2exp64(w, a, b)
+    ag, bg = a.to(dev), b.to(dev)
+    wide = torch.zeros(R, S, I, 2 * J)
+    wide[..., 1::2] = w
+    views = {
+        "every other element": wide.to(dev)[..., 1::2],
+        "every third element": torch.zeros(R, S, I, 3 * J).index_copy_(3, torch.arange(J) * 3, w).to(dev)[..., ::3],
+    }
+    for name, wg in views.items():
+        assert wg.stride(3) != 1 and torch.equal(wg.cpu(), w), name
+        wg.view(R, S, I * J)  # viewable, as the reference requires
+        lt2exp(wg, ag, bg, mode=mode)  # first call: library load, workspace query cache
+        torch.cuda.synchronize()
+        ws = _lib.load().trt_lt2exp_workspace_bytes(R, S, I, J, K, {"unsplit": _lib.MODE_UNSPLIT, "split": _lib.MODE_SPLIT}[mode])
+        before = torch.cuda.memory_allocated()
+        out = lt2exp(wg, ag, bg, mode=mode)
+        grown = torch.cuda.memory_allocated() - before
+        r = oracle64.compare(out, ref)
+        assert r["ok"], (name, r)
+        assert grown <= out.numel() * 4 + ws + 2048, (name, grown, out.numel() * 4, ws)
+    w1 = w[:1]
+    wg = w1.to(dev).expand(R, S, I, J)
+    out = lt2exp(wg, ag, bg, mode=mode)
+    assert oracle64.compare(out, oracle64.lt2exp64(w1.expand(R, S, I, J), a, b))["ok"]
+    # on the bf16 matrix pipe the wrapper materialises such a view: same result as from a dense w
+    dense = lt2exp(w.to(dev), ag, bg, mode=mode, _precision="bf16x6")
+    assert torch.equal(lt2exp(views["every other element"], ag, bg, mode=mode, _precision="bf16x6"), dense)
+
+
 def test_reduces_to_lm2exp_and_factorises(dev):
     g = torch.Generator().manual_seed(10)
     R, S, I, J, K = 2, 64, 16, 24, 192

@@ -32,7 +32,7 @@ struct Lt2Args {
     float *c;         // output (unsplit) -- or partial sums (split)
     float *shift;     // split only: [2][R][K] clamped column maxima
     int R, S, I, J, K;
-    int64_t sw0, sw1, sa0, sa1, sb0, sb1, sc0, sc1;
+    int64_t sw0, sw1, sw2, sa0, sa1, sb0, sb1, sc0, sc1;  // sw2: stride of the flat (i, j) axis of w
     int s_tiles, n_tiles, splits;
     int iters_per_split;  // (j-chunk, i) iterations per split
     int stream_out;       // rows of c are 16-byte aligned: non-temporal result stores
@@ -159,7 +159,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     const int wrows = (p.S - s0) < TS ? (p.S - s0) : TS;
     const float *wtile0 = wr + (int64_t)s0 * p.sw1;
     const __amdgpu_buffer_rsrc_t w_rsrc =
-        make_rsrc(wtile0, (uint32_t)(((int64_t)(wrows - 1) * p.sw1 + (int64_t)p.I * p.J) * 4));
+        make_rsrc(wtile0, (uint32_t)(((int64_t)(wrows - 1) * p.sw1 + ((int64_t)p.I * p.J - 1) * p.sw2 + 1) * 4));
     uint32_t woff[SLOTS];
 #pragma unroll
     for (int sidx = 0; sidx < SLOTS; ++sidx)
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     constexpr bool ELEM = !VEC && (NT % JC == 0) && ((TS * JC) % NT == 0) && (TS * JC / NT <= 4 * SLOTS);
     constexpr int NE = ELEM ? TS * JC / NT : 1;  // floats per thread
     const int ecol = tid % JC;
-    const uint32_t ebase = ((uint32_t)(tid / JC) * (uint32_t)p.sw1 + (uint32_t)ecol) * 4u;
+    const uint32_t ebase = ((uint32_t)(tid / JC) * (uint32_t)p.sw1 + (uint32_t)ecol * (uint32_t)p.sw2) * 4u;
     // (a slot past the tile loads some valid or out-of-extent address: the value is never used)
     auto load_tile = [&](int i, int jc) {
         // floats of the chunk that belong to this step (packed: of the flat (i, j) axis)
@@ -192,7 +192,7 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
         } else if (ELEM) {
             // rows that are not 16-byte aligned: single floats, consecutive lanes on consecutive
             // columns (coalesced), a thread's floats NT / JC rows apart (scalar offsets)
-            const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
+            const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * (uint32_t)p.sw2 * 4u;
             const bool inside = jc * JC + ecol < p.J;
 #pragma unroll
             for (int e = 0; e < NE; ++e) {
@@ -204,13 +204,13 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
             for (int sidx = 0; sidx < SLOTS; ++sidx) {
                 const int row = srow[sidx];
                 const int j = jc * JC + 4 * sc4[sidx];
-                const float *src = wtile0 + (int64_t)row * p.sw1 + (int64_t)i * p.J + j;
+                const float *src = wtile0 + (int64_t)row * p.sw1 + ((int64_t)i * p.J + j) * p.sw2;
                 floatx4 v = {0.f, 0.f, 0.f, 0.f};
                 if (sval[sidx] && row < wrows) {
                     if (j + 0 < p.J) v[0] = src[0];
-                    if (j + 1 < p.J) v[1] = src[1];
-                    if (j + 2 < p.J) v[2] = src[2];
-                    if (j + 3 < p.J) v[3] = src[3];
+                    if (j + 1 < p.J) v[1] = src[p.sw2];
+                    if (j + 2 < p.J) v[2] = src[2 * p.sw2];
+                    if (j + 3 < p.J) v[3] = src[3 * p.sw2];
                 }
                 stage[sidx] = v;
             }
@@ -602,14 +602,14 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (mode != TRT_MODE_AUTO && mode != TRT_MODE_SPLIT && mode != TRT_MODE_UNSPLIT) return TRT_E_INVALID;
     if (variant < 0 || variant > kNumVariants) return TRT_E_INVALID;
-    if (sw[2] != 1 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
+    if (sw[2] < 0 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     if (sc[1] < K) return TRT_E_LAYOUT;  // output rows must not overlap (stores rely on it)
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
     // byte offsets inside one batch slab of w, a and c are 32-bit (buffer addressing)
-    if (S * sw[1] + I * J >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
+    if (S * sw[1] + I * J * (sw[2] > 0 ? sw[2] : 1) >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
 
     // A single j under several i: the contraction is symmetric in (i, a) and (j, b), and with
     // J = 1 the same w is an R x S x 1 x I tensor, so the call runs with the roles exchanged
@@ -619,7 +619,8 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
                               stream);
 
     int v = resolve_variant(variant, R, S, I, J, K);
-    const bool w_aligned = (sw[0] % 4 == 0) && (sw[1] % 4 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
+    // (a flat axis of w with another stride than 1 -- a sliced view -- is read element by element, in place)
+    const bool w_aligned = sw[2] == 1 && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
     // packed rows need 16-byte loads along the flat (i, j) axis; any other call runs the same tile unpacked
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
     const Lt2Variant &vr = kVariants[v];
@@ -628,7 +629,7 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     Lt2Args args;
     args.w = w; args.a = a; args.b = b;
     args.R = (int)R; args.S = (int)S; args.I = (int)I; args.J = (int)J; args.K = (int)K;
-    args.sw0 = sw[0]; args.sw1 = sw[1];
+    args.sw0 = sw[0]; args.sw1 = sw[1]; args.sw2 = sw[2];
     args.sa0 = sa[0]; args.sa1 = sa[1];
     args.sb0 = sb[0]; args.sb1 = sb[1];
     args.sc0 = sc[0]; args.sc1 = sc[1];

@@ -127,7 +127,9 @@ def lt2exp(
         b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
         J = J4
     sw, sa, sb = w.stride(), a.stride(), b.stride()
-    if sw[2] != 1 or min(sw) < 0:
+    # w is read in place whatever the stride of its flat (i, j) axis (a sliced view: element
+    # loads instead of 16-byte ones); only the bf16 kernels and negative strides need a copy
+    if min(sw) < 0 or (sw[2] != 1 and _precision != "fp32"):
         w = _unit_inner(w)
         sw = w.stride()
     if sa[2] != 1 or min(sa) < 0:
