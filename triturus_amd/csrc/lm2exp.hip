@@ -615,6 +615,16 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
         return find_variant_shape(1, 2, 2);
     const int64_t kFill = 384;
     const int64_t ct = ceil_div(K, 128);
+    // Large grids of 256-row tiles under a contraction of a few hundred: the paired-wavefront
+    // kernel (exact shift first, no rescaling, an exp per workgroup and element).  Its time does
+    // not depend on the data; the online kernels rescale whenever a chunk towers over the shift
+    // so far, which b ~ N(-50, 20) does in most of the early chunks.  Measured at K = 4096 with
+    // that b: R=64 I=J=256 281 us against 293; with b ~ N(0, 1): 280 against 284, R=16 77
+    // against 80, R=32 I=1024 K=2048 271 against 280, J = 512 531 against 533; slower with
+    // fewer than two tiles per CU (R=8: +9 %), J = 192 (+1 %), or J not a multiple of 4 (+4 %).
+    const int64_t i256 = ceil_div(I, 256);
+    if (J >= 224 && J <= 512 && J % 4 == 0 && I >= 240 && i256 * 256 * 100 <= I * 107 && R * i256 * ct >= 512)
+        return find_pair_variant(4, 4);
     const int64_t n128 = R * ceil_div(I, 128) * ct, n64 = R * ceil_div(I, 64) * ct;
     int rt;
     if (I <= 32 || J <= 32) {
