@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TRT_ABI_VERSION 6
+#define TRT_ABI_VERSION 7
 
 #define TRT_OK 0
 #define TRT_E_INVALID (-1)   /* null pointer, non-positive size, bad enum   */

@@ -14,7 +14,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtriturus_hip.so"
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 TRT_F32, TRT_F64, TRT_F16, TRT_BF16 = 0, 1, 2, 3
 MODE_AUTO, MODE_SPLIT, MODE_UNSPLIT = 0, 1, 2
