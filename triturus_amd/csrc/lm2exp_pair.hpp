@@ -161,19 +161,18 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
     // kLoadVec: piece f = tid + s NT is row f / NPL, plane f % NPL
     // kLoadByCol: element g = tid + e NT is row g / JC, column g % JC = tid % JC
     // kLoadByRow: element g = tid + e NT is row g % TM = tid % TM, column g / TM
-    uint32_t aoff[LOADA == kLoadVec ? SLOTS : 1];
-    int lds_off[LOADA == kLoadVec ? SLOTS : 1];
+    // (kLoadVec: a thread keeps its plane, and its pieces lie NT / NPL rows apart: one lane
+    // offset, the slot in the scalar offset of the load and the immediate offset of the LDS
+    // write; rows past I lie outside the extent and read as zeros)
+    static_assert(NT % NPL == 0, "a thread's pieces share a plane");
+    uint32_t aoff[1];
+    int lds_off[1];
     int ecol = 0, erow = 0;
+    const uint32_t a_slot_bytes = (uint32_t)(NT / NPL) * (uint32_t)p.sa1 * 4u;  // wave-uniform
     if (LOADA == kLoadVec) {
-#pragma unroll
-        for (int s = 0; s < SLOTS; ++s) {
-            const int f = tid + s * NT;
-            int row = f / NPL;
-            const int c = f % NPL;
-            lds_off[s] = c * PLANE + row * 4;
-            row = row < arows ? row : arows - 1;
-            aoff[s] = ((uint32_t)row * (uint32_t)p.sa1 + 4u * (uint32_t)c) * 4u;
-        }
+        const int row = tid / NPL, c = tid % NPL;
+        lds_off[0] = c * PLANE + row * 4;
+        aoff[0] = ((uint32_t)row * (uint32_t)p.sa1 + 4u * (uint32_t)c) * 4u;
     } else if (LOADA == kLoadByCol) {
         ecol = tid % JC;
         erow = tid / JC;
@@ -190,8 +189,8 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
             const uint32_t soff = (uint32_t)(jc * JC) * 4u;
 #pragma unroll
             for (int s = 0; s < SLOTS; ++s) {
-                const floatx4 v = buf_load_f32x4(a_rsrc, aoff[s], soff);
-                const int j = jc * JC + 4 * ((tid + s * NT) % NPL);
+                const floatx4 v = buf_load_f32x4(a_rsrc, aoff[0], soff + (uint32_t)s * a_slot_bytes);
+                const int j = jc * JC + 4 * (tid % NPL);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sa[4 * s + e] = (!masked || j + e < p.J) ? v[e] : 0.f;
             }
@@ -218,7 +217,7 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
 #pragma unroll
             for (int s = 0; s < SLOTS; ++s) {
                 const floatx4 v = {sa[4 * s], sa[4 * s + 1], sa[4 * s + 2], sa[4 * s + 3]};
-                *reinterpret_cast<floatx4 *>(&dst[lds_off[s]]) = v;
+                *reinterpret_cast<floatx4 *>(&dst[lds_off[0] + s * (NT / NPL) * 4]) = v;
             }
         } else if (LOADA == kLoadByCol) {
 #pragma unroll
@@ -264,10 +263,18 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
     // to LDS buffer CUR ^ 1.  FAST: all those chunks exist and are full, no tests.
     const int rd_own = (2 * (wm * NH) + h) * PLANE + (wrow0 + m) * 4;
     const int rd_partner = (2 * ((wm ^ 1) * NH) + h) * PLANE + (wrow0 + m) * 4;
-    auto step = [&](auto cur_c, auto fast_c, int t, const float (&ecur)[NB], float (&enext)[NB],
-                    const float (&bnext)[NB], float (&bfree)[NB]) {
+    // Two register sets that swap roles from step to step, picked by the step's parity (a
+    // compile-time index: the sets must stay in registers): ee[CUR] the own exps of chunk t,
+    // ee[CUR ^ 1] those of chunk t + 1; bb[CUR ^ 1] the raw b values of chunk t + 1, bb[CUR]
+    // free for those of chunk t + 2.
+    float ee[2][NB], bb[2][NB];
+    auto step = [&](auto cur_c, auto fast_c, int t) {
         constexpr int CUR = decltype(cur_c)::value;
         constexpr bool FAST = decltype(fast_c)::value;
+        float (&ecur)[NB] = ee[CUR];
+        float (&enext)[NB] = ee[CUR ^ 1];
+        const float (&bnext)[NB] = bb[CUR ^ 1];
+        float (&bfree)[NB] = bb[CUR];
         const bool more = FAST || t + 1 < jc1;  // wave-uniform
         if (FAST) {
             load_a(t + 1, false);
@@ -316,15 +323,18 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
                     acc[rt0 + k] = __builtin_amdgcn_mfma_f32_32x32x2f32(
                         af[k][u], half ? ebp[qq][u] : ecur[4 * qq + u], acc[rt0 + k], 0, 0, 0);
                 // NB exps over the 2 NG u-pairs of the first half
-                if (more && half == 0 && (u % 2 == 1 || NB > NG) && nexp < NB) {
-                    enext[nexp] = exp_one(bnext[nexp]);
+                // (the count advances whether or not there is a next chunk: it must stay a
+                // compile-time index, or the register sets become arrays in scratch memory)
+                if (half == 0 && (u % 2 == 1 || NB > NG) && nexp < NB) {
+                    if (more) enext[nexp] = exp_one(bnext[nexp]);
                     ++nexp;
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
-            if (more && g == NG / 2 - 1) {
-                for (; nexp < NB; ++nexp) enext[nexp] = exp_one(bnext[nexp]);
-                publish(enext, CUR ^ 1);
+            if (g == NG / 2 - 1) {
+                for (; nexp < NB; ++nexp)
+                    if (more) enext[nexp] = exp_one(bnext[nexp]);
+                if (more) publish(enext, CUR ^ 1);
             }
         };
 #pragma unroll
@@ -340,7 +350,7 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
 
     // ---- prologue: the first chunk (a tile and b values) and the b values of the second
     using std::integral_constant;
-    float e0[NB], e1[NB], b0[NB], b1[NB];
+    float (&e0)[NB] = ee[0], (&b0)[NB] = bb[0], (&b1)[NB] = bb[1];
     if (jc0 >= n_full) {
         load_a(jc0, true);
         load_b(b0, jc0, true);
@@ -362,13 +372,13 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
     // last chunks, the ragged one among them, take the steps with tests
     int t = jc0;
     for (; t + 3 < full_end; t += 2) {
-        step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, t, e0, e1, b1, b0);
-        step(integral_constant<int, 1>{}, integral_constant<bool, true>{}, t + 1, e1, e0, b0, b1);
+        step(integral_constant<int, 0>{}, integral_constant<bool, true>{}, t);
+        step(integral_constant<int, 1>{}, integral_constant<bool, true>{}, t + 1);
     }
     while (t < jc1) {
-        step(integral_constant<int, 0>{}, integral_constant<bool, false>{}, t, e0, e1, b1, b0);
+        step(integral_constant<int, 0>{}, integral_constant<bool, false>{}, t);
         if (++t >= jc1) break;
-        step(integral_constant<int, 1>{}, integral_constant<bool, false>{}, t, e1, e0, b0, b1);
+        step(integral_constant<int, 1>{}, integral_constant<bool, false>{}, t);
         ++t;
     }
 
