@@ -127,7 +127,8 @@ def test_other_float_dtypes(dev, dtype):
 @pytest.mark.parametrize(
     "shape",
     [(1, 1), (1, 7), (7, 1), (23, 31), (64, 64), (65, 127), (200, 150), (1000, 3), (3, 1000), (2, 300000),
-     (300000, 2), (513, 1024), (4096, 256), (5, 65536), (65537, 5), (65536, 256), (40000, 64), (5000, 130)],
+     (300000, 2), (513, 1024), (4096, 256), (5, 65536), (65537, 5), (65536, 256), (40000, 64), (5000, 130),
+     (16400, 4100), (8200, 8196)],  # 256 MiB and more: two 16-byte pieces per lane along axis 0, ragged last block
 )
 def test_matmax_shapes(dev, shape):
     x = torch.randn(*shape)

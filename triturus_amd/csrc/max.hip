@@ -660,7 +660,8 @@ __global__ __launch_bounds__(kMatThreads) void colmax_kernel(
 // combines the block's partial rows (device-scope 8-byte accesses, see take_ticket) and writes y.
 // VPL: 16-byte vectors per lane.  With 2 a wavefront reads 2 KiB of a row at a time and a
 // workgroup owns 512 (fp32) columns: measured on 4096 x 4096 fp32 with 128 rows per workgroup,
-// the sweep alone takes 12.2 us against 13.6 us with 1 KiB pieces (16384^2: 173 against 182 us).
+// the sweep alone takes 12.9 us against 13.3 us with 1 KiB pieces (16384^2: 173 against 182 us);
+// the host picks it for large matrices only (colmax_fused_plan).
 constexpr int kColFusedSplits = 32;
 constexpr int kColFusedUnroll = 8;  // 16-byte loads in flight per lane
 template <int DT, int VPL>
@@ -753,34 +754,32 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
     if (!last_block) return;
     // the last workgroup of the column block: wavefront w takes splits w, w + 4, ...; all loads
     // of a batch are asked for before the first is looked at
-    constexpr int kBatch = 8 / VPL;  // splits per batch and wavefront
+    constexpr int kBatch = kColFusedSplits / kMatWaves;  // all splits in one batch: one round trip (a trip costs over 1 us here)
 #pragma unroll
     for (int e = 0; e < CN; ++e) best[e] = neg_inf<C>();
+    // (a split past the last one is replaced by split 0: folding a row twice changes nothing,
+    // and the loads carry no predicates)
+#pragma unroll
     for (int s0 = 0; s0 < kColFusedSplits; s0 += kBatch * kMatWaves) {
-        if (s0 >= splits) break;
+        if (s0 >= splits) break;  // wave-uniform
         unsigned long long w[kBatch][WORDS];
 #pragma unroll
         for (int q = 0; q < kBatch; ++q) {
             const int sp = s0 + wave + q * kMatWaves;
-            if (sp < splits) {
+            const unsigned long long *src = prow + (sp < splits ? sp : 0) * words_per_row;
 #pragma unroll
-                for (int k = 0; k < WORDS; ++k)
-                    w[q][k] = __hip_atomic_load(&prow[sp * words_per_row + k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            }
+            for (int k = 0; k < WORDS; ++k)
+                w[q][k] = __hip_atomic_load(&src[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
 #pragma unroll
-        for (int q = 0; q < kBatch; ++q) {
-            const int sp = s0 + wave + q * kMatWaves;
-            if (sp < splits) {
+        for (int q = 0; q < kBatch; ++q)
 #pragma unroll
-                for (int p = 0; p < VPL; ++p) {
-                    Piece u;
-                    u.w[0] = w[q][2 * p];
-                    u.w[1] = w[q][2 * p + 1];
-                    fold(u.v, p);
-                }
+            for (int p = 0; p < VPL; ++p) {
+                Piece u;
+                u.w[0] = w[q][2 * p];
+                u.w[1] = w[q][2 * p + 1];
+                fold(u.v, p);
             }
-        }
     }
     __syncthreads();  // sm is reused
     across_waves();
@@ -851,8 +850,13 @@ struct FusedPlan {
 static FusedPlan colmax_fused_plan(int64_t m, int64_t n, int vn) {
     FusedPlan none{0, 0, 1, m};
     if (n % vn != 0) return none;  // whole 16-byte pieces only (y is written in pieces)
-    // two pieces per lane where that still leaves a workgroup of at least 128 rows per CU
-    for (int vpl = 2; vpl >= 1; --vpl) {
+    // Two pieces per lane for matrices of 256 MiB and more, where that still leaves a workgroup
+    // of at least 128 rows per CU: the sweep is 5 % faster (16384^2 fp32: 175 against 182 us),
+    // but the last workgroup of a column block then has twice the partial words to fetch, and
+    // those device-scope loads are slow (4096^2 fp32: 3.6 us against 1.3 us, 16.7 us in all
+    // against 14.6 us).
+    const bool large = m * n * (16 / vn) >= ((int64_t)1 << 28);
+    for (int vpl = large ? 2 : 1; vpl >= 1; --vpl) {
         const int64_t colblocks = ceil_div(n, (int64_t)kWave * vn * vpl);
         if (colblocks > kMaxTickets) continue;
         int64_t splits = ceil_div((int64_t)(vpl == 2 ? 256 : 512), colblocks);
