@@ -663,6 +663,7 @@ __global__ __launch_bounds__(kMatThreads) void colmax_kernel(
 // the sweep alone takes 12.9 us against 13.3 us with 1 KiB pieces (16384^2: 173 against 182 us);
 // the host picks it for large matrices only (colmax_fused_plan).
 constexpr int kColFusedSplits = 32;
+constexpr int kDeviceScope = 16;  // cache-policy bit sc1 of a buffer access: past the caches that are not coherent across the device
 constexpr int kColFusedUnroll = 8;  // 16-byte loads in flight per lane
 template <int DT, int VPL>
 __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
@@ -732,20 +733,22 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
     // a partial row: VPL x 16 bytes per lane of wave 0, as 8-byte words (piece p, half q: word 2p + q)
     constexpr int WORDS = 2 * VPL;
     const int64_t words_per_row = (int64_t)colblocks * kWave * WORDS;
-    unsigned long long *prow = part + ((int64_t)cb * kWave + lane) * WORDS;
     union Piece {
         V v;
         unsigned long long w[2];
     };
+    // (partials travel as 16-byte buffer accesses with the device-scope bit: the last workgroup's
+    // trips to memory cost by the instruction, and this halves their number)
+    const __amdgpu_buffer_rsrc_t prsrc = make_rsrc(part, (uint32_t)(words_per_row * splits * 8));
+    const uint32_t plane = (uint32_t)(((int64_t)cb * kWave + lane) * WORDS * 8);
     if (wave == 0) {
 #pragma unroll
         for (int p = 0; p < VPL; ++p) {
             Piece u;
 #pragma unroll
             for (int e = 0; e < VN; ++e) u.v.e[e] = E::down(best[p * VN + e]);
-            __hip_atomic_store(&prow[split * words_per_row + 2 * p], u.w[0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            __hip_atomic_store(&prow[split * words_per_row + 2 * p + 1], u.w[1], __ATOMIC_RELAXED,
-                               __HIP_MEMORY_SCOPE_AGENT);
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uintx4, u), prsrc, plane + 16u * p,
+                                                   (uint32_t)(split * words_per_row * 8), kDeviceScope);
         }
         const unsigned t = take_ticket_wave(ticket + cb * kTicketStride);
         if (lane == 0) last_block = t == (unsigned)splits - 1;
@@ -762,24 +765,19 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
 #pragma unroll
     for (int s0 = 0; s0 < kColFusedSplits; s0 += kBatch * kMatWaves) {
         if (s0 >= splits) break;  // wave-uniform
-        unsigned long long w[kBatch][WORDS];
+        uintx4 w[kBatch][VPL];
 #pragma unroll
         for (int q = 0; q < kBatch; ++q) {
             const int sp = s0 + wave + q * kMatWaves;
-            const unsigned long long *src = prow + (sp < splits ? sp : 0) * words_per_row;
+            const uint32_t soff = (uint32_t)((sp < splits ? sp : 0) * words_per_row * 8);  // wave-uniform
 #pragma unroll
-            for (int k = 0; k < WORDS; ++k)
-                w[q][k] = __hip_atomic_load(&src[k], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            for (int p = 0; p < VPL; ++p)
+                w[q][p] = __builtin_amdgcn_raw_buffer_load_b128(prsrc, plane + 16u * p, soff, kDeviceScope);
         }
 #pragma unroll
         for (int q = 0; q < kBatch; ++q)
 #pragma unroll
-            for (int p = 0; p < VPL; ++p) {
-                Piece u;
-                u.w[0] = w[q][2 * p];
-                u.w[1] = w[q][2 * p + 1];
-                fold(u.v, p);
-            }
+            for (int p = 0; p < VPL; ++p) fold(__builtin_bit_cast(Piece, w[q][p]).v, p);
     }
     __syncthreads();  // sm is reused
     across_waves();
