@@ -59,6 +59,10 @@ constexpr int64_t kNoIdx = INT64_MAX;
 // max that ignores a NaN operand (both NaN: NaN), one instruction without canonicalisation moves
 __device__ __forceinline__ float max_ignoring_nan(float a, float b) { return max3_raw(a, b, b); }
 __device__ __forceinline__ double max_ignoring_nan(double a, double b) { return __builtin_fmax(a, b); }
+__device__ __forceinline__ float max3_ignoring_nan(float a, float b, float c) { return max3_raw(a, b, c); }
+__device__ __forceinline__ double max3_ignoring_nan(double a, double b, double c) {
+    return __builtin_fmax(__builtin_fmax(a, b), c);
+}
 
 template <typename C>
 __device__ __forceinline__ C vmax_nan(C a, C b) {
@@ -180,6 +184,11 @@ static_assert(kVmaxMaxBlocks / kVmaxGroup < kMaxTickets, "one counter per group 
 // well but writes back and invalidates whole caches, once per workgroup: measured 120 us
 // instead of 12 us on a 64 MiB vector.  Between its partial stores and its ticket a wavefront
 // waits for the stores to be acknowledged (a workgroup-scope release: a wait, no cache action).
+// Partial results themselves travel as 16-byte buffer accesses with the device-scope bit (sc1)
+// of the cache policy.  A wavefront's device-scope accesses do not overlap one another -- each
+// costs a trip of some 170 ns (measured: the last workgroup's time grows by that much per load
+// instruction) -- so a partial is one 16-byte record, not a word per field.
+constexpr int kDeviceScope = 16;
 __device__ __forceinline__ unsigned take_ticket(unsigned *ticket) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
@@ -204,7 +213,7 @@ __device__ __forceinline__ unsigned take_ticket_wave(unsigned *ticket) {
 template <int DT, bool WITH_IDX, bool FINAL>
 __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     const typename Elem<DT>::T *__restrict__ x, int64_t n, int64_t head, int64_t nvec,
-    typename Elem<DT>::C *pval, int64_t *pidx, unsigned *ticket,
+    uintx4 *prec, unsigned *ticket,
     typename Elem<DT>::T *__restrict__ out_val, int64_t *__restrict__ out_idx) {
     using E = Elem<DT>;
     using T = typename E::T;
@@ -376,11 +385,23 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     const int ngroups = (nblocks + kVmaxGroup - 1) / kVmaxGroup;
     const int gfirst = group * kVmaxGroup;
     const int gsize = nblocks - gfirst < kVmaxGroup ? nblocks - gfirst : kVmaxGroup;
+    union Record {
+        struct {
+            C val;  // (a 4-byte value leaves the rest of its 8-byte slot unused)
+            int64_t idx;
+        } f;
+        uintx4 bits;
+    };
+    static_assert(sizeof(Record) == 16, "one 16-byte access per partial");
+    const __amdgpu_buffer_rsrc_t prsrc = make_rsrc(prec, (uint32_t)kVmaxMaxBlocks * 16u);
     unsigned *tick1 = ticket + group * kTicketStride;
     unsigned *tick2 = ticket + (kMaxTickets - 1) * kTicketStride;
     if (tid == 0) {
-        __hip_atomic_store(&pval[blockIdx.x], best, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        if (WITH_IDX) __hip_atomic_store(&pidx[blockIdx.x], bidx, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // the partial: one 16-byte record (value in an 8-byte slot, index)
+        Record rec;
+        rec.f.val = best;
+        rec.f.idx = bidx;
+        __builtin_amdgcn_raw_buffer_store_b128(rec.bits, prsrc, (uint32_t)blockIdx.x * 16u, 0, kDeviceScope);
         bool last = take_ticket(tick1) == (unsigned)gsize - 1;
         if (last) {
             last = take_ticket(tick2) == (unsigned)ngroups - 1;
@@ -394,24 +415,19 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     bidx = kNoIdx;
     // every partial is asked for before the first is looked at: one round trip, not one per partial
     constexpr int kPer = (kVmaxMaxBlocks + kVmaxThreads - 1) / kVmaxThreads;
-    C pc[kPer];
-    int64_t pi[kPer];
+    // (a slot past the last workgroup is replaced by slot 0: seeing a partial twice changes nothing)
+    Record pr[kPer];
 #pragma unroll
     for (int u = 0; u < kPer; ++u) {
         const int i = tid + u * kVmaxThreads;
-        pc[u] = neg_inf<C>();
-        pi[u] = kNoIdx;
-        if (i < nblocks) {
-            pc[u] = __hip_atomic_load(&pval[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-            if (WITH_IDX) pi[u] = __hip_atomic_load(&pidx[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        }
+        pr[u].bits = __builtin_amdgcn_raw_buffer_load_b128(prsrc, (uint32_t)(i < nblocks ? i : 0) * 16u, 0, kDeviceScope);
     }
 #pragma unroll
     for (int u = 0; u < kPer; ++u) {
         if (WITH_IDX) {
-            feed(pc[u], pi[u]);
+            feed(pr[u].f.val, pr[u].f.idx);
         } else {
-            best = vmax_nan(best, pc[u]);
+            best = vmax_nan(best, pr[u].f.val);
         }
     }
     block_reduce();
@@ -438,7 +454,7 @@ static size_t elem_size(int dtype) {
     }
 }
 
-// workspace layout: [tickets][kVmaxMaxBlocks x 8-byte value slots][kVmaxMaxBlocks x int64];
+// workspace layout: [tickets][kVmaxMaxBlocks x 16-byte records (value slot, int64 index)];
 // vectors short enough for one workgroup need none
 static bool vmax_single_block(int64_t n, int dtype) {
     const int64_t vn = 16 / (int64_t)elem_size(dtype);
@@ -465,22 +481,21 @@ static int vmax_launch(const void *x, int64_t n, void *out_val, int64_t *out_idx
     if (vmax_single_block(n, DT)) {
         if (out_idx)
             hipLaunchKernelGGL((vmax_kernel<DT, true, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                               nvec, (C *)nullptr, (int64_t *)nullptr, (unsigned *)nullptr, ov, out_idx);
+                               nvec, (uintx4 *)nullptr, (unsigned *)nullptr, ov, out_idx);
         else
             hipLaunchKernelGGL((vmax_kernel<DT, false, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                               nvec, (C *)nullptr, (int64_t *)nullptr, (unsigned *)nullptr, ov, out_idx);
+                               nvec, (uintx4 *)nullptr, (unsigned *)nullptr, ov, out_idx);
         return (int)hipGetLastError();
     }
     const int blocks = vmax_blocks(nvec);
     unsigned *ticket = static_cast<unsigned *>(ws);
-    C *pval = reinterpret_cast<C *>(static_cast<char *>(ws) + kTicketBytes);
-    int64_t *pidx = reinterpret_cast<int64_t *>(static_cast<char *>(ws) + kTicketBytes + (size_t)kVmaxMaxBlocks * 8);
+    uintx4 *prec = reinterpret_cast<uintx4 *>(static_cast<char *>(ws) + kTicketBytes);
     if (out_idx)
         hipLaunchKernelGGL((vmax_kernel<DT, true, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                           nvec, pval, pidx, ticket, ov, out_idx);
+                           nvec, prec, ticket, ov, out_idx);
     else
         hipLaunchKernelGGL((vmax_kernel<DT, false, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                           nvec, pval, pidx, ticket, ov, out_idx);
+                           nvec, prec, ticket, ov, out_idx);
     return (int)hipGetLastError();
 }
 
@@ -663,7 +678,6 @@ __global__ __launch_bounds__(kMatThreads) void colmax_kernel(
 // the sweep alone takes 12.9 us against 13.3 us with 1 KiB pieces (16384^2: 173 against 182 us);
 // the host picks it for large matrices only (colmax_fused_plan).
 constexpr int kColFusedSplits = 32;
-constexpr int kDeviceScope = 16;  // cache-policy bit sc1 of a buffer access: past the caches that are not coherent across the device
 constexpr int kColFusedUnroll = 8;  // 16-byte loads in flight per lane
 template <int DT, int VPL>
 __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
@@ -696,10 +710,29 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
     int64_t poff[VPL];
 #pragma unroll
     for (int p = 0; p < VPL; ++p) poff[p] = have[p] ? (int64_t)p * kWave * VN : 0;
-    auto fold = [&](const V &b, int p) {
+    // One vector instruction per element: a maximum of three that ignores NaN takes two rows
+    // at a time, and one unordered test per pair of rows remembers, per column, whether a NaN
+    // went by; the flag is folded into the value once, after the sweep (NaN wins).
+    bool un[CN];
 #pragma unroll
-        for (int e = 0; e < VN; ++e) best[p * VN + e] = vmax_nan(best[p * VN + e], E::up(b.e[e]));
+    for (int e = 0; e < CN; ++e) un[e] = false;
+    auto fold2 = [&](const V &b0, const V &b1, int p) {
+#pragma unroll
+        for (int e = 0; e < VN; ++e) {
+            const C c0 = E::up(b0.e[e]), c1 = E::up(b1.e[e]);
+            best[p * VN + e] = max3_ignoring_nan(best[p * VN + e], c0, c1);
+            un[p * VN + e] |= __builtin_isunordered(c0, c1);
+        }
     };
+    auto fold = [&](const V &b, int p) { fold2(b, b, p); };
+    auto settle = [&]() {  // a column that has seen a NaN is NaN
+#pragma unroll
+        for (int e = 0; e < CN; ++e) {
+            best[e] = un[e] ? (C)__builtin_nanf("") : best[e];
+            un[e] = false;
+        }
+    };
+    static_assert(ROWS % 2 == 0, "rows are folded in pairs");
     int64_t r = r0 + wave;
     for (; r + (ROWS - 1) * kMatWaves < r1; r += ROWS * kMatWaves) {
         V b[ROWS][VPL];
@@ -709,9 +742,9 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
             for (int p = 0; p < VPL; ++p) b[u][p] = *reinterpret_cast<const V *>(xc + (r + u * kMatWaves) * ld + poff[p]);
         __builtin_amdgcn_sched_barrier(0);  // all loads of the step are under way before the first is looked at
 #pragma unroll
-        for (int u = 0; u < ROWS; ++u)
+        for (int u = 0; u < ROWS; u += 2)
 #pragma unroll
-            for (int p = 0; p < VPL; ++p) fold(b[u][p], p);
+            for (int p = 0; p < VPL; ++p) fold2(b[u][p], b[u + 1][p], p);
     }
     for (; r < r1; r += kMatWaves) {
 #pragma unroll
@@ -720,6 +753,7 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
     __shared__ C sm[kMatWaves][kWave * CN];
     __shared__ bool last_block;
     auto across_waves = [&]() {  // wave 0 ends up with the maxima of the workgroup
+        settle();
 #pragma unroll
         for (int e = 0; e < CN; ++e) sm[wave][e * kWave + lane] = best[e];
         __syncthreads();
@@ -775,9 +809,10 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
                 w[q][p] = __builtin_amdgcn_raw_buffer_load_b128(prsrc, plane + 16u * p, soff, kDeviceScope);
         }
 #pragma unroll
-        for (int q = 0; q < kBatch; ++q)
+        for (int q = 0; q < kBatch; q += 2)
 #pragma unroll
-            for (int p = 0; p < VPL; ++p) fold(__builtin_bit_cast(Piece, w[q][p]).v, p);
+            for (int p = 0; p < VPL; ++p)
+                fold2(__builtin_bit_cast(Piece, w[q][p]).v, __builtin_bit_cast(Piece, w[q + 1][p]).v, p);
     }
     __syncthreads();  // sm is reused
     across_waves();
