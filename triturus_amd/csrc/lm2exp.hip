@@ -423,7 +423,7 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
 template <bool CLAMP>
 __global__ __launch_bounds__(256) void lm2exp_colmax_kernel(const float *__restrict__ b, float *__restrict__ m, int R,
                                                             int J, int K, int64_t sb0, int64_t sb1, int chunk,
-                                                            int splits) {
+                                                            int /*splits*/) {
     __shared__ float part[4][256];
     const int blocks_per_batch = (K + 255) / 256;
     const int kb = blockIdx.x % blocks_per_batch;

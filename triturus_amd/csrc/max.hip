@@ -469,7 +469,6 @@ static int vmax_launch(const void *x, int64_t n, void *out_val, int64_t *out_idx
                        hipStream_t stream) {
     using E = Elem<DT>;
     using T = typename E::T;
-    using C = typename E::C;
     constexpr int VN = 16 / (int)sizeof(T);
     const T *xp = static_cast<const T *>(x);
     // elements before the first 16-byte boundary
