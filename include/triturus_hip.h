@@ -197,6 +197,10 @@ int trt_lm2exp_bf16_variant_count(void);
  * time need workspaces of their own.
  */
 #define TRT_MAX_TICKET_BYTES 65536
+/* Zeroes the arrival counters of a max workspace with a small kernel on `stream` (in place of a
+ * hipMemset; safe to record into a HIP graph).  No counterpart in the reference, whose
+ * reductions launch once per level.  workspace_bytes < TRT_MAX_TICKET_BYTES: TRT_E_WORKSPACE. */
+int trt_max_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * Max of a contiguous m x n row-major matrix along axis 0 (y has n entries)

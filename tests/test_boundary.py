@@ -127,6 +127,8 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_matmax(one, one, 1 << 33, 2, 1, _lib.TRT_F16, null, 0, null) == -4
     assert lib.trt_matmax(one, one, 1, 1 << 40, 0, _lib.TRT_F16, null, 0, null) == -4
     assert lib.trt_copy_bytes(one, one, 24, null) == -1
+    assert lib.trt_max_workspace_init(null, 1 << 20, null) == -3
+    assert lib.trt_max_workspace_init(one, 1024, null) == -3  # smaller than the arrival counters
     # mm, vadd
     assert lib.trt_mm_f32(one, null, one, 2, 2, 2, null) == -1
     assert lib.trt_mm_f32(one, one, one, 2, 0, 2, null) == -1

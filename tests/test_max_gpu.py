@@ -12,6 +12,7 @@ import torch
 
 from oracle import max_ref
 from triturus.max import matmax, vamax, vmax
+from triturus_amd import _lib
 
 pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
@@ -217,6 +218,37 @@ def test_runs_on_the_current_stream_without_synchronising(dev):
     s.synchronize()
     assert (v.item(), i.item()) == tuple(t.item() for t in torch.max(x, 0))
     _same(y, torch.amax(x.view(1024, 1024), 1))
+
+
+def test_c_abi_with_a_workspace_prepared_by_the_library(dev):
+    """A C caller's workspace: garbage from the allocator, its arrival counters zeroed once by
+    trt_max_workspace_init; several calls of both reductions then share it (every call leaves
+    the counters zero)."""
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(5)
+    x = torch.randn(3000, 4100, generator=g)
+    x[17, 33] = float("nan")
+    xg = x.to(dev)
+    n = x.numel()
+    need = max(lib.trt_vmax_workspace_bytes(n, _lib.TRT_F32), lib.trt_matmax_workspace_bytes(3000, 4100, 0, _lib.TRT_F32),
+               lib.trt_matmax_workspace_bytes(3000, 4100, 1, _lib.TRT_F32))
+    ws = torch.full((need,), 0xAB, dtype=torch.uint8, device=dev)
+    stream = _lib.raw_stream(dev)
+    with _lib.on_device(dev):
+        _lib.check(lib.trt_max_workspace_init(ws.data_ptr(), need, stream), "trt_max_workspace_init")
+        for _ in range(3):
+            val = torch.empty((), device=dev)
+            idx = torch.empty((), dtype=torch.int64, device=dev)
+            _lib.check(lib.trt_vmax(xg.data_ptr(), n, _lib.TRT_F32, val.data_ptr(), idx.data_ptr(), ws.data_ptr(), need,
+                                    stream), "trt_vmax")
+            gv, gi = torch.max(x.view(-1), 0)
+            assert torch.isnan(val).item() and idx.item() == gi.item()
+            for axis in (0, 1):
+                y = torch.empty(x.shape[1 - axis], device=dev)
+                _lib.check(lib.trt_matmax(xg.data_ptr(), y.data_ptr(), 3000, 4100, axis, _lib.TRT_F32, ws.data_ptr(),
+                                          need, stream), "trt_matmax")
+                _same(y, torch.amax(x, axis))
+    assert int(ws[:65536].max().item()) == 0  # the counters are back to zero
 
 
 # ---- batched column maxima: the front end of the contraction recipes

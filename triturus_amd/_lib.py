@@ -88,6 +88,7 @@ SIGNATURES = {
     "trt_mm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "trt_vadd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "trt_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
+    "trt_max_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
     "trt_lt2exp_kernel_name": (c_int, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_char_p, c_size_t]),
     "trt_lm2exp_kernel_name": (c_int, [c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_char_p, c_size_t]),
 }

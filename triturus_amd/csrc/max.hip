@@ -1101,6 +1101,20 @@ __global__ __launch_bounds__(256) void copy16_kernel(const trt::uintx4 *__restri
         if (base + u * 256 < nvec) __builtin_nontemporal_store(v[u], &dst[base + u * 256]);
 }
 
+// Arrival counters of a max workspace back to zero, by a kernel (a caller that prepares its
+// workspaces while a stream is being captured into a graph needs no memset node).
+__global__ __launch_bounds__(256) void zero_tickets_kernel(unsigned *ticket) {
+    for (unsigned i = threadIdx.x; i < trt::kTicketBytes / sizeof(unsigned); i += 256) ticket[i] = 0u;
+}
+
+extern "C" int trt_max_workspace_init(void *workspace, size_t workspace_bytes, void *stream) {
+    if (!workspace || workspace_bytes < trt::kTicketBytes) return TRT_E_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(workspace) & 3) return TRT_E_LAYOUT;
+    hipLaunchKernelGGL(zero_tickets_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<unsigned *>(workspace));
+    return (int)hipGetLastError();
+}
+
 extern "C" int trt_copy_bytes(const void *src, void *dst, size_t nbytes, void *stream) {
     if (!src || !dst || nbytes == 0 || (nbytes & 15)) return TRT_E_INVALID;
     if ((reinterpret_cast<uintptr_t>(src) | reinterpret_cast<uintptr_t>(dst)) & 15) return TRT_E_LAYOUT;
