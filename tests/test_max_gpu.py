@@ -110,6 +110,23 @@ def test_vmax_special_values(dev):
     assert v.item() == 0.0 and i.item() == 0
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("n", [3, 9, 41, 75, 8875, 70001, (1 << 20) + 3, 3790651])
+def test_vmax_of_nothing_but_minus_infinity(dev, dtype, n):
+    """Every element -inf: index 0 whatever the length -- also when the vector ends in elements
+    that do not fill a 16-byte piece, or starts off a 16-byte boundary -- and a finite value or a
+    later -inf must not disturb the first-occurrence rule."""
+    ninf = float("-inf")
+    for off in (0, 1, 3):
+        base = torch.full((n + off,), ninf, dtype=dtype)
+        v, i = vmax(base.to(dev)[off:])
+        assert (v.item(), i.item()) == (ninf, 0), (n, off)
+        base[off + n - 1] = -3.0  # the only finite value: last element (in the scalar tail for most n)
+        v, i = vmax(base.to(dev)[off:])
+        assert (v.item(), i.item()) == (-3.0, n - 1), (n, off)
+        assert vamax(base.to(dev)[off:]).item() == -3.0
+
+
 @pytest.mark.parametrize("dtype", [torch.float64, torch.float16, torch.bfloat16])
 def test_other_float_dtypes(dev, dtype):
     x = torch.randn(50001).to(dtype)

@@ -330,6 +330,10 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
                 }
             }
         }
+    } else if (k > 0) {
+        // ---- no piece rose above -inf: every element of this thread's share is -inf, and the
+        // first of them is its candidate (a later tail element must not win the tie)
+        bidx = head + piece_index(0) * VN;
     }
     // elements before the first and after the last whole 16-byte piece
     if (blockIdx.x == 0 && tid < head) feed(E::up(x[tid]), tid);
