@@ -192,7 +192,8 @@ int trt_lm2exp_bf16_variant_count(void);
  * Workspaces of the max reductions (trt_matmax, trt_vmax) start with arrival counters: the
  * workgroup that finishes last combines the partial results of all of them, so a reduction is
  * one launch.  The first TRT_MAX_TICKET_BYTES of such a workspace must be ZERO before the first
- * call that uses it (one hipMemset when it is allocated); every call leaves them zero, so a
+ * call that uses it (one hipMemset when it is allocated, or trt_max_workspace_init); every call
+ * leaves them zero, so a
  * workspace can be reused from call to call -- by one stream at a time: calls that overlap in
  * time need workspaces of their own.
  */
@@ -217,8 +218,7 @@ size_t trt_matmax_workspace_bytes(int64_t m, int64_t n, int axis, int dtype);
  * (element strides sb, trailing stride 1); m is R x K, contiguous.  A NaN in a
  * column gives NaN, like torch.amax(b, dim=1).  With clamp != 0 the maxima are
  * clamped to +-1e38: exactly the shift that the contraction recipes subtract
- * (baselines/lm2exp.py:11-12, baselines/lt2exp.py:15-19) and that the two-launch
- * lm2exp variant consumes.  The reference has the 2-D reduction only
+ * (baselines/lm2exp.py:11-12, baselines/lt2exp.py:15-19).  The reference has the 2-D reduction only
  * (`matmax`, triturus/max.py:125-188); this is its batched form along axis 1.
  * workspace: trt_colmax_batched_workspace_bytes(R, J, K) bytes (0 unless few
  * columns stand under a long reduced axis, which is then cut over J).
