@@ -193,9 +193,8 @@ int trt_lm2exp_bf16_variant_count(void);
  * workgroup that finishes last combines the partial results of all of them, so a reduction is
  * one launch.  The first TRT_MAX_TICKET_BYTES of such a workspace must be ZERO before the first
  * call that uses it (one hipMemset when it is allocated, or trt_max_workspace_init); every call
- * leaves them zero, so a
- * workspace can be reused from call to call -- by one stream at a time: calls that overlap in
- * time need workspaces of their own.
+ * leaves them zero, so a workspace can be reused from call to call -- by one stream at a time:
+ * calls that overlap in time need workspaces of their own.
  */
 #define TRT_MAX_TICKET_BYTES 65536
 /* Zeroes the arrival counters of a max workspace with a small kernel on `stream` (in place of a
