@@ -268,6 +268,53 @@ def test_c_abi_with_a_workspace_prepared_by_the_library(dev):
     assert int(ws[:65536].max().item()) == 0  # the counters are back to zero
 
 
+@pytest.mark.parametrize("seed", range(8))
+def test_random_vectors_and_matrices(dev, seed):
+    """A bracketed version of a one-off randomized scan (which found the all -inf tail case
+    above): lengths and shapes drawn log-uniformly, four dtypes, views off a 16-byte boundary,
+    ties, NaN, +inf and vectors of nothing but -inf, against torch.max / torch.amax."""
+    import random
+
+    rng = random.Random(1000 + seed)
+    dtypes = [torch.float32, torch.float64, torch.float16, torch.bfloat16]
+
+    def logu(lo, hi):
+        return int(round(2 ** rng.uniform(math.log2(lo), math.log2(hi))))
+
+    for case in range(40):
+        dt = rng.choice(dtypes)
+        g = torch.Generator().manual_seed(rng.randrange(1 << 30))
+        wide = (lambda t: t.float()) if dt in (torch.float16, torch.bfloat16) else (lambda t: t)
+        if case % 2 == 0:
+            n, off = logu(1, 1 << 21), rng.choice([0, 0, 1, 2, 3, 5])
+            x = torch.randn(n + off, generator=g)
+            if rng.random() < 0.3:
+                x = torch.round(x * 2) / 2  # many ties
+            if rng.random() < 0.2 and n > 2:
+                x[rng.randrange(n + off)] = float("nan")
+            if rng.random() < 0.15:
+                x[:] = float("-inf")
+            x = x.to(dt)
+            gv, gi = torch.max(wide(x[off:]), 0)
+            v, i = vmax(x.to(dev)[off:])
+            assert i.item() == gi.item(), (dt, n, off)
+            _same(v.float(), gv.float())
+            _same(vamax(x.to(dev)[off:]).float(), gv.float())
+        else:
+            m, n = logu(1, 6000), logu(1, 6000)
+            off = rng.choice([0, 0, 0, 1, 4])
+            base = torch.randn(m * n + off, generator=g)
+            if rng.random() < 0.3 and m * n > 2:
+                base[rng.randrange(m * n + off)] = float("nan")
+            if rng.random() < 0.2:
+                base[rng.randrange(m * n + off)] = float("inf")
+            base = base.to(dt)
+            x = base[off:].view(m, n)
+            xg = base.to(dev)[off:].view(m, n)
+            for axis in (0, 1):
+                _same(matmax(xg, axis), torch.amax(wide(x), axis).to(dt))
+
+
 # ---- batched column maxima: the front end of the contraction recipes
 @pytest.mark.parametrize("shape", [(1, 1, 1), (3, 7, 5), (4, 64, 256), (2, 300, 1000), (64, 64, 4096), (5, 33, 257),
                                    (1, 4096, 300), (2, 1000, 70), (16, 512, 512), (1, 129, 3),  # these four are cut over J
