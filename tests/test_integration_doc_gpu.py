@@ -29,6 +29,12 @@ def test_documented_ctypes_stubs_run(dev):
     c = torch.empty(3, 50, 90, device=dev)
     ns["_launch_lm2exp"](a, b, c)
     assert torch.equal(c, lm2exp(a, b))
+    # a transposed a goes through the stub as it is (the library reads it in place)
+    at = a.transpose(1, 2).contiguous().transpose(1, 2)
+    assert at.stride(2) != 1
+    ct = torch.empty(3, 50, 90, device=dev)
+    ns["_launch_lm2exp"](at, b, ct)
+    assert torch.equal(ct, lm2exp(at, b)) and torch.allclose(ct, c, rtol=1e-5, atol=1e-6)
     # a shape that splits over J (needs the workspace the stub allocates)
     a2 = torch.rand(1, 128, 4096, generator=g).to(dev)
     b2 = torch.randn(1, 4096, 128, generator=g).to(dev)
@@ -53,3 +59,13 @@ def test_documented_ctypes_stubs_run(dev):
         exec(compile(blocks[1], "INTEGRATION.md:lt2exp", "exec"), scope)
         assert scope["status"] == 0
         assert torch.equal(c3, lt2exp(w, a3, b3, mode=mode))
+    # every other element of a wider w: the flattened view keeps the stride, the library reads it in place
+    wide = torch.zeros(batch, m, j, 2 * k, device=dev)
+    wide[..., ::2] = w
+    ws_ = wide[..., ::2]
+    c4 = torch.empty(batch, m, n, device=dev)
+    scope = dict(ns, w=ws_.view(batch, m, -1), a=a3, b=b3, c=c4, batch=batch, m=m, j=j, k=k, n=n, mode="unsplit")
+    assert scope["w"].stride(2) == 2
+    exec(compile(blocks[1], "INTEGRATION.md:lt2exp", "exec"), scope)
+    assert scope["status"] == 0
+    assert torch.equal(c4, lt2exp(w, a3, b3, mode="unsplit"))
