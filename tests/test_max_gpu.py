@@ -59,6 +59,45 @@ def test_vmax_sizes(dev, n):
     assert vamax(x.to(dev)).item() == rv
 
 
+@pytest.mark.parametrize("n,offset", [((1 << 23) + 5, 0), (9_000_001, 3), (1 << 24, 0), (20_000_000, 1)])
+def test_vmax_of_vectors_too_large_for_the_cache(dev, n, offset):
+    """Operands of 32 MiB and more are swept with read-once loads, each workgroup over a run of
+    consecutive blocks: ties (lowest index wins), a NaN (first one wins) and all -inf are placed
+    across the seams of those runs."""
+    g = torch.Generator().manual_seed(n)
+    base = torch.round(torch.randn(n + offset, generator=g) * 4) / 4  # many ties
+    x = base[offset:]
+    xg = base.to(dev)[offset:]
+    gv, gi = torch.max(x, 0)
+    v, i = vmax(xg)
+    assert (v.item(), i.item()) == (gv.item(), gi.item())
+    assert vamax(xg).item() == gv.item()
+    # one maximum, planted at the seams of the workgroups' runs and at both ends
+    top = gv.item() + 1.0
+    for pos in (0, 1, 2047 * 4, 2048 * 4, n // 512, n // 512 + 1, n // 2 - 1, n // 2, n - 2049 * 4, n - 2, n - 1):
+        y = xg.clone()
+        y[pos] = top
+        v, i = vmax(y)
+        assert (v.item(), i.item()) == (top, pos), pos
+    # two equal maxima in different runs: the first is reported
+    y = xg.clone()
+    y[n - 3] = top
+    y[n // 3] = top
+    v, i = vmax(y)
+    assert (v.item(), i.item()) == (top, n // 3)
+    # a NaN wins, the first of two is reported
+    y = xg.clone()
+    y[n - 7] = float("nan")
+    y[n // 5] = float("nan")
+    v, i = vmax(y)
+    assert math.isnan(v.item()) and i.item() == n // 5
+    assert math.isnan(vamax(y).item())
+    # nothing but -inf: index 0
+    y = torch.full_like(xg, float("-inf"))
+    v, i = vmax(y)
+    assert (v.item(), i.item()) == (float("-inf"), 0)
+
+
 @pytest.mark.parametrize("offset", [1, 2, 3, 5])
 def test_vmax_unaligned_views(dev, offset):
     base = torch.randn(5000)
@@ -235,6 +274,35 @@ def test_runs_on_the_current_stream_without_synchronising(dev):
     s.synchronize()
     assert (v.item(), i.item()) == tuple(t.item() for t in torch.max(x, 0))
     _same(y, torch.amax(x.view(1024, 1024), 1))
+
+
+def test_a_captured_graph_survives_the_growth_of_its_workspace(dev):
+    """A graph captured on a stream launches kernels that count in the workspace that was current
+    for the stream at capture time.  A later call on that stream that needs a larger workspace
+    must not hand the old one back to the allocator while the graph can still be replayed."""
+    x = torch.randn(1 << 21)
+    xg = x.to(dev)
+    want = tuple(t.item() for t in torch.max(x, 0))
+    s = torch.cuda.Stream(device=dev)
+    s.wait_stream(torch.cuda.current_stream(dev))
+    with torch.cuda.stream(s):
+        vmax(xg)  # the stream's first workspace: the small one of vmax
+    s.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        v, i = vmax(xg)
+    wide = torch.randn(4096, 8192, device=dev)
+    with torch.cuda.stream(s):
+        y = matmax(wide, 0)  # partial rows of 32 splits: a larger workspace replaces the first
+        fill = [torch.full((1 << 14,), float(k), device=dev) for k in range(64)]  # would land in a freed block
+    s.synchronize()
+    _same(y, torch.amax(wide, 0).cpu())
+    for _ in range(3):
+        g.replay()
+        torch.cuda.synchronize()
+        assert (v.item(), i.item()) == want
+    for k, f in enumerate(fill):
+        assert torch.all(f == float(k))
 
 
 def test_c_abi_with_a_workspace_prepared_by_the_library(dev):

@@ -9,6 +9,8 @@
 //
 // Replaces: _ker_vamax / _ker_vmax / _ker_matmax, triturus/max.py:8-32,62-93,125-168.
 
+#include <type_traits>
+
 #include "common.hpp"
 
 #include <hip/hip_fp16.h>
@@ -203,6 +205,39 @@ __device__ __forceinline__ unsigned take_ticket_wave(unsigned *ticket) {
     return t;
 }
 
+// Workgroups go to the 8 dies (each with an L2 of its own) round-robin: logical position of a
+// workgroup such that each die owns a run of consecutive positions.  A column reduction hands
+// each die whole row splits -- all column blocks of them -- and not one column block of every
+// split (rows a power of two apart map to the same few channels of a die's L2: measured 14.6 us
+// against 18.2 us on a 4096 x 4096 fp32 matrix); a sweep of a vector gives each die one
+// contiguous eighth.
+constexpr int kDies = 8;
+__device__ __forceinline__ int64_t die_major(int64_t block, int64_t total) {
+    return (total % kDies == 0) ? (block % kDies) * (total / kDies) + block / kDies : block;
+}
+
+// One 16-byte piece.  ONCE: a non-temporal load, for operands too large to be found in L2 by a
+// later call (kStreamBytes): the sweep of a 64 MiB operand then runs at 7.0-7.5 TB/s where
+// ordinary loads of the same pattern reach 6.1, provided the engine clock is up (at the few
+// hundred MHz of a GPU that has just been idle the two are level).  Operands that fit L2 keep
+// ordinary loads: read again by the next call, they are served from L2 (16 MiB: 5.6 us against
+// 6.8 with non-temporal loads).
+constexpr int64_t kStreamBytes = (int64_t)32 << 20;
+template <bool ONCE, class V>
+__device__ __forceinline__ V load_piece(const V *p) {
+    static_assert(sizeof(V) == 16, "a 16-byte piece");
+    if constexpr (ONCE) {
+        const uintx4 bits = __builtin_nontemporal_load(reinterpret_cast<const uintx4 *>(p));
+        V v;
+        __builtin_memcpy(&v, &bits, 16);
+        return v;
+    } else {
+        return *p;
+    }
+}
+using OnceT = std::true_type;
+using AgainT = std::false_type;
+
 // Max and first-occurrence argmax in one launch.  Every 16-byte piece costs a couple of vector
 // instructions: the maximum of its elements (NaN ignored), one unordered test per pair of elements
 // to notice NaNs, and a compare-and-select of (value, piece number) -- the position inside the
@@ -213,7 +248,7 @@ __device__ __forceinline__ unsigned take_ticket_wave(unsigned *ticket) {
 template <int DT, bool WITH_IDX, bool FINAL>
 __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     const typename Elem<DT>::T *__restrict__ x, int64_t n, int64_t head, int64_t nvec,
-    uintx4 *prec, unsigned *ticket,
+    int64_t share_q, int share_rem, int once, uintx4 *prec, unsigned *ticket,
     typename Elem<DT>::T *__restrict__ out_val, int64_t *__restrict__ out_idx) {
     using E = Elem<DT>;
     using T = typename E::T;
@@ -243,32 +278,45 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
 #pragma unroll
         for (int e = 0; e + 1 < VN; e += 2) un |= __builtin_isunordered(c[e], c[e + 1]);
     };
-    // Workgroups walk the vector in contiguous blocks of kVmaxUnroll * kVmaxThreads 16-byte
-    // pieces (block-cyclic over the grid): measured 6.3 TB/s against 4.7 TB/s for the same
-    // loads spread a whole grid apart.  Piece numbers increase with the index within a thread.
+    // The vector is cut into blocks of kVmaxUnroll * kVmaxThreads 16-byte pieces; a workgroup
+    // takes a run of consecutive blocks (share_q of them, one more for the first share_rem
+    // workgroups), and the workgroups of a die take consecutive runs, so each die streams one
+    // contiguous eighth of the vector.  Measured on 64 MiB: 9.6 us for the bare sweep against
+    // 10.5 with the blocks dealt round-robin over the grid (and 11.1 with ordinary loads).
+    // Piece numbers increase with the index within a thread.
+    const int64_t logical = die_major(blockIdx.x, gridDim.x);
+    const int64_t first_block = logical * share_q + (logical < share_rem ? logical : share_rem);
+    const int64_t end_block = first_block + share_q + (logical < share_rem ? 1 : 0);
     unsigned k = 0;
-    for (int64_t blk = blockIdx.x; blk < full_blocks; blk += gridDim.x) {
-        const int64_t v = blk * kBlock + tid;
-        V buf[kVmaxUnroll];
-#pragma unroll
-        for (int u = 0; u < kVmaxUnroll; ++u) buf[u] = xv[v + u * kVmaxThreads];
-#pragma unroll
-        for (int u = 0; u < kVmaxUnroll; ++u) {
-            C m;
-            piece_max(buf[u], m, saw_nan);
-            const bool take = m > bv;
-            bv = take ? m : bv;
-            if (WITH_IDX) {
-                bk = take ? k + u : bk;
-#pragma unroll
-                for (int e = 0; e < VN; ++e) bpiece.e[e] = take ? buf[u].e[e] : bpiece.e[e];
+    auto sweep = [&](auto once_tag) {
+        for (int64_t blk = first_block; blk < end_block; ++blk) {
+            const int64_t v = blk * kBlock + tid;
+            V buf[kVmaxUnroll];
+    #pragma unroll
+                for (int u = 0; u < kVmaxUnroll; ++u)
+                buf[u] = load_piece<decltype(once_tag)::value>(&xv[v + u * kVmaxThreads]);
+            // every load of the block is issued before the first piece is looked at
+            __builtin_amdgcn_sched_barrier(0);
+    #pragma unroll
+            for (int u = 0; u < kVmaxUnroll; ++u) {
+                C m;
+                piece_max(buf[u], m, saw_nan);
+                const bool take = m > bv;
+                bv = take ? m : bv;
+                if (WITH_IDX) {
+                    bk = take ? k + u : bk;
+    #pragma unroll
+                    for (int e = 0; e < VN; ++e) bpiece.e[e] = take ? buf[u].e[e] : bpiece.e[e];
+                }
             }
+            k += kVmaxUnroll;
         }
-        k += kVmaxUnroll;
-    }
+    };
+    if (once) sweep(OnceT{});
+    else sweep(AgainT{});
     const unsigned in_full = k;  // pieces of whole blocks come first in the visiting order
-    // the last, partial block goes to the workgroup whose turn it would be
-    const bool has_tail_block = (int64_t)blockIdx.x == full_blocks % gridDim.x;
+    // the last, partial block goes to the workgroup of the last run
+    const bool has_tail_block = logical == (int64_t)gridDim.x - 1;
     if (has_tail_block) {
         for (int64_t v = full_blocks * kBlock + tid; v < nvec; v += kVmaxThreads) {
             C m;
@@ -287,7 +335,7 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     // piece number -> absolute piece index (the inverse of the two loops above)
     auto piece_index = [&](unsigned kk) -> int64_t {
         if (kk < in_full)
-            return ((int64_t)blockIdx.x + (int64_t)(kk / kVmaxUnroll) * gridDim.x) * kBlock + tid +
+            return (first_block + (int64_t)(kk / kVmaxUnroll)) * kBlock + tid +
                    (int64_t)(kk % kVmaxUnroll) * kVmaxThreads;
         return full_blocks * kBlock + tid + (int64_t)(kk - in_full) * kVmaxThreads;
     };
@@ -302,7 +350,7 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     };
     if (__builtin_amdgcn_ballot_w64(saw_nan) != 0) {
         // ---- a NaN somewhere in this wavefront's share: element by element, exact rule
-        for (int64_t blk = blockIdx.x; blk < full_blocks; blk += gridDim.x)
+        for (int64_t blk = first_block; blk < end_block; ++blk)
             for (int u = 0; u < kVmaxUnroll; ++u) {
                 const int64_t v = blk * kBlock + tid + u * kVmaxThreads;
                 const V b = xv[v];
@@ -480,25 +528,29 @@ static int vmax_launch(const void *x, int64_t n, void *out_val, int64_t *out_idx
     int64_t head = (int64_t)(((16 - (addr & 15)) & 15) / sizeof(T));
     if (head > n) head = n;
     const int64_t nvec = (n - head) / VN;
+    const int64_t full_blocks = nvec / ((int64_t)kVmaxUnroll * kVmaxThreads);  // whole blocks of pieces
     T *ov = static_cast<T *>(out_val);
     if (vmax_single_block(n, DT)) {
         if (out_idx)
             hipLaunchKernelGGL((vmax_kernel<DT, true, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                               nvec, (uintx4 *)nullptr, (unsigned *)nullptr, ov, out_idx);
+                               nvec, full_blocks, 0, 0, (uintx4 *)nullptr, (unsigned *)nullptr, ov, out_idx);
         else
             hipLaunchKernelGGL((vmax_kernel<DT, false, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                               nvec, (uintx4 *)nullptr, (unsigned *)nullptr, ov, out_idx);
+                               nvec, full_blocks, 0, 0, (uintx4 *)nullptr, (unsigned *)nullptr, ov, out_idx);
         return (int)hipGetLastError();
     }
     const int blocks = vmax_blocks(nvec);
+    const int64_t share_q = full_blocks / blocks;
+    const int share_rem = (int)(full_blocks % blocks);
+    const int once = n * (int64_t)sizeof(T) >= kStreamBytes;
     unsigned *ticket = static_cast<unsigned *>(ws);
     uintx4 *prec = reinterpret_cast<uintx4 *>(static_cast<char *>(ws) + kTicketBytes);
     if (out_idx)
         hipLaunchKernelGGL((vmax_kernel<DT, true, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                           nvec, prec, ticket, ov, out_idx);
+                           nvec, share_q, share_rem, once, prec, ticket, ov, out_idx);
     else
         hipLaunchKernelGGL((vmax_kernel<DT, false, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                           nvec, prec, ticket, ov, out_idx);
+                           nvec, share_q, share_rem, once, prec, ticket, ov, out_idx);
     return (int)hipGetLastError();
 }
 
@@ -511,7 +563,7 @@ constexpr int kMatWaves = kMatThreads / kWave;
 template <int DT, bool VEC>
 __global__ __launch_bounds__(kMatThreads) void rowmax_kernel(
     const typename Elem<DT>::T *__restrict__ x, int64_t ld, int64_t m, int64_t n, int64_t chunk,
-    int64_t splits, typename Elem<DT>::T *__restrict__ y, int64_t ldy) {
+    int64_t splits, int once, typename Elem<DT>::T *__restrict__ y, int64_t ldy) {
     using E = Elem<DT>;
     using T = typename E::T;
     using C = typename E::C;
@@ -531,16 +583,22 @@ __global__ __launch_bounds__(kMatThreads) void rowmax_kernel(
         const int64_t nv = (c1 - c0) / VN;
         const V *xv = reinterpret_cast<const V *>(xr + c0);
         int64_t v = lane;
-        for (; v + 3 * kWave < nv; v += 4 * kWave) {
-            V b0 = xv[v], b1 = xv[v + kWave], b2 = xv[v + 2 * kWave], b3 = xv[v + 3 * kWave];
+        auto sweep = [&](auto once_tag) {
+            constexpr bool ONCE = decltype(once_tag)::value;
+            for (; v + 3 * kWave < nv; v += 4 * kWave) {
+                V b0 = load_piece<ONCE>(&xv[v]), b1 = load_piece<ONCE>(&xv[v + kWave]),
+                  b2 = load_piece<ONCE>(&xv[v + 2 * kWave]), b3 = load_piece<ONCE>(&xv[v + 3 * kWave]);
 #pragma unroll
-            for (int e = 0; e < VN; ++e) {
-                best = vmax_nan(best, E::up(b0.e[e]));
-                best = vmax_nan(best, E::up(b1.e[e]));
-                best = vmax_nan(best, E::up(b2.e[e]));
-                best = vmax_nan(best, E::up(b3.e[e]));
+                for (int e = 0; e < VN; ++e) {
+                    best = vmax_nan(best, E::up(b0.e[e]));
+                    best = vmax_nan(best, E::up(b1.e[e]));
+                    best = vmax_nan(best, E::up(b2.e[e]));
+                    best = vmax_nan(best, E::up(b3.e[e]));
+                }
             }
-        }
+        };
+        if (once) sweep(OnceT{});
+        else sweep(AgainT{});
         for (; v < nv; v += kWave) {
             V b0 = xv[v];
 #pragma unroll
@@ -559,7 +617,7 @@ __global__ __launch_bounds__(kMatThreads) void rowmax_kernel(
 // than four wavefronts on four different rows (measured on 16384^2 fp32: 174 us against 189 us).
 template <int DT>
 __global__ __launch_bounds__(kMatThreads) void rowmax_wide_kernel(const typename Elem<DT>::T *__restrict__ x,
-                                                                  int64_t ld, int64_t n,
+                                                                  int64_t ld, int64_t n, int once,
                                                                   typename Elem<DT>::T *__restrict__ y) {
     using E = Elem<DT>;
     using T = typename E::T;
@@ -567,20 +625,25 @@ __global__ __launch_bounds__(kMatThreads) void rowmax_wide_kernel(const typename
     using V = Vec16<T>;
     constexpr int VN = V::N;
     const int tid = threadIdx.x;
-    const T *xr = x + (int64_t)blockIdx.x * ld;
+    const int64_t row = die_major(blockIdx.x, gridDim.x);  // each die streams a run of consecutive rows
+    const T *xr = x + row * ld;
     const V *xv = reinterpret_cast<const V *>(xr);
     const int64_t nv = n / VN;
     C best = neg_inf<C>();
     int64_t v = tid;
-    for (; v + 3 * kMatThreads < nv; v += 4 * kMatThreads) {
-        V b[4];
+    auto sweep = [&](auto once_tag) {
+        for (; v + 3 * kMatThreads < nv; v += 4 * kMatThreads) {
+            V b[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) b[u] = xv[v + u * kMatThreads];
+            for (int u = 0; u < 4; ++u) b[u] = load_piece<decltype(once_tag)::value>(&xv[v + u * kMatThreads]);
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+            for (int u = 0; u < 4; ++u)
 #pragma unroll
-            for (int e = 0; e < VN; ++e) best = vmax_nan(best, E::up(b[u].e[e]));
-    }
+                for (int e = 0; e < VN; ++e) best = vmax_nan(best, E::up(b[u].e[e]));
+        }
+    };
+    if (once) sweep(OnceT{});
+    else sweep(AgainT{});
     for (; v < nv; v += kMatThreads) {
         V b0 = xv[v];
 #pragma unroll
@@ -594,17 +657,8 @@ __global__ __launch_bounds__(kMatThreads) void rowmax_wide_kernel(const typename
     if (tid == 0) {
 #pragma unroll
         for (int w = 1; w < kMatWaves; ++w) best = vmax_nan(best, part[w]);
-        y[blockIdx.x] = E::down(best);
+        y[row] = E::down(best);
     }
-}
-
-// Workgroups go to the 8 dies (each with an L2 of its own) round-robin, and rows a power of two
-// apart map to the same few channels of a die's L2.  A column reduction therefore hands each
-// die whole row splits -- all column blocks of them -- and not one column block of every split:
-// measured 14.6 us against 18.2 us on a 4096 x 4096 fp32 matrix.
-constexpr int kDies = 8;
-__device__ __forceinline__ int64_t die_major(int64_t block, int64_t total) {
-    return (total % kDies == 0) ? (block % kDies) * (total / kDies) + block / kDies : block;
 }
 
 // Column maxima (reduction along the strided axis).  Each thread owns CN
@@ -685,7 +739,8 @@ constexpr int kColFusedUnroll = 8;  // 16-byte loads in flight per lane
 template <int DT, int VPL>
 __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
     const typename Elem<DT>::T *__restrict__ x, int64_t ld, int64_t m, int64_t n, int64_t rchunk,
-    int colblocks, int splits, unsigned long long *part, unsigned *ticket, typename Elem<DT>::T *__restrict__ y) {
+    int colblocks, int splits, int once, unsigned long long *part, unsigned *ticket,
+    typename Elem<DT>::T *__restrict__ y) {
     using E = Elem<DT>;
     using T = typename E::T;
     using C = typename E::C;
@@ -737,18 +792,24 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
     };
     static_assert(ROWS % 2 == 0, "rows are folded in pairs");
     int64_t r = r0 + wave;
-    for (; r + (ROWS - 1) * kMatWaves < r1; r += ROWS * kMatWaves) {
-        V b[ROWS][VPL];
+    auto sweep = [&](auto once_tag) {
+        for (; r + (ROWS - 1) * kMatWaves < r1; r += ROWS * kMatWaves) {
+            V b[ROWS][VPL];
 #pragma unroll
-        for (int u = 0; u < ROWS; ++u)
+            for (int u = 0; u < ROWS; ++u)
 #pragma unroll
-            for (int p = 0; p < VPL; ++p) b[u][p] = *reinterpret_cast<const V *>(xc + (r + u * kMatWaves) * ld + poff[p]);
-        __builtin_amdgcn_sched_barrier(0);  // all loads of the step are under way before the first is looked at
+                for (int p = 0; p < VPL; ++p)
+                    b[u][p] = load_piece<decltype(once_tag)::value>(
+                        reinterpret_cast<const V *>(xc + (r + u * kMatWaves) * ld + poff[p]));
+            __builtin_amdgcn_sched_barrier(0);  // all loads of the step are under way before the first is looked at
 #pragma unroll
-        for (int u = 0; u < ROWS; u += 2)
+            for (int u = 0; u < ROWS; u += 2)
 #pragma unroll
-            for (int p = 0; p < VPL; ++p) fold2(b[u][p], b[u + 1][p], p);
-    }
+                for (int p = 0; p < VPL; ++p) fold2(b[u][p], b[u + 1][p], p);
+        }
+    };
+    if (once) sweep(OnceT{});
+    else sweep(AgainT{});
     for (; r < r1; r += kMatWaves) {
 #pragma unroll
         for (int p = 0; p < VPL; ++p) fold(*reinterpret_cast<const V *>(xc + r * ld + poff[p]), p);
@@ -919,14 +980,14 @@ static bool vec_ok(const void *p, int64_t ld) {
 
 template <int DT>
 static void rowmax_launch(const typename Elem<DT>::T *x, int64_t ld, int64_t m, int64_t n, MatPlan p,
-                          typename Elem<DT>::T *y, int64_t ldy, hipStream_t stream) {
+                          typename Elem<DT>::T *y, int64_t ldy, hipStream_t stream, int once = 0) {
     const int64_t blocks = p.splits * ceil_div(m, (int64_t)kMatWaves);
     if (vec_ok<DT>(x, ld))
         hipLaunchKernelGGL((rowmax_kernel<DT, true>), dim3((unsigned)blocks), dim3(kMatThreads), 0, stream,
-                           x, ld, m, n, p.chunk, p.splits, y, ldy);
+                           x, ld, m, n, p.chunk, p.splits, once, y, ldy);
     else
         hipLaunchKernelGGL((rowmax_kernel<DT, false>), dim3((unsigned)blocks), dim3(kMatThreads), 0, stream,
-                           x, ld, m, n, p.chunk, p.splits, y, ldy);
+                           x, ld, m, n, p.chunk, p.splits, once, y, ldy);
 }
 
 template <int DT>
@@ -976,14 +1037,16 @@ static int matmax_launch(const void *xv, void *yv, int64_t m, int64_t n, int axi
     T *part = reinterpret_cast<T *>(static_cast<char *>(ws) + kTicketBytes);
     if (matmax_ws<DT>(m, n, axis) > ws_bytes) return TRT_E_WORKSPACE;
     if (matmax_ws<DT>(m, n, axis) > 0 && ws == nullptr) return TRT_E_WORKSPACE;
+    const int once = m * n * (int64_t)sizeof(T) >= kStreamBytes;  // too large to be found in L2 again
     if (axis == 1 && rowmax_wide<DT>(x, m, n)) {
-        hipLaunchKernelGGL((rowmax_wide_kernel<DT>), dim3((unsigned)m), dim3(kMatThreads), 0, stream, x, n, n, y);
+        hipLaunchKernelGGL((rowmax_wide_kernel<DT>), dim3((unsigned)m), dim3(kMatThreads), 0, stream, x, n, n, once,
+                           y);
     } else if (axis == 1) {
         MatPlan p = rowmax_plan(m, n, VN);
         if (p.splits == 1) {
-            rowmax_launch<DT>(x, n, m, n, p, y, 1, stream);
+            rowmax_launch<DT>(x, n, m, n, p, y, 1, stream, once);
         } else {
-            rowmax_launch<DT>(x, n, m, n, p, part, p.splits, stream);
+            rowmax_launch<DT>(x, n, m, n, p, part, p.splits, stream, once);
             MatPlan p2{1, p.splits};
             rowmax_launch<DT>(part, p.splits, m, p.splits, p2, y, 1, stream);
         }
@@ -994,11 +1057,11 @@ static int matmax_launch(const void *xv, void *yv, int64_t m, int64_t n, int axi
         const bool fused = vec && (reinterpret_cast<uintptr_t>(y) & 15) == 0;  // y is written in 16-byte pieces
         if (fused && pf.vpl == 2) {
             hipLaunchKernelGGL((colmax_fused_kernel<DT, 2>), dim3((unsigned)(pf.colblocks * pf.splits)),
-                               dim3(kMatThreads), 0, stream, x, n, m, n, pf.chunk, pf.colblocks, pf.splits,
+                               dim3(kMatThreads), 0, stream, x, n, m, n, pf.chunk, pf.colblocks, pf.splits, once,
                                reinterpret_cast<unsigned long long *>(part), static_cast<unsigned *>(ws), y);
         } else if (fused && pf.vpl == 1) {
             hipLaunchKernelGGL((colmax_fused_kernel<DT, 1>), dim3((unsigned)(pf.colblocks * pf.splits)),
-                               dim3(kMatThreads), 0, stream, x, n, m, n, pf.chunk, pf.colblocks, pf.splits,
+                               dim3(kMatThreads), 0, stream, x, n, m, n, pf.chunk, pf.colblocks, pf.splits, once,
                                reinterpret_cast<unsigned long long *>(part), static_cast<unsigned *>(ws), y);
         } else if (p.splits == 1) {
             colmax_launch<DT>(x, n, m, n, vec, p, y, n, stream);

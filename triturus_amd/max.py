@@ -21,12 +21,18 @@ _ws_bytes: dict = {}  # (op, shape..., dtype code) -> workspace bytes, as report
 # results), so the workspace is allocated once per stream, zero-filled, and kept: calls on one
 # stream run one after the other, calls on different streams never share one.
 _workspaces: dict = {}
+# Workspaces that a larger one has replaced.  They are kept for the life of the process: a HIP
+# graph captured while one of them was current still launches kernels that count in it.
+_retired: list = []
 
 
 def _workspace(dev: torch.device, nbytes: int):
     key = (dev.index, _lib.raw_stream(dev))
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
+        if ws is not None:
+            _retired.append(ws)
+            nbytes = max(nbytes, 2 * ws.numel())  # grow geometrically: what is retired stays below what is live
         ws = _workspaces[key] = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=dev)
     return ws
 
