@@ -138,8 +138,8 @@ def graph_time(fn, calls: int = 20, reps: int = 20, prewarm_ms: float = 0.0, bot
     up, and the streaming kernels follow it.  `both`: returns (seconds after the prewarm,
     seconds of the same measurement taken before it)."""
     # (warm-up on the launch stream itself: once a second stream has run kernels in the process,
-    # every short kernel on the first pays 1.5-2 us more per launch, which is not what a caller
-    # with one stream sees)
+    # vmax's sweep runs 2 us slower for the rest of it, which is not what a caller with one
+    # stream sees)
     for _ in range(3):
         fn()
     torch.cuda.synchronize()

@@ -292,12 +292,12 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
         for (int64_t blk = first_block; blk < end_block; ++blk) {
             const int64_t v = blk * kBlock + tid;
             V buf[kVmaxUnroll];
-    #pragma unroll
-                for (int u = 0; u < kVmaxUnroll; ++u)
+#pragma unroll
+            for (int u = 0; u < kVmaxUnroll; ++u)
                 buf[u] = load_piece<decltype(once_tag)::value>(&xv[v + u * kVmaxThreads]);
             // every load of the block is issued before the first piece is looked at
             __builtin_amdgcn_sched_barrier(0);
-    #pragma unroll
+#pragma unroll
             for (int u = 0; u < kVmaxUnroll; ++u) {
                 C m;
                 piece_max(buf[u], m, saw_nan);
@@ -305,7 +305,7 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
                 bv = take ? m : bv;
                 if (WITH_IDX) {
                     bk = take ? k + u : bk;
-    #pragma unroll
+#pragma unroll
                     for (int e = 0; e < VN; ++e) bpiece.e[e] = take ? buf[u].e[e] : bpiece.e[e];
                 }
             }
