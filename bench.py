@@ -130,23 +130,32 @@ def do_bench(fn, *, warmup_ms=150.0, rep_ms=1000.0, flush_bytes=512 << 20):
     return {"median_ms": q(0.5), "q10_ms": q(0.1), "q90_ms": q(0.9), "reps": n_rep}
 
 
-def graph_time(fn, calls: int = 20, reps: int = 20, prewarm_ms: float = 0.0, both: bool = False):
+def graph_time(fn, calls: int = 20, reps: int = 20, prewarm_ms: float = 0.0, both: bool = False, operands=None):
     """Average seconds per call of a short kernel: `calls` launches captured in one HIP
     graph (no host launch gaps), replayed `reps` times between HIP events.  With `prewarm_ms`
     the graph is first replayed, untimed, for that long (as `timed_region` does): after an
     idle or host-bound phase the engine clock takes some hundred milliseconds of load to come
     up, and the streaming kernels follow it.  `both`: returns (seconds after the prewarm,
-    seconds of the same measurement taken before it)."""
+    seconds of the same measurement taken before it).  With `operands` the calls of the graph
+    are fn(operands[0]), fn(operands[1]), ... in turn: enough copies of an operand that none of
+    them is still in a cache when its turn comes again."""
+    if operands is not None:
+        n_ops = len(operands)
+        calls = max(calls, n_ops) // n_ops * n_ops
+        turn = iter(range(1 << 60))
+        call = lambda: fn(operands[next(turn) % n_ops])
+    else:
+        call = fn
     # (warm-up on the launch stream itself: once a second stream has run kernels in the process,
     # vmax's sweep runs 2 us slower for the rest of it, which is not what a caller with one
     # stream sees)
     for _ in range(3):
-        fn()
+        fn(operands[0]) if operands is not None else fn()
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
     with torch.cuda.graph(g):
         for _ in range(calls):
-            fn()
+            call()
     g.replay()
     torch.cuda.synchronize()
 
@@ -415,21 +424,35 @@ def main() -> int:
             f"{result['c1']['hip_graph_us_per_call']:.2f} us inside a HIP graph")
 
         # ------------------------------------------------ max reductions (HBM bound)
+        # Two figures per reduction.  `us`: the same 64 MiB operand call after call, as a caller
+        # that reduces one tensor repeatedly sees it -- the operand then sits in the 256 MB
+        # memory-side cache (and, with the library's read-once loads, half of it stays in the
+        # dies' L2s from one call to the next).  `out_of_cache`: 8 copies of the operand
+        # (512 MiB) taken in turn, so that every call streams from HBM.
         x = cfg["b"].to(dev)  # 64 x 64 x 4096
         nbytes = x.numel() * 4
-        flat, mat = x.view(-1), x.view(4096, 4096)
+        copies = [x] + [x.clone() for _ in range(7)]
         mx = {"bytes": nbytes, "unit": "GB/s", "peak": PEAK_HBM_GBPS}
-        for name, fn in (("vmax", lambda: vmax(flat)), ("matmax_axis0", lambda: matmax(mat, 0)),
-                         ("matmax_axis1", lambda: matmax(mat, 1)),
-                         ("bmatmax_shift", lambda: bmatmax(x, clamp=True)),  # 64 x 64 x 4096 -> 64 x 4096: the shift m
-                         ("torch_amax_batched", lambda: torch.amax(x, 1)),
-                         ("torch_max", lambda: torch.max(flat, 0)), ("torch_amax_axis0", lambda: torch.amax(mat, 0)),
-                         ("torch_amax_axis1", lambda: torch.amax(mat, 1))):
-            sec, before = graph_time(fn, prewarm_ms=PREWARM_MS, both=True)
+        fns = (("vmax", lambda z: vmax(z.view(-1))), ("matmax_axis0", lambda z: matmax(z.view(4096, 4096), 0)),
+               ("matmax_axis1", lambda z: matmax(z.view(4096, 4096), 1)),
+               ("bmatmax_shift", lambda z: bmatmax(z, clamp=True)),  # 64 x 64 x 4096 -> 64 x 4096: the shift m
+               ("torch_amax_batched", lambda z: torch.amax(z, 1)),
+               ("torch_max", lambda z: torch.max(z.view(-1), 0)),
+               ("torch_amax_axis0", lambda z: torch.amax(z.view(4096, 4096), 0)),
+               ("torch_amax_axis1", lambda z: torch.amax(z.view(4096, 4096), 1)))
+        # (all the one-operand figures first: what a sweep over 512 MiB leaves in the caches is
+        # not what a caller that keeps reducing one tensor finds there)
+        for name, fn in fns:
+            sec, before = graph_time(lambda: fn(x), prewarm_ms=PREWARM_MS, both=True)
             mx[name] = {"us": round(sec * 1e6, 2), "achieved": round(nbytes / sec / 1e9, 1),
                         "frac": round(nbytes / sec / 1e9 / PEAK_HBM_GBPS, 4),
                         "us_before_prewarm": round(before * 1e6, 2)}
             log(f"{name}: {sec * 1e6:.2f} us, {nbytes / sec / 1e9:.0f} GB/s ({before * 1e6:.2f} us before the prewarm)")
+        for name, fn in fns:
+            cold = graph_time(fn, calls=24, prewarm_ms=PREWARM_MS / 2, operands=copies)
+            mx[name]["out_of_cache"] = {"us": round(cold * 1e6, 2), "achieved": round(nbytes / cold / 1e9, 1),
+                                        "frac": round(nbytes / cold / 1e9 / PEAK_HBM_GBPS, 4)}
+            log(f"{name}, 8 operands in turn (out of cache): {cold * 1e6:.2f} us, {nbytes / cold / 1e9:.0f} GB/s")
         mx["prewarm_ms"] = PREWARM_MS
         result["max"] = mx
 
