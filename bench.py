@@ -146,9 +146,9 @@ def graph_time(fn, calls: int = 20, reps: int = 20, prewarm_ms: float = 0.0, bot
         call = lambda: fn(operands[next(turn) % n_ops])
     else:
         call = fn
-    # (warm-up on the launch stream itself: once a second stream has run kernels in the process,
-    # vmax's sweep runs 2 us slower for the rest of it, which is not what a caller with one
-    # stream sees)
+    # (warm-up on the launch stream itself: a kernel on a second stream displaces what the
+    # read-once sweeps find in the dies' L2s from one call to the next, and vmax then runs 2 us
+    # slower for the rest of the process -- not what a caller with one stream sees)
     for _ in range(3):
         fn(operands[0]) if operands is not None else fn()
     torch.cuda.synchronize()
