@@ -413,8 +413,8 @@ constexpr int kLt2Waves = 4;
 // 32 accumulator registers, j-chunks of 32) runs at 87-89 % of the fp32 MFMA peak, the
 // 64 x 64 tiles at 81-85 %: occupancy beats operand reuse here.
 // Row tile: 32 rows unless the 64-row tile pays.  Its Khatri-Rao multiply is shared by two
-// MFMAs, worth 2-6 % per row on long contractions (I*J >= 4096) when the grid gives every CU
-// a workgroup (measured at S = 64..256 on R = 32..128, and at the large configuration);
+// MFMAs, worth 3-6 % per row on contractions of I*J >= 1024 when the tiles divide evenly over
+// the CUs (the rule is below, beside the counts it uses);
 // everywhere else the 32-row tile is as fast or faster -- twice the workgroups hide more
 // latency and balance better (over 288 random shapes: 4-30 % ahead on grids of 1-4 workgroups
 // per CU, 27 % (median) when S leaves the last 64-row tile at most half full, e.g. S = 96,
@@ -452,8 +452,16 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
     if (S > 32) {
         const int64_t last = S % 64;
         const bool same_padding = last == 0 || last > 32;
-        const int64_t n64 = R * ceil_div(S, 64) * ceil_div(K, 128);
-        if (same_padding && I * J >= 4096 && n64 >= 256) rt = 2;
+        const int64_t ct = ceil_div(K, 128);
+        const int64_t n64 = R * ceil_div(S, 64) * ct, n32 = R * ceil_div(S, 32) * ct;
+        // The busiest of the 256 CUs decides: it holds ceil(n / 256) tiles, a 64-row tile costs
+        // 1.91 32-row tiles (9 % more when it is the only workgroup on its CU).  Measured over
+        // 200 shapes with I*J = 1024..16384 and 256..2048 64-row tiles, this ranks the two
+        // tiles right every time: 64 rows are 3-6 % ahead at 448-512, 768, 1024, 2048 tiles,
+        // 26 % behind at 320-384 and 14 % behind at 640, 3-5 % behind at 256.
+        const int64_t q64 = ceil_div(n64, 256), q32 = ceil_div(n32, 256);
+        const int64_t c64 = 191 * q64 * (q64 == 1 ? 109 : 100), c32 = 100 * q32 * 100;
+        if (same_padding && I * J >= 1024 && c64 < c32) rt = 2;
         // packed rows spend more vector instructions per step (a factor of a per row of the chunk):
         // sharing them between two MFMAs pays from half a wave of workgroups on, whatever the
         // length of the contraction (measured: 6-13 % at 256..2048 tiles, level at 192, from 4 %
