@@ -642,8 +642,15 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     // that b: R=64 I=J=256 281 us against 293; with b ~ N(0, 1): 280 against 284, R=16 77
     // against 80, R=32 I=1024 K=2048 271 against 280, J = 512 531 against 533; slower with
     // fewer than two tiles per CU (R=8: +9 %), J = 192 (+1 %), or J not a multiple of 4 (+4 %).
+    // Both kernels run in steps of the busiest CU's tile count: measured at I = J = 256, K = 1024..
+    // 4096, R = 8..64 the paired tile takes 34.3 us per ceil(tiles / 256) and the 128-row tile
+    // 18.5 us per ceil(2 tiles / 256), so with 513..640, 769..896 or 1025..1152 paired tiles the
+    // online kernel is 4-22 % ahead (576 tiles: 108 against 90-95 us) and the pair is taken only
+    // where 1.85 of its steps undercut the online kernel's.
     const int64_t i256 = ceil_div(I, 256);
-    if (J >= 224 && J <= 512 && J % 4 == 0 && I >= 240 && i256 * 256 * 100 <= I * 107 && R * i256 * ct >= 512)
+    const int64_t t256 = R * i256 * ct;
+    if (J >= 224 && J <= 512 && J % 4 == 0 && I >= 240 && i256 * 256 * 100 <= I * 107 && t256 >= 512 &&
+        185 * ceil_div(t256, 256) <= 100 * ceil_div(2 * t256, 256))
         return find_pair_variant(4, 4);
     const int64_t n128 = R * ceil_div(I, 128) * ct, n64 = R * ceil_div(I, 64) * ct;
     int rt;
