@@ -595,10 +595,32 @@ static int pick_chunk(int64_t J) {
 // (measured on large grids) and only ever wins by avoiding such a tail.
 // Fitted at R=384 and R=64, I=J=64..1024, K=256: ranks the tiles as measured in 26 of 28 shapes
 // (both misses within 5 %); I = 96, 160, 192, 288 move to 96 rows (-15..23 %), I = 320 to 64.
-static int pick_tile(int64_t R, int64_t I, int64_t K, int overhead_quarters, bool wide, int max_rt = 4) {
+static int pick_tile(int64_t R, int64_t I, int64_t K, int overhead_quarters, bool wide, int max_rt = 4,
+                     int64_t chunks = 0) {
     const int64_t kFill = 256, kCuCount = 256;  // at least one workgroup per CU
     int best = 0;
     int64_t best_cost = 0;
+    const int64_t ct128 = ceil_div(K, 128);
+    // Grids of fewer than four 128-row tiles per CU (chunks > 0: the caller contracts that many
+    // chunks of 32): the busiest CU decides.  It holds q = ceil(tiles / 256) tiles of
+    // chunks * (rt + 1/4) + 3 rt blocks each (the exp work of a chunk does not shrink with the
+    // tile; prologue and epilogue do), 10 % more for a tile that is alone on its CU.  Fitted to
+    // 155 shapes (I = 128..768, J = 96..640, K = 256..2048, 200..1280 128-row tiles) timed on all
+    // four tiles: on the 137 below 1024 tiles the mean regret against the best tile is 0.3 %
+    // (the tail model below: 2.4 %, 13 shapes more than 10 % off, e.g. 576-640 tiles of 128 rows
+    // where 64 rows are 10 % ahead); from 1024 tiles on short contractions favour the 64-row tile
+    // by more than either model says, and the tail model is kept.
+    if (chunks > 0 && R * ceil_div(I, 128) * ct128 < 1024) {
+        for (int rt = max_rt; rt >= 1; --rt) {
+            const int64_t q = ceil_div(R * ceil_div(I, 32 * rt) * ct128, kCuCount);
+            const int64_t cost = q * (chunks * (4 * rt + 1) + 12 * rt) * (q == 1 ? 11 : 10);
+            if (best == 0 || cost < best_cost) {
+                best = rt;
+                best_cost = cost;
+            }
+        }
+        return best;
+    }
     auto consider = [&](int id, int64_t n, int64_t c, int res) {
         if (n < kFill) return;
         const int64_t T = ceil_div(n, kCuCount);
@@ -665,7 +687,7 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
         // at most 1.5 workgroups per CU and a long contraction: it will be cut over J, which
         // fills the chip; take the largest tile that leaves >= 128 tiles
         rt = n128 >= 128 ? 4 : (n64 >= 128 ? 2 : 1);
-    } else if ((rt = pick_tile(R, I, K, 3, true, J <= 64 ? 2 : 4)) != 0) {  // two chunks: 64 rows at most (+2..13 %)
+    } else if ((rt = pick_tile(R, I, K, 3, true, J <= 64 ? 2 : 4, ceil_div(J, 32))) != 0) {  // two chunks: 64 rows at most (+2..13 %)
         if (rt == 8) return find_variant(4, 8, kOnline);
     } else {
         rt = 1;
