@@ -455,12 +455,13 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
         const int64_t ct = ceil_div(K, 128);
         const int64_t n64 = R * ceil_div(S, 64) * ct, n32 = R * ceil_div(S, 32) * ct;
         // The busiest of the 256 CUs decides: it holds ceil(n / 256) tiles, a 64-row tile costs
-        // 1.91 32-row tiles (9 % more when it is the only workgroup on its CU).  Measured over
-        // 200 shapes with I*J = 1024..16384 and 256..2048 64-row tiles, this ranks the two
-        // tiles right every time: 64 rows are 3-6 % ahead at 448-512, 768, 1024, 2048 tiles,
-        // 26 % behind at 320-384 and 14 % behind at 640, 3-5 % behind at 256.
+        // 1.91 32-row tiles.  Measured over 200 shapes with I*J = 1024..16384 and 256..2048
+        // 64-row tiles, this ranks the two tiles right: 64 rows are 3-6 % ahead at 448-512, 768,
+        // 1024, 2048 tiles, 26 % behind at 320-384 and 14 % behind at 640.  With exactly one
+        // 64-row tile per CU the two are level (3-5 % behind launched back to back, 4-5 % ahead
+        // on inputs that are not in cache, as the reference's benchmarks time them): 64 rows.
         const int64_t q64 = ceil_div(n64, 256), q32 = ceil_div(n32, 256);
-        const int64_t c64 = 191 * q64 * (q64 == 1 ? 109 : 100), c32 = 100 * q32 * 100;
+        const int64_t c64 = 191 * q64 * (q64 == 1 ? 104 : 100), c32 = 100 * q32 * 100;
         if (same_padding && I * J >= 1024 && c64 < c32) rt = 2;
         // packed rows spend more vector instructions per step (a factor of a per row of the chunk):
         // sharing them between two MFMAs pays from half a wave of workgroups on, whatever the
