@@ -687,7 +687,11 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
         // at most 1.5 workgroups per CU and a long contraction: it will be cut over J, which
         // fills the chip; take the largest tile that leaves >= 128 tiles
         rt = n128 >= 128 ? 4 : (n64 >= 128 ? 2 : 1);
-    } else if ((rt = pick_tile(R, I, K, 3, true, J <= 64 ? 2 : 4, ceil_div(J, 32))) != 0) {  // two chunks: 64 rows at most (+2..13 %)
+    } else if ((rt = pick_tile(R, I, K, 3, true, (J <= 64 || (J <= 128 && n128 >= 1024 && n128 < 6144)) ? 2 : 4,
+                               ceil_div(J, 32))) != 0) {
+        // (two chunks: 64 rows at most (+2..13 %); three or four chunks on 4..24 128-row tiles
+        // per CU as well: timed on 47 such shapes the 64-row tile is 1-29 % ahead of the 128-row
+        // one on 45 and 1-2 % behind on 2; with more tiles, or longer contractions, 128 rows win)
         if (rt == 8) return find_variant(4, 8, kOnline);
     } else {
         rt = 1;
