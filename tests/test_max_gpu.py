@@ -181,6 +181,31 @@ def test_other_float_dtypes(dev, dtype):
         _same(matmax(m.to(dev), axis), torch.amax(m, axis))
 
 
+@pytest.mark.parametrize("dtype", [torch.float64, torch.float16, torch.bfloat16])
+def test_other_float_dtypes_beyond_the_cache(dev, dtype):
+    """Operands of 32 MiB and more take the read-once loads in every element width."""
+    wide = dtype == torch.float64
+    n = 5_000_003 if wide else 18_000_005
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(n, generator=g).to(dtype)
+    ref = x if wide else x.float()
+    gv, gi = torch.max(ref, 0)
+    xg = x.to(dev)
+    v, i = vmax(xg)
+    assert v.dtype == dtype and v.item() == gv.item() and i.item() == gi.item()
+    assert vamax(xg).item() == gv.item()
+    rows, cols = (2100, 2048) if wide else (4200, 4096)
+    m = xg[: rows * cols].view(rows, cols)
+    mref = ref[: rows * cols].view(rows, cols)
+    for axis in (0, 1):
+        _same(matmax(m, axis), torch.amax(mref, axis).to(dtype))
+    m[rows // 2, 17] = float("nan")
+    m[3, cols - 1] = float("-inf")
+    mref = m.cpu() if wide else m.cpu().float()
+    for axis in (0, 1):
+        _same(matmax(m, axis), torch.amax(mref, axis).to(dtype))
+
+
 @pytest.mark.parametrize(
     "shape",
     [(1, 1), (1, 7), (7, 1), (23, 31), (64, 64), (65, 127), (200, 150), (1000, 3), (3, 1000), (2, 300000),
