@@ -411,7 +411,8 @@ def test_random_vectors_and_matrices(dev, seed):
 # ---- batched column maxima: the front end of the contraction recipes
 @pytest.mark.parametrize("shape", [(1, 1, 1), (3, 7, 5), (4, 64, 256), (2, 300, 1000), (64, 64, 4096), (5, 33, 257),
                                    (1, 4096, 300), (2, 1000, 70), (16, 512, 512), (1, 129, 3),  # these four are cut over J
-                                   (1, 70000, 40), (2, 9000, 300)])  # more than 128 pieces: combined in two levels
+                                   (1, 70000, 40), (2, 9000, 300),  # more than 128 pieces: combined in two levels
+                                   (66, 75, 2048), (2, 40000, 128), (3, 1111, 3000)])  # 32 MiB and more: read-once loads
 @pytest.mark.parametrize("clamp", [False, True])
 def test_bmatmax(dev, shape, clamp):
     from triturus_amd.max import bmatmax
