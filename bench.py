@@ -425,9 +425,9 @@ def main() -> int:
 
         # ------------------------------------------------ max reductions (HBM bound)
         # Two figures per reduction.  `us`: the same 64 MiB operand call after call, as a caller
-        # that reduces one tensor repeatedly sees it -- the operand then sits in the 256 MB
-        # memory-side cache (and, with the library's read-once loads, half of it stays in the
-        # dies' L2s from one call to the next).  `out_of_cache`: 8 copies of the operand
+        # that reduces one tensor repeatedly sees it -- the operand then fits the 256 MB
+        # memory-side cache, and the library's read-once loads leave in place whatever part of
+        # it an earlier pass left in the dies' L2s.  `out_of_cache`: 8 copies of the operand
         # (512 MiB) taken in turn, so that every call streams from HBM.
         x = cfg["b"].to(dev)  # 64 x 64 x 4096
         nbytes = x.numel() * 4
