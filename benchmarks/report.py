@@ -19,8 +19,7 @@ same metrics (GB/s of input bytes for lm2exp / lt2exp; comparisons per second, l
 reductions) and the same protocol (median of event-timed calls, each preceded by a 512 MiB cache flush).
 `torch` is the reference's eager torch recipe on the same GPU (rocBLAS bmm + elementwise kernels); `triturus` is
 this repository; `triturus (allow_tf32)` is the same call after `set_tf32_enabled(True)` (split-bf16 matrix path).  Run with
-`python -m benchmarks.lm2exp|lt2exp|max|mm <dir>` (and `python -m benchmarks.random_shapes <dir>` for the scan of
-random shapes at the end), then `python -m benchmarks.report <dir>`.
+`python -m benchmarks.lm2exp|lt2exp|max|mm <dir>`, then `python -m benchmarks.report <dir>`.
 """
 
 
@@ -52,9 +51,7 @@ def main():
     dst = Path(sys.argv[2]) if len(sys.argv) > 2 else Path(__file__).with_name("RESULTS.md")
     sweeps = [json.loads(p.read_text()) for p in sorted(src.glob("*.json"))]
     sweeps.sort(key=lambda s: (next((i for i, o in enumerate(ORDER) if s["name"].startswith(o)), 99), s["name"]))
-    extra = src / "random_shapes.md"  # written by benchmarks.random_shapes
-    tail = "\n" + extra.read_text() if extra.exists() else ""
-    dst.write_text(HEADER + "\n" + "\n\n".join(table(s) for s in sweeps) + "\n" + tail)
+    dst.write_text(HEADER + "\n" + "\n\n".join(table(s) for s in sweeps) + "\n")
     print(f"wrote {dst} ({len(sweeps)} sweeps)")
 
 

@@ -1,7 +1,9 @@
 // matmax / vmax / vamax for gfx950: every element is read once from HBM with
 // 16-byte coalesced loads, reduced in registers, then across the 64-lane
-// wavefront, then across the workgroup through LDS.  Large inputs take one
-// streaming launch plus one tiny combine launch over per-workgroup partials.
+// wavefront, then across the workgroup through LDS.  A reduction is one launch:
+// the workgroups leave partial results in the caller's workspace and the one that
+// finishes last combines them (unaligned or very wide matrices keep a tree of
+// two or three launches, colmax_kernel / rowmax_kernel).
 //
 // Semantics follow torch, the oracle the reference tests use
 // (tests/max.py:13,22,32): NaN propagates; argmax ties go to the lowest index

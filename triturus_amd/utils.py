@@ -47,8 +47,9 @@ def ensure_reproducibility(
     else:
         torch.set_default_device(device)
     if determinism:
-        # every kernel of this library is deterministic (fixed summation order,
-        # no atomics); the flag only concerns torch's own ops
+        # every kernel of this library is deterministic (fixed summation order; the
+        # only atomics are the arrival counters of the max reductions, which decide who
+        # combines the partial results, never the result); the flag only concerns torch's own ops
         torch.use_deterministic_algorithms(True, warn_only=True)
         torch.backends.cudnn.benchmark = False
         os.environ["CUBLAS_WORKSPACE_CONFIG"] = ":16:8"
