@@ -3,7 +3,7 @@
  *
  * Every entry point takes raw DEVICE pointers, sizes, element strides and a
  * hipStream_t (as void*).  The library allocates nothing, keeps no state,
- * never synchronises and never throws: each call enqueues its kernels on the
+ * never synchronises (trt_max_workspace_check, a debugging aid, excepted) and never throws: each call enqueues its kernels on the
  * given stream and returns an int status
  *      0            success
  *      < 0          argument / layout error (TRT_E_*), nothing was enqueued
@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TRT_ABI_VERSION 7
+#define TRT_ABI_VERSION 8
 
 #define TRT_OK 0
 #define TRT_E_INVALID (-1)   /* null pointer, non-positive size, bad enum   */
@@ -35,6 +35,7 @@ extern "C" {
 #define TRT_E_WORKSPACE (-3) /* workspace missing or smaller than required  */
 #define TRT_E_RANGE (-4)     /* a size exceeds what the index math supports */
 #define TRT_E_SCRATCH (-5)   /* the call needs more than the library's static scratch holds */
+#define TRT_E_STATE (-6)     /* trt_max_workspace_check: arrival counters not idle           */
 
 /* Element types of the max reductions (triturus/max.py:37,98,178 accept any
  * floating dtype). */
@@ -191,16 +192,33 @@ int trt_lm2exp_bf16_variant_count(void);
 /*
  * Workspaces of the max reductions (trt_matmax, trt_vmax) start with arrival counters: the
  * workgroup that finishes last combines the partial results of all of them, so a reduction is
- * one launch.  The first TRT_MAX_TICKET_BYTES of such a workspace must be ZERO before the first
- * call that uses it (one hipMemset when it is allocated, or trt_max_workspace_init); every call
- * leaves them zero, so a workspace can be reused from call to call -- by one stream at a time:
- * calls that overlap in time need workspaces of their own.
+ * one launch.  The first TRT_MAX_TICKET_BYTES of such a workspace must be prepared with
+ * trt_max_workspace_init before the first call that uses it (a hipMemset to zero does NOT do:
+ * an idle counter carries a tag); every call leaves the counters idle, so a workspace is
+ * prepared once and reused from call to call -- by one stream at a time: calls that overlap in
+ * time need workspaces of their own.  Workspaces must be 16-byte aligned (TRT_E_LAYOUT).
+ * What a broken contract looks like: a reduction that finds a counter without the tag (a
+ * workspace never prepared, or written over) or with more arrivals than its launch makes
+ * elects no combining workgroup and writes NaN -- with index -1 from trt_vmax -- where the
+ * result belongs (the launch itself cannot report a status: it is asynchronous); the counters
+ * stay as they are until trt_max_workspace_init runs again.  Two calls that use one workspace
+ * at the same time are detected only when their counts happen to overshoot.
  */
 #define TRT_MAX_TICKET_BYTES 65536
-/* Zeroes the arrival counters of a max workspace with a small kernel on `stream` (in place of a
- * hipMemset; safe to record into a HIP graph).  No counterpart in the reference, whose
- * reductions launch once per level.  workspace_bytes < TRT_MAX_TICKET_BYTES: TRT_E_WORKSPACE. */
+/* Sets the arrival counters of a max workspace idle with a small kernel on `stream` (no memset
+ * node: safe to record into a HIP graph).  No counterpart in the reference, whose reductions
+ * launch once per level.  workspace_bytes < TRT_MAX_TICKET_BYTES: TRT_E_WORKSPACE. */
 int trt_max_workspace_init(void *workspace, size_t workspace_bytes, void *stream);
+/* Debugging aid, no counterpart in the reference: waits for `stream` (this one call of the
+ * library synchronises), reads the counters back and returns TRT_E_STATE unless all of them
+ * are idle -- which they are between any two reductions of a sound program. */
+int trt_max_workspace_check(const void *workspace, size_t workspace_bytes, void *stream);
+
+/* *capture_id = the identity of the HIP graph capture `stream` is in, 0 when it is in none.  Host
+ * only; no counterpart in the reference.  A caller that keeps one max workspace per stream
+ * needs it to give every capture a workspace (and a trt_max_workspace_init node) of its own:
+ * a workspace prepared while capturing is idle only when the graph runs. */
+int trt_stream_capture_id(void *stream, unsigned long long *capture_id);
 
 /*
  * Max of a contiguous m x n row-major matrix along axis 0 (y has n entries)

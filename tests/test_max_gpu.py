@@ -358,7 +358,124 @@ def test_c_abi_with_a_workspace_prepared_by_the_library(dev):
                 _lib.check(lib.trt_matmax(xg.data_ptr(), y.data_ptr(), 3000, 4100, axis, _lib.TRT_F32, ws.data_ptr(),
                                           need, stream), "trt_matmax")
                 _same(y, torch.amax(x, axis))
-    assert int(ws[:65536].max().item()) == 0  # the counters are back to zero
+    assert lib.trt_max_workspace_check(ws.data_ptr(), need, stream) == 0  # the counters are idle again
+    assert lib.trt_vmax(xg.data_ptr(), n, _lib.TRT_F32, val.data_ptr(), idx.data_ptr(), ws.data_ptr() + 4, need - 4,
+                        stream) == -2  # a workspace that is not 16-byte aligned is refused
+    assert lib.trt_matmax(xg.data_ptr(), y.data_ptr(), 3000, 4100, 0, _lib.TRT_F32, ws.data_ptr() + 8, need - 8,
+                          stream) == -2
+
+
+@pytest.mark.parametrize("dirt", ["never prepared", "zeroed", "one counter zeroed", "random bytes"])
+def test_a_workspace_with_foreign_counters_shows_in_the_result(dev, dirt):
+    """Counters that no call of the library left behind (written here from the host side with torch;
+    every kernel still runs to its end): the reductions then return NaN -- vmax with index -1 --
+    instead of leaving garbage, trt_max_workspace_check reports TRT_E_STATE, and after
+    trt_max_workspace_init the same workspace serves again."""
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(2048, 4096, generator=g)
+    xg = x.to(dev)
+    n = x.numel()
+    need = max(lib.trt_vmax_workspace_bytes(n, _lib.TRT_F32), lib.trt_matmax_workspace_bytes(2048, 4096, 0, _lib.TRT_F32))
+    ws = torch.empty(need, dtype=torch.uint8, device=dev)
+    stream = _lib.raw_stream(dev)
+    val = torch.empty((), device=dev)
+    idx = torch.empty((), dtype=torch.int64, device=dev)
+    y = torch.empty(4096, device=dev)
+
+    def run_both():
+        val.fill_(123.0), idx.fill_(123), y.fill_(123.0)
+        with _lib.on_device(dev):
+            _lib.check(lib.trt_vmax(xg.data_ptr(), n, _lib.TRT_F32, val.data_ptr(), idx.data_ptr(), ws.data_ptr(), need,
+                                    stream), "trt_vmax")
+            _lib.check(lib.trt_matmax(xg.data_ptr(), y.data_ptr(), 2048, 4096, 0, _lib.TRT_F32, ws.data_ptr(), need,
+                                      stream), "trt_matmax")
+        torch.cuda.synchronize()
+
+    with _lib.on_device(dev):
+        _lib.check(lib.trt_max_workspace_init(ws.data_ptr(), need, stream), "trt_max_workspace_init")
+    head = ws[:65536]
+    if dirt == "never prepared":
+        head.fill_(0xAB)
+    elif dirt == "zeroed":
+        head.zero_()
+    elif dirt == "one counter zeroed":  # the first group of vmax, the first column block of matmax
+        head[:8].zero_()
+    else:
+        head.copy_(torch.randint(0, 256, (65536,), generator=g, dtype=torch.uint8))
+    torch.cuda.synchronize()
+    assert lib.trt_max_workspace_check(ws.data_ptr(), need, stream) == _lib.E_STATE
+    run_both()
+    gv, gi = torch.max(x.view(-1), 0)
+    right = (val.item(), idx.item()) == (gv.item(), gi.item())
+    assert right or (torch.isnan(val).item() and idx.item() == -1), (val.item(), idx.item())
+    col_right = y.cpu() == torch.amax(x, 0)
+    assert bool(torch.all(col_right | torch.isnan(y.cpu())))
+    assert not (right and bool(col_right.all()))  # this dirt is not survivable: it must show
+    with _lib.on_device(dev):
+        _lib.check(lib.trt_max_workspace_init(ws.data_ptr(), need, stream), "trt_max_workspace_init")
+    run_both()
+    assert (val.item(), idx.item()) == (gv.item(), gi.item())
+    _same(y, torch.amax(x, 0))
+    assert lib.trt_max_workspace_check(ws.data_ptr(), need, stream) == 0
+
+
+def test_the_first_reduction_of_a_stream_inside_a_graph_capture(dev):
+    """A stream whose first reduction ever is recorded into a HIP graph: the workspace prepared
+    during the capture is idle only when that graph runs, so neither an eager call on the stream
+    nor a second graph may count in it before the first replay."""
+    import triturus_amd.max as tmax
+
+    x = torch.randn(1 << 22)
+    x2 = torch.randn(3000, 1000)
+    xg, x2g = x.to(dev), x2.to(dev)
+    want = tuple(t.item() for t in torch.max(x, 0))
+    s = torch.cuda.Stream(device=dev)
+    s.wait_stream(torch.cuda.current_stream(dev))
+    key = (dev.index, s.cuda_stream)
+    assert key not in tmax._workspaces
+    g1 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g1, stream=s):
+        v1, i1 = vmax(xg)
+        y1 = matmax(x2g, 0)
+    assert key not in tmax._workspaces  # nothing prepared under capture is kept for eager calls
+    with torch.cuda.stream(s):
+        v, i = vmax(xg)  # eager, before the first replay
+        y = matmax(x2g, 0)
+    s.synchronize()
+    assert (v.item(), i.item()) == want
+    _same(y, torch.amax(x2, 0))
+    g2 = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g2, stream=s):
+        v2, i2 = vmax(xg)
+    for _ in range(3):
+        g2.replay()
+        torch.cuda.synchronize()
+        assert (v2.item(), i2.item()) == want
+        with torch.cuda.stream(s):
+            v, i = vmax(xg)
+        s.synchronize()
+        assert (v.item(), i.item()) == want
+        g1.replay()
+        torch.cuda.synchronize()
+        assert (v1.item(), i1.item()) == want
+        _same(y1, torch.amax(x2, 0))
+
+
+def test_workspaces_are_kept_for_a_bounded_number_of_streams(dev):
+    import triturus_amd.max as tmax
+
+    x = torch.randn(1 << 18)
+    xg = x.to(dev)
+    want = tuple(t.item() for t in torch.max(x, 0))
+    streams = [torch.cuda.Stream(device=dev) for _ in range(tmax._MAX_STREAMS + 8)]
+    for s in streams:
+        s.wait_stream(torch.cuda.current_stream(dev))
+        with torch.cuda.stream(s):
+            v, i = vmax(xg)
+        s.synchronize()
+        assert (v.item(), i.item()) == want
+    assert len(tmax._workspaces) <= tmax._MAX_STREAMS
 
 
 @pytest.mark.parametrize("seed", range(8))

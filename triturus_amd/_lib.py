@@ -14,12 +14,13 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtriturus_hip.so"
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 TRT_F32, TRT_F64, TRT_F16, TRT_BF16 = 0, 1, 2, 3
 MODE_AUTO, MODE_SPLIT, MODE_UNSPLIT = 0, 1, 2
 STATIC_SCRATCH_BYTES = 16 << 20  # TRT_STATIC_SCRATCH_BYTES
 E_SCRATCH = -5
+E_STATE = -6
 
 DTYPE_CODES = {
     torch.float32: TRT_F32,
@@ -89,6 +90,8 @@ SIGNATURES = {
     "trt_vadd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "trt_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "trt_max_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),
+    "trt_max_workspace_check": (c_int, [c_void_p, c_size_t, c_void_p]),
+    "trt_stream_capture_id": (c_int, [c_void_p, POINTER(ctypes.c_ulonglong)]),
     "trt_lt2exp_kernel_name": (c_int, [c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_char_p, c_size_t]),
     "trt_lm2exp_kernel_name": (c_int, [c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_int, c_char_p, c_size_t]),
 }

@@ -172,14 +172,26 @@ constexpr int kVmaxGroup = 32;  // workgroups that draw from one arrival counter
 
 // Arrival counters ("tickets") at the head of a max workspace: a launch whose workgroups leave
 // partial results takes one ticket per workgroup; the workgroup that draws the last one
-// combines the partials and puts the counter back to zero.  The counters must be zero before
-// the first call that uses a workspace and every call leaves them zero, so one launch does the
-// work of two and the library still keeps no state of its own.
+// combines the partials and puts the counter back to its idle value.  The counters must be idle
+// before the first call that uses a workspace (trt_max_workspace_init) and every call leaves
+// them idle, so one launch does the work of two and the library still keeps no state of its own.
+// A counter is a 64-bit word: a fixed tag in the upper half, the number of arrivals in the lower.
+// A workgroup that draws a word with another tag, or a count its launch cannot have produced,
+// knows that the workspace was never prepared or has been written over: it elects nobody and
+// writes a NaN (index -1) where the result belongs, so that a broken workspace shows in the
+// output instead of leaving it unwritten.
 constexpr size_t kTicketBytes = TRT_MAX_TICKET_BYTES;
+using Ticket = unsigned long long;
+constexpr Ticket kTicketTag = (Ticket)0x7452544Bu << 32;  // "tRTK": idle counter = tag, no arrivals
 // Counters that different groups of workgroups draw from sit 256 bytes apart: device-scope atomics on
 // one memory line are served one after the other (measured ~10 ns each), on different lines side by side.
-constexpr int kTicketStride = 256 / (int)sizeof(unsigned);
+constexpr int kTicketStride = 256 / (int)sizeof(Ticket);
 constexpr int kMaxTickets = (int)(kTicketBytes / 256);
+// drawn: what the counter held before this workgroup's arrival; of: arrivals the launch makes
+__device__ __forceinline__ bool ticket_last(Ticket drawn, int of) { return drawn == (kTicketTag | (Ticket)(of - 1)); }
+__device__ __forceinline__ bool ticket_sound(Ticket drawn, int of) {
+    return (drawn >> 32) == (kTicketTag >> 32) && (unsigned)drawn < (unsigned)of;
+}
 static_assert(kVmaxMaxBlocks / kVmaxGroup < kMaxTickets, "one counter per group and one for the groups");
 
 // The partials of the other workgroups were written on other compute units (and other dies,
@@ -193,18 +205,21 @@ static_assert(kVmaxMaxBlocks / kVmaxGroup < kMaxTickets, "one counter per group 
 // costs a trip of some 170 ns (measured: the last workgroup's time grows by that much per load
 // instruction) -- so a partial is one 16-byte record, not a word per field.
 constexpr int kDeviceScope = 16;
-__device__ __forceinline__ unsigned take_ticket(unsigned *ticket) {
+__device__ __forceinline__ Ticket take_ticket(Ticket *ticket) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
-    return __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    return __hip_atomic_fetch_add(ticket, (Ticket)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 // The same for a whole wavefront that has stored: lane 0 draws, the others wait with it.
-__device__ __forceinline__ unsigned take_ticket_wave(unsigned *ticket) {
+__device__ __forceinline__ Ticket take_ticket_wave(Ticket *ticket) {
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
     __builtin_amdgcn_s_waitcnt(0);
-    unsigned t = 0;
-    if (lane_id() == 0) t = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    Ticket t = 0;
+    if (lane_id() == 0) t = __hip_atomic_fetch_add(ticket, (Ticket)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     return t;
+}
+__device__ __forceinline__ void ticket_idle(Ticket *ticket) {  // ready for the next call
+    __hip_atomic_store(ticket, kTicketTag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 // Workgroups go to the 8 dies (each with an L2 of its own) round-robin: logical position of a
@@ -250,7 +265,7 @@ using AgainT = std::false_type;
 template <int DT, bool WITH_IDX, bool FINAL>
 __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     const typename Elem<DT>::T *__restrict__ x, int64_t n, int64_t head, int64_t nvec,
-    int64_t share_q, int share_rem, int once, uintx4 *prec, unsigned *ticket,
+    int64_t share_q, int share_rem, int once, uintx4 *prec, Ticket *ticket,
     typename Elem<DT>::T *__restrict__ out_val, int64_t *__restrict__ out_idx) {
     using E = Elem<DT>;
     using T = typename E::T;
@@ -448,18 +463,26 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     };
     static_assert(sizeof(Record) == 16, "one 16-byte access per partial");
     const __amdgpu_buffer_rsrc_t prsrc = make_rsrc(prec, (uint32_t)kVmaxMaxBlocks * 16u);
-    unsigned *tick1 = ticket + group * kTicketStride;
-    unsigned *tick2 = ticket + (kMaxTickets - 1) * kTicketStride;
+    Ticket *tick1 = ticket + group * kTicketStride;
+    Ticket *tick2 = ticket + (kMaxTickets - 1) * kTicketStride;
     if (tid == 0) {
         // the partial: one 16-byte record (value in an 8-byte slot, index)
         Record rec;
         rec.f.val = best;
         rec.f.idx = bidx;
         __builtin_amdgcn_raw_buffer_store_b128(rec.bits, prsrc, (uint32_t)blockIdx.x * 16u, 0, kDeviceScope);
-        bool last = take_ticket(tick1) == (unsigned)gsize - 1;
+        Ticket drawn = take_ticket(tick1);
+        bool sound = ticket_sound(drawn, gsize);
+        bool last = ticket_last(drawn, gsize);
         if (last) {
-            last = take_ticket(tick2) == (unsigned)ngroups - 1;
-            __hip_atomic_store(tick1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);  // ready for the next call
+            drawn = take_ticket(tick2);
+            sound = ticket_sound(drawn, ngroups);
+            last = ticket_last(drawn, ngroups);
+            ticket_idle(tick1);
+        }
+        if (!sound) {  // counters that no launch of this library left behind: say so in the result
+            *out_val = E::down((C)__builtin_nanf(""));
+            if (WITH_IDX) *out_idx = -1;
         }
         last_block = last;
     }
@@ -487,7 +510,7 @@ __global__ __launch_bounds__(kVmaxThreads) void vmax_kernel(
     block_reduce();
     if (tid == 0) {
         write_result();
-        __hip_atomic_store(tick2, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        ticket_idle(tick2);
     }
 }
 
@@ -535,17 +558,17 @@ static int vmax_launch(const void *x, int64_t n, void *out_val, int64_t *out_idx
     if (vmax_single_block(n, DT)) {
         if (out_idx)
             hipLaunchKernelGGL((vmax_kernel<DT, true, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                               nvec, full_blocks, 0, 0, (uintx4 *)nullptr, (unsigned *)nullptr, ov, out_idx);
+                               nvec, full_blocks, 0, 0, (uintx4 *)nullptr, (Ticket *)nullptr, ov, out_idx);
         else
             hipLaunchKernelGGL((vmax_kernel<DT, false, true>), dim3(1), dim3(kVmaxThreads), 0, stream, xp, n, head,
-                               nvec, full_blocks, 0, 0, (uintx4 *)nullptr, (unsigned *)nullptr, ov, out_idx);
+                               nvec, full_blocks, 0, 0, (uintx4 *)nullptr, (Ticket *)nullptr, ov, out_idx);
         return (int)hipGetLastError();
     }
     const int blocks = vmax_blocks(nvec);
     const int64_t share_q = full_blocks / blocks;
     const int share_rem = (int)(full_blocks % blocks);
     const int once = n * (int64_t)sizeof(T) >= kStreamBytes;
-    unsigned *ticket = static_cast<unsigned *>(ws);
+    Ticket *ticket = static_cast<Ticket *>(ws);
     uintx4 *prec = reinterpret_cast<uintx4 *>(static_cast<char *>(ws) + kTicketBytes);
     if (out_idx)
         hipLaunchKernelGGL((vmax_kernel<DT, true, false>), dim3(blocks), dim3(kVmaxThreads), 0, stream, xp, n, head,
@@ -741,7 +764,7 @@ constexpr int kColFusedUnroll = 8;  // 16-byte loads in flight per lane
 template <int DT, int VPL>
 __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
     const typename Elem<DT>::T *__restrict__ x, int64_t ld, int64_t m, int64_t n, int64_t rchunk,
-    int colblocks, int splits, int once, unsigned long long *part, unsigned *ticket,
+    int colblocks, int splits, int once, unsigned long long *part, Ticket *ticket,
     typename Elem<DT>::T *__restrict__ y) {
     using E = Elem<DT>;
     using T = typename E::T;
@@ -850,8 +873,20 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
             __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(uintx4, u), prsrc, plane + 16u * p,
                                                    (uint32_t)(split * words_per_row * 8), kDeviceScope);
         }
-        const unsigned t = take_ticket_wave(ticket + cb * kTicketStride);
-        if (lane == 0) last_block = t == (unsigned)splits - 1;
+        const Ticket drawn = take_ticket_wave(ticket + cb * kTicketStride);
+        if (lane == 0) last_block = ticket_last(drawn, splits);
+        // counters that no launch of this library left behind: NaN in this block's part of y
+        const bool broken = __builtin_amdgcn_readfirstlane((int)!ticket_sound(drawn, splits)) != 0;
+        if (broken) {
+#pragma unroll
+            for (int p = 0; p < VPL; ++p) {
+                if (!have[p]) continue;
+                V out;
+#pragma unroll
+                for (int e = 0; e < VN; ++e) out.e[e] = E::down((C)__builtin_nanf(""));
+                *reinterpret_cast<V *>(y + col + (int64_t)p * kWave * VN) = out;
+            }
+        }
     }
     __syncthreads();
     if (!last_block) return;
@@ -891,7 +926,7 @@ __global__ __launch_bounds__(kMatThreads) void colmax_fused_kernel(
             for (int e = 0; e < VN; ++e) out.e[e] = E::down(best[p * VN + e]);
             *reinterpret_cast<V *>(y + col + (int64_t)p * kWave * VN) = out;
         }
-        if (lane == 0) __hip_atomic_store(ticket + cb * kTicketStride, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (lane == 0) ticket_idle(ticket + cb * kTicketStride);
     }
 }
 
@@ -1060,11 +1095,11 @@ static int matmax_launch(const void *xv, void *yv, int64_t m, int64_t n, int axi
         if (fused && pf.vpl == 2) {
             hipLaunchKernelGGL((colmax_fused_kernel<DT, 2>), dim3((unsigned)(pf.colblocks * pf.splits)),
                                dim3(kMatThreads), 0, stream, x, n, m, n, pf.chunk, pf.colblocks, pf.splits, once,
-                               reinterpret_cast<unsigned long long *>(part), static_cast<unsigned *>(ws), y);
+                               reinterpret_cast<unsigned long long *>(part), static_cast<Ticket *>(ws), y);
         } else if (fused && pf.vpl == 1) {
             hipLaunchKernelGGL((colmax_fused_kernel<DT, 1>), dim3((unsigned)(pf.colblocks * pf.splits)),
                                dim3(kMatThreads), 0, stream, x, n, m, n, pf.chunk, pf.colblocks, pf.splits, once,
-                               reinterpret_cast<unsigned long long *>(part), static_cast<unsigned *>(ws), y);
+                               reinterpret_cast<unsigned long long *>(part), static_cast<Ticket *>(ws), y);
         } else if (p.splits == 1) {
             colmax_launch<DT>(x, n, m, n, vec, p, y, n, stream);
         } else {
@@ -1119,6 +1154,8 @@ extern "C" int trt_vmax(const void *x, int64_t n, int dtype, void *out_val, int6
     const size_t need = vmax_ws_bytes(n, dtype);
     if (need && (!workspace || workspace_bytes < need)) return TRT_E_WORKSPACE;
     if ((reinterpret_cast<uintptr_t>(x) % elem_size(dtype)) != 0) return TRT_E_LAYOUT;
+    // counters are 8-byte atomics, partial results 16-byte accesses
+    if (need && (reinterpret_cast<uintptr_t>(workspace) & 15)) return TRT_E_LAYOUT;
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (dtype) {
         case TRT_F32: return vmax_launch<TRT_F32>(x, n, out_val, out_idx, workspace, s);
@@ -1144,6 +1181,7 @@ extern "C" int trt_matmax(const void *x, void *y, int64_t m, int64_t n, int axis
     if (!x || !y || m <= 0 || n <= 0 || (axis != 0 && axis != 1) || !elem_size(dtype))
         return TRT_E_INVALID;
     if ((reinterpret_cast<uintptr_t>(x) % elem_size(dtype)) != 0) return TRT_E_LAYOUT;
+    if (workspace && (reinterpret_cast<uintptr_t>(workspace) & 15)) return TRT_E_LAYOUT;
     if (m > (int64_t)1 << 40 || n > (int64_t)1 << 40) return TRT_E_RANGE;
     // workgroup ids are 32-bit: every launch of the call must stay below 2^31 workgroups
     if (matmax_max_blocks(m, n, axis, dtype) >= ((int64_t)1 << 31)) return TRT_E_RANGE;
@@ -1170,18 +1208,33 @@ __global__ __launch_bounds__(256) void copy16_kernel(const trt::uintx4 *__restri
         if (base + u * 256 < nvec) __builtin_nontemporal_store(v[u], &dst[base + u * 256]);
 }
 
-// Arrival counters of a max workspace back to zero, by a kernel (a caller that prepares its
+// Arrival counters of a max workspace set idle, by a kernel (a caller that prepares its
 // workspaces while a stream is being captured into a graph needs no memset node).
-__global__ __launch_bounds__(256) void zero_tickets_kernel(unsigned *ticket) {
-    for (unsigned i = threadIdx.x; i < trt::kTicketBytes / sizeof(unsigned); i += 256) ticket[i] = 0u;
+__global__ __launch_bounds__(256) void idle_tickets_kernel(trt::Ticket *ticket) {
+    for (unsigned i = threadIdx.x; i < trt::kTicketBytes / sizeof(trt::Ticket); i += 256) ticket[i] = trt::kTicketTag;
 }
 
 extern "C" int trt_max_workspace_init(void *workspace, size_t workspace_bytes, void *stream) {
     if (!workspace || workspace_bytes < trt::kTicketBytes) return TRT_E_WORKSPACE;
-    if (reinterpret_cast<uintptr_t>(workspace) & 3) return TRT_E_LAYOUT;
-    hipLaunchKernelGGL(zero_tickets_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<unsigned *>(workspace));
+    if (reinterpret_cast<uintptr_t>(workspace) & 15) return TRT_E_LAYOUT;
+    hipLaunchKernelGGL(idle_tickets_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<trt::Ticket *>(workspace));
     return (int)hipGetLastError();
+}
+
+// Debugging aid: waits for `stream`, copies the counters to the host and looks at them.
+extern "C" int trt_max_workspace_check(const void *workspace, size_t workspace_bytes, void *stream) {
+    if (!workspace || workspace_bytes < trt::kTicketBytes) return TRT_E_WORKSPACE;
+    if (reinterpret_cast<uintptr_t>(workspace) & 15) return TRT_E_LAYOUT;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipError_t err = hipStreamSynchronize(s);
+    if (err != hipSuccess) return (int)err;
+    static thread_local trt::Ticket host[trt::kTicketBytes / sizeof(trt::Ticket)];
+    err = hipMemcpy(host, workspace, trt::kTicketBytes, hipMemcpyDeviceToHost);
+    if (err != hipSuccess) return (int)err;
+    for (size_t i = 0; i < trt::kTicketBytes / sizeof(trt::Ticket); ++i)
+        if (host[i] != trt::kTicketTag) return TRT_E_STATE;
+    return TRT_OK;
 }
 
 extern "C" int trt_copy_bytes(const void *src, void *dst, size_t nbytes, void *stream) {

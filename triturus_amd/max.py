@@ -10,30 +10,73 @@ NaN handling follows torch.amax / torch.max (NaN propagates).
 
 from __future__ import annotations
 
+import ctypes
+import os
+from collections import OrderedDict
+
 import torch
 
 from triturus_amd import _lib
 
 _ws_bytes: dict = {}  # (op, shape..., dtype code) -> workspace bytes, as reported by the library
-# (device index, raw stream) -> workspace of the reductions launched on that stream.  The library
-# wants the arrival counters at the head of a max workspace zero before the first use and leaves
-# them zero (one launch per reduction: the workgroup that finishes last combines the partial
-# results), so the workspace is allocated once per stream, zero-filled, and kept: calls on one
-# stream run one after the other, calls on different streams never share one.
-_workspaces: dict = {}
-# Workspaces that a larger one has replaced.  They are kept for the life of the process: a HIP
-# graph captured while one of them was current still launches kernels that count in it.
-_retired: list = []
+
+# The library wants the arrival counters at the head of a max workspace idle before the first
+# use (trt_max_workspace_init) and leaves them idle (one launch per reduction: the workgroup
+# that finishes last combines the partial results).  So a workspace is allocated and prepared
+# once per device and stream and kept: calls on one stream run one after the other, calls on
+# different streams never share one.  At most _MAX_STREAMS of them are kept, the least recently
+# used one going first (the allocator hands its block to later work on the same stream only).
+_MAX_STREAMS = 16
+_workspaces: "OrderedDict[tuple, torch.Tensor]" = OrderedDict()  # (device index, raw stream) -> workspace
+# A stream that is being captured into a HIP graph gets a workspace of its own per capture,
+# allocated inside the capture (from the graph's memory pool) and prepared by a kernel node of
+# that graph: whatever is prepared while capturing is idle only once the graph runs, so it must
+# never serve an eager call, and an eager workspace must never serve a graph (the replays would
+# count in it while eager calls on the stream do).  (device index, raw stream) -> (capture id,
+# workspace); the entry of a finished capture is dropped when the stream is next seen -- the
+# graph's pool keeps the block for the replays.
+_capture_workspaces: dict = {}
+_CHECK = os.environ.get("TRITURUS_CHECK_WORKSPACE", "0") not in ("", "0")  # debugging: verify the counters before every call
+
+try:
+    _is_capturing = torch._C._cuda_isCurrentStreamCapturing
+except AttributeError:  # pragma: no cover
+    _is_capturing = torch.cuda.is_current_stream_capturing
+
+
+def _new_workspace(dev: torch.device, nbytes: int, stream: int) -> torch.Tensor:
+    ws = torch.empty(max(nbytes, 1 << 16), dtype=torch.uint8, device=dev)
+    with _lib.on_device(dev):
+        _lib.check(_lib.load().trt_max_workspace_init(ws.data_ptr(), ws.numel(), stream), "trt_max_workspace_init")
+    return ws
 
 
 def _workspace(dev: torch.device, nbytes: int):
-    key = (dev.index, _lib.raw_stream(dev))
+    stream = _lib.raw_stream(dev)
+    key = (dev.index, stream)
+    if torch.cuda.is_available() and _is_capturing():
+        cid = ctypes.c_ulonglong(0)
+        _lib.check(_lib.load().trt_stream_capture_id(stream, ctypes.byref(cid)), "trt_stream_capture_id")
+        if cid.value:
+            held = _capture_workspaces.get(key)
+            if held is None or held[0] != cid.value or held[1].numel() < nbytes:
+                held = _capture_workspaces[key] = (cid.value, _new_workspace(dev, nbytes, stream))
+            return held[1]
+    if _capture_workspaces:
+        _capture_workspaces.pop(key, None)
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < nbytes:
         if ws is not None:
-            _retired.append(ws)
-            nbytes = max(nbytes, 2 * ws.numel())  # grow geometrically: what is retired stays below what is live
-        ws = _workspaces[key] = torch.zeros(max(nbytes, 1 << 16), dtype=torch.uint8, device=dev)
+            nbytes = max(nbytes, 2 * ws.numel())  # grow geometrically
+        ws = _workspaces[key] = _new_workspace(dev, nbytes, stream)
+        while len(_workspaces) > _MAX_STREAMS:
+            _workspaces.popitem(last=False)
+    else:
+        _workspaces.move_to_end(key)
+        if _CHECK:
+            with _lib.on_device(dev):
+                _lib.check(_lib.load().trt_max_workspace_check(ws.data_ptr(), ws.numel(), stream),
+                           "trt_max_workspace_check")
     return ws
 
 
