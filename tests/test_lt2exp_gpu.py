@@ -20,7 +20,7 @@ from triturus_amd import _lib, workloads
 pytestmark = pytest.mark.gpu
 GOLDEN = Path(__file__).resolve().parent / "golden"
 NINF = float("-inf")
-N_VARIANTS = 14
+N_VARIANTS = 16
 N_BF16_VARIANTS = 16  # 1..4, 9..12 tiles; 5..8, 13..16 the same tiles with the contraction cut over workgroups
 # Accuracy gates of the split-bf16 paths against the float64 oracle.  Two pieces (3 MFMAs per
 # product) carry 16 significand bits: looser than fp32, ten times tighter than the rtol 5e-4

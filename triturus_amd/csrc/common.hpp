@@ -44,17 +44,19 @@ __host__ __device__ __forceinline__ int64_t ceil_div(int64_t a, int64_t b) { ret
 // smallest estimate; a split must win by 20 %.  The merge constants are pessimistic on purpose
 // (2 TB/s, 5 us): splits the model rates as marginal were losses when measured.  per_split_us
 // adds a cost per split for callers whose merge is bound by its chain of loads; must_win is the
-// fraction of the uncut estimate a cut has to stay under.
+// fraction of the uncut estimate a cut has to stay under.  eff_few: the rate with one and with
+// two workgroups on a CU, for kernels that measure other than 45 % and 65 % there (the 64-row
+// lt2exp tile, whose steps hold 32 MFMAs: 67 % and 82 %).
 inline int choose_splits(int64_t tiles, int64_t units, int64_t mfmas_per_unit, int64_t out_elems,
                          int min_units_per_split, int max_splits, bool forced, double per_split_us = 0.0,
-                         double must_win = 0.8) {
+                         double must_win = 0.8, double eff_one = 0.45, double eff_two = 0.65) {
     constexpr double kCyclesPerUs = 2400.0;
     constexpr int64_t kCuCount = 256;
     const double unit_us = (double)mfmas_per_unit * 64.0 / kCyclesPerUs;
     auto estimate = [&](int sp) {
         const double chain_us = (double)ceil_div(units, sp) * unit_us;  // one workgroup at the full MFMA rate
         const int64_t q = ceil_div(tiles * sp, kCuCount);               // workgroups on the busiest CU
-        const double eff = q >= 4 ? 0.9 : (q == 3 ? 0.8 : (q == 2 ? 0.65 : 0.45));
+        const double eff = q >= 4 ? 0.9 : (q == 3 ? (eff_two > 0.8 ? 0.88 : 0.8) : (q == 2 ? eff_two : eff_one));
         const double body = (double)q * chain_us / eff;
         const double merge_us =
             sp > 1 ? 5.0 + (double)sp * per_split_us + (double)(sp + 1) * (double)out_elems * 4.0 / 2.0e6 : 0.0;

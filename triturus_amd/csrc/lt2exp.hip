@@ -45,10 +45,17 @@ struct Lt2Args {
 // w is contiguous over (i, j), so the kernel walks that flat axis in chunks of 16 instead: a chunk
 // holds 16 / PJ values of i, and MFMA slot f = 8q + 4h + u of it multiplies exp a[i0 + f / PJ]
 // by exp b[f % PJ] (the factors of b are the same in every chunk).
-template <int RT, int CT, int NQ, int NWAVES, bool VEC, bool SPLIT, int WM = 1, int PJ = 0>
-__global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args p) {
+// GS: groups of NWAVES wavefronts in the workgroup.  With 2, the two groups own the SAME output
+// tile and contract the two halves of the (j-chunk, i) iteration range, each through w tiles
+// of its own in LDS; at the end they exchange, through LDS, the half of the accumulators that
+// the other group finishes.  A grid of one or two tiles per compute unit then runs with twice
+// the wavefronts per SIMD -- what such grids lack (one or two wavefronts per SIMD hide neither
+// LDS nor barrier latency) -- without the partial sums ever leaving the compute unit.
+template <int RT, int CT, int NQ, int NWAVES, bool VEC, bool SPLIT, int WM = 1, int PJ = 0, int GS = 1>
+__global__ __launch_bounds__(NWAVES *kWave *GS, 2 * GS) void lt2exp_kernel(const Lt2Args p) {
     static_assert(PJ == 0 || (VEC && NQ == 2 && (PJ == 2 || PJ == 4 || PJ == 8)), "packed rows: chunks of 16");
-    constexpr int NT = NWAVES * kWave;
+    static_assert(GS == 1 || (GS == 2 && VEC && !SPLIT && WM == 1 && PJ == 0 && CT == 1), "paired groups: plain aligned tiles");
+    constexpr int NT = NWAVES * kWave;  // threads of a group
     constexpr int WN = NWAVES / WM;
     constexpr int TS = 32 * RT * WM;      // rows of S per workgroup
     constexpr int JC = 8 * NQ;            // j per chunk
@@ -64,7 +71,8 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 
     // (a thread whose last slot lies past the tile stages into a private 16 bytes behind it:
     // the steady state carries no predicates)
-    __shared__ __attribute__((aligned(16))) float wt[2][TS * LDW + (REGULAR ? 0 : 4 * NT)];
+    static_assert(GS == 1 || REGULAR, "paired groups stage whole slots");
+    __shared__ __attribute__((aligned(16))) float wt_all[GS][2][TS * LDW + (REGULAR ? 0 : 4 * NT)];
 
     const int64_t L = xcd_logical_id(blockIdx.x, p.padded_wgs);
     if (L >= p.total_wgs) return;
@@ -78,7 +86,9 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     const int st = __builtin_amdgcn_readfirstlane((int)(rest % p.s_tiles));
     const int r = __builtin_amdgcn_readfirstlane((int)(rest / p.s_tiles));
 
-    const int tid = threadIdx.x;
+    const int grp = GS == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)threadIdx.x / NT);  // wave-uniform
+    const int tid = GS == 1 ? (int)threadIdx.x : (int)threadIdx.x - grp * NT;             // within the group
+    float(*wt)[TS * LDW + (REGULAR ? 0 : 4 * NT)] = wt_all[grp];
     const int wave = tid / kWave;
     const int lane = tid % kWave;
     const int h = lane / 32;
@@ -107,13 +117,26 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     for (int ct = 0; ct < CT; ++ct) {
         float x = -__builtin_inff();
 #pragma unroll 8
-        for (int i = h; i < p.I; i += 2) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + ncl[ct]]);
+        for (int i = 2 * grp + h; i < p.I; i += 2 * GS) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + ncl[ct]]);
         x = __builtin_fmaxf(x, __shfl_xor(x, 32, kWave));
-        ma[ct] = clamp_shift(x);
         float y = -__builtin_inff();
 #pragma unroll 8
-        for (int j = h; j < p.J; j += 2) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + ncl[ct]]);
+        for (int j = 2 * grp + h; j < p.J; j += 2 * GS) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + ncl[ct]]);
         y = __builtin_fmaxf(y, __shfl_xor(y, 32, kWave));
+        if (GS == 2) {
+            // each group has swept half of the rows: the halves meet in LDS (the tile buffers are
+            // not in use yet)
+            float *mx = &wt_all[0][0][0];
+            if (h == 0) {
+                mx[(grp * 2 + 0) * TN + wave * 32 + m] = x;
+                mx[(grp * 2 + 1) * TN + wave * 32 + m] = y;
+            }
+            __syncthreads();
+            x = __builtin_fmaxf(x, mx[((grp ^ 1) * 2 + 0) * TN + wave * 32 + m]);
+            y = __builtin_fmaxf(y, mx[((grp ^ 1) * 2 + 1) * TN + wave * 32 + m]);
+            __syncthreads();
+        }
+        ma[ct] = clamp_shift(x);
         mb[ct] = clamp_shift(y);
     }
 
@@ -123,6 +146,13 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
     int it = split * p.iters_per_split;
     int it_end = it + p.iters_per_split;
     if (it_end > total_iters) it_end = total_iters;
+    // paired groups: the first takes the first half of the range (the longer one when the count
+    // is odd); both make the same number of trips through the loop, for the barriers' sake
+    const int trips = GS == 1 ? it_end - it : (total_iters + 1) / 2;
+    if (GS == 2) {
+        it = grp * trips;
+        it_end = grp == 0 ? trips : total_iters;
+    }
 
     floatx16 acc[RT][CT];
 #pragma unroll
@@ -281,60 +311,129 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
             }
     };
 
-    if (it < it_end) {
-        int jc = it / n_i;
-        int i = it - jc * n_i;
-        load_tile(i, jc);
-        load_eb(jc);
-        load_ea(i);
-        finish_ea(i);
-        store_tile(0);
-        __syncthreads();
-
-        // ---- MFMA block over one (i, j-chunk): 4*NQ*RT*CT MFMAs per wavefront
-        auto mfma_block = [&](const float *tile) {
+    // ---- MFMA block over one (i, j-chunk): 4*NQ*RT*CT MFMAs per wavefront
+    auto mfma_block = [&](const float *tile) {
 #pragma unroll
-            for (int q = 0; q < NQ; ++q) {
-                floatx4 af[RT];
+        for (int q = 0; q < NQ; ++q) {
+            floatx4 af[RT];
 #pragma unroll
-                for (int rt = 0; rt < RT; ++rt)
-                    af[rt] = *reinterpret_cast<const floatx4 *>(&tile[(32 * rt + m) * LDW + 8 * q + 4 * h]);
+            for (int rt = 0; rt < RT; ++rt)
+                af[rt] = *reinterpret_cast<const floatx4 *>(&tile[(32 * rt + m) * LDW + 8 * q + 4 * h]);
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
+            for (int u = 0; u < 4; ++u) {
 #pragma unroll
-                    for (int ct = 0; ct < CT; ++ct) {
-                        const float bop = ea[ct][PJ == 2 ? 2 * q + u / 2 : (PJ ? q : 0)] * eb[ct][4 * q + u];
+                for (int ct = 0; ct < CT; ++ct) {
+                    const float bop = ea[ct][PJ == 2 ? 2 * q + u / 2 : (PJ ? q : 0)] * eb[ct][4 * q + u];
 #pragma unroll
-                        for (int rt = 0; rt < RT; ++rt)
-                            acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[rt][u], bop, acc[rt][ct], 0, 0, 0);
-                    }
+                    for (int rt = 0; rt < RT; ++rt)
+                        acc[rt][ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(af[rt][u], bop, acc[rt][ct], 0, 0, 0);
                 }
             }
-        };
+        }
+    };
 
-        // Steady state: every iteration prefetches the next tile unconditionally and
-        // consumes it before the back edge (no load is ever left in flight across the
-        // loop header); the last iteration is peeled.
+    if constexpr (GS == 1) {
+        if (it < it_end) {
+            int jc = it / n_i;
+            int i = it - jc * n_i;
+            load_tile(i, jc);
+            load_eb(jc);
+            load_ea(i);
+            finish_ea(i);
+            store_tile(0);
+            __syncthreads();
+
+            // Steady state: every iteration prefetches the next tile unconditionally and
+            // consumes it before the back edge (no load is ever left in flight across the
+            // loop header); the last iteration is peeled.
+            int cur = 0;
+            for (; it + 1 < it_end; ++it) {
+                int ni = i + 1, njc = jc;
+                if (ni == n_i) {
+                    ni = 0;
+                    njc = jc + 1;
+                }
+                load_tile(ni, njc);
+                load_ea(ni);
+                __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block, not sunk into it
+                mfma_block(wt[cur] + wrow0 * LDW);
+                store_tile(cur ^ 1);
+                if (njc != jc) load_eb(njc);
+                finish_ea(ni);
+                __syncthreads();
+                cur ^= 1;
+                i = ni;
+                jc = njc;
+            }
+            mfma_block(wt[cur] + wrow0 * LDW);
+        }
+    } else {
+        // Paired groups: the same pipeline, with every step guarded by wave-uniform tests so that
+        // both groups meet at every barrier whatever the lengths of their halves.
+        // (Measured and not kept: the barrier in the middle of a step's MFMAs, with the fragments
+        // of the second half read before it and those of the next tile's first half right after
+        // it -- 39.6 us against 38.9 at R=16, S=64, I=J=32, K=2048; with neither stores, loads
+        // nor barriers the same loop takes 36.7 us: the MFMAs and the Khatri-Rao multiplies
+        // alone run at 89 % of the matrix peak.)
+        bool live = it < it_end;
+        int jc = live ? it / n_i : 0;
+        int i = live ? it - jc * n_i : 0;
+        if (live) {
+            load_tile(i, jc);
+            load_eb(jc);
+            load_ea(i);
+            finish_ea(i);
+            store_tile(0);
+        }
+        __syncthreads();
         int cur = 0;
-        for (; it + 1 < it_end; ++it) {
+        for (int t = 0; t + 1 < trips; ++t) {
+            const bool more = it + 1 < it_end;
             int ni = i + 1, njc = jc;
             if (ni == n_i) {
                 ni = 0;
                 njc = jc + 1;
             }
-            load_tile(ni, njc);
-            load_ea(ni);
-            __builtin_amdgcn_sched_barrier(0);  // the prefetch is issued before the MFMA block, not sunk into it
-            mfma_block(wt[cur] + wrow0 * LDW);
-            store_tile(cur ^ 1);
-            if (njc != jc) load_eb(njc);
-            finish_ea(ni);
+            if (more) {
+                load_tile(ni, njc);
+                load_ea(ni);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            if (live) mfma_block(wt[cur] + wrow0 * LDW);
+            if (more) {
+                store_tile(cur ^ 1);
+                if (njc != jc) load_eb(njc);
+                finish_ea(ni);
+            }
             __syncthreads();
             cur ^= 1;
+            ++it;
             i = ni;
             jc = njc;
+            live = more;
         }
-        mfma_block(wt[cur] + wrow0 * LDW);
+        if (live) mfma_block(wt[cur] + wrow0 * LDW);
+
+        // ---- the groups exchange halves of their sums: group g finishes registers 8g .. 8g+7 of
+        // every 32 x 32 block (rows 16g + 4h + {0..3, 8..11}) and hands the other eight over.
+        __syncthreads();  // the tile buffers are free
+        float *xb = &wt_all[0][0][0];
+        static_assert(sizeof(wt_all) >= (size_t)GS * NWAVES * RT * 8 * kWave * sizeof(float), "room for the exchange");
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const float theirs = grp == 0 ? acc[rt][0][8 + v] : acc[rt][0][v];
+                xb[(((grp * NWAVES + wave) * RT + rt) * 8 + v) * kWave + lane] = theirs;
+            }
+        __syncthreads();
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int v = 0; v < 8; ++v) {
+                const float mine = grp == 0 ? acc[rt][0][v] : acc[rt][0][8 + v];
+                acc[rt][0][v] = mine + xb[((((grp ^ 1) * NWAVES + wave) * RT + rt) * 8 + v) * kWave + lane];
+            }
     }
 
     // ---- epilogue.  D layout of 32x32x2: register v of lane (h, m) holds
@@ -372,8 +471,9 @@ __global__ __launch_bounds__(NWAVES *kWave, 2) void lt2exp_kernel(const Lt2Args 
 #pragma unroll
             for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4);  // + 4h in the lane offset
+                for (int v = 0; v < 16 / GS; ++v) {
+                    // (paired groups: register v of group g is accumulator register 8g + v)
+                    const uint32_t trow_c = 32 * rt + 8 * (v / 4) + (v % 4) + (GS == 2 ? 16 * grp : 0);  // + 4h in the lane offset
                     buf_store_f32_out(p.stream_out != 0, log_plus(acc[rt][ct][v], mm), c_rsrc, co,
                                       trow_c * c_row_bytes);
                 }
@@ -386,6 +486,7 @@ struct Lt2Variant {
     int rt, ct, nq;
     int wm = 1;     // wavefronts stacked over rows
     bool pack = false;  // J = 2, 4 or 8: chunks of 16 over the flat (i, j) axis
+    int gs = 1;         // 2: two groups of four wavefronts halve the contraction of one tile between them
 };
 // variant ids (1-based in the C ABI; 0 = choose by shape)
 // (Tiles of two 32-column groups per wavefront -- 64 x 256 and 32 x 256 -- were measured and
@@ -405,6 +506,8 @@ static const Lt2Variant kVariants[] = {
     {1, 1, 4, 2},  // 12: 64 x 64 tile (outputs of <= 64 columns)
     {1, 1, 2, 1, true},  // 13, 14: short rows of w packed into chunks of 16 (other shapes: as 5 and 8)
     {2, 1, 2, 1, true},
+    {1, 1, 4, 1, false, 2},  // 15, 16: tiles 4 and 2 with the contraction halved between two groups of
+    {2, 1, 4, 1, false, 2},  //         wavefronts in the workgroup (grids of one or two tiles per compute unit)
 };
 constexpr int kNumVariants = sizeof(kVariants) / sizeof(kVariants[0]);
 constexpr int kLt2Waves = 4;
@@ -427,10 +530,10 @@ static bool packs(int64_t I, int64_t J) {
     return (J == 2 || J == 4 || J == 8) && (I * J) % 4 == 0 && I * J >= 32;
 }
 
-static int find_lt2_variant(int rt, int nq, bool pack) {
+static int find_lt2_variant(int rt, int nq, bool pack, int gs = 1) {
     for (int v = 0; v < kNumVariants; ++v)
         if (kVariants[v].rt == rt && kVariants[v].ct == 1 && kVariants[v].nq == nq && kVariants[v].wm == 1 &&
-            kVariants[v].pack == pack)
+            kVariants[v].pack == pack && kVariants[v].gs == gs)
             return v;
     return 0;
 }
@@ -526,7 +629,18 @@ static void launch_packed(const Lt2Args &args, bool split, hipStream_t stream) {
     else launch_packed_pj<RT, 2>(args, split, stream);
 }
 
+template <int RT>
+static void launch_paired(const Lt2Args &args, hipStream_t stream) {
+    hipLaunchKernelGGL((lt2exp_kernel<RT, 1, 4, kLt2Waves, true, false, 1, 0, 2>), dim3((unsigned)args.padded_wgs),
+                       dim3(2 * kLt2Waves * kWave), 0, stream, args);
+}
+
 static void launch_variant(int v, const Lt2Args &args, bool vec, bool split, hipStream_t stream) {
+    if (kVariants[v].gs == 2) {  // (the caller has made sure of aligned rows and an uncut contraction)
+        if (kVariants[v].rt == 2) launch_paired<2>(args, stream);
+        else launch_paired<1>(args, stream);
+        return;
+    }
     if (kVariants[v].pack) {
         if (kVariants[v].rt == 2) launch_packed<2>(args, split, stream);
         else launch_packed<1>(args, split, stream);
@@ -553,6 +667,25 @@ struct SplitPlan {
     int splits;
     int iters_per_split;
 };
+static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode, int variant);
+
+// Grids of at most two 32-row tiles per compute unit that are not worth cutting over workgroups
+// (plan_split) run with the contraction halved between two groups of wavefronts of one
+// workgroup instead: 3-27 % faster over 70 random such shapes (R=16, S=64, I=J=32, K=2048: 40.7 ->
+// 38.9 us; R=128, S=128, I=64, J=32, K=128: 77 -> 73; R=16, S=32, I=J=32, K=2048: 26.4 -> 24.2).
+// 64 rows where the contraction is short (I*J <= 1024) and 64-row tiles fill more than half of
+// the CUs, else 32 rows.  Only for aligned rows of w and j-chunks of 32 (the caller checks).
+static int paired_variant(int v, int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode) {
+    const Lt2Variant &vr = kVariants[v];
+    if (mode == TRT_MODE_SPLIT || vr.nq != 4 || vr.pack || vr.wm != 1 || vr.gs != 1) return v;
+    if (plan_split(R, S, I, J, K, mode, v).split) return v;
+    const int64_t ct = ceil_div(K, 128);
+    const int64_t n32 = R * ceil_div(S, 32) * ct, n64 = R * ceil_div(S, 64) * ct;
+    if (n32 > 512 || I * ceil_div(J, 32) < 2) return v;
+    const int64_t last = S % 64;
+    const bool rows64 = I * J <= 1024 && S > 32 && (last == 0 || last > 32) && n64 > 128;
+    return find_lt2_variant(rows64 ? 2 : 1, 4, false, 2);
+}
 
 // AUTO follows the reference in kind -- a small output grid with a long contraction is
 // split (triturus/lt2exp.py:535 tests R*S*K < 1048576 and I*J > 512) -- but decides with a
@@ -561,9 +694,13 @@ struct SplitPlan {
 static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode, int variant) {
     const Lt2Variant &v = kVariants[variant];
     const int64_t iters = v.pack ? ceil_div(I * J, 8 * v.nq) : ceil_div(J, 8 * v.nq) * I;
-    if (mode == TRT_MODE_UNSPLIT) return {false, 1, (int)iters};
+    if (mode == TRT_MODE_UNSPLIT || v.gs == 2) return {false, 1, (int)iters};
     const int64_t base = R * ceil_div(S, 32 * v.rt * v.wm) * ceil_div(K, 32 * v.ct * (kLt2Waves / v.wm));
-    int64_t splits = choose_splits(base, iters, 4 * v.nq * v.rt * v.ct, R * S * K, 4, 32, mode == TRT_MODE_SPLIT);
+    // (the 64-row tile alone on a CU runs at 67 % of the MFMA rate, two of them at 82 %: measured
+    // at R=16 / 32, S=64, I=J=32, K=2048, 40.6 and 66.5 us)
+    const bool tall = v.rt >= 2;
+    int64_t splits = choose_splits(base, iters, 4 * v.nq * v.rt * v.ct, R * S * K, 4, 32, mode == TRT_MODE_SPLIT, 0.0,
+                                   0.8, tall ? 0.67 : 0.45, tall ? 0.82 : 0.65);
     if (splits <= 1) return {false, 1, (int)iters};
     const int64_t per = ceil_div(iters, splits);
     splits = ceil_div(iters, per);
@@ -632,6 +769,10 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     const bool w_aligned = sw[2] == 1 && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
     // packed rows need 16-byte loads along the flat (i, j) axis; any other call runs the same tile unpacked
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
+    if (variant == 0 && (J % 4 == 0) && w_aligned) v = paired_variant(v, R, S, I, J, K, mode);
+    // paired groups: aligned rows only, and never under a forced cut over workgroups
+    if (kVariants[v].gs == 2 && (!((J % 4 == 0) && w_aligned) || mode == TRT_MODE_SPLIT))
+        v = find_lt2_variant(kVariants[v].rt, kVariants[v].nq, false);
     const Lt2Variant &vr = kVariants[v];
     const SplitPlan sp = plan_split(R, S, I, J, K, mode, v);
 
@@ -679,12 +820,15 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
     }
     int v = resolve_variant(variant, R, S, I, J, K);
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
+    if (variant == 0 && (J % 4 == 0) && w_aligned) v = paired_variant(v, R, S, I, J, K, mode);
+    if (kVariants[v].gs == 2 && (!((J % 4 == 0) && w_aligned) || mode == TRT_MODE_SPLIT))
+        v = find_lt2_variant(kVariants[v].rt, kVariants[v].nq, false);
     const Lt2Variant &vr = kVariants[v];
     const SplitPlan sp = plan_split(R, S, I, J, K, mode, v);
     const bool vec = vr.pack || ((J % 4 == 0) && w_aligned);
-    const int n = snprintf(buf, buf_bytes, "trt::lt2exp_kernel<%d, %d, %d, %d, %s, %s, %d, %d>", vr.rt, vr.ct,
+    const int n = snprintf(buf, buf_bytes, "trt::lt2exp_kernel<%d, %d, %d, %d, %s, %s, %d, %d, %d>", vr.rt, vr.ct,
                            vr.pack ? 2 : vr.nq, kLt2Waves, vec ? "true" : "false", sp.split ? "true" : "false", vr.wm,
-                           vr.pack ? (int)J : 0);
+                           vr.pack ? (int)J : 0, vr.gs);
     return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
 }
 
