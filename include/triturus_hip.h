@@ -59,10 +59,12 @@ const char *trt_error_string(int status);
  * c[r,i,k] = log sum_j a[r,i,j] * exp(b[r,j,k])            (fp32)
  * a: R x I x J linear-space, b: R x J x K log-space, c: R x I x K.
  * sa/sb/sc: element strides of the three axes, all non-negative (zero: an
- * expanded operand).  a may have any strides, as the reference forwards them to its
- * kernel (triturus/lm2exp.py:190-198): a transposed or column-strided a is read in
- * place.  The trailing stride of b and c must be 1 (TRT_E_LAYOUT otherwise); their two
- * leading strides are free.  Replaces the `_ker_lm2exp[grid](...)` launch,
+ * expanded operand).  a and b may have any strides, as the reference forwards them to its
+ * kernel (triturus/lm2exp.py:190-198): a transposed or column-strided operand is read in
+ * place (a lane owns a column of b, so its trailing stride only scales the lane's offsets;
+ * fastest with a unit trailing stride, where a half-wave reads 128-byte row segments).  The
+ * trailing stride of c must be 1 (TRT_E_LAYOUT otherwise); its two leading strides are
+ * free.  Replaces the `_ker_lm2exp[grid](...)` launch,
  * triturus/lm2exp.py:186-205; arithmetic contract baselines/lm2exp.py:11-14 (column
  * max clamped to +-1e38, an all -inf column gives -inf, never NaN).
  * variant: 0 = choose by shape; 1..trt_lm2exp_variant_count() force a tile shape and
@@ -88,10 +90,11 @@ int trt_lm2exp_variant_count(void);
  * c[r,s,k] = log sum_{i,j} w[r,s,i,j] * exp(a[r,i,k]) * exp(b[r,j,k])   (fp32)
  * w: R x S x (I*J) linear-space (the reference flattens the two trailing axes
  * with w.view(batch, m, -1), triturus/lt2exp.py:549, so sw has 3 entries),
- * a: R x I x K, b: R x J x K log-space, c: R x S x K.  Trailing strides of a, b
- * and c must be 1; w takes any non-negative strides (a flat axis with another
- * stride than 1 -- a sliced view -- is read in place, element by element; the
- * reference's kernels take the stride too, triturus/lt2exp.py:577-579).  Replaces the `_ker_lt2exp_unsplit[grid](...)` launch,
+ * a: R x I x K, b: R x J x K log-space, c: R x S x K.  The trailing stride of c
+ * must be 1; w, a and b take any non-negative strides, as the reference's kernels do
+ * (triturus/lt2exp.py:577-585, :606-620): a flat axis of w with another stride than 1
+ * -- a sliced view -- is read in place, element by element, and so are transposed or
+ * column-strided a and b (a lane owns a column: the stride scales its offsets).  Replaces the `_ker_lt2exp_unsplit[grid](...)` launch,
  * triturus/lt2exp.py:601-629, and the `_ker_lt2exp_split[grid](...)` launch,
  * triturus/lt2exp.py:564-597; arithmetic contract baselines/lt2exp.py:15-25.
  * mode: TRT_MODE_*.  AUTO decides like the reference does -- by the size of the
@@ -140,7 +143,8 @@ int trt_lt2exp_f32_static(const float *w, const float *a, const float *b, float 
 
 /*
  * The same contraction as trt_lt2exp_f32 (fp32 tensors in and out, same layouts and status
- * codes; every trailing stride, that of w included, must be 1) on the bf16 matrix pipe: every fp32 operand is cut into `pieces` bf16
+ * codes; the trailing strides of w and c must be 1, a and b take any non-negative strides) on
+ * the bf16 matrix pipe: every fp32 operand is cut into `pieces` bf16
  * pieces and a product is the sum of the piece products that matter, accumulated in fp32.
  *   pieces = 2 (TRT_PIECES_BF16X3): 3 MFMAs per product, relative error ~2^-16 per product
  *   pieces = 3 (TRT_PIECES_BF16X6): 6 MFMAs per product, relative error ~2^-23 per product
@@ -168,8 +172,8 @@ size_t trt_lt2exp_bf16_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t 
 
 /*
  * trt_lm2exp_f32 on the bf16 matrix pipe, in the same way (ALLOW_TF32 at
- * triturus/lm2exp.py:152 is the reference's counterpart): same tensors, layouts, strides and
- * status codes; pieces as above.  splits as for trt_lm2exp_f32: 0 = decide by shape, 1 = never,
+ * triturus/lm2exp.py:152 is the reference's counterpart): same tensors, layouts and status
+ * codes (strides as there, except that the trailing stride of a must be 1); pieces as above.  splits as for trt_lm2exp_f32: 0 = decide by shape, 1 = never,
  * > 1 = cut the contraction that many times (capped by its length).  With variant 0, a grid too
  * small to be matrix bound has its contraction cut over workgroups (as the workspace allows) or
  * is handed to trt_lm2exp_f32, so the workspace is the larger of

@@ -68,8 +68,8 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_lm2exp_f32(one, one, one, 0, 1, 1, 1, ok, ok, ok, *tail) == -1
     assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, ok, 99, 0, null, 0, null) == -1
     assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, ok, 0, -1, null, 0, null) == -1
-    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, s3(12, 1, 4), ok, *tail) == -2  # b, c: unit trailing stride
-    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, s3(12, 1, 4), *tail) == -2
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, s3(12, 4, -1), ok, *tail) == -2  # b: any stride but a negative one
+    assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, ok, ok, s3(12, 1, 4), *tail) == -2  # c: unit trailing stride
     assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, s3(12, 4, -1), ok, ok, *tail) == -2
     # a may have any non-negative strides, except under a forced tile that reads rows 16 bytes at a time
     assert lib.trt_lm2exp_f32(one, one, one, 1, 1, 1, 1, s3(12, 1, 4), ok, ok, 1, 0, null, 0, null) == -2
@@ -83,7 +83,8 @@ def test_c_abi_argument_errors_are_statuses():
     args = (1, 1, 1, 1, 1, ok, ok, ok, ok)
     assert lib.trt_lt2exp_f32(one, null, one, one, *args, 0, 0, null, 0, null) == -1
     assert lib.trt_lt2exp_f32(one, one, one, one, *args, 7, 0, null, 0, null) == -1
-    assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, s3(1, 1, 2), ok, 0, 0, null, 0, null) == -2
+    assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, s3(1, 1, -2), ok, 0, 0, null, 0, null) == -2  # a, b: any stride but a negative one
+    assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, s3(1, -1, 1), ok, ok, 0, 0, null, 0, null) == -2
     assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, -1), ok, ok, ok, 0, 0, null, 0, null) == -2
     assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, ok, s3(1, 1, 2), 0, 0, null, 0, null) == -2
     big4 = (2, 8, 16, 16, 64, s3(2048, 256, 1), s3(1024, 64, 1), s3(1024, 64, 1), s3(512, 64, 1))
@@ -110,7 +111,8 @@ def test_c_abi_argument_errors_are_statuses():
     nv = lib.trt_lm2exp_bf16_variant_count()
     assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, ok, ok, 2, nv + 1, 0, null, 0, null) == -1
     assert lib.trt_lm2exp_bf16(one, null, one, 1, 1, 1, 1, ok, ok, ok, 3, *mtail) == -1
-    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, s3(4, 1, 2), ok, 2, *mtail) == -2
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, s3(4, 1, -2), ok, 2, *mtail) == -2  # b: any stride but a negative one
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, s3(4, 1, 2), ok, ok, 2, *mtail) == -2  # a: unit trailing stride on this pipe
     assert lib.trt_lm2exp_bf16(one, one, one, 1, 2, 2, 8, ok, ok, s3(16, 4, 1), 2, *mtail) == -2
     assert lib.trt_lm2exp_bf16(one, one, one, 1, 1 << 30, 1, 1, ok, ok, ok, 2, *mtail) == -4
     assert lib.trt_lm2exp_bf16(one, one, one, 1, 1024, 1024, 1024, big, big, big, 2, 0, 4, null, 0, null) == -3

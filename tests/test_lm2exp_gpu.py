@@ -7,6 +7,8 @@ against the fp32 torch recipe."""
 
 from pathlib import Path
 
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -292,6 +294,70 @@ def test_views_of_a_are_read_in_place(dev, shape):
     out = lm2exp(ag, bg)
     assert torch.cuda.memory_allocated() - before <= out.numel() * 4 + 1024
     assert oracle64.compare(out, oracle64.lm2exp64(a1.expand(R, I, J), b))["ok"]
+
+
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+@pytest.mark.parametrize("shape", [(2, 256, 64, 128), (3, 300, 50, 129), (2, 70, 333, 40), (1, 130, 18, 257), (5, 16, 33, 7),
+                                   (2, 256, 256, 384)])  # the last one: the paired-wavefront tile
+def test_views_of_b_are_read_in_place(dev, shape, precision):
+    """The log-space operand with a trailing stride other than 1 -- transposed (J contiguous),
+    every other column of a wider tensor, one column expanded over K -- is read where it lies, as
+    the reference forwards every stride to its kernel (triturus/lm2exp.py:190-198): the call may
+    allocate its output (and the workspace of a cut contraction) and nothing else."""
+    R, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(R, I, J, generator=g)
+    b = -5 + 4 * torch.randn(R, J, K, generator=g)
+    b[torch.rand(b.shape, generator=g) < 0.1] = NINF
+    b[0, :, K // 2] = NINF
+    ref = oracle64.lm2exp64(a, b)
+    gate = {"rtol": 1e-4, "atol": 5e-5} if precision == "bf16x3" else {}
+    ag = a.to(dev)
+    wide = torch.zeros(R, J, 2 * K + 1)
+    wide[:, :, 1::2] = b
+    views = {
+        "transposed": b.transpose(1, 2).contiguous().to(dev).transpose(1, 2),
+        "every other column": wide.to(dev)[:, :, 1::2],
+        "batch first in memory": b.permute(1, 2, 0).contiguous().to(dev).permute(2, 0, 1),
+    }
+    if R == 1:
+        del views["batch first in memory"]
+    lib = _lib.load()
+    pieces = {"fp32": 0, "bf16x3": 2, "bf16x6": 3}[precision]
+    ws_bytes = lib.trt_lm2exp_workspace_bytes(R, I, J, K, 0, 0)
+    if pieces:
+        ws_bytes = max(ws_bytes, lib.trt_lm2exp_bf16_workspace_bytes(R, I, J, K, pieces, 0))
+    for name, bg in views.items():
+        assert bg.stride(2) != 1 and torch.equal(bg.cpu(), b), name
+        lm2exp(ag, bg, _precision=precision)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        out = lm2exp(ag, bg, _precision=precision)
+        grown = torch.cuda.memory_allocated() - before
+        r = oracle64.compare(out, ref, **gate)
+        assert r["ok"], (name, r)
+        assert grown <= out.numel() * 4 + ws_bytes + 2048, (name, grown, out.numel() * 4, ws_bytes)
+    # one column of b for every k (stride 0): every output column is the same
+    b1 = b[:, :, 1:2]
+    out = lm2exp(ag, b1.to(dev).expand(R, J, K), _precision=precision)
+    assert oracle64.compare(out, oracle64.lm2exp64(a, b1.expand(R, J, K)), **gate)["ok"]
+
+
+def test_c_abi_takes_a_strided_b(dev):
+    """trt_lm2exp_f32 itself (no Python wrapper in between) with sb[2] != 1."""
+    lib = _lib.load()
+    R, I, J, K = 2, 96, 40, 200
+    g = torch.Generator().manual_seed(5)
+    a = torch.rand(R, I, J, generator=g)
+    bt = torch.randn(R, K, J, generator=g) * 3   # b[r, j, k] = bt[r, k, j]
+    ag, btg = a.to(dev), bt.to(dev)
+    c = torch.empty(R, I, K, device=dev)
+    s3 = ctypes.c_int64 * 3
+    with _lib.on_device(dev):
+        st = lib.trt_lm2exp_f32(ag.data_ptr(), btg.data_ptr(), c.data_ptr(), R, I, J, K, s3(I * J, J, 1),
+                                s3(K * J, 1, J), s3(I * K, K, 1), 0, 1, None, 0, _lib.raw_stream(dev))
+    assert st == 0
+    assert oracle64.compare(c, oracle64.lm2exp64(a, bt.transpose(1, 2)))["ok"]
 
 
 def test_algebraic_properties_on_the_gpu(dev):

@@ -200,7 +200,7 @@ def test_strided_inputs(dev):
     w, a, b = w_big[sl], a_big[::2, :, 7:90], b_big[::2, 10:30, 7:90]
     out = lt2exp(w_big.to(dev)[sl], a_big.to(dev)[::2, :, 7:90], b_big.to(dev)[::2, 10:30, 7:90])
     _check(out, w, a, b)
-    # inner-strided log operands are materialised by the wrapper
+    # log-space operands with a trailing stride other than 1 are read in place as well
     at = torch.randn(2, 83, 12, generator=g)
     out = lt2exp(w_big.to(dev)[sl], at.to(dev).transpose(1, 2), b_big.to(dev)[::2, 10:30, 7:90])
     _check(out, w, at.transpose(1, 2), b)
@@ -247,6 +247,80 @@ def test_views_of_w_are_read_in_place(dev, shape, mode):
     # on the bf16 matrix pipe the wrapper materialises such a view: same result as from a dense w
     dense = lt2exp(w.to(dev), ag, bg, mode=mode, _precision="bf16x6")
     assert torch.equal(lt2exp(views["every other element"], ag, bg, mode=mode, _precision="bf16x6"), dense)
+
+
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
+@pytest.mark.parametrize("mode", ["unsplit", "split"])
+@pytest.mark.parametrize("shape", [(2, 70, 12, 20, 130), (3, 33, 7, 5, 64), (1, 200, 4, 8, 40), (2, 64, 40, 1, 256),
+                                   (2, 64, 32, 32, 256), (4, 64, 64, 64, 512)])  # the last two: paired wavefront groups
+def test_views_of_a_and_b_are_read_in_place(dev, shape, mode, precision):
+    """The log-space operands with trailing strides other than 1 -- transposed (the contracted
+    axis contiguous), every other column of a wider tensor, batch innermost -- are read where they
+    lie, as the reference forwards every stride to its kernels (triturus/lt2exp.py:606-620): the
+    call may allocate its output and its workspace and nothing else."""
+    R, S, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    w = torch.rand(R, S, I, J, generator=g)
+    a = 3 * torch.randn(R, I, K, generator=g)
+    b = -2 + 3 * torch.randn(R, J, K, generator=g)
+    a[torch.rand(a.shape, generator=g) < 0.05] = NINF
+    b[0, :, K // 3] = NINF
+    ref = oracle64.lt2exp64(w, a, b)
+    gate = PRECISION_GATES.get(precision, {})
+    wg = w.to(dev)
+    wide_a = torch.zeros(R, I, 2 * K + 1)
+    wide_a[:, :, 1::2] = a
+    pairs = {
+        "both transposed": (a.transpose(1, 2).contiguous().to(dev).transpose(1, 2),
+                            b.transpose(1, 2).contiguous().to(dev).transpose(1, 2)),
+        "a every other column, b batch first in memory": (wide_a.to(dev)[:, :, 1::2],
+                                                          b.permute(1, 2, 0).contiguous().to(dev).permute(2, 0, 1)),
+        "a dense, b one column for all": (a.to(dev), None),
+    }
+    lib = _lib.load()
+    mode_code = {"unsplit": _lib.MODE_UNSPLIT, "split": _lib.MODE_SPLIT}[mode]
+    pieces = {"fp32": 0, "bf16x3": 2, "bf16x6": 3}[precision]
+    ws = lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, mode_code)
+    if pieces:
+        ws = max(ws, lib.trt_lt2exp_bf16_workspace_bytes(R, S, I, J, K, pieces, mode_code))
+    for name, (ag, bg) in pairs.items():
+        want = ref
+        if bg is None:
+            b1 = b[:, :, 1:2]
+            bg = b1.to(dev).expand(R, J, K)
+            want = oracle64.lt2exp64(w, a, b1.expand(R, J, K))
+        elif R > 1 or "batch" not in name:
+            assert ag.stride(2) != 1 or bg.stride(2) != 1, name
+        lt2exp(wg, ag, bg, mode=mode, _precision=precision)
+        torch.cuda.synchronize()
+        before = torch.cuda.memory_allocated()
+        out = lt2exp(wg, ag, bg, mode=mode, _precision=precision)
+        grown = torch.cuda.memory_allocated() - before
+        r = oracle64.compare(out, want, **gate)
+        assert r["ok"], (name, r)
+        if J >= 4:  # (shorter rows of w may be padded or exchanged on copies by the wrapper: not this test's subject)
+            assert grown <= out.numel() * 4 + ws + 2048, (name, grown, out.numel() * 4, ws)
+
+
+def test_c_abi_takes_strided_a_and_b(dev):
+    """trt_lt2exp_f32 itself (no Python wrapper in between) with sa[2] != 1 and sb[2] != 1."""
+    import ctypes
+
+    lib = _lib.load()
+    R, S, I, J, K = 2, 40, 6, 20, 150
+    g = torch.Generator().manual_seed(6)
+    w = torch.rand(R, S, I, J, generator=g)
+    at = torch.randn(R, K, I, generator=g) * 3      # a[r, i, k] = at[r, k, i]
+    b2 = torch.randn(R, J, 2 * K, generator=g) * 3  # b = every other column of b2
+    wg, atg, b2g = w.to(dev), at.to(dev), b2.to(dev)
+    c = torch.empty(R, S, K, device=dev)
+    s3 = ctypes.c_int64 * 3
+    with _lib.on_device(dev):
+        st = lib.trt_lt2exp_f32(wg.data_ptr(), atg.data_ptr(), b2g.data_ptr(), c.data_ptr(), R, S, I, J, K,
+                                s3(S * I * J, I * J, 1), s3(K * I, 1, I), s3(J * 2 * K, 2 * K, 2), s3(S * K, K, 1),
+                                _lib.MODE_UNSPLIT, 0, None, 0, _lib.raw_stream(dev))
+    assert st == 0
+    _check(c, w, at.transpose(1, 2), b2[:, :, ::2])
 
 
 def test_reduces_to_lm2exp_and_factorises(dev):

@@ -43,6 +43,7 @@ struct Lm2Args {
     int R, I, J, K;
     int64_t sa0, sa1, sb0, sb1, sc0, sc1;
     int64_t sa2;  // trailing stride of a (1 for every kernel but the paired-wavefront one)
+    int64_t sb2;  // trailing stride of b: a lane owns a column, so it only scales the lane offsets
     int i_tiles, n_tiles, splits, chunks_per_split;
     int stream_out;  // rows of c are 16-byte aligned: non-temporal result stores
     int64_t total_wgs, padded_wgs;
@@ -109,7 +110,7 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     for (int ct = 0; ct < CT; ++ct) {
         ncol[ct] = n0 + 32 * ct + m;
         ncl[ct] = ncol[ct] < p.K ? ncol[ct] : p.K - 1;
-        boff[ct] = ((uint32_t)(4 * h) * (uint32_t)p.sb1 + (uint32_t)ncl[ct]) * 4u;
+        boff[ct] = ((uint32_t)(4 * h) * (uint32_t)p.sb1 + (uint32_t)ncl[ct] * (uint32_t)p.sb2) * 4u;
     }
     const float *ar = p.a + (int64_t)r * p.sa0;
     const float *br = p.b + (int64_t)r * p.sb0;
@@ -229,7 +230,8 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     // every VALU instruction in the steady state costs matrix throughput: addresses
     // are kept in scalar registers and exp/log use the bare hardware instructions.
     float braw[CT][NB], eb[CT][NB];
-    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(br, (uint32_t)(((int64_t)(p.J - 1) * p.sb1 + p.K) * 4));
+    const __amdgpu_buffer_rsrc_t b_rsrc =
+        make_rsrc(br, (uint32_t)(((int64_t)(p.J - 1) * p.sb1 + (int64_t)(p.K - 1) * p.sb2 + 1) * 4));
     const uint32_t b_row_bytes = (uint32_t)p.sb1 * 4u;
     auto load_b_full = [&](int jc) {
 #pragma unroll
@@ -817,14 +819,14 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     if (!a || !b || !c || !sa || !sb || !sc) return TRT_E_INVALID;
     if (R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (variant < 0 || variant > kNumVariants || splits < 0) return TRT_E_INVALID;
-    if (sb[2] != 1 || sc[2] != 1 || sa[2] < 0) return TRT_E_LAYOUT;
+    if (sc[2] != 1 || sa[2] < 0 || sb[2] < 0) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     if (sc[1] < K || sc[0] < 0) return TRT_E_LAYOUT;  // output rows must not overlap (stores rely on it)
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || I >= lim || J >= lim || K >= lim) return TRT_E_RANGE;
     // byte offsets inside one batch slab of a, b and c are 32-bit (buffer addressing)
-    if (J * sb[1] + K >= lim || I * sa[1] + J * sa[2] >= lim || I * sc[1] + K >= lim || I * K >= lim)
+    if (J * sb[1] + K * sb[2] >= lim || I * sa[1] + J * sa[2] >= lim || I * sc[1] + K >= lim || I * K >= lim)
         return TRT_E_RANGE;
 
     Lm2Plan pl = make_plan(R, I, J, K, variant, splits);
@@ -854,6 +856,7 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     args.sb0 = sb[0]; args.sb1 = sb[1];
     args.sc0 = sc[0]; args.sc1 = sc[1];
     args.sa2 = sa[2];
+    args.sb2 = sb[2];
     args.i_tiles = (int)ceil_div(I, 32 * vr.rt * vr.wm);
     args.n_tiles = (int)ceil_div(K, 32 * vr.ct * vr.wn);
     args.splits = pl.splits;
@@ -1010,6 +1013,7 @@ extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, i
     args.sb0 = k * n; args.sb1 = n;
     args.sc0 = m * n; args.sc1 = n;
     args.sa2 = 1;
+    args.sb2 = 1;
     args.i_tiles = (int)ceil_div(m, 32 * rt);
     args.n_tiles = (int)ceil_div(n, 128);
     args.splits = 1;

@@ -31,6 +31,7 @@ struct Lm2BfArgs {
     float *shift;  // splits > 1: [splits][R][K] the shift each partial sum is relative to
     int R, I, J, K;
     int64_t sa0, sa1, sb0, sb1, sc0, sc1;
+    int64_t sb2;  // trailing stride of b (a lane owns a column: it only scales the lane offsets)
     int i_tiles, n_tiles, splits, chunks_per_split;
     int stream_out;  // rows of c are 16-byte aligned: non-temporal result stores
     int64_t total_wgs, padded_wgs;
@@ -176,9 +177,10 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 
     // ---- b chunk: global -> registers; rows past J read as -inf
     float braw[KS][8];
-    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(br, (uint32_t)(((int64_t)(p.J - 1) * p.sb1 + p.K) * 4));
+    const __amdgpu_buffer_rsrc_t b_rsrc =
+        make_rsrc(br, (uint32_t)(((int64_t)(p.J - 1) * p.sb1 + (int64_t)(p.K - 1) * p.sb2 + 1) * 4));
     const uint32_t b_row_bytes = (uint32_t)p.sb1 * 4u;
-    const uint32_t boff = ((uint32_t)(8 * h) * (uint32_t)p.sb1 + (uint32_t)ncl) * 4u;
+    const uint32_t boff = ((uint32_t)(8 * h) * (uint32_t)p.sb1 + (uint32_t)ncl * (uint32_t)p.sb2) * 4u;
     auto load_b = [&](int jc) {
         if (jc * JC + JC <= p.J) {  // wave-uniform: a full chunk needs no masks
 #pragma unroll
@@ -423,14 +425,14 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     if (R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
     if (variant < 0 || variant > kNumLmBfVariants || splits < 0) return TRT_E_INVALID;
-    if (sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
+    if (sa[2] != 1 || sb[2] < 0 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     if (sc[1] < K) return TRT_E_LAYOUT;  // output rows must not overlap
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || I >= lim || J >= lim || K >= lim) return TRT_E_RANGE;
     // byte offsets inside one batch slab are 32-bit (buffer addressing)
-    if (I * sa[1] + J >= lim || J * sb[1] + K >= lim || I * sc[1] + K >= lim) return TRT_E_RANGE;
+    if (I * sa[1] + J >= lim || J * sb[1] + K * sb[2] >= lim || I * sc[1] + K >= lim) return TRT_E_RANGE;
 
     // Tile and hand-over rules, fitted to 223 random shapes (R 1..256, I, J 16..1024, K 64..8192)
     // timed with every tile and on the fp32 path; against the best of those the rules below lose
@@ -506,7 +508,7 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     args.a = a; args.b = b; args.c = c;
     args.R = (int)R; args.I = (int)I; args.J = (int)J; args.K = (int)K;
     args.sa0 = sa[0]; args.sa1 = sa[1];
-    args.sb0 = sb[0]; args.sb1 = sb[1];
+    args.sb0 = sb[0]; args.sb1 = sb[1]; args.sb2 = sb[2];
     args.sc0 = sc[0]; args.sc1 = sc[1];
     args.i_tiles = (int)ceil_div(I, 32 * vr.rt);
     args.n_tiles = (int)ceil_div(K, 128);
@@ -570,7 +572,7 @@ extern "C" int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, 
     args.a = a; args.b = b; args.c = c;
     args.R = 1; args.I = (int)m; args.J = (int)k; args.K = (int)n;
     args.sa0 = m * k; args.sa1 = k;
-    args.sb0 = k * n; args.sb1 = n;
+    args.sb0 = k * n; args.sb1 = n; args.sb2 = 1;
     args.sc0 = m * n; args.sc1 = n;
     args.i_tiles = (int)ceil_div(m, 32 * rt);
     args.n_tiles = (int)ct;

@@ -98,7 +98,8 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
     const int jbeg = jc0 * JC;
     const int jend = jc1 * JC < p.J ? jc1 * JC : p.J;
 
-    const __amdgpu_buffer_rsrc_t b_rsrc = make_rsrc(br, (uint32_t)(((int64_t)(p.J - 1) * p.sb1 + p.K) * 4));
+    const __amdgpu_buffer_rsrc_t b_rsrc =
+        make_rsrc(br, (uint32_t)(((int64_t)(p.J - 1) * p.sb1 + (int64_t)(p.K - 1) * p.sb2 + 1) * 4));
     const uint32_t b_row_bytes = (uint32_t)p.sb1 * 4u;
 
     // ---- column maxima of rows [jbeg, jend): the four (wm, h) classes take every fourth row.
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
     // a workgroup starts with overlap.)
     float msh = 0.f;  // the shift: the clamped column maximum
     auto find_shift = [&]() {
-        const uint32_t poff = ((uint32_t)h * (uint32_t)p.sb1 + (uint32_t)ncl) * 4u;
+        const uint32_t poff = ((uint32_t)h * (uint32_t)p.sb1 + (uint32_t)ncl * (uint32_t)p.sb2) * 4u;
         float x0 = -__builtin_inff(), x1 = x0;
         int j = jbeg + 2 * wm;  // wave-uniform: this lane reads row j + h
         // 64 loads in flight per lane (256 rows of the panel per step), then 8 at a time: the
@@ -233,7 +234,7 @@ __global__ __launch_bounds__(128 * WN, 4) void lm2exp_pair_kernel(const Lm2Args 
 
     // ---- b: this wavefront's half of a chunk, rows 8 (wm NH + qq) + 4h + u, column ncl, raw,
     // two chunks ahead (two register sets that swap roles from step to step)
-    const uint32_t boff = ((uint32_t)(4 * h) * (uint32_t)p.sb1 + (uint32_t)ncl) * 4u;
+    const uint32_t boff = ((uint32_t)(4 * h) * (uint32_t)p.sb1 + (uint32_t)ncl * (uint32_t)p.sb2) * 4u;
     auto load_b = [&](float (&raw)[NB], int jc, bool masked) {
 #pragma unroll
         for (int qq = 0; qq < NH; ++qq)

@@ -33,6 +33,7 @@ struct Lt2Args {
     float *shift;     // split only: [2][R][K] clamped column maxima
     int R, S, I, J, K;
     int64_t sw0, sw1, sw2, sa0, sa1, sb0, sb1, sc0, sc1;  // sw2: stride of the flat (i, j) axis of w
+    int64_t sa2, sb2;  // trailing strides of a and b: a lane owns a column, so they only scale lane offsets
     int s_tiles, n_tiles, splits;
     int iters_per_split;  // (j-chunk, i) iterations per split
     int stream_out;       // rows of c are 16-byte aligned: non-temporal result stores
@@ -117,11 +118,11 @@ __global__ __launch_bounds__(NWAVES *kWave *GS, 2 * GS) void lt2exp_kernel(const
     for (int ct = 0; ct < CT; ++ct) {
         float x = -__builtin_inff();
 #pragma unroll 8
-        for (int i = 2 * grp + h; i < p.I; i += 2 * GS) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + ncl[ct]]);
+        for (int i = 2 * grp + h; i < p.I; i += 2 * GS) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + (int64_t)ncl[ct] * p.sa2]);
         x = __builtin_fmaxf(x, __shfl_xor(x, 32, kWave));
         float y = -__builtin_inff();
 #pragma unroll 8
-        for (int j = 2 * grp + h; j < p.J; j += 2 * GS) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + ncl[ct]]);
+        for (int j = 2 * grp + h; j < p.J; j += 2 * GS) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + (int64_t)ncl[ct] * p.sb2]);
         y = __builtin_fmaxf(y, __shfl_xor(y, 32, kWave));
         if (GS == 2) {
             // each group has swept half of the rows: the halves meet in LDS (the tile buffers are
@@ -257,11 +258,12 @@ __global__ __launch_bounds__(NWAVES *kWave *GS, 2 * GS) void lt2exp_kernel(const
     };
 
     // a rows for the scalar factor exp(a[i,n] - ma[n]): same addressing scheme
-    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ar, (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + p.K) * 4));
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        make_rsrc(ar, (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + (int64_t)(p.K - 1) * p.sa2 + 1) * 4));
     const uint32_t a_row_bytes = (uint32_t)p.sa1 * 4u;
     uint32_t aoff[CT];
 #pragma unroll
-    for (int ct = 0; ct < CT; ++ct) aoff[ct] = (uint32_t)ncl[ct] * 4u;
+    for (int ct = 0; ct < CT; ++ct) aoff[ct] = (uint32_t)ncl[ct] * (uint32_t)p.sa2 * 4u;
 
     float eb[CT][4 * NQ];
     auto load_eb = [&](int jc) {
@@ -273,7 +275,7 @@ __global__ __launch_bounds__(NWAVES *kWave *GS, 2 * GS) void lt2exp_kernel(const
                 for (int u = 0; u < 4; ++u) {
                     const int j = PJ ? (8 * q + 4 * h + u) % (PJ ? PJ : 1) : jc * JC + 8 * q + 4 * h + u;
                     float raw = -__builtin_inff();
-                    if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl[ct]];
+                    if (j < p.J) raw = br[(int64_t)j * p.sb1 + (int64_t)ncl[ct] * p.sb2];
                     eb[ct][4 * q + u] = exp_shifted(raw - mb[ct]);
                 }
     };
@@ -748,14 +750,16 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     if (R <= 0 || S <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (mode != TRT_MODE_AUTO && mode != TRT_MODE_SPLIT && mode != TRT_MODE_UNSPLIT) return TRT_E_INVALID;
     if (variant < 0 || variant > kNumVariants) return TRT_E_INVALID;
-    if (sw[2] < 0 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
+    if (sw[2] < 0 || sa[2] < 0 || sb[2] < 0 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     if (sc[1] < K) return TRT_E_LAYOUT;  // output rows must not overlap (stores rely on it)
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
     // byte offsets inside one batch slab of w, a and c are 32-bit (buffer addressing)
-    if (S * sw[1] + I * J * (sw[2] > 0 ? sw[2] : 1) >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
+    if (S * sw[1] + I * J * (sw[2] > 0 ? sw[2] : 1) >= lim || I * sa[1] + K * sa[2] >= lim ||
+        J * sb[1] + K * sb[2] >= lim || S * sc[1] + K >= lim)
+        return TRT_E_RANGE;
 
     // A single j under several i: the contraction is symmetric in (i, a) and (j, b), and with
     // J = 1 the same w is an R x S x 1 x I tensor, so the call runs with the roles exchanged
@@ -780,8 +784,8 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     args.w = w; args.a = a; args.b = b;
     args.R = (int)R; args.S = (int)S; args.I = (int)I; args.J = (int)J; args.K = (int)K;
     args.sw0 = sw[0]; args.sw1 = sw[1]; args.sw2 = sw[2];
-    args.sa0 = sa[0]; args.sa1 = sa[1];
-    args.sb0 = sb[0]; args.sb1 = sb[1];
+    args.sa0 = sa[0]; args.sa1 = sa[1]; args.sa2 = sa[2];
+    args.sb0 = sb[0]; args.sb1 = sb[1]; args.sb2 = sb[2];
     args.sc0 = sc[0]; args.sc1 = sc[1];
     args.s_tiles = (int)ceil_div(S, 32 * vr.rt * vr.wm);
     args.n_tiles = (int)ceil_div(K, 32 * vr.ct * (kLt2Waves / vr.wm));

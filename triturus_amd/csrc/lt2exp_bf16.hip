@@ -34,6 +34,7 @@ struct Lt2BfArgs {
     float *shift;  // split only: [2][R][K] clamped column maxima
     int R, S, I, J, K;
     int64_t sw0, sw1, sa0, sa1, sb0, sb1, sc0, sc1;
+    int64_t sa2, sb2;  // trailing strides of a and b (a lane owns a column: they only scale lane offsets)
     int s_tiles, n_tiles, splits;
     int iters_per_split;  // (j-chunk, i) iterations per split
     int stream_out;       // rows of c are 16-byte aligned: non-temporal result stores
@@ -85,12 +86,12 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     // alternate rows and exchange once
     float x = -__builtin_inff();
 #pragma unroll 8
-    for (int i = h; i < p.I; i += 2) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + ncl]);
+    for (int i = h; i < p.I; i += 2) x = __builtin_fmaxf(x, ar[(int64_t)i * p.sa1 + (int64_t)ncl * p.sa2]);
     x = __builtin_fmaxf(x, __shfl_xor(x, 32, kWave));
     const float ma = clamp_shift(x);
     float y = -__builtin_inff();
 #pragma unroll 8
-    for (int j = h; j < p.J; j += 2) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + ncl]);
+    for (int j = h; j < p.J; j += 2) y = __builtin_fmaxf(y, br[(int64_t)j * p.sb1 + (int64_t)ncl * p.sb2]);
     y = __builtin_fmaxf(y, __shfl_xor(y, 32, kWave));
     const float mb = clamp_shift(y);
 
@@ -207,9 +208,10 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
         }
     };
 
-    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ar, (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + p.K) * 4));
+    const __amdgpu_buffer_rsrc_t a_rsrc =
+        make_rsrc(ar, (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + (int64_t)(p.K - 1) * p.sa2 + 1) * 4));
     const uint32_t a_row_bytes = (uint32_t)p.sa1 * 4u;
-    const uint32_t aoff = (uint32_t)ncl * 4u;
+    const uint32_t aoff = (uint32_t)ncl * (uint32_t)p.sa2 * 4u;
 
     // B operand: exp(b[j,n] - mb[n]) of the current j-chunk, split, in MFMA layout
     uintx4 ebp[NS][KS];
@@ -221,7 +223,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
             for (int u = 0; u < 8; ++u) {
                 const int j = jc * JC + 16 * ks + 8 * h + u;
                 float raw = -__builtin_inff();
-                if (j < p.J) raw = br[(int64_t)j * p.sb1 + ncl];
+                if (j < p.J) raw = br[(int64_t)j * p.sb1 + (int64_t)ncl * p.sb2];
                 e[u] = exp_shifted(raw - mb);
             }
 #pragma unroll
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
         int i = it0 - jc * p.I;
         load_tile(i, jc);
         load_eb(jc);
-        float ea = exp_shifted(ar[(int64_t)i * p.sa1 + ncl] - ma);
+        float ea = exp_shifted(ar[(int64_t)i * p.sa1 + (int64_t)ncl * p.sa2] - ma);
         float ea_raw;
         store_tile(0);
         __syncthreads();
@@ -494,13 +496,14 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
     if (mode != TRT_MODE_AUTO && mode != TRT_MODE_SPLIT && mode != TRT_MODE_UNSPLIT) return TRT_E_INVALID;
     if (variant < 0 || variant > 16) return TRT_E_INVALID;
-    if (sw[2] != 1 || sa[2] != 1 || sb[2] != 1 || sc[2] != 1) return TRT_E_LAYOUT;
+    if (sw[2] != 1 || sa[2] < 0 || sb[2] < 0 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     if (sc[1] < K) return TRT_E_LAYOUT;
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
-    if (S * sw[1] + I * J >= lim || I * sa[1] + K >= lim || S * sc[1] + K >= lim) return TRT_E_RANGE;
+    if (S * sw[1] + I * J >= lim || I * sa[1] + K * sa[2] >= lim || J * sb[1] + K * sb[2] >= lim || S * sc[1] + K >= lim)
+        return TRT_E_RANGE;
 
     // a single j under several i: run with the roles of (i, a) and (j, b) exchanged (see trt_lt2exp_f32)
     if (J == 1 && I > 1 && variant == 0)
@@ -591,8 +594,8 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     }
     args.R = (int)R; args.S = (int)S; args.I = (int)I; args.J = (int)J; args.K = (int)K;
     args.sw0 = sw[0]; args.sw1 = sw[1];
-    args.sa0 = sa[0]; args.sa1 = sa[1];
-    args.sb0 = sb[0]; args.sb1 = sb[1];
+    args.sa0 = sa[0]; args.sa1 = sa[1]; args.sa2 = sa[2];
+    args.sb0 = sb[0]; args.sb1 = sb[1]; args.sb2 = sb[2];
     args.sc0 = sc[0]; args.sc1 = sc[1];
     args.s_tiles = (int)ceil_div(S, 32 * rt);
     args.n_tiles = (int)ceil_div(K, 128);

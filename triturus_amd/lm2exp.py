@@ -72,15 +72,18 @@ def lm2exp(
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
     fp32 = _precision == "fp32"
-    # a goes to the fp32 kernels with whatever non-negative strides it has (a transposed or
-    # strided view is read in place, as the reference does: triturus/lm2exp.py:190-198); the
-    # bf16 kernels and every kernel's b want a unit trailing stride
+    # Operands go to the kernels with whatever non-negative strides they have, as the reference
+    # forwards them (triturus/lm2exp.py:190-198): b in every kernel (a lane owns a column of b,
+    # so a trailing stride only scales its offsets), a in the fp32 kernels (the paired-wavefront
+    # tiles read a transposed or strided a in place; a forced tile of another family and the
+    # bf16 kernels want unit-stride rows of a).  Only negative strides always need a copy.
     sa, sb = a.stride(), b.stride()
-    if (not fp32 and sa[2] != 1) or min(sa) < 0:
+    pair_tile = _variant == 0 or _variant > lib.trt_lm2exp_variant_count() - 5
+    if ((not fp32 or not pair_tile) and sa[2] != 1) or min(sa) < 0:
         a = _unit_inner(a)
         sa = a.stride()
-    if sb[2] != 1 or min(sb) < 0:
-        b = _unit_inner(b)
+    if min(sb) < 0:
+        b = b.contiguous()
         sb = b.stride()
     if _variant == 0 and _splits == 0 and sa[2] == 1 and autotune.is_autotune_enabled():
         cands = _FP32_CANDIDATES if fp32 else _BF16_CANDIDATES

@@ -132,11 +132,13 @@ def lt2exp(
     if min(sw) < 0 or (sw[2] != 1 and _precision != "fp32"):
         w = _unit_inner(w)
         sw = w.stride()
-    if sa[2] != 1 or min(sa) < 0:
-        a = _unit_inner(a)
+    # a and b are read in place whatever their strides, as the reference forwards them
+    # (triturus/lt2exp.py:606-620): a lane owns a column, so a trailing stride only scales its offsets
+    if min(sa) < 0:
+        a = a.contiguous()
         sa = a.stride()
-    if sb[2] != 1 or min(sb) < 0:
-        b = _unit_inner(b)
+    if min(sb) < 0:
+        b = b.contiguous()
         sb = b.stride()
     if _variant == 0 and autotune.is_autotune_enabled() and not _tuning:
         cands = _FP32_CANDIDATES if _precision == "fp32" else _BF16_CANDIDATES
