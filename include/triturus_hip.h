@@ -143,8 +143,7 @@ int trt_lt2exp_f32_static(const float *w, const float *a, const float *b, float 
 
 /*
  * The same contraction as trt_lt2exp_f32 (fp32 tensors in and out, same layouts and status
- * codes; the trailing strides of w and c must be 1, a and b take any non-negative strides) on
- * the bf16 matrix pipe: every fp32 operand is cut into `pieces` bf16
+ * codes and strides) on the bf16 matrix pipe: every fp32 operand is cut into `pieces` bf16
  * pieces and a product is the sum of the piece products that matter, accumulated in fp32.
  *   pieces = 2 (TRT_PIECES_BF16X3): 3 MFMAs per product, relative error ~2^-16 per product
  *   pieces = 3 (TRT_PIECES_BF16X6): 6 MFMAs per product, relative error ~2^-23 per product
@@ -172,8 +171,8 @@ size_t trt_lt2exp_bf16_workspace_bytes(int64_t R, int64_t S, int64_t I, int64_t 
 
 /*
  * trt_lm2exp_f32 on the bf16 matrix pipe, in the same way (ALLOW_TF32 at
- * triturus/lm2exp.py:152 is the reference's counterpart): same tensors, layouts and status
- * codes (strides as there, except that the trailing stride of a must be 1); pieces as above.  splits as for trt_lm2exp_f32: 0 = decide by shape, 1 = never,
+ * triturus/lm2exp.py:152 is the reference's counterpart): same tensors, layouts, strides and
+ * status codes; pieces as above.  splits as for trt_lm2exp_f32: 0 = decide by shape, 1 = never,
  * > 1 = cut the contraction that many times (capped by its length).  With variant 0, a grid too
  * small to be matrix bound has its contraction cut over workgroups (as the workspace allows) or
  * is handed to trt_lm2exp_f32, so the workspace is the larger of

@@ -101,7 +101,8 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 2, 0, 17, null, 0, null) == -1
     assert lib.trt_lt2exp_bf16(one, one, one, one, *args, 2, 5, 0, null, 0, null) == -1
     assert lib.trt_lt2exp_bf16(null, one, one, one, *args, 2, *btail) == -1
-    assert lib.trt_lt2exp_bf16(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, 2), ok, ok, ok, 2, *btail) == -2
+    assert lib.trt_lt2exp_bf16(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, -2), ok, ok, ok, 2, *btail) == -2  # any stride but a negative one
+    assert lib.trt_lt2exp_bf16(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, ok, s3(1, 1, 2), 2, *btail) == -2  # c: unit trailing stride
     assert lib.trt_lt2exp_bf16(one, one, one, one, 1 << 31, 1, 1, 1, 1, ok, ok, ok, ok, 3, *btail) == -4
     # a grid the fp32 path would split is handed to it, and then needs its workspace
     assert lib.trt_lt2exp_bf16(one, one, one, one, *big4, 2, _lib.MODE_SPLIT, 0, null, 0, null) == -3
@@ -112,7 +113,8 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, ok, ok, 2, nv + 1, 0, null, 0, null) == -1
     assert lib.trt_lm2exp_bf16(one, null, one, 1, 1, 1, 1, ok, ok, ok, 3, *mtail) == -1
     assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, s3(4, 1, -2), ok, 2, *mtail) == -2  # b: any stride but a negative one
-    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, s3(4, 1, 2), ok, ok, 2, *mtail) == -2  # a: unit trailing stride on this pipe
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, s3(4, 1, -2), ok, ok, 2, *mtail) == -2
+    assert lib.trt_lm2exp_bf16(one, one, one, 1, 1, 1, 1, ok, ok, s3(4, 1, 2), 2, *mtail) == -2  # c: unit trailing stride
     assert lib.trt_lm2exp_bf16(one, one, one, 1, 2, 2, 8, ok, ok, s3(16, 4, 1), 2, *mtail) == -2
     assert lib.trt_lm2exp_bf16(one, one, one, 1, 1 << 30, 1, 1, ok, ok, ok, 2, *mtail) == -4
     assert lib.trt_lm2exp_bf16(one, one, one, 1, 1024, 1024, 1024, big, big, big, 2, 0, 4, null, 0, null) == -3

@@ -255,8 +255,9 @@ def test_strided_inputs(dev):
     assert torch.equal(ag.cpu(), a_big) and torch.equal(bg.cpu(), b_big)
 
 
+@pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
 @pytest.mark.parametrize("shape", [(2, 256, 64, 128), (3, 300, 50, 129), (2, 70, 333, 40), (1, 130, 18, 257), (64, 16, 33, 7)])
-def test_views_of_a_are_read_in_place(dev, shape):
+def test_views_of_a_are_read_in_place(dev, shape, precision):
     """The reference hands any strides to its kernel (triturus/lm2exp.py:190-198).  A transposed,
     column-strided or expanded a must give the oracle's result without a copy: the call may
     allocate its output and nothing else."""
@@ -266,6 +267,12 @@ def test_views_of_a_are_read_in_place(dev, shape):
     b = -5 + 4 * torch.randn(R, J, K, generator=g)
     b[torch.rand(b.shape, generator=g) < 0.1] = NINF
     ref = oracle64.lm2exp64(a, b)
+    gate = BF16X3_GATE if precision == "bf16x3" else {}
+    lib = _lib.load()
+    pieces = {"fp32": 0, "bf16x3": 2, "bf16x6": 3}[precision]
+    ws_bytes = lib.trt_lm2exp_workspace_bytes(R, I, J, K, 0, 0)
+    if pieces:
+        ws_bytes = max(ws_bytes, lib.trt_lm2exp_bf16_workspace_bytes(R, I, J, K, pieces, 0))
     bg = b.to(dev)
     wide = torch.zeros(R, I, 2 * J + 1)
     wide[:, :, 1::2] = a
@@ -278,22 +285,22 @@ def test_views_of_a_are_read_in_place(dev, shape):
         del views["batch first in memory"]  # the trailing stride is the batch size
     for name, ag in views.items():
         assert ag.stride(2) != 1 and torch.equal(ag.cpu(), a), name
-        lm2exp(ag, bg)  # first call: library load, workspace query cache
+        lm2exp(ag, bg, _precision=precision)  # first call: library load, workspace query cache
         torch.cuda.synchronize()
         before = torch.cuda.memory_allocated()
-        out = lm2exp(ag, bg)
+        out = lm2exp(ag, bg, _precision=precision)
         grown = torch.cuda.memory_allocated() - before
-        r = oracle64.compare(out, ref)
+        r = oracle64.compare(out, ref, **gate)
         assert r["ok"], (name, r)
-        assert grown <= out.numel() * 4 + 1024, (name, grown, out.numel() * 4)
+        assert grown <= out.numel() * 4 + ws_bytes + 1024, (name, grown, out.numel() * 4, ws_bytes)
     # an expanded operand (stride 0) is read in place as well
     a1 = a[:1]
     ag = a1.to(dev).expand(R, I, J)
-    lm2exp(ag, bg)
+    lm2exp(ag, bg, _precision=precision)
     before = torch.cuda.memory_allocated()
-    out = lm2exp(ag, bg)
-    assert torch.cuda.memory_allocated() - before <= out.numel() * 4 + 1024
-    assert oracle64.compare(out, oracle64.lm2exp64(a1.expand(R, I, J), b))["ok"]
+    out = lm2exp(ag, bg, _precision=precision)
+    assert torch.cuda.memory_allocated() - before <= out.numel() * 4 + ws_bytes + 1024
+    assert oracle64.compare(out, oracle64.lm2exp64(a1.expand(R, I, J), b), **gate)["ok"]
 
 
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])

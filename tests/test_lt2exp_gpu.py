@@ -244,9 +244,20 @@ def test_views_of_w_are_read_in_place(dev, shape, mode):
     wg = w1.to(dev).expand(R, S, I, J)
     out = lt2exp(wg, ag, bg, mode=mode)
     assert oracle64.compare(out, oracle64.lt2exp64(w1.expand(R, S, I, J), a, b))["ok"]
-    # on the bf16 matrix pipe the wrapper materialises such a view: same result as from a dense w
-    dense = lt2exp(w.to(dev), ag, bg, mode=mode, _precision="bf16x6")
-    assert torch.equal(lt2exp(views["every other element"], ag, bg, mode=mode, _precision="bf16x6"), dense)
+    # on the bf16 matrix pipe such a view is staged element by element, in place as well
+    for precision in ("bf16x3", "bf16x6"):
+        wg = views["every other element"]
+        lt2exp(wg, ag, bg, mode=mode, _precision=precision)
+        torch.cuda.synchronize()
+        ws = max(_lib.load().trt_lt2exp_workspace_bytes(R, S, I, J, K, {"unsplit": _lib.MODE_UNSPLIT, "split": _lib.MODE_SPLIT}[mode]),
+                 _lib.load().trt_lt2exp_bf16_workspace_bytes(R, S, I, J, K, 2 if precision == "bf16x3" else 3,
+                                                             {"unsplit": _lib.MODE_UNSPLIT, "split": _lib.MODE_SPLIT}[mode]))
+        before = torch.cuda.memory_allocated()
+        out = lt2exp(wg, ag, bg, mode=mode, _precision=precision)
+        grown = torch.cuda.memory_allocated() - before
+        assert oracle64.compare(out, ref, **PRECISION_GATES[precision])["ok"]
+        if J >= 4 and not (J < I and K >= 256):  # (the wrapper may pad or exchange short rows of w on copies: not this test's subject)
+            assert grown <= out.numel() * 4 + ws + 2048, (precision, grown, out.numel() * 4, ws)
 
 
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])

@@ -32,6 +32,7 @@ struct Lm2BfArgs {
     int R, I, J, K;
     int64_t sa0, sa1, sb0, sb1, sc0, sc1;
     int64_t sb2;  // trailing stride of b (a lane owns a column: it only scales the lane offsets)
+    int64_t sa2;  // trailing stride of a: other than 1 in the builds without 16-byte loads only
     int i_tiles, n_tiles, splits, chunks_per_split;
     int stream_out;  // rows of c are 16-byte aligned: non-temporal result stores
     int64_t total_wgs, padded_wgs;
@@ -98,19 +99,20 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
     for (int sidx = 0; sidx < SLOTS; ++sidx) {
         int row = i0 + trow + sidx * ROWS_PER_SLOT;
         row = row < p.I ? row : p.I - 1;
-        aoff[sidx] = ((uint32_t)(row - i0) * (uint32_t)p.sa1 + 4u * tc4) * 4u;
+        aoff[sidx] = ((uint32_t)(row - i0) * (uint32_t)p.sa1 + 4u * tc4 * (uint32_t)p.sa2) * 4u;
     }
     const float *atile0 = ar + (int64_t)i0 * p.sa1;
     const int arows = (p.I - i0) < TM ? (p.I - i0) : TM;
     const __amdgpu_buffer_rsrc_t a_rsrc =
-        make_rsrc(atile0, (uint32_t)(((int64_t)(arows - 1) * p.sa1 + p.J) * 4));
+        make_rsrc(atile0, (uint32_t)(((int64_t)(arows - 1) * p.sa1 + (int64_t)(p.J - 1) * p.sa2 + 1) * 4));
     // pair-wise staging of the unaligned build (chunks that divide the workgroup evenly)
     constexpr bool ELEM = !VEC && (NT % (JC / 2) == 0) && ((TM * JC / 2) % NT == 0) && (TM * JC / 2 / NT <= 2 * SLOTS);
     constexpr int NP = ELEM ? TM * JC / 2 / NT : 1;  // column pairs per thread
     const int ecp = tid % (JC / 2);
-    const uint32_t ebase = ((uint32_t)(tid / (JC / 2)) * (uint32_t)p.sa1 + 2u * (uint32_t)ecp) * 4u;
+    const uint32_t ebase = ((uint32_t)(tid / (JC / 2)) * (uint32_t)p.sa1 + 2u * (uint32_t)ecp * (uint32_t)p.sa2) * 4u;
+    const uint32_t acol_bytes = (uint32_t)p.sa2 * 4u;  // one column further (4 in the builds with 16-byte loads)
     auto load_tile = [&](int jc) {
-        const uint32_t soff = (uint32_t)(jc * JC) * 4u;  // wave-uniform
+        const uint32_t soff = (uint32_t)(jc * JC) * acol_bytes;  // wave-uniform
         const bool full = VEC && (jc * JC + JC <= p.J);
         if (full) {
 #pragma unroll
@@ -134,7 +136,7 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
 #pragma unroll
             for (int e = 0; e < NP; ++e) {
                 const uint32_t so = soff + (uint32_t)(e * (2 * NT / JC)) * (uint32_t)p.sa1 * 4u;
-                const float v0 = buf_load_f32(a_rsrc, ebase, so), v1 = buf_load_f32(a_rsrc, ebase + 4u, so);
+                const float v0 = buf_load_f32(a_rsrc, ebase, so), v1 = buf_load_f32(a_rsrc, ebase + acol_bytes, so);
                 stage[e / 2][2 * (e % 2)] = in0 ? v0 : 0.f;
                 stage[e / 2][2 * (e % 2) + 1] = in1 ? v1 : 0.f;
             }
@@ -144,7 +146,7 @@ __global__ __launch_bounds__(256, 2) void lm2exp_bf16_kernel(const Lm2BfArgs p) 
             for (int sidx = 0; sidx < SLOTS; ++sidx)
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const float v = buf_load_f32(a_rsrc, aoff[sidx] + 4u * e, soff);
+                    const float v = buf_load_f32(a_rsrc, aoff[sidx] + acol_bytes * e, soff);
                     stage[sidx][e] = (j + e < p.J) ? v : 0.f;
                 }
         }
@@ -425,14 +427,14 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     if (R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
     if (variant < 0 || variant > kNumLmBfVariants || splits < 0) return TRT_E_INVALID;
-    if (sa[2] != 1 || sb[2] < 0 || sc[2] != 1) return TRT_E_LAYOUT;
+    if (sa[2] < 0 || sb[2] < 0 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     if (sc[1] < K) return TRT_E_LAYOUT;  // output rows must not overlap
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || I >= lim || J >= lim || K >= lim) return TRT_E_RANGE;
     // byte offsets inside one batch slab are 32-bit (buffer addressing)
-    if (I * sa[1] + J >= lim || J * sb[1] + K * sb[2] >= lim || I * sc[1] + K >= lim) return TRT_E_RANGE;
+    if (I * sa[1] + J * sa[2] >= lim || J * sb[1] + K * sb[2] >= lim || I * sc[1] + K >= lim) return TRT_E_RANGE;
 
     // Tile and hand-over rules, fitted to 223 random shapes (R 1..256, I, J 16..1024, K 64..8192)
     // timed with every tile and on the fp32 path; against the best of those the rules below lose
@@ -508,7 +510,7 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     args.a = a; args.b = b; args.c = c;
     args.R = (int)R; args.I = (int)I; args.J = (int)J; args.K = (int)K;
     args.sa0 = sa[0]; args.sa1 = sa[1];
-    args.sb0 = sb[0]; args.sb1 = sb[1]; args.sb2 = sb[2];
+    args.sb0 = sb[0]; args.sb1 = sb[1]; args.sb2 = sb[2]; args.sa2 = sa[2];
     args.sc0 = sc[0]; args.sc1 = sc[1];
     args.i_tiles = (int)ceil_div(I, 32 * vr.rt);
     args.n_tiles = (int)ceil_div(K, 128);
@@ -523,7 +525,7 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     // (J itself need not be a multiple of 4 when the row stride is: the piece that straddles J
     // is masked by element)
-    const bool vec = (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
+    const bool vec = sa[2] == 1 && (sa[0] % 4 == 0) && (sa[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
     int status;
@@ -572,7 +574,7 @@ extern "C" int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, 
     args.a = a; args.b = b; args.c = c;
     args.R = 1; args.I = (int)m; args.J = (int)k; args.K = (int)n;
     args.sa0 = m * k; args.sa1 = k;
-    args.sb0 = k * n; args.sb1 = n; args.sb2 = 1;
+    args.sb0 = k * n; args.sb1 = n; args.sb2 = 1; args.sa2 = 1;
     args.sc0 = m * n; args.sc1 = n;
     args.i_tiles = (int)ceil_div(m, 32 * rt);
     args.n_tiles = (int)ct;

@@ -35,6 +35,7 @@ struct Lt2BfArgs {
     int R, S, I, J, K;
     int64_t sw0, sw1, sa0, sa1, sb0, sb1, sc0, sc1;
     int64_t sa2, sb2;  // trailing strides of a and b (a lane owns a column: they only scale lane offsets)
+    int64_t sw2;       // stride of the flat (i, j) axis of w: other than 1 in the builds without 16-byte loads only
     int s_tiles, n_tiles, splits;
     int iters_per_split;  // (j-chunk, i) iterations per split
     int stream_out;       // rows of c are 16-byte aligned: non-temporal result stores
@@ -131,18 +132,19 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
     const int wrows = (p.S - s0) < TS ? (p.S - s0) : TS;
     const float *wtile0 = wr + (int64_t)s0 * p.sw1;
     const __amdgpu_buffer_rsrc_t w_rsrc =
-        make_rsrc(wtile0, (uint32_t)(((int64_t)(wrows - 1) * p.sw1 + (int64_t)p.I * p.J) * 4));
+        make_rsrc(wtile0, (uint32_t)(((int64_t)(wrows - 1) * p.sw1 + ((int64_t)p.I * p.J - 1) * p.sw2 + 1) * 4));
     uint32_t woff[SLOTS];
 #pragma unroll
     for (int sidx = 0; sidx < SLOTS; ++sidx)
-        woff[sidx] = ((uint32_t)srow[sidx] * (uint32_t)p.sw1 + 4u * (uint32_t)sc4[sidx]) * 4u;
+        woff[sidx] = ((uint32_t)srow[sidx] * (uint32_t)p.sw1 + 4u * (uint32_t)sc4[sidx] * (uint32_t)p.sw2) * 4u;
     // pair-wise staging of the unaligned build (chunks that divide the workgroup evenly)
     constexpr bool ELEM = !VEC && (NT % (JC / 2) == 0) && ((TS * JC / 2) % NT == 0) && (TS * JC / 2 / NT <= 2 * SLOTS);
     constexpr int NP = ELEM ? TS * JC / 2 / NT : 1;  // column pairs per thread
     const int ecp = tid % (JC / 2);
-    const uint32_t ebase = ((uint32_t)(tid / (JC / 2)) * (uint32_t)p.sw1 + 2u * (uint32_t)ecp) * 4u;
+    const uint32_t ebase = ((uint32_t)(tid / (JC / 2)) * (uint32_t)p.sw1 + 2u * (uint32_t)ecp * (uint32_t)p.sw2) * 4u;
+    const uint32_t wcol_bytes = (uint32_t)p.sw2 * 4u;  // one element of the flat axis further (4 in the builds with 16-byte loads)
     auto load_tile = [&](int i, int jc) __attribute__((always_inline)) {
-        const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * 4u;
+        const uint32_t soff = (uint32_t)(i * p.J + jc * JC) * wcol_bytes;
         const bool full = VEC && (jc * JC + JC <= p.J);  // wave-uniform
         if (full) {
 #pragma unroll
@@ -164,7 +166,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
 #pragma unroll
             for (int e = 0; e < NP; ++e) {
                 const uint32_t so = soff + (uint32_t)(e * (2 * NT / JC)) * (uint32_t)p.sw1 * 4u;
-                const float v0 = buf_load_f32(w_rsrc, ebase, so), v1 = buf_load_f32(w_rsrc, ebase + 4u, so);
+                const float v0 = buf_load_f32(w_rsrc, ebase, so), v1 = buf_load_f32(w_rsrc, ebase + wcol_bytes, so);
                 stage[e / 2][2 * (e % 2)] = in0 ? v0 : 0.f;
                 stage[e / 2][2 * (e % 2) + 1] = in1 ? v1 : 0.f;
             }
@@ -176,7 +178,7 @@ __global__ __launch_bounds__(256, 2) void lt2exp_bf16_kernel(const Lt2BfArgs p) 
                 const int j = jc * JC + 4 * sc4[sidx];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
-                    const float v = buf_load_f32(w_rsrc, woff[sidx] + 4u * e, soff);
+                    const float v = buf_load_f32(w_rsrc, woff[sidx] + wcol_bytes * e, soff);
                     stage[sidx][e] = (j + e < p.J) ? v : 0.f;
                 }
             }
@@ -496,13 +498,13 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
     if (mode != TRT_MODE_AUTO && mode != TRT_MODE_SPLIT && mode != TRT_MODE_UNSPLIT) return TRT_E_INVALID;
     if (variant < 0 || variant > 16) return TRT_E_INVALID;
-    if (sw[2] != 1 || sa[2] < 0 || sb[2] < 0 || sc[2] != 1) return TRT_E_LAYOUT;
+    if (sw[2] < 0 || sa[2] < 0 || sb[2] < 0 || sc[2] != 1) return TRT_E_LAYOUT;
     for (int d = 0; d < 2; ++d)
         if (sw[d] < 0 || sa[d] < 0 || sb[d] < 0 || sc[d] < 0) return TRT_E_LAYOUT;
     if (sc[1] < K) return TRT_E_LAYOUT;
     const int64_t lim = (int64_t)1 << 30;
     if (R >= lim || S >= lim || I >= lim || J >= lim || K >= lim || I * J >= lim) return TRT_E_RANGE;
-    if (S * sw[1] + I * J >= lim || I * sa[1] + K * sa[2] >= lim || J * sb[1] + K * sb[2] >= lim || S * sc[1] + K >= lim)
+    if (S * sw[1] + I * J * (sw[2] > 0 ? sw[2] : 1) >= lim || I * sa[1] + K * sa[2] >= lim || J * sb[1] + K * sb[2] >= lim || S * sc[1] + K >= lim)
         return TRT_E_RANGE;
 
     // a single j under several i: run with the roles of (i, a) and (j, b) exchanged (see trt_lt2exp_f32)
@@ -594,7 +596,7 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     }
     args.R = (int)R; args.S = (int)S; args.I = (int)I; args.J = (int)J; args.K = (int)K;
     args.sw0 = sw[0]; args.sw1 = sw[1];
-    args.sa0 = sa[0]; args.sa1 = sa[1]; args.sa2 = sa[2];
+    args.sa0 = sa[0]; args.sa1 = sa[1]; args.sa2 = sa[2]; args.sw2 = sw[2];
     args.sb0 = sb[0]; args.sb1 = sb[1]; args.sb2 = sb[2];
     args.sc0 = sc[0]; args.sc1 = sc[1];
     args.s_tiles = (int)ceil_div(S, 32 * rt);
@@ -603,7 +605,7 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
     args.stream_out = rows_16_byte_aligned(c, sc[0], sc[1]);
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
-    const bool vec = (J % 4 == 0) && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) &&
+    const bool vec = sw[2] == 1 && (J % 4 == 0) && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) &&
                      ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (pieces == 2) launch_bf_shape<2>(args, rt, ks, vec, split, s);

@@ -74,12 +74,13 @@ def lm2exp(
     fp32 = _precision == "fp32"
     # Operands go to the kernels with whatever non-negative strides they have, as the reference
     # forwards them (triturus/lm2exp.py:190-198): b in every kernel (a lane owns a column of b,
-    # so a trailing stride only scales its offsets), a in the fp32 kernels (the paired-wavefront
-    # tiles read a transposed or strided a in place; a forced tile of another family and the
-    # bf16 kernels want unit-stride rows of a).  Only negative strides always need a copy.
+    # so a trailing stride only scales its offsets) and a (on the fp32 pipe the paired-wavefront
+    # tiles read a transposed or strided a in place -- a forced tile of another family wants
+    # unit-stride rows --, on the bf16 pipe the element-staging builds do).  Only negative
+    # strides always need a copy.
     sa, sb = a.stride(), b.stride()
     pair_tile = _variant == 0 or _variant > lib.trt_lm2exp_variant_count() - 5
-    if ((not fp32 or not pair_tile) and sa[2] != 1) or min(sa) < 0:
+    if (fp32 and not pair_tile and sa[2] != 1) or min(sa) < 0:
         a = _unit_inner(a)
         sa = a.stride()
     if min(sb) < 0:

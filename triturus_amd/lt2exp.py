@@ -128,8 +128,8 @@ def lt2exp(
         J = J4
     sw, sa, sb = w.stride(), a.stride(), b.stride()
     # w is read in place whatever the stride of its flat (i, j) axis (a sliced view: element
-    # loads instead of 16-byte ones); only the bf16 kernels and negative strides need a copy
-    if min(sw) < 0 or (sw[2] != 1 and _precision != "fp32"):
+    # loads instead of 16-byte ones); only negative strides need a copy
+    if min(sw) < 0:
         w = _unit_inner(w)
         sw = w.stride()
     # a and b are read in place whatever their strides, as the reference forwards them
