@@ -67,15 +67,47 @@ def test_static_scratch_entry_point_matches_the_workspace_entry_point(dev):
     assert lib.trt_lt2exp_workspace_bytes(3, 75, 50, 50, 100, _lib.MODE_SPLIT) > 0  # the scratch array was in use
 
 
+def test_static_scratch_entry_point_takes_no_memory_from_the_driver(dev):
+    """torch's own counters cannot see a hipMalloc made inside the library: the free memory that
+    the driver reports must be the same before and after a call whose tensors all exist already
+    (a warm-up call first: the first call on a device looks up the scratch array's address)."""
+    lib = _lib.load()
+    shape = (3, 75, 50, 50, 100)
+    R, S, I, J, K = shape
+    (w, a, b), (wg, ag, bg) = _inputs(shape, 100, dev)
+    w3 = wg.view(R, S, I * J)
+    c = torch.empty(R, S, K, device=dev)
+    args = (w3.data_ptr(), ag.data_ptr(), bg.data_ptr(), c.data_ptr(), R, S, I, J, K,
+            _lib.strides3(w3), _lib.strides3(ag), _lib.strides3(bg), _lib.strides3(c), _lib.MODE_SPLIT, 0)
+    stream = _lib.raw_stream(dev)
+    assert lib.trt_lt2exp_f32_static(*args, stream) == 0
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info(dev)
+    reserved_before = torch.cuda.memory_reserved(dev)
+    for _ in range(3):
+        assert lib.trt_lt2exp_f32_static(*args, stream) == 0
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info(dev)
+    assert torch.cuda.memory_reserved(dev) == reserved_before  # torch took nothing from the driver in between
+    assert free_after == free_before, (free_before, free_after)
+    assert oracle64.compare(c, oracle64.lt2exp64(w, a, b))["ok"]
+
+
 def test_static_scratch_entry_point_refuses_what_does_not_fit(dev):
     lib = _lib.load()
     shape = (64, 512, 8, 8, 1024)  # split mode: some ten copies of a 128 MiB output
     R, S, I, J, K = shape
     assert lib.trt_lt2exp_workspace_bytes(R, S, I, J, K, _lib.MODE_SPLIT) > _lib.STATIC_SCRATCH_BYTES
-    one = ctypes.c_void_p(256)  # never dereferenced: the call is refused before anything is enqueued
+    # real tensors of that shape (were the refusal to regress, the kernels would run on valid memory)
+    wg = torch.rand(R, S, I * J, device=dev)
+    ag, bg = torch.randn(R, I, K, device=dev), torch.randn(R, J, K, device=dev)
+    c = torch.full((R, S, K), 7.0, device=dev)
     s3 = (ctypes.c_int64 * 3)
-    args = (one, one, one, one, R, S, I, J, K, s3(S * I * J, I * J, 1), s3(I * K, K, 1), s3(J * K, K, 1), s3(S * K, K, 1))
-    assert lib.trt_lt2exp_f32_static(*args, _lib.MODE_SPLIT, 0, None) == _lib.E_SCRATCH
+    args = (wg.data_ptr(), ag.data_ptr(), bg.data_ptr(), c.data_ptr(), R, S, I, J, K,
+            s3(S * I * J, I * J, 1), s3(I * K, K, 1), s3(J * K, K, 1), s3(S * K, K, 1))
+    assert lib.trt_lt2exp_f32_static(*args, _lib.MODE_SPLIT, 0, _lib.raw_stream(dev)) == _lib.E_SCRATCH
+    torch.cuda.synchronize()
+    assert bool((c == 7.0).all())  # nothing was enqueued
     assert b"scratch" in lib.trt_error_string(_lib.E_SCRATCH)
     # unsplit needs no scratch at all, whatever the size
     (w, a, b), (wg, ag, bg) = _inputs((2, 33, 5, 7, 40), 7, dev)
