@@ -361,3 +361,22 @@ def test_short_row_rule_of_the_lt2exp_wrapper():
     assert not _packs(3, 2)        # 6 floats: not a multiple of 4
     assert not _packs(2, 8)        # a single chunk
     assert not _packs(64, 16) and not _packs(64, 3) and not _packs(64, 1)
+
+
+def test_paired_wavefront_groups_take_grids_of_at_most_two_tiles_per_cu():
+    """Host-side tile rule of lt2exp (no GPU needed: trt_lt2exp_kernel_name reports what a call
+    would launch).  The last template argument is the number of wavefront groups that share a
+    tile's contraction inside a workgroup."""
+    name = lambda *sh, mode=_lib.MODE_AUTO, aligned=1: _lib.kernel_name("lt2exp", *sh, mode, 0, aligned)
+    # R=16, S=64, I=J=32, K=2048: 256 tiles of 64 rows, a short contraction: 64 rows, two groups
+    assert name(16, 64, 32, 32, 2048) == "trt::lt2exp_kernel<2, 1, 4, 4, true, false, 1, 0, 2>"
+    # one 32-row tile per CU, or a long contraction: 32 rows, two groups
+    assert name(16, 32, 32, 32, 2048) == "trt::lt2exp_kernel<1, 1, 4, 4, true, false, 1, 0, 2>"
+    assert name(16, 64, 64, 64, 2048) == "trt::lt2exp_kernel<1, 1, 4, 4, true, false, 1, 0, 2>"
+    # the large configuration fills the machine many times over: one group per tile
+    assert name(64, 64, 64, 64, 4096) == "trt::lt2exp_kernel<2, 1, 4, 4, true, false, 1, 0, 1>"
+    # never under a forced cut over workgroups, for rows of w that are not 16-byte aligned, or
+    # where another j-chunk than 32 fits J better
+    assert name(16, 64, 32, 32, 2048, mode=_lib.MODE_SPLIT).endswith("true, true, 1, 0, 1>")
+    assert name(16, 64, 32, 32, 2048, aligned=0).endswith("false, false, 1, 0, 1>")
+    assert name(16, 64, 32, 16, 2048).endswith(", 1>") and ", 2, 4, " in name(16, 64, 32, 16, 2048)
