@@ -26,6 +26,8 @@ _ws_bytes: dict = {}  # (op, shape..., dtype code) -> workspace bytes, as report
 # once per device and stream and kept: calls on one stream run one after the other, calls on
 # different streams never share one.  At most _MAX_STREAMS of them are kept, the least recently
 # used one going first (the allocator hands its block to later work on the same stream only).
+# The key is the raw stream handle: a stream created after another one was destroyed may get its
+# handle and with it its workspace, which is as good as a new one -- every call leaves it idle.
 _MAX_STREAMS = 16
 _workspaces: "OrderedDict[tuple, torch.Tensor]" = OrderedDict()  # (device index, raw stream) -> workspace
 # A stream that is being captured into a HIP graph gets a workspace of its own per capture,
