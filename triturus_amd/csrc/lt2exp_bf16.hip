@@ -533,7 +533,7 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     //  - j-chunks of 64, 48, 32 or 16: the one that pads J least, weighed by its cost per j
     //    (bf16_chunk).
     const int64_t ctk = ceil_div(K, 128);
-    const int64_t t32 = R * ceil_div(S, 32) * ctk, t64 = R * ceil_div(S, 64) * ctk;
+    const int64_t t64 = R * ceil_div(S, 64) * ctk;
     const int64_t s_last = S % 64;
     int rt = (S > 32 && (s_last == 0 || s_last > 32) && t64 >= 512) ? 2 : 1;
     int ks = bf16_chunk(J, pieces);
