@@ -363,6 +363,26 @@ def test_short_row_rule_of_the_lt2exp_wrapper():
     assert not _packs(64, 16) and not _packs(64, 3) and not _packs(64, 1)
 
 
+def test_small_lm2exp_grids_get_tile_and_cut_chosen_together():
+    """Host-side plan of lm2exp (no GPU needed: trt_lm2exp_kernel_name reports the tile,
+    trt_lm2exp_workspace_bytes the cut: splits * (R*I*K partial sums + R*K shifts) floats)."""
+    lib = _lib.load()
+    name = lambda R, I, J, K: _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1)
+    cut = lambda R, I, J, K: lib.trt_lm2exp_workspace_bytes(R, I, J, K, 0, 0) // (4 * (R * I * K + R * K))
+    # a batch-1 square of 1536: 96-row tiles cut four ways are 768 workgroups, three per CU
+    assert name(1, 1536, 1536, 1536) == "trt::lm2exp_kernel<3, 1, 1, 4, 4, true, 1>" and cut(1, 1536, 1536, 1536) == 4
+    assert name(2, 1536, 1536, 1536) == "trt::lm2exp_kernel<3, 1, 1, 4, 4, true, 1>" and cut(2, 1536, 1536, 1536) == 2
+    # 256 tiles of 64 rows under 16 chunks: one workgroup per tile (a cut would cost more than it hides)
+    assert name(16, 512, 512, 512) == "trt::lm2exp_kernel<2, 1, 1, 4, 4, true, 1>" and cut(16, 512, 512, 512) == 0
+    # a forced cut keeps its count; the tile follows it
+    assert lib.trt_lm2exp_workspace_bytes(1, 1536, 1536, 1536, 0, 3) == 3 * 4 * (1536 * 1536 + 1536)
+    # outside the region (a short contraction, a large grid, a contraction that wants chunks of 16)
+    # the tile rules decide as before
+    assert name(64, 256, 256, 4096) == "trt::lm2exp_pair_kernel<4, 4, 2, 0>"
+    assert name(6, 325, 464, 1266) == "trt::lm2exp_kernel<3, 1, 1, 4, 2, true, 1>"
+    assert cut(1, 128, 64, 128) == 0
+
+
 def test_paired_wavefront_groups_take_grids_of_at_most_two_tiles_per_cu():
     """Host-side tile rule of lt2exp (no GPU needed: trt_lt2exp_kernel_name reports what a call
     would launch).  The last template argument is the number of wavefront groups that share a

@@ -125,6 +125,27 @@ def test_small_grid_long_contraction_splits_by_itself(dev):
     assert torch.allclose(torch_baseline.lm2exp_fp32(a, b), out.cpu())  # the reference's bar
 
 
+@pytest.mark.parametrize(
+    "shape",
+    [(1, 768, 1536, 768), (2, 200, 704, 900), (5, 333, 992, 257), (1, 96, 2496, 1173), (12, 420, 2688, 273), (1, 1536, 1536, 1536)],
+)
+def test_small_grids_whose_tile_and_cut_are_chosen_together(dev, shape):
+    """Shapes whose plan comes from the joint model of tile height and cut (every tile height,
+    cuts of 1..8): against float64 on the GPU -- these are too large for the CPU oracle to be
+    quick -- with -inf columns, zero rows and a batch-dependent offset in b."""
+    R, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(R, I, J, generator=g).to(dev)
+    b = (5 * torch.randn(R, J, K, generator=g) - 30 * torch.arange(R).view(R, 1, 1)).to(dev)
+    a[:, 3, :] = 0.0
+    b[:, :, 7] = NINF
+    out = lm2exp(a, b)
+    ref = oracle64.lm2exp64(a, b, device=dev)  # float64 torch on the device
+    r = oracle64.compare(out, ref)
+    assert r["ok"] and r["n_neg_inf"] >= R * (I + K - 1), (shape, r)
+    assert torch.equal(out, lm2exp(a, b))  # deterministic, cut or not
+
+
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
 @pytest.mark.parametrize("shape", [(3, 37, 41, 70), (2, 130, 129, 257), (1, 64, 7, 64), (2, 33, 301, 31), (24, 150, 99, 200)])
 def test_padded_rows_of_a(dev, precision, shape, monkeypatch):

@@ -769,18 +769,75 @@ struct Lm2Plan {
 
 constexpr int kMaxSplits = 32;
 
+// Small grids under a contraction of some length -- at most nine 32-row tiles per CU, J >= 160,
+// 0.1 GFLOP and more -- get the height of their tile and the cut over J chosen TOGETHER, by
+// modelled time.  (choose_variant's rules fix the tile first and choose_splits then cuts it; on
+// such grids what counts is how many whole workgroups the busiest CU ends up with, which only
+// the pair (tile, cut) decides: I=J=K=1536 takes 80 us on 96-row tiles cut four ways -- 768
+// workgroups, three per CU -- against 93 on the 128-row tile the rules pick; R=12, I=420, J=2688,
+// K=273: 108 against 129.)  The model: a workgroup's chain is its chunks times (MFMAs + the exp
+// work of a chunk, which does not shrink with the tile), the busiest of the 256 CUs runs
+// q = ceil(workgroups / 256) chains at 77 % of that rate alone, 92 % with two, in full from three
+// on, a launch costs 4.8 us, a cut 4.1 us more plus its partial sums' trip through memory at
+// 2.46 TB/s.  Constants fitted to 28 tile-and-cut combinations on each of 30 batch-1..3 shapes of
+// 640..3072; on 46 other random shapes of the region its pick is 0.9 % (mean) behind the best
+// combination measured, the rules' 3.1 %, with the worst case 6 % against 20 %.  Outside the
+// region the rules stay: they are ahead on short contractions (J < 160: 2 % against 7 %), on the
+// reference's grid shapes below 0.1 GFLOP and where J wants j-chunks of 16 or 24 (the exp work per
+// chunk is fitted for chunks of 32 only), and level on larger grids.
+struct TileCut {
+    int rt, splits;
+    double us;
+};
+static bool joint_region(int64_t R, int64_t I, int64_t J, int64_t K) {
+    const int64_t n32 = R * ceil_div(I, 32) * ceil_div(K, 128);
+    return K > 64 && I > 32 && J >= 160 && pick_chunk(J) == 4 && n32 <= 2304 &&
+           (double)R * (double)I * (double)J * (double)K >= 1e8;
+}
+// splits_fixed: 0 = any cut, n >= 1 = exactly n (1: uncut)
+static TileCut choose_tile_and_cut(int64_t R, int64_t I, int64_t J, int64_t K, int splits_fixed) {
+    constexpr int nq = 4;
+    const int64_t units = ceil_div(J, 8 * nq);
+    TileCut best{1, 1, 1e300};
+    for (int rt = 1; rt <= 4; ++rt) {
+        const int64_t tiles = R * ceil_div(I, 32 * rt) * ceil_div(K, 128);
+        const double unit_us = (256.0 * nq * rt + 107.5 * nq) / 2400.0;
+        for (int sp = 1; sp <= kMaxSplits && (sp == 1 || 2 * sp <= units); ++sp) {
+            if (splits_fixed && sp != splits_fixed) continue;
+            const int64_t per = ceil_div(units, sp);
+            if (!splits_fixed && ceil_div(units, per) != sp) continue;  // the same cut as a smaller count
+            const int64_t q = ceil_div(tiles * ceil_div(units, per), 256);
+            const double eff = q >= 3 ? 1.0 : (q == 2 ? 0.92 : 0.77);
+            double us = 4.8 + (double)q * (double)per * unit_us / eff;
+            if (sp > 1) us += 4.1 + (double)(sp + 1) * (double)(R * I * K) * 4.0 / 2.46e6;
+            if (us < best.us) best = {rt, sp, us};
+        }
+    }
+    return best;
+}
+
 // splits_req: 0 = decide here, 1 = never split, n > 1 = split n ways (capped).
 // A small grid with a long contraction is cut over J so that the 256 CUs have work:
 // e.g. batch 1, I=J=K=1024 is 64 tiles of 128 x 128 but 32 chunks deep.
 static Lm2Plan make_plan(int64_t R, int64_t I, int64_t J, int64_t K, int variant, int splits_req) {
     Lm2Plan pl;
-    pl.variant = (variant >= 1) ? variant - 1 : choose_variant(R, I, J, K);
+    const bool joint = variant < 1 && joint_region(R, I, J, K);
+    TileCut tc{1, 1, 0.0};
+    if (joint) {
+        tc = choose_tile_and_cut(R, I, J, K, splits_req);
+        if (tc.us >= 1e300) tc = choose_tile_and_cut(R, I, J, K, 0);  // a cut the contraction is too short for
+        pl.variant = find_variant(tc.rt, 4, kOnline);
+    } else {
+        pl.variant = (variant >= 1) ? variant - 1 : choose_variant(R, I, J, K);
+    }
     const Lm2Variant &vr = kVariants[pl.variant];
     const int64_t chunks = ceil_div(J, 8 * vr.nq);
     const int64_t base = R * ceil_div(I, 32 * vr.rt * vr.wm) * ceil_div(K, 32 * vr.ct * vr.wn);
     int64_t splits = 1;
     if (vr.mode == kPlain)
         splits = 1;  // this build does not write partial sums
+    else if (splits_req == 0 && joint)
+        splits = tc.splits;
     else if (splits_req == 0)
         // measured: R=16 I=J=K=512 (256 tiles, 16 chunks) is 1.5x slower split, batch-1
         // squares of 512..1536 are 1.2-1.9x faster; the model below reproduces both
