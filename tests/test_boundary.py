@@ -400,3 +400,16 @@ def test_paired_wavefront_groups_take_grids_of_at_most_two_tiles_per_cu():
     assert name(16, 64, 32, 32, 2048, mode=_lib.MODE_SPLIT).endswith("true, true, 1, 0, 1>")
     assert name(16, 64, 32, 32, 2048, aligned=0).endswith("false, false, 1, 0, 1>")
     assert name(16, 64, 32, 16, 2048).endswith(", 1>") and ", 2, 4, " in name(16, 64, 32, 16, 2048)
+
+
+def test_lt2exp_takes_64_column_tiles_where_128_column_tiles_would_stand_half_empty():
+    """Host-side tile rule (seventh template argument: wavefronts stacked over rows; 2 is the
+    64 x 64 tile).  K = 192 is three tiles of 64 columns or two of 128."""
+    name = lambda *sh, aligned=1: _lib.kernel_name("lt2exp", *sh, _lib.MODE_AUTO, 0, aligned)
+    wm = lambda n: int(n.split(", ")[6])
+    assert wm(name(1, 192, 192, 192, 192)) == 2      # one of the reference's benchmark shapes
+    assert wm(name(1, 535, 26, 64, 136)) == 2
+    assert wm(name(1, 192, 192, 192, 256)) == 1      # whole 128-column tiles
+    assert wm(name(1, 192, 192, 192, 448)) == 1      # 7 tiles of 64 against 4 of 128: 0.875 of the area
+    assert wm(name(1, 535, 26, 64, 136, aligned=0)) == 1 and wm(name(1, 535, 26, 24, 136)) == 1  # aligned rows, chunks of 32 only
+    assert name(16, 382, 10, 32, 184).endswith(", 2>")  # paired groups keep their grids

@@ -689,6 +689,26 @@ static int paired_variant(int v, int64_t R, int64_t S, int64_t I, int64_t J, int
     return find_lt2_variant(rows64 ? 2 : 1, 4, false, 2);
 }
 
+// A 64 x 64 tile (the wavefronts 2 x 2) in place of the 32 x 128 one where tiles of 128 columns
+// would stand half empty: K = 192 is three tiles of 64 columns or two of 128, the second half
+// idle.  Taken when the 64 x 64 tiles cover at most 0.8 of the padded area (rows included: they
+// pad S to 64), for aligned rows of w and j-chunks of 32 only (the tile has no other build).
+// Measured: S=I=J=K=192, batch 1 (one of the reference's benchmark shapes) 61.8 -> 51.3 us;
+// R=1, S=535, I=26, J=64, K=136: 18.5 -> 16.5; R=6, S=449, I=10, J=92, K=192: 30.5 -> 27.0;
+// R=32, S=60, I=11, J=96, K=192: 25.3 -> 23.2; at 0.88 of the area (R=32, S=41, I=52, J=160,
+// K=424) still 5 % ahead, at 0.9 and above level or behind; where paired groups apply they
+// stay (R=16, S=382, I=10, J=32, K=184: 16.4 against 17.5).
+static int narrow_variant(int v, int64_t S, int64_t K) {
+    const Lt2Variant &vr = kVariants[v];
+    if (vr.gs != 1 || vr.wm != 1 || vr.pack || vr.nq != 4 || vr.rt != 1 || S <= 32) return v;
+    const int64_t area128 = ceil_div(S, 32) * 32 * ceil_div(K, 128) * 128;
+    const int64_t area64 = ceil_div(S, 64) * 64 * ceil_div(K, 64) * 64;
+    if (5 * area64 > 4 * area128) return v;
+    for (int u = 0; u < kNumVariants; ++u)
+        if (kVariants[u].wm == 2) return u;
+    return v;
+}
+
 // AUTO follows the reference in kind -- a small output grid with a long contraction is
 // split (triturus/lt2exp.py:535 tests R*S*K < 1048576 and I*J > 512) -- but decides with a
 // cost model fitted to this machine (measured: R=16 S=64 I=J=32 K=2048, 256 tiles of 32
@@ -773,7 +793,7 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     const bool w_aligned = sw[2] == 1 && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
     // packed rows need 16-byte loads along the flat (i, j) axis; any other call runs the same tile unpacked
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
-    if (variant == 0 && (J % 4 == 0) && w_aligned) v = paired_variant(v, R, S, I, J, K, mode);
+    if (variant == 0 && (J % 4 == 0) && w_aligned) v = narrow_variant(paired_variant(v, R, S, I, J, K, mode), S, K);
     // paired groups: aligned rows only, and never under a forced cut over workgroups
     if (kVariants[v].gs == 2 && (!((J % 4 == 0) && w_aligned) || mode == TRT_MODE_SPLIT))
         v = find_lt2_variant(kVariants[v].rt, kVariants[v].nq, false);
@@ -824,7 +844,7 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
     }
     int v = resolve_variant(variant, R, S, I, J, K);
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
-    if (variant == 0 && (J % 4 == 0) && w_aligned) v = paired_variant(v, R, S, I, J, K, mode);
+    if (variant == 0 && (J % 4 == 0) && w_aligned) v = narrow_variant(paired_variant(v, R, S, I, J, K, mode), S, K);
     if (kVariants[v].gs == 2 && (!((J % 4 == 0) && w_aligned) || mode == TRT_MODE_SPLIT))
         v = find_lt2_variant(kVariants[v].rt, kVariants[v].nq, false);
     const Lt2Variant &vr = kVariants[v];
