@@ -413,3 +413,16 @@ def test_lt2exp_takes_64_column_tiles_where_128_column_tiles_would_stand_half_em
     assert wm(name(1, 192, 192, 192, 448)) == 1      # 7 tiles of 64 against 4 of 128: 0.875 of the area
     assert wm(name(1, 535, 26, 64, 136, aligned=0)) == 1 and wm(name(1, 535, 26, 24, 136)) == 1  # aligned rows, chunks of 32 only
     assert name(16, 382, 10, 32, 184).endswith(", 2>")  # paired groups keep their grids
+
+
+def test_lt2exp_cuts_64_row_tiles_where_the_contraction_is_cut_anyway():
+    """Host-side tile rule (first template argument: rows of S in units of 32; sixth: the
+    contraction is cut over workgroups)."""
+    name = lambda *sh, mode=_lib.MODE_AUTO: _lib.kernel_name("lt2exp", *sh, mode, 0, 1)
+    # R=32, S=I=J=64, K=256 (one of the reference's benchmark shapes): 64 tiles of 64 rows, cut
+    assert name(32, 64, 64, 64, 256) == "trt::lt2exp_kernel<2, 1, 4, 4, true, true, 1, 0, 1>"
+    assert name(4, 170, 90, 128, 245).startswith("trt::lt2exp_kernel<2, 1, 4, 4, true, true")
+    # fewer than twelve 64-row tiles, rows that 64 pads further than 32, or no cut: 32 rows
+    assert name(1, 128, 128, 128, 128).startswith("trt::lt2exp_kernel<1, 1, 4, 4, true, true")
+    assert name(32, 82, 131, 64, 184).startswith("trt::lt2exp_kernel<1, 1, 4, 4, true, true")
+    assert name(32, 64, 64, 64, 256, mode=_lib.MODE_UNSPLIT).startswith("trt::lt2exp_kernel<1, 1, 4, 4, true, false")

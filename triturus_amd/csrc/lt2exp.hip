@@ -709,6 +709,23 @@ static int narrow_variant(int v, int64_t S, int64_t K) {
     return v;
 }
 
+// A grid whose contraction is cut over workgroups anyway does not need its tiles to be many: the
+// cut fills the CUs, and the 64-row tile's Khatri-Rao multiply serves two MFMAs.  So a 32-row
+// tile that would be cut gives way to the 64-row tile of the same j-chunk when S pads alike and
+// at least twelve 64-row tiles are left (fewer, and the 32-row tile's finer grain wins: batch 1,
+// S=I=J=K=128 29 us against 37).  Measured: R=32, S=I=J=64, K=256 (one of the reference's
+// benchmark shapes) 53.8 -> 47.1 us; R=4, S=170, I=90, J=128, K=245 59.9 -> 54.3; R=1, S=570,
+// I=26, J=128, K=1309 66.5 -> 61.9; R=32, S=I=J=128, K=256 281 -> 267.
+static int tall_variant(int v, int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode) {
+    const Lt2Variant &vr = kVariants[v];
+    if (mode == TRT_MODE_UNSPLIT || vr.rt != 1 || vr.gs != 1 || vr.wm != 1 || vr.pack || S <= 32) return v;
+    const int64_t last = S % 64;
+    if (!(last == 0 || last > 32) || R * ceil_div(S, 64) * ceil_div(K, 128) < 12) return v;
+    const int tall = find_lt2_variant(2, vr.nq, false);
+    if (kVariants[tall].rt != 2 || kVariants[tall].nq != vr.nq) return v;
+    return plan_split(R, S, I, J, K, mode, v).split && plan_split(R, S, I, J, K, mode, tall).split ? tall : v;
+}
+
 // AUTO follows the reference in kind -- a small output grid with a long contraction is
 // split (triturus/lt2exp.py:535 tests R*S*K < 1048576 and I*J > 512) -- but decides with a
 // cost model fitted to this machine (measured: R=16 S=64 I=J=32 K=2048, 256 tiles of 32
@@ -793,6 +810,7 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     const bool w_aligned = sw[2] == 1 && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
     // packed rows need 16-byte loads along the flat (i, j) axis; any other call runs the same tile unpacked
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
+    if (variant == 0) v = tall_variant(v, R, S, I, J, K, mode);
     if (variant == 0 && (J % 4 == 0) && w_aligned) v = narrow_variant(paired_variant(v, R, S, I, J, K, mode), S, K);
     // paired groups: aligned rows only, and never under a forced cut over workgroups
     if (kVariants[v].gs == 2 && (!((J % 4 == 0) && w_aligned) || mode == TRT_MODE_SPLIT))
@@ -844,6 +862,7 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
     }
     int v = resolve_variant(variant, R, S, I, J, K);
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
+    if (variant == 0) v = tall_variant(v, R, S, I, J, K, mode);
     if (variant == 0 && (J % 4 == 0) && w_aligned) v = narrow_variant(paired_variant(v, R, S, I, J, K, mode), S, K);
     if (kVariants[v].gs == 2 && (!((J % 4 == 0) && w_aligned) || mode == TRT_MODE_SPLIT))
         v = find_lt2_variant(kVariants[v].rt, kVariants[v].nq, false);
