@@ -110,7 +110,7 @@ def test_edge_shapes(dev, shape, mode):
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
 @pytest.mark.parametrize("shape", [(2, 40, 150, 2, 300), (1, 20, 64, 8, 260), (2, 33, 21, 7, 257), (2, 35, 9, 13, 45),
                                    (1, 70, 20, 33, 300), (2, 16, 5, 50, 64), (2, 40, 30, 3, 100), (1, 70, 9, 5, 64),
-                                   (2, 33, 11, 6, 130)])
+                                   (2, 33, 11, 6, 130), (2, 33, 9, 21, 130)])
 def test_reshaping_front_ends(dev, precision, shape, monkeypatch):
     """The wrapper's two front ends -- roles of (i, a) and (j, b) exchanged on a transposed copy
     of w for a short j axis, and w / b padded to a multiple of 4 in J (for aligned rows, or for
@@ -130,9 +130,11 @@ def test_reshaping_front_ends(dev, precision, shape, monkeypatch):
     a[torch.rand(a.shape, generator=g) < 0.1] = NINF
     b[:, :, 0] = NINF
     for mode in ("auto", "split", "unsplit"):
-        out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision)
-        r = _check(out, w, a, b, **PRECISION_GATES.get(precision, {}))
-        assert r["n_neg_inf"] > 0
+        # (the rule pads J = 21 for its chunk of 24; _pad=True pads the other unaligned J as well)
+        for pad in (None, True):
+            out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision, _pad=pad)
+            r = _check(out, w, a, b, **PRECISION_GATES.get(precision, {}))
+            assert r["n_neg_inf"] > 0
 
 
 def test_empty_inputs(dev):

@@ -56,6 +56,11 @@ def _padded(n: int) -> int:
     return min(-(-n // c) * c for c in (16, 24, 32, 48))
 
 
+def _padded_by_element(n: int) -> int:
+    """The same for rows of w that are not 16-byte aligned: staged by element, in chunks of 16 or 32 only."""
+    return min(-(-n // c) * c for c in (16, 32))
+
+
 def _packs(I: int, J: int) -> bool:
     """Rows of w short enough for the fp32 kernel to walk (i, j) as one flat axis (no padding of j)."""
     return J in (2, 4, 8) and (I * J) % 4 == 0 and I * J >= 32
@@ -63,7 +68,7 @@ def _packs(I: int, J: int) -> bool:
 
 def lt2exp(
     w: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, mode: str = "auto", _variant: int = 0,
-    _precision: str | None = None, _tuning: bool = False,
+    _precision: str | None = None, _tuning: bool = False, _pad: bool | None = None,
 ) -> torch.Tensor:
     wsh, ash, bsh = w.shape, a.shape, b.shape
     assert len(wsh) == 4
@@ -108,12 +113,21 @@ def lt2exp(
         a, b = b, a
         I, J = J, I
     # Rows of w are read 16 bytes at a time only when J is a multiple of 4 (every (s, i) row then
-    # starts aligned); otherwise the kernels fall back to element loads, 15-60 % slower.  A call
-    # with enough work runs on copies padded to the next multiple of 4 instead: zeros in w, -inf
-    # rows in b (terms of weight 0: the result is the same).
-    if (_variant == 0 and J % 4 != 0 and J > 4 and K >= _PAD_MIN_K
-            and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS):
-        J4 = J + (-J) % 4
+    # starts aligned); otherwise the kernels stage w element by element, in j-chunks of 16 or 32
+    # only.  The element loads themselves no longer cost what a padded copy of w and b does (timed
+    # on 70 shapes with J = 9..237: the copies lose by 2-20 % on large calls and up to 2.5x on small
+    # ones), but the chunks do where a chunk of 24 would fit and 32 has to serve: J = 17..23 runs
+    # a third more MFMAs unpadded.  So a call with enough work runs on copies padded to the next
+    # multiple of 4 (zeros in w, -inf rows in b: terms of weight 0, the result is the same) when
+    # that shortens the padded contraction to 0.8 or less (R=64, S=34, I=199, J=17, K=3707:
+    # 1493 -> 1195 us; R=32, S=452, I=97, J=21, K=2188: 1653 -> 1318).
+    # _pad: True / False force the copies / their absence (tests, timing).
+    J4 = J + (-J) % 4
+    # (the bf16 paths, whose unaligned builds stage pairs of columns, keep padding from that work on:
+    # R=S=I=64, K=4096, J = 33 runs in ~300 us padded against 483 with two pieces)
+    pad = (K >= _PAD_MIN_K and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS
+           and (_precision != "fp32" or 5 * _padded(J4) <= 4 * _padded_by_element(J))) if _pad is None else _pad
+    if _variant == 0 and J % 4 != 0 and J > 4 and pad:
         w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
         b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
         J = J4
