@@ -163,9 +163,12 @@ def test_padded_rows_of_a(dev, precision, shape, monkeypatch):
     b[torch.rand(b.shape, generator=g) < 0.05] = NINF
     b[:, :, 0] = NINF
     for splits in (0, 1, 3):
-        out = lm2exp(a.to(dev), b.to(dev), _precision=precision, _splits=splits)
+        # (the fp32 path pads only on request; the bf16 paths by the lowered thresholds)
+        out = lm2exp(a.to(dev), b.to(dev), _precision=precision, _splits=splits, _pad=True)
         r = _check(out, a, b, **PRECISION_GATES.get(precision, {}))
         assert r["n_neg_inf"] > 0
+        _check(lm2exp(a.to(dev), b.to(dev), _precision=precision, _splits=splits, _pad=False), a, b,
+               **PRECISION_GATES.get(precision, {}))
     # a caller's own padded rows (a view of a wider tensor) qualify as well
     wide = torch.full((R, I, J + (-J) % 4 + 4), float("nan"))
     wide[..., :J] = a

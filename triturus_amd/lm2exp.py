@@ -37,7 +37,7 @@ def _unit_inner(t: torch.Tensor) -> torch.Tensor:
 
 _PIECES = {"bf16x3": 2, "bf16x6": 3}
 # from this output width and this much work on, rows of a that are not a multiple of 4 long are
-# padded (tests lower the thresholds to reach that path on small inputs)
+# padded on the bf16 paths (tests lower the thresholds, or pass _pad, to reach that path on small inputs)
 _PAD_MIN_K = 2048
 _PAD_MIN_FLOPS = 2e9
 # tile variants worth timing when tuning is on (0 = the library's rule)
@@ -46,7 +46,8 @@ _BF16_CANDIDATES = (0, 1, 2, 3, 4, 8, 9)
 
 
 def lm2exp(
-    a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0, _splits: int = 0, _precision: str | None = None
+    a: torch.Tensor, b: torch.Tensor, *, _variant: int = 0, _splits: int = 0, _precision: str | None = None,
+    _pad: bool | None = None,
 ) -> torch.Tensor:
     ash, bsh = a.shape, b.shape
     assert len(ash) == len(bsh) == 3
@@ -91,10 +92,13 @@ def lm2exp(
         _variant = autotune.pick(("lm2exp", R, I, J, K, _precision), cands,
                                  lambda v: lm2exp(a, b, _variant=v, _splits=-1, _precision=_precision))
     # Rows of a are read 16 bytes at a time when they start aligned; with J not a multiple of 4 a
-    # contiguous a does not qualify and the kernels fall back to element loads (10-50 % slower).
-    # A call with enough work per element of a (the copy costs ~3 ps per element, the element loads
-    # ~15 % of 20 fs x K) runs on a copy of a whose rows are padded to a multiple of 4.
-    if J % 4 != 0 and J > 4 and sa[2] == 1 and K >= _PAD_MIN_K and 2 * R * I * J * K >= _PAD_MIN_FLOPS:
+    # contiguous a does not qualify and the kernels stage it element by element.  The bf16 paths
+    # then run a call with enough work on a copy of a whose rows are padded to a multiple of 4; on
+    # the fp32 path the copy no longer pays (timed on 50 shapes with J = 9..1347: of the nine the
+    # work thresholds would have padded, six ran 3-18 % slower and three 1-3 % faster).
+    # _pad: True / False force the copy / its absence (tests, timing).
+    pad = (not fp32 and K >= _PAD_MIN_K and 2 * R * I * J * K >= _PAD_MIN_FLOPS) if _pad is None else _pad
+    if J % 4 != 0 and J > 4 and sa[2] == 1 and pad:
         a = torch.nn.functional.pad(a, (0, (-J) % 4))[..., :J]
         sa = a.stride()
     if _splits < 0:  # tuning launch: the library decides the split for this tile
