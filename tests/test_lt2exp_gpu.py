@@ -130,9 +130,11 @@ def test_reshaping_front_ends(dev, precision, shape, monkeypatch):
     a[torch.rand(a.shape, generator=g) < 0.1] = NINF
     b[:, :, 0] = NINF
     for mode in ("auto", "split", "unsplit"):
-        # (the rule pads J = 21 for its chunk of 24; _pad=True pads the other unaligned J as well)
-        for pad in (None, True):
-            out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision, _pad=pad)
+        # (with the thresholds lowered the rules pad J = 21 for its chunk of 24 and, on the bf16
+        # paths, exchange and pad the rest; the fp32 path weighs the copies against the work they
+        # save, so small inputs take them on request)
+        for pad, swap in ((None, None), (True, None), (None, True), (True, True)):
+            out = lt2exp(w.to(dev), a.to(dev), b.to(dev), mode=mode, _precision=precision, _pad=pad, _swap=swap)
             r = _check(out, w, a, b, **PRECISION_GATES.get(precision, {}))
             assert r["n_neg_inf"] > 0
 

@@ -61,6 +61,21 @@ def _padded_by_element(n: int) -> int:
     return min(-(-n // c) * c for c in (16, 32))
 
 
+def _exchange_pays(R: int, S: int, I: int, J: int, K: int) -> bool:
+    """fp32 path: does running with the roles of (i, a) and (j, b) exchanged save more than the
+    transposed copy of w costs?  Saved: the share of the padded contraction that the exchange
+    removes, of a kernel priced at 80 TFLOP/s; cost: w read and written at 2.5 TB/s plus 8 us for
+    the extra launch, with a margin of 20 %.  Timed on 70 shapes with J = 2..24 under I = 9..350:
+    the rule's choice is the faster of the two on 64 of them and within 5 % on the rest, where
+    the former thresholds (a third of the work saved, K >= 256, 4 GFLOP) left the exchange out
+    on 14 shapes that it speeds up by 1.2-2.2x (R=64, S=282, I=64, J=6, K=222: 95 -> 57 us;
+    R=32, S=50, I=196, J=5, K=1219: 177 -> 80, where padding J to 8 gives 135)."""
+    saved = 1.0 - (J * _padded(I)) / (I * _padded(J))
+    kernel_s = 2.0 * R * S * I * _padded(J) * K / 80e12
+    copy_s = 8.0 * R * S * I * J / 2.5e12 + 8e-6
+    return saved * kernel_s >= 1.2 * copy_s
+
+
 def _packs(I: int, J: int) -> bool:
     """Rows of w short enough for the fp32 kernel to walk (i, j) as one flat axis (no padding of j)."""
     return J in (2, 4, 8) and (I * J) % 4 == 0 and I * J >= 32
@@ -68,7 +83,7 @@ def _packs(I: int, J: int) -> bool:
 
 def lt2exp(
     w: torch.Tensor, a: torch.Tensor, b: torch.Tensor, *, mode: str = "auto", _variant: int = 0,
-    _precision: str | None = None, _tuning: bool = False, _pad: bool | None = None,
+    _precision: str | None = None, _tuning: bool = False, _pad: bool | None = None, _swap: bool | None = None,
 ) -> torch.Tensor:
     wsh, ash, bsh = w.shape, a.shape, b.shape
     assert len(wsh) == 4
@@ -99,16 +114,23 @@ def lt2exp(
     # The kernels walk j in chunks of at least 16 and i one at a time: a short j axis under a
     # long i axis wastes most of every chunk.  The contraction is symmetric in (i, a) and (j, b),
     # so such a call runs with the roles exchanged on a transposed copy of w (J = 1 needs no
-    # copy: the library does that exchange itself), when that saves a third of the padded work
-    # and the output is wide enough for the copy not to matter.  Not for forced tiles (tests, tuning),
-    # nor where the fp32 kernel packs the short rows itself.
+    # copy: the library does that exchange itself) when the padded work that saves is worth the
+    # copy (_exchange_pays: fp32) / a third of the padded work on a wide enough output (bf16 paths).
+    # Not for forced tiles (tests, tuning), nor where the fp32 kernel packs the short rows itself.
+    # _swap: True / False force the exchange / its absence (tests, timing).
     if _precision is None:
         _precision = matrix_precision()
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
     packed = _precision == "fp32" and _packs(I, J)
-    if (_variant == 0 and 2 <= J < I and not packed and K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
-            and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS):  # worth a copy kernel: some 40 us of work
+    if _swap is not None:
+        swap = _swap
+    elif _precision == "fp32":
+        swap = _exchange_pays(R, S, I, J, K)
+    else:
+        swap = (K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
+                and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS)  # worth a copy kernel: some 40 us of work
+    if _variant == 0 and 2 <= J < I and not packed and swap:
         w = w.view(R, S, I, J).transpose(2, 3).contiguous().view(R, S, I * J)
         a, b = b, a
         I, J = J, I
@@ -134,8 +156,8 @@ def lt2exp(
     # Rows of 3, 5, 6 or 7 fill a fifth to a half of a j-chunk; padded to 4 or 8 the fp32 kernel
     # packs them (measured R=86 S=482 I=193 K=145: J = 3 574 -> 244 us, J = 5..7 576-594 -> 453-480;
     # at a tenth of that work the copies cost more than they save).
-    if (_variant == 0 and _precision == "fp32" and J in (3, 5, 6, 7) and I * (4 if J == 3 else 8) >= 32
-            and 2 * R * S * I * 16 * K >= _PACK_PAD_MIN_FLOPS):
+    pack_pad = 2 * R * S * I * 16 * K >= _PACK_PAD_MIN_FLOPS if _pad is None else _pad
+    if _variant == 0 and _precision == "fp32" and J in (3, 5, 6, 7) and I * (4 if J == 3 else 8) >= 32 and pack_pad:
         J4 = 4 if J == 3 else 8
         w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
         b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
