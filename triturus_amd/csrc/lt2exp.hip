@@ -668,6 +668,7 @@ struct SplitPlan {
     bool split;
     int splits;
     int iters_per_split;
+    double us = 0.0;  // modelled time of the call (0: this plan comes from a rule, not from the fitted model)
 };
 static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode, int variant);
 
@@ -680,12 +681,34 @@ static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t 
 static int paired_variant(int v, int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode) {
     const Lt2Variant &vr = kVariants[v];
     if (mode == TRT_MODE_SPLIT || vr.nq != 4 || vr.pack || vr.wm != 1 || vr.gs != 1) return v;
-    if (plan_split(R, S, I, J, K, mode, v).split) return v;
+    const SplitPlan sp = plan_split(R, S, I, J, K, mode, v);
     const int64_t ct = ceil_div(K, 128);
     const int64_t n32 = R * ceil_div(S, 32) * ct, n64 = R * ceil_div(S, 64) * ct;
     if (n32 > 512 || I * ceil_div(J, 32) < 2) return v;
     const int64_t last = S % 64;
-    const bool rows64 = I * J <= 1024 && S > 32 && (last == 0 || last > 32) && n64 > 128;
+    const bool pads_alike = S > 32 && (last == 0 || last > 32);
+    if (sp.us > 0.0) {
+        // the plan is the fitted model's (plan_split): paired groups are priced by the same model --
+        // the whole chain on one CU, which two groups of wavefronts keep at 90 % of the rate
+        // (97 % with a second workgroup beside them), half a microsecond for the exchange -- and
+        // taken where that is the cheaper plan (timed on 56 shapes of at most 512 tiles: 0.2 %
+        // behind the better of the two on average; never pairing would lose 1.8 %)
+        const int64_t iters = ceil_div(J, 32) * I;
+        auto paired_us = [&](int rt) {
+            const int64_t q = ceil_div(rt == 2 ? n64 : n32, 256);
+            const double unit_us = (256.0 * 4 * rt + 85.0 + 25.0 * 4) / 2400.0;
+            return 6.4 + (double)q * ((double)iters * unit_us + 0.0062 * (double)(I + J)) / (q >= 2 ? 0.97 : 0.9) + 0.5;
+        };
+        int rt = 1;
+        double us = paired_us(1);
+        if (pads_alike && paired_us(2) < us) {
+            rt = 2;
+            us = paired_us(2);
+        }
+        return us < sp.us ? find_lt2_variant(rt, 4, false, 2) : v;
+    }
+    if (sp.split) return v;
+    const bool rows64 = I * J <= 1024 && pads_alike && n64 > 128;
     return find_lt2_variant(rows64 ? 2 : 1, 4, false, 2);
 }
 
@@ -707,6 +730,15 @@ static int narrow_variant(int v, int64_t S, int64_t K) {
     for (int u = 0; u < kNumVariants; ++u)
         if (kVariants[u].wm == 2) return u;
     return v;
+}
+
+// Where both apply, the 64 x 64 tile goes first under a long contraction (64 steps and more: R=6,
+// S=656, I=40, J=160, K=186 takes 100 us on it, cut, against 129 on paired groups), paired groups
+// under a short one (R=16, S=382, I=10, J=32, K=184: 16.4 against 17.5).
+static int narrow_or_paired_variant(int v, int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, int mode) {
+    const int narrow = narrow_variant(v, S, K);
+    if (narrow != v && I * ceil_div(J, 32) >= 64) return narrow;
+    return narrow_variant(paired_variant(v, R, S, I, J, K, mode), S, K);
 }
 
 // A grid whose contraction is cut over workgroups anyway does not need its tiles to be many: the
@@ -735,6 +767,38 @@ static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t 
     const int64_t iters = v.pack ? ceil_div(I * J, 8 * v.nq) : ceil_div(J, 8 * v.nq) * I;
     if (mode == TRT_MODE_UNSPLIT || v.gs == 2) return {false, 1, (int)iters};
     const int64_t base = R * ceil_div(S, 32 * v.rt * v.wm) * ceil_div(K, 32 * v.ct * (kLt2Waves / v.wm));
+    // 128-column tiles on aligned rows of w: the cut with the least modelled time, where the model
+    // is the one fitted for lm2exp's small grids (csrc/lm2exp.hip, choose_tile_and_cut) with this
+    // kernel's constants: a step costs its MFMAs plus 85 + 25 nq cycles of vector work, a
+    // workgroup's sweeps for the column maxima 6.2 ns per row of a and b, the busiest CU runs
+    // q = ceil(workgroups / 256) chains at 73 % of that rate alone, 93.5 % with two, 95 % with
+    // three, in full from four on; a launch costs 6.4 us, a cut 4.8 us more plus its partial
+    // sums' trip at 3.36 TB/s.  Fitted to cuts of 1..32 timed on 32- and 64-row tiles of 88
+    // shapes; on 83 other shapes (166 tiles) the cut it picks is 1.4 % (mean) behind the best
+    // one timed, the cut of the model below 4.6 % (R=8, S=296, I=184, J=28, K=1556, 64 rows:
+    // 562 us uncut, 435 cut four ways; R=16, S=74, I=55, J=92, K=2372: 488 -> 417).
+    if (!v.pack && v.wm == 1 && v.ct == 1 && J % 4 == 0) {
+        const double unit_us = (256.0 * v.nq * v.rt + 85.0 + 25.0 * v.nq) / 2400.0;
+        const double sweep_us = 0.0062 * (double)(I + J);
+        int best = 1;
+        double best_us = 1e300;
+        const bool forced = mode == TRT_MODE_SPLIT && iters >= 2;  // a cut is asked for: two ways at least
+        for (int sp = forced ? 2 : 1; sp <= 32; ++sp) {
+            if (sp > 1 && 4 * sp > iters && !(forced && sp == 2)) break;  // four steps per workgroup at least
+            const int64_t per = ceil_div(iters, sp);
+            if (ceil_div(iters, per) != sp) continue;  // the same cut as a smaller count
+            const int64_t q = ceil_div(base * sp, 256);
+            const double eff = q >= 4 ? 1.0 : (q == 3 ? 0.95 : (q == 2 ? 0.935 : 0.73));
+            double us = 6.4 + (double)q * ((double)per * unit_us + sweep_us) / eff;
+            if (sp > 1) us += 4.8 + (double)(sp + 1) * (double)(R * S * K) * 4.0 / 3.36e6;
+            if (us < best_us) {
+                best_us = us;
+                best = sp;
+            }
+        }
+        if (best <= 1) return {false, 1, (int)iters, best_us};
+        return {true, best, (int)ceil_div(iters, best), best_us};
+    }
     // (the 64-row tile alone on a CU runs at 67 % of the MFMA rate, two of them at 82 %: measured
     // at R=16 / 32, S=64, I=J=32, K=2048, 40.6 and 66.5 us)
     const bool tall = v.rt >= 2;
@@ -811,7 +875,7 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     // packed rows need 16-byte loads along the flat (i, j) axis; any other call runs the same tile unpacked
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
     if (variant == 0) v = tall_variant(v, R, S, I, J, K, mode);
-    if (variant == 0 && (J % 4 == 0) && w_aligned) v = narrow_variant(paired_variant(v, R, S, I, J, K, mode), S, K);
+    if (variant == 0 && (J % 4 == 0) && w_aligned) v = narrow_or_paired_variant(v, R, S, I, J, K, mode);
     // paired groups: aligned rows only, and never under a forced cut over workgroups
     if (kVariants[v].gs == 2 && (!((J % 4 == 0) && w_aligned) || mode == TRT_MODE_SPLIT))
         v = find_lt2_variant(kVariants[v].rt, kVariants[v].nq, false);
@@ -863,7 +927,7 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
     int v = resolve_variant(variant, R, S, I, J, K);
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
     if (variant == 0) v = tall_variant(v, R, S, I, J, K, mode);
-    if (variant == 0 && (J % 4 == 0) && w_aligned) v = narrow_variant(paired_variant(v, R, S, I, J, K, mode), S, K);
+    if (variant == 0 && (J % 4 == 0) && w_aligned) v = narrow_or_paired_variant(v, R, S, I, J, K, mode);
     if (kVariants[v].gs == 2 && (!((J % 4 == 0) && w_aligned) || mode == TRT_MODE_SPLIT))
         v = find_lt2_variant(kVariants[v].rt, kVariants[v].nq, false);
     const Lt2Variant &vr = kVariants[v];
