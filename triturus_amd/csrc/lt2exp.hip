@@ -699,13 +699,8 @@ static int paired_variant(int v, int64_t R, int64_t S, int64_t I, int64_t J, int
             const double unit_us = (256.0 * 4 * rt + 85.0 + 25.0 * 4) / 2400.0;
             return 6.4 + (double)q * ((double)iters * unit_us + 0.0062 * (double)(I + J)) / (q >= 2 ? 0.97 : 0.9) + 0.5;
         };
-        int rt = 1;
-        double us = paired_us(1);
-        if (pads_alike && paired_us(2) < us) {
-            rt = 2;
-            us = paired_us(2);
-        }
-        return us < sp.us ? find_lt2_variant(rt, 4, false, 2) : v;
+        const int rt = (I * J <= 1024 && pads_alike && n64 > 128) ? 2 : 1;
+        return paired_us(rt) < sp.us ? find_lt2_variant(rt, 4, false, 2) : v;
     }
     if (sp.split) return v;
     const bool rows64 = I * J <= 1024 && pads_alike && n64 > 128;
@@ -781,7 +776,7 @@ static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t 
         const double unit_us = (256.0 * v.nq * v.rt + 85.0 + 25.0 * v.nq) / 2400.0;
         const double sweep_us = 0.0062 * (double)(I + J);
         int best = 1;
-        double best_us = 1e300;
+        double best_us = 1e300, uncut_us = 0.0;
         const bool forced = mode == TRT_MODE_SPLIT && iters >= 2;  // a cut is asked for: two ways at least
         for (int sp = forced ? 2 : 1; sp <= 32; ++sp) {
             if (sp > 1 && 4 * sp > iters && !(forced && sp == 2)) break;  // four steps per workgroup at least
@@ -791,10 +786,18 @@ static SplitPlan plan_split(int64_t R, int64_t S, int64_t I, int64_t J, int64_t 
             const double eff = q >= 4 ? 1.0 : (q == 3 ? 0.95 : (q == 2 ? 0.935 : 0.73));
             double us = 6.4 + (double)q * ((double)per * unit_us + sweep_us) / eff;
             if (sp > 1) us += 4.8 + (double)(sp + 1) * (double)(R * S * K) * 4.0 / 3.36e6;
+            if (sp == 1) uncut_us = us;
             if (us < best_us) {
                 best_us = us;
                 best = sp;
             }
+        }
+        // a cut must win by 3 % (that margin costs nothing on the timed shapes, and on inputs that
+        // are not in cache, as the reference's benchmarks time them, a marginal cut loses: R=128,
+        // S=I=J=96, K=256 runs 2 % slower cut two ways)
+        if (best > 1 && uncut_us > 0.0 && best_us > 0.97 * uncut_us) {
+            best = 1;
+            best_us = uncut_us;
         }
         if (best <= 1) return {false, 1, (int)iters, best_us};
         return {true, best, (int)ceil_div(iters, best), best_us};
