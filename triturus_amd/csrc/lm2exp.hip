@@ -581,11 +581,15 @@ static int find_pair_variant(int rt, int wn = 2) {
 // j-chunk of the 128-, 64- and 32-row tiles: 32, or 16 or 24 where those pad J less.  Per padded j
 // they cost 3-4 % more (R=64, I=256, K=4096: J = 256 takes 281 us on chunks of 32, 287 / 297 on
 // 16 / 24), so J = 16, 24, 40, 48, 72, 80, 144, 200 run 17, 8, 15, 13, 16, 12, 9, 6 % faster.
-// (Not when J is not a multiple of 4: rows of a are then read by element unless the caller padded
-// them, and the smaller chunks, whose tiles leave part of the workgroup without a piece to stage,
-// bear that worst: R=2, I=87, J=482, K=2925 runs 47 % slower on chunks of 16.)
-static int pick_chunk(int64_t J) {
-    if (J % 4 != 0) return 4;
+// J not a multiple of 4 (rows of a are then staged by element unless the caller padded them):
+// chunks of 32, or of 16 where those shorten the padded contraction to 0.9 or less (J = 37, 45,
+// 47: 21-23 % faster; 75, 106: 10-12 %; with less to gain they lose -- a chunk of 16 is twice
+// the steps -- R=2, I=87, J=482, K=2925: 21 % slower) and on the 128-row tile, whose 32-wide
+// chunk is 16 element loads per thread and step (rt = 4; timed on five such shapes: 4-19 % faster
+// on chunks of 16, R=32, I=633, J=273, K=660: 104 -> 84 us).  Chunks of 24 do not divide the
+// workgroup evenly and keep the slow staging for such J.
+static int pick_chunk(int64_t J, int rt = 0) {
+    if (J % 4 != 0) return (10 * ceil_div(J, 16) * 16 <= 9 * ceil_div(J, 32) * 32 || rt == 4) ? 2 : 4;
     int nq = 4;
     int64_t best = ceil_div(J, 32) * 32 * 100;
     const int cand[2] = {2, 3};
@@ -714,7 +718,7 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     } else {
         rt = 1;
     }
-    return find_variant(rt, 4, kOnline, pick_chunk(J));
+    return find_variant(rt, 4, kOnline, pick_chunk(J, rt));
 }
 
 template <int RT, int CT, int WM, int WN, int NQ, bool VEC, int MODE>
@@ -826,7 +830,7 @@ static Lm2Plan make_plan(int64_t R, int64_t I, int64_t J, int64_t K, int variant
     if (joint) {
         tc = choose_tile_and_cut(R, I, J, K, splits_req);
         if (tc.us >= 1e300) tc = choose_tile_and_cut(R, I, J, K, 0);  // a cut the contraction is too short for
-        pl.variant = find_variant(tc.rt, 4, kOnline);
+        pl.variant = find_variant(tc.rt, 4, kOnline, pick_chunk(J, tc.rt));
     } else {
         pl.variant = (variant >= 1) ? variant - 1 : choose_variant(R, I, J, K);
     }
