@@ -383,6 +383,19 @@ def test_small_lm2exp_grids_get_tile_and_cut_chosen_together():
     assert cut(1, 128, 64, 128) == 0
 
 
+def test_lm2exp_takes_64_column_pair_tiles_where_128_column_tiles_would_stand_partly_empty():
+    """Host-side tile rule of lm2exp on large grids (lm2exp_pair_kernel<rows / 64, wavefront
+    columns, ...>: two wavefront columns are a 64-column tile)."""
+    name = lambda R, I, J, K: _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1)
+    assert name(384, 2039, 420, 180) == "trt::lm2exp_pair_kernel<2, 2, 2, 0>"   # 128 rows pad 2039 less than 192
+    assert name(64, 2085, 772, 268) == "trt::lm2exp_pair_kernel<3, 2, 2, 0>"
+    assert name(16, 1755, 268, 652) == "trt::lm2exp_pair_kernel<2, 2, 2, 0>"    # 0.92 of the columns, long and tall
+    assert name(64, 256, 256, 4096) == "trt::lm2exp_pair_kernel<4, 4, 2, 0>"    # whole 128-column tiles
+    assert name(32, 2496, 112, 276).startswith("trt::lm2exp_kernel<")           # a short contraction
+    assert name(384, 654, 96, 564).startswith("trt::lm2exp_kernel<")            # 0.9 of the columns, short
+    assert name(384, 2039, 421, 180).startswith("trt::lm2exp_kernel<")          # rows of a not 16-byte aligned
+
+
 def test_paired_wavefront_groups_take_grids_of_at_most_two_tiles_per_cu():
     """Host-side tile rule of lt2exp (no GPU needed: trt_lt2exp_kernel_name reports what a call
     would launch).  The last template argument is the number of wavefront groups that share a

@@ -146,6 +146,22 @@ def test_small_grids_whose_tile_and_cut_are_chosen_together(dev, shape):
     assert torch.equal(out, lm2exp(a, b))  # deterministic, cut or not
 
 
+@pytest.mark.parametrize("shape", [(64, 700, 200, 180), (96, 390, 256, 144), (40, 1100, 260, 268)])
+def test_large_grids_on_64_column_pair_tiles(dev, shape):
+    """Shapes that the tile rule hands to the 64-column tiles of the paired kernel (K = 144, 180,
+    268 on grids of some hundred tiles): against float64 on the GPU, with -inf columns and zero rows."""
+    R, I, J, K = shape
+    assert "pair_kernel" in _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1)
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(R, I, J, generator=g).to(dev)
+    b = (4 * torch.randn(R, J, K, generator=g) - 10).to(dev)
+    a[:, 5, :] = 0.0
+    b[:, :, K - 1] = NINF
+    out = lm2exp(a, b)
+    r = oracle64.compare(out, oracle64.lm2exp64(a, b, device=dev))
+    assert r["ok"] and r["n_neg_inf"] >= R * (I + K - 1), (shape, r)
+
+
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
 @pytest.mark.parametrize("shape", [(3, 37, 41, 70), (2, 130, 129, 257), (1, 64, 7, 64), (2, 33, 301, 31), (24, 150, 99, 200)])
 def test_padded_rows_of_a(dev, precision, shape, monkeypatch):

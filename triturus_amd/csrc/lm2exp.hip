@@ -677,6 +677,24 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     if (K <= 32 && I > 64 && R * ceil_div(I, 128) >= 96) return find_variant_shape(1, 4, 1);
     if (K <= 64 && I > 32 && !(K <= 32 && I > 64) && R * ceil_div(I, 64) * ceil_div(K, 64) >= 96)
         return find_variant_shape(1, 2, 2);
+    // 64-column tiles of the paired kernel where tiles of 128 columns would stand partly empty:
+    // K = 180 is three tiles of 64 columns or two of 128.  Taken when the 64-column tiling covers
+    // at most 0.85 of the padded columns -- or 0.92 under a long contraction on a tall matrix
+    // (J >= 256, I >= 512) -- on grids of two such tiles per CU and more, for rows of a that are
+    // 16-byte aligned; 192 or 128 rows, whichever pads I less.  Timed on 48 large grids with
+    // K = 144..3168: R=384, I=2039, J=420, K=180 1344 -> 1139 us; R=64, I=2085, J=772, K=268
+    // 688 -> 531; R=128, I=1383, J=1404, K=144 1014 -> 793; R=384, I=358, J=472, K=192 299 -> 234;
+    // R=16, I=1755, J=268, K=652 (0.92) 120 -> 102; between 0.85 and 0.92 on short contractions
+    // the 96-row online tile is as good or better, and under J < 192 the online tiles win whatever
+    // the padding (R=32, I=2496, J=112, K=276: 67 us against 81).
+    {
+        const int64_t c128 = ceil_div(K, 128) * 128, c64 = ceil_div(K, 64) * 64;
+        if (J % 4 == 0 && J >= 192 && I > 96 &&
+            (100 * c64 <= 85 * c128 || (100 * c64 <= 92 * c128 && J >= 256 && I >= 512))) {
+            const int rt = ceil_div(I, 192) * 192 <= ceil_div(I, 128) * 128 ? 3 : 2;
+            if (R * ceil_div(I, 64 * rt) * (c64 / 64) >= 512) return find_pair_variant(rt, 2);
+        }
+    }
     const int64_t kFill = 384;
     const int64_t ct = ceil_div(K, 128);
     // Large grids of 256-row tiles under a contraction of a few hundred: the paired-wavefront
