@@ -567,7 +567,12 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
         // on inputs that are not in cache, as the reference's benchmarks time them): 64 rows.
         const int64_t q64 = ceil_div(n64, 256), q32 = ceil_div(n32, 256);
         const int64_t c64 = 191 * q64 * (q64 == 1 ? 104 : 100), c32 = 100 * q32 * 100;
-        if (same_padding && I * J >= 1024 && c64 < c32) rt = 2;
+        // (Short contractions, I*J < 1024, were measured level on grids of a few tiles per CU; from
+        // four 64-row tiles per CU on they want 64 rows too -- half the workgroups, so half the
+        // sweeps, first loads and result stores that a short chain cannot hide: over 44 large
+        // grids 7-17 % on every such shape, R=64, S=765, I=5, J=108, K=1739: 897 -> 790 us;
+        // R=256, S=52, I=4, J=36, K=2286: 155 -> 132.)
+        if (same_padding && (I * J >= 1024 || n64 >= 1024) && c64 < c32) rt = 2;
         // packed rows spend more vector instructions per step (a factor of a per row of the chunk):
         // sharing them between two MFMAs pays from half a wave of workgroups on, whatever the
         // length of the contraction (measured: 6-13 % at 256..2048 tiles, level at 192, from 4 %
