@@ -364,7 +364,7 @@ def main() -> int:
     kernel = _lib.kernel_name("lt2exp", R, S, I, J, K, _lib.MODE_AUTO, 0, 1)
     head = contraction_line("lt2exp R=64 S=64 I=64 J=64 K=4096 (unsplit)", step, flops,
                             W.lt2exp_bytes(R, S, I, J, K), kernel, args, required_traffic=True,
-                            sibling=lambda: lt2exp(w, a, b, _precision="fp32", _variant=1))  # j-chunks of 64
+                            sibling=lambda: lt2exp(w, a, b, _precision="fp32", _variant=2))  # j-chunks of 32
     value = head["value"]
     launch_ms = head["roofline"]["launch_ms"]["mean"]
     result = {

@@ -407,7 +407,7 @@ def test_paired_wavefront_groups_take_grids_of_at_most_two_tiles_per_cu():
     assert name(16, 32, 32, 32, 2048) == "trt::lt2exp_kernel<1, 1, 4, 4, true, false, 1, 0, 2>"
     assert name(16, 64, 64, 64, 2048).endswith("4, 4, true, false, 1, 0, 2>")
     # the large configuration fills the machine many times over: one group per tile
-    assert name(64, 64, 64, 64, 4096) == "trt::lt2exp_kernel<2, 1, 4, 4, true, false, 1, 0, 1>"
+    assert name(64, 64, 64, 64, 4096) == "trt::lt2exp_kernel<2, 1, 8, 4, true, false, 1, 0, 1>"  # (j-chunks of 64)
     # never under a forced cut over workgroups, for rows of w that are not 16-byte aligned, or
     # where another j-chunk than 32 fits J better
     assert name(16, 64, 32, 32, 2048, mode=_lib.MODE_SPLIT).endswith("true, true, 1, 0, 1>")

@@ -599,6 +599,13 @@ static int choose_variant(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K)
             nq = cand[c];
         }
     }
+    // 64-row tiles on a large grid (four per CU and more) under a J that whole chunks of 64 fit:
+    // chunks of 64 -- half the steps and barriers, and with J = 64 a single j-chunk, so every row
+    // of a is loaded and exponentiated once per tile instead of twice.  Timed side by side,
+    // alternating: R=64, S=I=J=64, K=4096 975.2 -> 967.2 us (every one of 12 pairs within 1 us
+    // of that); R=128, S=I=J=K=256 7675 -> 7560; R=32, S=64, I=128, J=64, K=4096 982 -> 965.  (On
+    // small grids the 64-wide chunk's 16 more registers and coarser steps cost up to 25 %.)
+    if (rt == 2 && nq == 4 && J % 64 == 0 && R * ceil_div(S, 64) * ceil_div(K, 128) >= 1024) nq = 8;
     return find_lt2_variant(rt, nq, false);
 }
 
