@@ -122,18 +122,20 @@ def lt2exp(
         _precision = matrix_precision()
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
-    packed = _precision == "fp32" and _packs(I, J)
-    if _swap is not None:
-        swap = _swap
-    elif _precision == "fp32":
-        swap = _exchange_pays(R, S, I, J, K)
-    else:
-        swap = (K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
-                and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS)  # worth a copy kernel: some 40 us of work
-    if _variant == 0 and 2 <= J < I and not packed and swap:
-        w = w.view(R, S, I, J).transpose(2, 3).contiguous().view(R, S, I * J)
-        a, b = b, a
-        I, J = J, I
+    fp32 = _precision == "fp32"
+    # (the shape tests come first: most calls meet none of them and pay for no rule)
+    if _variant == 0 and 2 <= J < I and not (fp32 and _packs(I, J)):
+        if _swap is not None:
+            swap = _swap
+        elif fp32:
+            swap = _exchange_pays(R, S, I, J, K)
+        else:
+            swap = (K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
+                    and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS)  # worth a copy kernel: some 40 us of work
+        if swap:
+            w = w.view(R, S, I, J).transpose(2, 3).contiguous().view(R, S, I * J)
+            a, b = b, a
+            I, J = J, I
     # Rows of w are read 16 bytes at a time only when J is a multiple of 4 (every (s, i) row then
     # starts aligned); otherwise the kernels stage w element by element, in j-chunks of 16 or 32
     # only.  The element loads themselves no longer cost what a padded copy of w and b does (timed
@@ -144,20 +146,21 @@ def lt2exp(
     # that shortens the padded contraction to 0.8 or less (R=64, S=34, I=199, J=17, K=3707:
     # 1493 -> 1195 us; R=32, S=452, I=97, J=21, K=2188: 1653 -> 1318).
     # _pad: True / False force the copies / their absence (tests, timing).
-    J4 = J + (-J) % 4
     # (the bf16 paths, whose unaligned builds stage pairs of columns, keep padding from that work on:
     # R=S=I=64, K=4096, J = 33 runs in ~300 us padded against 483 with two pieces)
-    pad = (K >= _PAD_MIN_K and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS
-           and (_precision != "fp32" or 5 * _padded(J4) <= 4 * _padded_by_element(J))) if _pad is None else _pad
-    if _variant == 0 and J % 4 != 0 and J > 4 and pad:
-        w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
-        b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
-        J = J4
+    if _variant == 0 and J % 4 != 0 and J > 4:
+        J4 = J + (-J) % 4
+        pad = (K >= _PAD_MIN_K and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS
+               and (not fp32 or 5 * _padded(J4) <= 4 * _padded_by_element(J))) if _pad is None else _pad
+        if pad:
+            w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
+            b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
+            J = J4
     # Rows of 3, 5, 6 or 7 fill a fifth to a half of a j-chunk; padded to 4 or 8 the fp32 kernel
     # packs them (measured R=86 S=482 I=193 K=145: J = 3 574 -> 244 us, J = 5..7 576-594 -> 453-480;
     # at a tenth of that work the copies cost more than they save).
-    pack_pad = 2 * R * S * I * 16 * K >= _PACK_PAD_MIN_FLOPS if _pad is None else _pad
-    if _variant == 0 and _precision == "fp32" and J in (3, 5, 6, 7) and I * (4 if J == 3 else 8) >= 32 and pack_pad:
+    if (_variant == 0 and fp32 and J in (3, 5, 6, 7) and I * (4 if J == 3 else 8) >= 32
+            and (2 * R * S * I * 16 * K >= _PACK_PAD_MIN_FLOPS if _pad is None else _pad)):
         J4 = 4 if J == 3 else 8
         w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
         b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))

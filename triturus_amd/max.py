@@ -53,10 +53,9 @@ def _new_workspace(dev: torch.device, nbytes: int, stream: int) -> torch.Tensor:
     return ws
 
 
-def _workspace(dev: torch.device, nbytes: int):
-    stream = _lib.raw_stream(dev)
+def _workspace(dev: torch.device, nbytes: int, stream: int):
     key = (dev.index, stream)
-    if torch.cuda.is_available() and _is_capturing():
+    if _is_capturing():  # the callers hold a tensor on `dev`, so the runtime is up
         cid = ctypes.c_ulonglong(0)
         _lib.check(_lib.load().trt_stream_capture_id(stream, ctypes.byref(cid)), "trt_stream_capture_id")
         if cid.value:
@@ -103,11 +102,12 @@ def _vmax_impl(x: torch.Tensor, with_index: bool):
     ws_bytes = _ws_bytes.get(key)
     if ws_bytes is None:
         ws_bytes = _ws_bytes[key] = lib.trt_vmax_workspace_bytes(n, code)
-    ws = _workspace(dev, ws_bytes) if ws_bytes else None
+    stream = _lib.raw_stream(dev)
+    ws = _workspace(dev, ws_bytes, stream) if ws_bytes else None
     with _lib.on_device(dev):
         status = lib.trt_vmax(
             x.data_ptr(), n, code, val.data_ptr(), idx.data_ptr() if with_index else None,
-            ws.data_ptr() if ws_bytes else None, ws_bytes, _lib.raw_stream(dev),
+            ws.data_ptr() if ws_bytes else None, ws_bytes, stream,
         )
     if status:
         _lib.check(status, "trt_vmax")
@@ -145,11 +145,12 @@ def matmax(x: torch.Tensor, axis: int = 0, *, block_size: int = 32) -> torch.Ten
     ws_bytes = _ws_bytes.get(key)
     if ws_bytes is None:
         ws_bytes = _ws_bytes[key] = lib.trt_matmax_workspace_bytes(m, n, axis, code)
-    ws = _workspace(dev, ws_bytes) if ws_bytes else None
+    stream = _lib.raw_stream(dev)
+    ws = _workspace(dev, ws_bytes, stream) if ws_bytes else None
     with _lib.on_device(dev):
         status = lib.trt_matmax(
             x.data_ptr(), y.data_ptr(), m, n, axis, code,
-            ws.data_ptr() if ws_bytes else None, ws_bytes, _lib.raw_stream(dev),
+            ws.data_ptr() if ws_bytes else None, ws_bytes, stream,
         )
     if status:
         _lib.check(status, "trt_matmax")
