@@ -27,7 +27,7 @@
 extern "C" {
 #endif
 
-#define TRT_ABI_VERSION 8
+#define TRT_ABI_VERSION 9
 
 #define TRT_OK 0
 #define TRT_E_INVALID (-1)   /* null pointer, non-positive size, bad enum   */
@@ -264,17 +264,24 @@ size_t trt_vmax_workspace_bytes(int64_t n, int dtype);
  * on the fp32 matrix pipe (the lm2exp contraction kernel without shift, exp and log).
  * Replaces the `_ker_mm[grid](...)` launch, triturus/mm.py:199-213.  Not on the log-space
  * path: provided so that the reference's module surface is complete.
+ * variant: 0 = row tile by rule, 1..4 = tiles of 32..128 rows.  splits: 0 = the library
+ * decides whether to cut the product over k (grids of few tiles), 1 = never, n > 1 = n ways
+ * (capped at 32 and at 32 values of k per piece); the partial products are summed in split
+ * order by a second launch, so the result is deterministic.  workspace:
+ * trt_mm_workspace_bytes(m, k, n, variant, splits) bytes, 16-byte aligned; without it a cut
+ * the library chose itself is dropped and an explicit one fails with TRT_E_WORKSPACE.
  */
 int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n,
-               void *stream);
+               int variant, int splits, void *workspace, size_t workspace_bytes, void *stream);
+size_t trt_mm_workspace_bytes(int64_t m, int64_t k, int64_t n, int variant, int splits);
 
 /*
  * trt_mm_f32 on the bf16 matrix pipe with split operands (pieces as for trt_lt2exp_bf16;
  * counterpart of ALLOW_TF32 at triturus/mm.py:212).  Grids too small for the bf16 kernels
- * are handed to trt_mm_f32.
+ * are handed to trt_mm_f32 with the workspace (trt_mm_workspace_bytes(m, k, n, 0, 0) bytes).
  */
 int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n,
-                int pieces, void *stream);
+                int pieces, void *workspace, size_t workspace_bytes, void *stream);
 
 /*
  * r = x + y for contiguous vectors of n elements of `dtype` (TRT_F32 ...).  Replaces the

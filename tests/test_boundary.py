@@ -134,12 +134,19 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_max_workspace_init(null, 1 << 20, null) == -3
     assert lib.trt_max_workspace_init(one, 1024, null) == -3  # smaller than the arrival counters
     # mm, vadd
-    assert lib.trt_mm_f32(one, null, one, 2, 2, 2, null) == -1
-    assert lib.trt_mm_f32(one, one, one, 2, 0, 2, null) == -1
-    assert lib.trt_mm_f32(one, one, one, 1 << 30, 2, 2, null) == -4
-    assert lib.trt_mm_bf16(one, one, one, 2, 2, 2, 4, null) == -1
-    assert lib.trt_mm_bf16(null, one, one, 2, 2, 2, 2, null) == -1
-    assert lib.trt_mm_bf16(one, one, one, 2, 1 << 30, 2, 3, null) == -4
+    assert lib.trt_mm_f32(one, null, one, 2, 2, 2, 0, 0, null, 0, null) == -1
+    assert lib.trt_mm_f32(one, one, one, 2, 0, 2, 0, 0, null, 0, null) == -1
+    assert lib.trt_mm_f32(one, one, one, 2, 2, 2, 5, 0, null, 0, null) == -1
+    assert lib.trt_mm_f32(one, one, one, 2, 2, 2, 0, -1, null, 0, null) == -1
+    assert lib.trt_mm_f32(one, one, one, 1 << 30, 2, 2, 0, 0, null, 0, null) == -4
+    # an explicit cut over k needs its workspace: 2 pieces of a 64 x 64 product
+    assert lib.trt_mm_workspace_bytes(64, 64, 64, 0, 2) == 2 * 64 * 64 * 4
+    assert lib.trt_mm_workspace_bytes(64, 64, 64, 0, 1) == 0
+    assert lib.trt_mm_workspace_bytes(64, 32, 64, 0, 8) == 0  # one chunk of k: nothing to cut
+    assert lib.trt_mm_f32(one, one, one, 64, 64, 64, 0, 2, null, 0, null) == -3
+    assert lib.trt_mm_bf16(one, one, one, 2, 2, 2, 4, null, 0, null) == -1
+    assert lib.trt_mm_bf16(null, one, one, 2, 2, 2, 2, null, 0, null) == -1
+    assert lib.trt_mm_bf16(one, one, one, 2, 1 << 30, 2, 3, null, 0, null) == -4
     assert lib.trt_vadd(one, one, null, 5, 0, null) == -1
     assert lib.trt_vadd(one, one, one, 0, 0, null) == -1
     assert lib.trt_vadd(one, one, one, 5, 7, null) == -1

@@ -64,6 +64,39 @@ def test_mm_on_the_bf16_pipe(dev, precision, shape):
     assert torch.equal(mm(ai, bi, _precision=precision), (ai.double() @ bi.double()).float())
 
 
+@pytest.mark.parametrize("shape", [(512, 512, 512), (256, 4096, 256), (128, 8192, 128), (85, 1594, 82),
+                                   (33, 3001, 131), (64, 4096, 512), (768, 3072, 256), (1, 2000, 1)])
+@pytest.mark.parametrize("tile, cut", [(0, 0), (1, 2), (2, 5), (3, 7), (4, 32), (0, 3)])
+def test_mm_cut_over_k(dev, shape, tile, cut):
+    """Products of few tiles under a long k are cut over k and the pieces summed in split order
+    by a second launch (the rule's choice with tile = cut = 0, else forced): same bounds as the
+    uncut product, exact on small integers, and the same bits call after call."""
+    m, k, n = shape
+    g = torch.Generator().manual_seed(m + k + n)
+    a = torch.randn(m, k, generator=g).to(dev)
+    b = torch.randn(k, n, generator=g).to(dev)
+    c = mm(a, b, _variant=tile, _splits=cut)
+    ref = a.double() @ b.double()
+    # k products of magnitude ~1 added in fp32: the running sum grows like sqrt(j) and each
+    # addition rounds it, so the error's deviation is ~eps k / 5 (5e-5 at k = 4096), its
+    # maximum over the matrix 4-5 of those
+    assert torch.allclose(c.double(), ref, rtol=1e-5, atol=1.5e-7 * k + 1e-6)
+    assert torch.equal(c, mm(a, b, _variant=tile, _splits=cut))
+    ai = torch.randint(-3, 4, (m, k), generator=g).float().to(dev)
+    bi = torch.randint(-3, 4, (k, n), generator=g).float().to(dev)
+    assert torch.equal(mm(ai, bi, _variant=tile, _splits=cut), (ai.double() @ bi.double()).float())
+
+
+def test_mm_rule_cuts_long_products_of_few_tiles(dev):
+    """What the rule decides shows in the workspace it asks for: none for a grid that fills the
+    machine, some for 256 x 4096 x 256 (4 tiles of 128 columns and 32 rows each)."""
+    from triturus_amd import _lib
+    lib = _lib.load()
+    assert lib.trt_mm_workspace_bytes(4096, 512, 4096, 0, 0) == 0
+    assert lib.trt_mm_workspace_bytes(256, 4096, 256, 0, 0) >= 2 * 256 * 256 * 4
+    assert lib.trt_mm_workspace_bytes(256, 4096, 256, 0, 1) == 0
+
+
 def test_mm_rejects_what_the_reference_rejects(dev):
     a = torch.rand(4, 5, device=dev)
     with pytest.raises(AssertionError):

@@ -14,7 +14,7 @@ from pathlib import Path
 import torch
 
 LIB_PATH = Path(__file__).resolve().parent / "lib" / "libtriturus_hip.so"
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 TRT_F32, TRT_F64, TRT_F16, TRT_BF16 = 0, 1, 2, 3
 MODE_AUTO, MODE_SPLIT, MODE_UNSPLIT = 0, 1, 2
@@ -85,8 +85,11 @@ SIGNATURES = {
         [c_void_p, c_void_p, c_int64, c_int64, c_int64, POINTER(c_int64), c_int, c_void_p, c_size_t, c_void_p],
     ),
     "trt_colmax_batched_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64]),
-    "trt_mm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
-    "trt_mm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
+    "trt_mm_f32": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_size_t,
+                           c_void_p]),
+    "trt_mm_workspace_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int, c_int]),
+    "trt_mm_bf16": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p, c_size_t,
+                            c_void_p]),
     "trt_vadd": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int, c_void_p]),
     "trt_copy_bytes": (c_int, [c_void_p, c_void_p, c_size_t, c_void_p]),
     "trt_max_workspace_init": (c_int, [c_void_p, c_size_t, c_void_p]),

@@ -415,7 +415,7 @@ __global__ __launch_bounds__(WM *WN *kWave, 2) void lm2exp_kernel(const Lm2Args 
     for (int ct = 0; ct < CT; ++ct) {
         if (ncol[ct] >= p.K) continue;
         const uint32_t co = ((uint32_t)(4 * h) * orow + (uint32_t)ncol[ct]) * 4u;
-        if (split_out && itile == 0 && wm == 0 && h == 0)
+        if (MODE != kPlain && split_out && itile == 0 && wm == 0 && h == 0)
             p.shift[((int64_t)split * p.R + r) * p.K + ncol[ct]] = mref[ct];
 #pragma unroll
         for (int rt = 0; rt < RT; ++rt)
@@ -1075,22 +1075,110 @@ extern "C" int trt_colmax_batched_f32(const float *b, float *m, int64_t R, int64
     return (int)hipGetLastError();
 }
 
+namespace trt {
+
+// Sum of the partial products of a matrix product that was cut over k, in split order
+// (deterministic).  part: [splits][total]; four elements per lane when VEC.
+template <bool VEC>
+static __global__ __launch_bounds__(256) void mm_merge_kernel(const float *__restrict__ part, float *__restrict__ c,
+                                                              int64_t total, int splits) {
+    const int64_t stride = (int64_t)gridDim.x * 256;
+    if (VEC) {
+        const int64_t quads = total / 4;
+        for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < quads; e += stride) {
+            float4 sum = reinterpret_cast<const float4 *>(part)[e];
+            for (int sp = 1; sp < splits; ++sp) {
+                const float4 x = reinterpret_cast<const float4 *>(part + (int64_t)sp * total)[e];
+                sum.x += x.x; sum.y += x.y; sum.z += x.z; sum.w += x.w;
+            }
+            reinterpret_cast<float4 *>(c)[e] = sum;
+        }
+    } else {
+        for (int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x; e < total; e += stride) {
+            float sum = part[e];
+            for (int sp = 1; sp < splits; ++sp) sum += part[(int64_t)sp * total + e];
+            c[e] = sum;
+        }
+    }
+}
+
+struct MmPlan {
+    int rt;      // rows of the tile / 32
+    int splits;  // workgroups sharing one output tile (cut over k)
+};
+
+// Row tile and cut over k by modelled time.  variant: 0 = any row tile, 1..4 = 32..128 rows.
+// splits_req: 0 = any cut, 1 = never cut, n > 1 = cut n ways (capped at kMaxSplits and at one
+// 32-wide chunk of k per piece).  The model, fitted to 200 random shapes (m, n = 32..4096,
+// k = 64..16384, up to 30 GFLOP) timed on every tile under cuts of 1..32: the busiest CU runs
+// q = ceil(workgroups / 256) workgroups of `per` chunks each, a chunk costing 1096 cycles per 32
+// rows of the tile plus 306; one or two workgroups on a CU reach 0.84 / 0.98 of that rate, and
+// of the 128-row tile three are resident at a time; a launch costs 2.8 us, the merge 3.6 us
+// plus its traffic at 3.0 TB/s.  Its pick is 1.9 % (mean) behind the best combination timed,
+// the worst 17 %; the uncut rule it replaces was 1.99x (geometric mean) behind.
+static MmPlan mm_plan(int64_t m, int64_t k, int64_t n, int variant, int splits_req) {
+    const int64_t chunks = ceil_div(k, 32);
+    const int64_t ct = ceil_div(n, 128);
+    if (splits_req > 1) {  // the count this request comes to
+        int64_t sp = splits_req > kMaxSplits ? kMaxSplits : splits_req;
+        if (sp > chunks) sp = chunks;
+        splits_req = (int)ceil_div(chunks, ceil_div(chunks, sp));
+    }
+    auto rate = [](int64_t x) { return x >= 3 ? 1.0 : x == 2 ? 0.977 : 0.84; };
+    MmPlan best{variant ? variant : 1, 1};
+    double best_us = 1e300;
+    for (int rt = 1; rt <= 4; ++rt) {
+        if (variant ? rt != variant : (rt > 1 && 32 * (rt - 1) >= m)) continue;
+        const int64_t tiles = ceil_div(m, 32 * rt) * ct;
+        const double unit_us = (1096.0 * rt + 306.0) / 2400.0;
+        const int64_t resident = rt == 4 ? 3 : 1 << 20;
+        for (int64_t sp = 1; sp <= kMaxSplits; ++sp) {
+            if (splits_req ? sp != splits_req : (sp > 1 && 2 * sp > chunks)) continue;
+            const int64_t per = ceil_div(chunks, sp);
+            if (ceil_div(chunks, per) != sp) continue;  // the same cut as a smaller count
+            if (sp > 1 && !splits_req && (double)sp * m * n * 4.0 > (double)(1 << 30)) break;
+            const int64_t q = ceil_div(tiles * sp, 256);
+            const int64_t full = q / resident, rem = q % resident;
+            double us = 2.8 + per * unit_us * (full * resident / rate(resident) + (rem ? rem / rate(rem) : 0.0));
+            if (sp > 1) us += 3.6 + (double)(sp + 1) * m * n * 4.0 / 3.03e6;
+            if (us < best_us) {
+                best_us = us;
+                best = MmPlan{rt, (int)sp};
+            }
+        }
+    }
+    return best;
+}
+
+}  // namespace trt
+
+extern "C" size_t trt_mm_workspace_bytes(int64_t m, int64_t k, int64_t n, int variant, int splits) {
+    if (m <= 0 || k <= 0 || n <= 0 || variant < 0 || variant > 4 || splits < 0) return 0;
+    const MmPlan pl = mm_plan(m, k, n, variant, splits);
+    return pl.splits > 1 ? (size_t)pl.splits * m * n * sizeof(float) : 0;
+}
+
 // c = a b for row-major fp32 matrices (m x k times k x n): the contraction kernel above without
-// shift, exp and log.  Replaces the `_ker_mm[grid](...)` launch, triturus/mm.py:199-213.
-extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, void *stream) {
+// shift, exp and log; small grids are cut over k, the partial products summed in split order.
+// Replaces the `_ker_mm[grid](...)` launch, triturus/mm.py:199-213.
+extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, int variant,
+                          int splits, void *workspace, size_t workspace_bytes, void *stream) {
     if (!a || !b || !c) return TRT_E_INVALID;
     if (m <= 0 || k <= 0 || n <= 0) return TRT_E_INVALID;
+    if (variant < 0 || variant > 4 || splits < 0) return TRT_E_INVALID;
     const int64_t lim = (int64_t)1 << 30;
     if (m >= lim || k >= lim || n >= lim) return TRT_E_RANGE;
     if (k * n + n >= lim || m * k + k >= lim || m * n + n >= lim) return TRT_E_RANGE;
-    // row tile by modelled time as for lm2exp with one batch (the per-tile overhead is smaller
-    // without the exp work), else by grid fill
-    const int64_t ct = ceil_div(n, 128);
-    int rt = m > 64 ? pick_tile(1, m, n, 1, false) : 0;
-    if (rt == 0) rt = (m > 32 && ceil_div(m, 64) * ct >= 256) ? 2 : 1;
+    MmPlan pl = mm_plan(m, k, n, variant, splits);
+    if (pl.splits > 1 && (!workspace || workspace_bytes < (size_t)pl.splits * m * n * sizeof(float))) {
+        if (splits > 1) return TRT_E_WORKSPACE;  // an explicit request must be met
+        pl.splits = 1;                            // the rule's cut is an optimisation only
+    }
+    const int rt = pl.rt;
     Lm2Args args;
     args.a = a; args.b = b; args.c = c;
-    args.part = nullptr; args.shift = nullptr;
+    args.part = pl.splits > 1 ? static_cast<float *>(workspace) : nullptr;
+    args.shift = nullptr;
     args.R = 1; args.I = (int)m; args.J = (int)k; args.K = (int)n;
     args.sa0 = m * k; args.sa1 = k;
     args.sb0 = k * n; args.sb1 = n;
@@ -1099,17 +1187,28 @@ extern "C" int trt_mm_f32(const float *a, const float *b, float *c, int64_t m, i
     args.sb2 = 1;
     args.i_tiles = (int)ceil_div(m, 32 * rt);
     args.n_tiles = (int)ceil_div(n, 128);
-    args.splits = 1;
-    args.chunks_per_split = (int)ceil_div(k, 32);
-    args.total_wgs = (int64_t)args.i_tiles * args.n_tiles;
+    args.splits = pl.splits;
+    args.chunks_per_split = (int)ceil_div(ceil_div(k, 32), pl.splits);
+    args.total_wgs = (int64_t)args.i_tiles * args.n_tiles * pl.splits;
     args.padded_wgs = ceil_div(args.total_wgs, kXcds) * kXcds;
     args.stream_out = rows_16_byte_aligned(c, args.sc0, args.sc1);
     if (args.padded_wgs >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const bool vec = (k % 4 == 0) && ((reinterpret_cast<uintptr_t>(a) & 15) == 0);
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (rt == 4) return launch_v<4, 1, 1, 4, 4, kPlain>(args, vec, s);
-    if (rt == 3) return launch_v<3, 1, 1, 4, 4, kPlain>(args, vec, s);
-    if (rt == 2) return launch_v<2, 1, 1, 4, 4, kPlain>(args, vec, s);
-    return launch_v<1, 1, 1, 4, 4, kPlain>(args, vec, s);
+    int st;
+    if (rt == 4) st = launch_v<4, 1, 1, 4, 4, kPlain>(args, vec, s);
+    else if (rt == 3) st = launch_v<3, 1, 1, 4, 4, kPlain>(args, vec, s);
+    else if (rt == 2) st = launch_v<2, 1, 1, 4, 4, kPlain>(args, vec, s);
+    else st = launch_v<1, 1, 1, 4, 4, kPlain>(args, vec, s);
+    if (st != 0 || pl.splits <= 1) return st;
+    const int64_t total = m * n;
+    const bool vec4 = total % 4 == 0 && ((reinterpret_cast<uintptr_t>(c) | reinterpret_cast<uintptr_t>(workspace)) & 15) == 0;
+    int64_t blocks = ceil_div(vec4 ? total / 4 : total, 256);
+    if (blocks > 4096) blocks = 4096;
+    if (vec4)
+        hipLaunchKernelGGL(mm_merge_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, s, args.part, c, total, pl.splits);
+    else
+        hipLaunchKernelGGL(mm_merge_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, s, args.part, c, total, pl.splits);
+    return (int)hipGetLastError();
 }
 

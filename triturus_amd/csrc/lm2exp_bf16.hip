@@ -557,7 +557,7 @@ static int launch_mm_bf(const Lm2BfArgs &args, int pieces, bool vec, hipStream_t
 }
 
 extern "C" int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, int64_t k, int64_t n, int pieces,
-                           void *stream) {
+                           void *workspace, size_t workspace_bytes, void *stream) {
     if (!a || !b || !c) return TRT_E_INVALID;
     if (m <= 0 || k <= 0 || n <= 0) return TRT_E_INVALID;
     if (pieces != 2 && pieces != 3) return TRT_E_INVALID;
@@ -569,7 +569,7 @@ extern "C" int trt_mm_bf16(const float *a, const float *b, float *c, int64_t m, 
     int rt;
     if (m > 64 && n128 >= 384) rt = 4;
     else if (m > 32 && n64 >= 256) rt = 2;
-    else return trt_mm_f32(a, b, c, m, k, n, stream);
+    else return trt_mm_f32(a, b, c, m, k, n, 0, 0, workspace, workspace_bytes, stream);
     Lm2BfArgs args;
     args.a = a; args.b = b; args.c = c;
     args.R = 1; args.I = (int)m; args.J = (int)k; args.K = (int)n;

@@ -17,7 +17,11 @@ from triturus_amd import _lib
 from triturus_amd.utils import is_triturus_tf32_enabled, pinned_matrix_precision
 
 
-def mm(a: torch.Tensor, b: torch.Tensor, *, _precision: str | None = None) -> torch.Tensor:
+_ws_bytes: dict = {}  # (m, k, n, row tile, cut) -> workspace bytes
+
+
+def mm(a: torch.Tensor, b: torch.Tensor, *, _precision: str | None = None, _variant: int = 0,
+       _splits: int = 0) -> torch.Tensor:
     assert len(a.shape) == len(b.shape) == 2
     assert a.shape[1] == b.shape[0]
     assert a.dtype == b.dtype == torch.float32
@@ -35,12 +39,23 @@ def mm(a: torch.Tensor, b: torch.Tensor, *, _precision: str | None = None) -> to
     # the flag alone selects three pieces: inside the reference's fp32-level test tolerance
     # (tests/mm.py:16 uses torch.allclose defaults with the flag on as well)
     precision = _precision or pinned_matrix_precision() or ("bf16x6" if is_triturus_tf32_enabled() else "fp32")
+    # grids of few tiles are cut over k (the partial products meet in a workspace); _variant
+    # and _splits force the row tile (1..4: 32..128 rows) and the cut (tests, timing)
+    fp32 = precision == "fp32"
+    key = (m, k, n, _variant if fp32 else 0, _splits if fp32 else 0)
+    ws_bytes = _ws_bytes.get(key)
+    if ws_bytes is None:
+        ws_bytes = _ws_bytes[key] = lib.trt_mm_workspace_bytes(*key)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=a.device) if ws_bytes else None
+    ws_ptr = ws.data_ptr() if ws_bytes else None
     with _lib.on_device(a.device):
-        if precision == "fp32":
-            status = lib.trt_mm_f32(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, k, n, _lib.raw_stream(a.device))
+        if fp32:
+            status = lib.trt_mm_f32(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, k, n, _variant, _splits,
+                                    ws_ptr, ws_bytes, _lib.raw_stream(a.device))
         else:
             status = lib.trt_mm_bf16(a.data_ptr(), b.data_ptr(), c.data_ptr(), m, k, n,
-                                     {"bf16x3": 2, "bf16x6": 3}[precision], _lib.raw_stream(a.device))
+                                     {"bf16x3": 2, "bf16x6": 3}[precision], ws_ptr, ws_bytes,
+                                     _lib.raw_stream(a.device))
     if status:
         _lib.check(status, "trt_mm")
     return c
