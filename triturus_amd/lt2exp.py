@@ -61,15 +61,37 @@ def _padded_by_element(n: int) -> int:
     return min(-(-n // c) * c for c in (16, 32))
 
 
+def _kernel_us(R: int, S: int, I: int, J: int, K: int) -> float:
+    """Rough time of the fp32 contraction kernel on these sizes, for weighing one front end
+    against another (microseconds, without the launch): the padded work -- S to tiles of 32
+    rows, K to one 64-column tile or tiles of 128, J to whole chunks -- at 109 TFLOP/s, less on
+    a grid that leaves compute units idle (fill ** 0.38) and on rows of w that are not 16-byte
+    aligned (0.89), or w streamed at 2.65 TB/s where that takes longer."""
+    tiles = R * -(-S // 32) * (1 if K <= 64 else -(-K // 128))
+    fill = min(1.0, tiles / 256.0)
+    padded_j = _padded(J) if J % 4 == 0 else _padded_by_element(J)
+    flops = 2.0 * R * (-(-S // 32) * 32) * I * padded_j * (64 if K <= 64 else -(-K // 128) * 128)
+    compute = flops / (109e6 * fill ** 0.38 * (1.0 if J % 4 == 0 else 0.89))
+    stream = R * S * I * J * 4 / 2.65e6
+    return max(compute, stream)
+
+
 def _exchange_pays(R: int, S: int, I: int, J: int, K: int) -> bool:
-    """fp32 path: does running with the roles of (i, a) and (j, b) exchanged save more than the
-    transposed copy of w costs?  Saved: the share of the padded contraction that the exchange
-    removes, of a kernel priced at 80 TFLOP/s; cost: w read and written at 2.5 TB/s plus 8 us for
-    the extra launch, with a margin of 20 %.  Timed on 70 shapes with J = 2..24 under I = 9..350:
-    the rule's choice is the faster of the two on 64 of them and within 5 % on the rest, where
-    the former thresholds (a third of the work saved, K >= 256, 4 GFLOP) left the exchange out
-    on 14 shapes that it speeds up by 1.2-2.2x (R=64, S=282, I=64, J=6, K=222: 95 -> 57 us;
-    R=32, S=50, I=196, J=5, K=1219: 177 -> 80, where padding J to 8 gives 135)."""
+    """fp32 path: is the call faster with the roles of (i, a) and (j, b) exchanged, transposed
+    copy of w included?
+    Rows of at most 8 values: by the model above, the copy at 6.2 us and its traffic at 9.7 TB/s
+    (w is often still in cache).  The constants here and in _kernel_us were fitted to 378 shapes
+    timed both ways (R = 1..256, S = 4..1024, J = 2..24 under I = 3..400, K = 1..4096); on the
+    220 of them with J <= 8 and 74 others the rule's choice is 0.6-0.8 % (mean) behind the faster
+    of the two, where the rule below stood 8-10 % behind -- it leaves out narrow and short
+    outputs, which pad S and K (R=227, S=4, I=31, J=3, K=891: 65 -> 26 us; R=36, S=44, I=355,
+    J=2, K=47: 54 -> 24).
+    Longer rows: the padded work saved, of a kernel priced at 80 TFLOP/s, against w read and
+    written at 2.5 TB/s plus 8 us, with a margin of 20 % (0.6-1.1 % behind the faster of the two
+    on 278 shapes with J = 9..249, where the model above, which does not see what rows that are
+    not 16-byte aligned cost on either side of the exchange, stood 1.4-7.5 % behind)."""
+    if J <= 8:
+        return _kernel_us(R, S, J, I, K) + 6.2 + 8.0 * R * S * I * J / 9.7e6 < _kernel_us(R, S, I, J, K)
     saved = 1.0 - (J * _padded(I)) / (I * _padded(J))
     kernel_s = 2.0 * R * S * I * _padded(J) * K / 80e12
     copy_s = 8.0 * R * S * I * J / 2.5e12 + 8e-6
