@@ -403,6 +403,19 @@ def test_lm2exp_takes_64_column_pair_tiles_where_128_column_tiles_would_stand_pa
     assert name(384, 2039, 421, 180).startswith("trt::lm2exp_kernel<")          # rows of a not 16-byte aligned
 
 
+def test_lm2exp_outputs_of_at_most_64_columns_take_the_narrow_tiles():
+    """Host-side tile rule of lm2exp for K <= 64 (lm2exp_kernel<rows / 32, column blocks, wavefronts
+    over rows, wavefronts over columns, ...>): the wavefronts are stacked over rows whatever the
+    number of tiles; large grids of 33..64 columns take the paired kernel's 128 x 64 tile."""
+    name = lambda R, I, J, K: _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1)
+    assert name(30, 283, 2788, 10) == "trt::lm2exp_kernel<1, 1, 4, 1, 4, true, 1>"    # 128 x 32, 90 tiles
+    assert name(10, 162, 1324, 39) == "trt::lm2exp_kernel<1, 1, 2, 2, 4, true, 1>"    # 64 x 64, 30 tiles
+    assert name(101, 1510, 48, 48) == "trt::lm2exp_pair_kernel<2, 2, 2, 0>"           # 2424 tiles of 64 rows
+    assert name(14, 2464, 2688, 48) == "trt::lm2exp_pair_kernel<2, 2, 2, 0>"          # 546, a long contraction
+    assert name(203, 267, 2788, 63) == "trt::lm2exp_kernel<1, 1, 2, 2, 4, true, 1>"   # 128 rows would pad 267 to 384
+    assert name(40, 30, 500, 20) == "trt::lm2exp_kernel<1, 1, 1, 4, 4, true, 1>"      # I <= 32: the 32 x 128 tile
+
+
 def test_paired_wavefront_groups_take_grids_of_at_most_two_tiles_per_cu():
     """Host-side tile rule of lt2exp (no GPU needed: trt_lt2exp_kernel_name reports what a call
     would launch).  The last template argument is the number of wavefront groups that share a

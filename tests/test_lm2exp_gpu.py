@@ -162,6 +162,29 @@ def test_large_grids_on_64_column_pair_tiles(dev, shape):
     assert r["ok"] and r["n_neg_inf"] >= R * (I + K - 1), (shape, r)
 
 
+@pytest.mark.parametrize("shape, kernel", [
+    ((30, 283, 700, 10), "lm2exp_kernel<1, 1, 4, 1,"),     # 128 x 32 tiles, 90 of them, cut over J
+    ((3, 170, 1500, 47), "lm2exp_kernel<1, 1, 2, 2,"),     # 64 x 64 tiles, 9 of them, cut over J
+    ((101, 1510, 48, 48), "lm2exp_pair_kernel<2, 2,"),     # 128 x 64 paired tiles on a large grid
+    ((14, 2464, 1001, 48), "lm2exp_pair_kernel<2, 2,"),    # ... under a long contraction, rows of a unaligned
+    ((436, 89, 300, 46), "lm2exp_pair_kernel<2, 2,"),
+])
+def test_outputs_of_at_most_64_columns(dev, shape, kernel):
+    """The narrow tiles that K <= 64 takes whatever the size of the grid, and the paired 128 x 64
+    tile of large grids: against float64 on the GPU, with -inf columns and zero rows."""
+    R, I, J, K = shape
+    assert kernel in _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, int(J % 4 == 0))
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(R, I, J, generator=g).to(dev)
+    b = (4 * torch.randn(R, J, K, generator=g) - 10).to(dev)
+    a[:, 5, :] = 0.0
+    b[:, :, K - 1] = NINF
+    out = lm2exp(a, b)
+    r = oracle64.compare(out, oracle64.lm2exp64(a, b, device=dev))
+    assert r["ok"] and r["n_neg_inf"] >= R * (I + K - 1), (shape, r)
+    assert torch.equal(out, lm2exp(a, b))
+
+
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
 @pytest.mark.parametrize("shape", [(3, 37, 41, 70), (2, 130, 129, 257), (1, 64, 7, 64), (2, 33, 301, 31), (24, 150, 99, 200)])
 def test_padded_rows_of_a(dev, precision, shape, monkeypatch):

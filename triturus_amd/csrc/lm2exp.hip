@@ -675,12 +675,23 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     // 128-column tile idle: the wavefronts are stacked over rows instead (128 x 32 and 64 x 64
     // tiles).  R=31, I=2527, J=2423, K=20: 479 -> 269 us; R=26, I=820, J=2949, K=14: 187 -> 91;
     // R=96, I=2932, J=135, K=34: 112 -> 81.
-    // (only with some hundred such tiles: below that the call is latency bound and wants the
-    // most workgroups, which the 32-row tiles of the rules below give; over 80 random narrow
-    // shapes this threshold took the loss against the best tile from 5.6 to 2.6 %)
-    if (K <= 32 && I > 64 && R * ceil_div(I, 128) >= 96) return find_variant_shape(1, 4, 1);
-    if (K <= 64 && I > 32 && !(K <= 32 && I > 64) && R * ceil_div(I, 64) * ceil_div(K, 64) >= 96)
+    // Whatever the number of tiles: few of them under a long contraction are cut over J like any
+    // other tile, and over 250 random shapes with K = 9..64 (every tile timed) a threshold of 96
+    // tiles left the rule 8.6 % (mean) behind the best tile -- R=30, I=283, J=2788, K=10: 72 us on
+    // 32 x 128 tiles against 39 -- where taking the narrow tiles throughout stands 4.0 % behind.
+    // Large grids of 33..64 columns go to the paired-wavefront kernel's 128 x 64 tile when its
+    // 128 rows pad I little more than 64 would (at most 1.1x): the exps of a column shared by two
+    // wavefronts, 10-25 % ahead from some 600 tiles of 64 rows on, from 200 under a contraction of
+    // 32 chunks and more (R=101, I=1510, J=48, K=48: 23 -> 18 us; R=436, I=89, J=1384, K=46: 127 ->
+    // 113; R=14, I=2464, J=2688, K=48: 180 -> 134), which takes the rule to 2.9 % over those 250
+    // shapes and 200 others.
+    if (K <= 32 && I > 64) return find_variant_shape(1, 4, 1);
+    if (K <= 64 && I > 32) {
+        const int64_t t64 = R * ceil_div(I, 64);
+        if ((t64 >= 600 || (t64 >= 200 && J >= 32 * 31 + 1)) && 10 * ceil_div(I, 128) * 128 <= 11 * ceil_div(I, 64) * 64)
+            return find_pair_variant(2, 2);
         return find_variant_shape(1, 2, 2);
+    }
     // 64-column tiles of the paired kernel where tiles of 128 columns would stand partly empty:
     // K = 180 is three tiles of 64 columns or two of 128.  Taken when the 64-column tiling covers
     // at most 0.85 of the padded columns -- or 0.92 under a long contraction on a tall matrix
