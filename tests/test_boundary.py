@@ -400,7 +400,14 @@ def test_lm2exp_takes_64_column_pair_tiles_where_128_column_tiles_would_stand_pa
     assert name(64, 256, 256, 4096) == "trt::lm2exp_pair_kernel<4, 4, 2, 0>"    # whole 128-column tiles
     assert name(32, 2496, 112, 276).startswith("trt::lm2exp_kernel<")           # a short contraction
     assert name(384, 654, 96, 564).startswith("trt::lm2exp_kernel<")            # 0.9 of the columns, short
-    assert name(384, 2039, 421, 180).startswith("trt::lm2exp_kernel<")          # rows of a not 16-byte aligned
+    # rows of a that are not 16-byte aligned take the same tiles (last argument: how a is loaded)
+    assert _lib.kernel_name("lm2exp", 384, 2039, 421, 180, 0, 0, 0) == "trt::lm2exp_pair_kernel<2, 2, 2, 1>"
+    # smaller grids whose K leaves a quarter of the 128-column tiling empty: 64 x 64 tiles from 100 on
+    assert name(6, 1159, 2880, 159) == "trt::lm2exp_pair_kernel<1, 2, 2, 0>"
+    assert _lib.kernel_name("lm2exp", 3, 2878, 587, 158, 0, 0, 0) == "trt::lm2exp_pair_kernel<1, 2, 2, 1>"
+    assert name(3, 2878, 100, 158).startswith("trt::lm2exp_kernel<")            # a short contraction
+    assert name(1, 1159, 2880, 159).startswith("trt::lm2exp_kernel<")           # 57 tiles
+    assert name(6, 1159, 2880, 300).startswith("trt::lm2exp_kernel<")           # 320 of 384 columns
 
 
 def test_lm2exp_outputs_of_at_most_64_columns_take_the_narrow_tiles():

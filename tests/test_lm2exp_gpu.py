@@ -146,12 +146,14 @@ def test_small_grids_whose_tile_and_cut_are_chosen_together(dev, shape):
     assert torch.equal(out, lm2exp(a, b))  # deterministic, cut or not
 
 
-@pytest.mark.parametrize("shape", [(64, 700, 200, 180), (96, 390, 256, 144), (40, 1100, 260, 268)])
+@pytest.mark.parametrize("shape", [(64, 700, 200, 180), (96, 390, 256, 144), (40, 1100, 260, 268),
+                                   (64, 700, 201, 180), (96, 390, 131, 144),  # rows of a not 16-byte aligned
+                                   (3, 2878, 587, 158), (6, 1159, 1000, 159)])  # smaller grids: 64 x 64 tiles
 def test_large_grids_on_64_column_pair_tiles(dev, shape):
     """Shapes that the tile rule hands to the 64-column tiles of the paired kernel (K = 144, 180,
     268 on grids of some hundred tiles): against float64 on the GPU, with -inf columns and zero rows."""
     R, I, J, K = shape
-    assert "pair_kernel" in _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1)
+    assert "pair_kernel" in _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, int(J % 4 == 0))
     g = torch.Generator().manual_seed(sum(shape))
     a = torch.rand(R, I, J, generator=g).to(dev)
     b = (4 * torch.randn(R, J, K, generator=g) - 10).to(dev)

@@ -670,6 +670,33 @@ static int pick_tile(int64_t R, int64_t I, int64_t K, int overhead_quarters, boo
     return best;
 }
 
+// 64-column tiles of the paired kernel where tiles of 128 columns would stand partly empty:
+// K = 180 is three tiles of 64 columns or two of 128.  Taken when the 64-column tiling covers
+// at most 0.85 of the padded columns -- or 0.92 under a long contraction on a tall matrix
+// (J >= 256, I >= 512) -- on grids of two such tiles per CU and more; 192 or 128 rows,
+// whichever pads I less.  Timed on 48 large grids with
+// K = 144..3168: R=384, I=2039, J=420, K=180 1344 -> 1139 us; R=64, I=2085, J=772, K=268
+// 688 -> 531; R=128, I=1383, J=1404, K=144 1014 -> 793; R=384, I=358, J=472, K=192 299 -> 234;
+// R=16, I=1755, J=268, K=652 (0.92) 120 -> 102; between 0.85 and 0.92 on short contractions
+// the 96-row online tile is as good or better, and under J < 128 the online tiles are level or
+// ahead whatever the padding (R=32, I=2496, J=112, K=276: 65-67 us on either).  Rows of a that are not 16-byte aligned take them too (R=146, I=586, J=317,
+// K=146: 138 -> 112 us; R=45, I=3374, J=211, K=144: 162 -> 126), and smaller grids whose K
+// leaves a quarter of the 128-column tiling empty (K = 129..192) take the 64 x 64 tile of the
+// same kernel from 100 tiles on (R=3, I=2878, J=587, K=158: 45 -> 32 us; R=6, I=1159, J=2879,
+// K=159: 114 -> 95).  Over 200 random shapes with K = 128 m + 1..64 on which every tile was
+// timed: 4.7 % -> 2.8 % (mean) behind the best tile.
+static int pair64_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
+    if (K <= 64) return -1;
+    const int64_t c128 = ceil_div(K, 128) * 128, c64 = ceil_div(K, 64) * 64;
+    if (J >= 128 && I > 96 && (100 * c64 <= 85 * c128 || (100 * c64 <= 92 * c128 && J >= 256 && I >= 512))) {
+        const int rt = ceil_div(I, 192) * 192 <= ceil_div(I, 128) * 128 ? 3 : 2;
+        if (R * ceil_div(I, 64 * rt) * (c64 / 64) >= 512) return find_pair_variant(rt, 2);
+    }
+    if (J >= 192 && I > 64 && 100 * c64 <= 76 * c128 && R * ceil_div(I, 64) * (c64 / 64) >= 100)
+        return find_pair_variant(1, 2);
+    return -1;
+}
+
 static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
     // Outputs of at most 32 (64) columns would leave three (two) of the four wavefronts of a
     // 128-column tile idle: the wavefronts are stacked over rows instead (128 x 32 and 64 x 64
@@ -692,23 +719,9 @@ static int choose_variant(int64_t R, int64_t I, int64_t J, int64_t K) {
             return find_pair_variant(2, 2);
         return find_variant_shape(1, 2, 2);
     }
-    // 64-column tiles of the paired kernel where tiles of 128 columns would stand partly empty:
-    // K = 180 is three tiles of 64 columns or two of 128.  Taken when the 64-column tiling covers
-    // at most 0.85 of the padded columns -- or 0.92 under a long contraction on a tall matrix
-    // (J >= 256, I >= 512) -- on grids of two such tiles per CU and more, for rows of a that are
-    // 16-byte aligned; 192 or 128 rows, whichever pads I less.  Timed on 48 large grids with
-    // K = 144..3168: R=384, I=2039, J=420, K=180 1344 -> 1139 us; R=64, I=2085, J=772, K=268
-    // 688 -> 531; R=128, I=1383, J=1404, K=144 1014 -> 793; R=384, I=358, J=472, K=192 299 -> 234;
-    // R=16, I=1755, J=268, K=652 (0.92) 120 -> 102; between 0.85 and 0.92 on short contractions
-    // the 96-row online tile is as good or better, and under J < 192 the online tiles win whatever
-    // the padding (R=32, I=2496, J=112, K=276: 67 us against 81).
     {
-        const int64_t c128 = ceil_div(K, 128) * 128, c64 = ceil_div(K, 64) * 64;
-        if (J % 4 == 0 && J >= 192 && I > 96 &&
-            (100 * c64 <= 85 * c128 || (100 * c64 <= 92 * c128 && J >= 256 && I >= 512))) {
-            const int rt = ceil_div(I, 192) * 192 <= ceil_div(I, 128) * 128 ? 3 : 2;
-            if (R * ceil_div(I, 64 * rt) * (c64 / 64) >= 512) return find_pair_variant(rt, 2);
-        }
+        const int pv = pair64_variant(R, I, J, K);
+        if (pv >= 0) return pv;
     }
     const int64_t kFill = 384;
     const int64_t ct = ceil_div(K, 128);
@@ -858,7 +871,9 @@ static TileCut choose_tile_and_cut(int64_t R, int64_t I, int64_t J, int64_t K, i
 // e.g. batch 1, I=J=K=1024 is 64 tiles of 128 x 128 but 32 chunks deep.
 static Lm2Plan make_plan(int64_t R, int64_t I, int64_t J, int64_t K, int variant, int splits_req) {
     Lm2Plan pl;
-    const bool joint = variant < 1 && joint_region(R, I, J, K);
+    // (the 64-column tiles of the paired kernel go before the joint model, which knows the
+    // 128-column tiles only)
+    const bool joint = variant < 1 && joint_region(R, I, J, K) && pair64_variant(R, I, J, K) < 0;
     TileCut tc{1, 1, 0.0};
     if (joint) {
         tc = choose_tile_and_cut(R, I, J, K, splits_req);
