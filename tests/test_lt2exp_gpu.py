@@ -560,3 +560,58 @@ def test_bf16_paths_c5_full_size(dev, precision):
     assert torch.allclose(out_shift[fin], (out - t)[fin], rtol=1e-4, atol=2e-4)
     out_scaled = lt2exp(w * 8.0, a, b, _precision=precision)
     assert torch.allclose(out_scaled[fin], (out + float(np.log(8.0)))[fin], rtol=1e-6, atol=1e-5)
+
+
+SWEEP_SHAPES = [
+    (64, 64, 64, 64, 1), (64, 64, 64, 64, 8), (16, 100, 33, 28, 3), (8, 64, 16, 4, 5),     # a wavefront per row
+    (200, 3, 5, 24, 2), (130, 1, 64, 64, 7), (3, 333, 12, 20, 4), (1, 700, 100, 8, 6),
+    (4, 64, 64, 64, 4), (2, 70, 17, 12, 1), (1, 128, 3, 300, 8), (16, 8, 40, 40, 2),      # a workgroup per row
+    (64, 64, 1, 64, 2), (64, 64, 64, 1, 2), (5, 130, 1024, 4, 3), (2, 300, 2, 1024, 8),   # J = 1 exchanged; long axes
+]
+
+
+@pytest.mark.parametrize("shape", SWEEP_SHAPES)
+def test_outputs_of_at_most_8_columns_take_the_sweep(dev, shape):
+    """K <= 8 with rows of w that can be read 16 bytes at a time: the vector-ALU sweep over w
+    (csrc/lt2exp_smallk.hpp) against the float64 oracle, -inf and NaN columns included, and
+    against the matrix-pipe kernel on the same operands."""
+    R, S, I, J, K = shape
+    assert "smallk_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1)
+    g = torch.Generator().manual_seed(sum(shape))
+    w = torch.rand(R, S, I, J, generator=g)
+    w[:, S // 2] = 0.0
+    a = 5 * torch.randn(R, I, K, generator=g) - 10
+    b = 5 * torch.randn(R, J, K, generator=g) + 3
+    a[0, :, 0] = NINF                       # a whole column of a: -inf out
+    b[R - 1, J // 2, K - 1] = NINF          # a single -inf entry: finite out
+    ref = oracle64.lt2exp64(w, a, b, batch_chunk=8)
+    out = lt2exp(w.to(dev), a.to(dev), b.to(dev))
+    r = oracle64.compare(out, ref)
+    assert r["ok"], (shape, r)
+    assert torch.isneginf(out[0, :, 0]).all() and torch.isneginf(out[:, S // 2]).all()
+    assert torch.equal(out, lt2exp(w.to(dev), a.to(dev), b.to(dev)))
+    mfma = lt2exp(w.to(dev), a.to(dev), b.to(dev), _variant=4)
+    assert torch.allclose(out, mfma, rtol=1e-5, atol=1e-5)
+    for prec in ("bf16x3", "bf16x6"):        # handed over to the same sweep
+        assert torch.equal(out, lt2exp(w.to(dev), a.to(dev), b.to(dev), _precision=prec))
+    an = a.clone()
+    an[R // 2, I // 2, K // 2] = float("nan")
+    outn = lt2exp(w.to(dev), an.to(dev), b.to(dev))
+    assert torch.isnan(outn[R // 2, :, K // 2]).all()
+    mask = torch.ones_like(outn, dtype=torch.bool)
+    mask[R // 2, :, K // 2] = False
+    assert torch.equal(outn[mask], out[mask])
+
+
+def test_the_sweep_reads_strided_a_and_b_and_sliced_w_in_place(dev):
+    R, S, I, J, K = 12, 50, 24, 16, 5
+    g = torch.Generator().manual_seed(5)
+    wide = torch.rand(R, S + 3, I, J, generator=g).to(dev)
+    w = wide[:, 2:S + 2]                                           # rows stay 16-byte aligned
+    a = (3 * torch.randn(R, K, I, generator=g)).to(dev).transpose(1, 2)   # K-major
+    b = (3 * torch.randn(R, J, 2 * K, generator=g)).to(dev)[:, :, ::2]    # every other column
+    assert "smallk_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1)
+    out = lt2exp(w, a, b)
+    r = oracle64.compare(out, oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=4))
+    assert r["ok"], r
+    assert torch.equal(out, lt2exp(w.contiguous(), a.contiguous(), b.contiguous()))

@@ -21,6 +21,7 @@
 
 #include "common.hpp"
 #include "lt2exp_merge.hpp"
+#include "lt2exp_smallk.hpp"
 
 #include <cstdio>
 #include <mutex>
@@ -858,6 +859,14 @@ extern "C" size_t trt_lt2exp_workspace_bytes(int64_t R, int64_t S, int64_t I, in
     return need;
 }
 
+namespace trt {
+// for trt_lt2exp_bf16, which hands such calls over: would trt_lt2exp_f32 take the sweep of
+// csrc/lt2exp_smallk.hpp?
+bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned) {
+    return smallk_applies(R, S, I, J, K, w_aligned);
+}
+}  // namespace trt
+
 extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c, int64_t R, int64_t S,
                               int64_t I, int64_t J, int64_t K, const int64_t sw[3], const int64_t sa[3],
                               const int64_t sb[3], const int64_t sc[3], int mode, int variant, void *workspace,
@@ -884,9 +893,13 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
         return trt_lt2exp_f32(w, b, a, c, R, S, 1, I, K, sw, sb, sa, sc, mode, variant, workspace, workspace_bytes,
                               stream);
 
-    int v = resolve_variant(variant, R, S, I, J, K);
     // (a flat axis of w with another stride than 1 -- a sliced view -- is read element by element, in place)
     const bool w_aligned = sw[2] == 1 && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
+    // outputs of at most 8 columns: a sweep over w on the vector ALU (csrc/lt2exp_smallk.hpp); no
+    // cut, no workspace, whatever the mode asks for
+    if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned))
+        return launch_lt2exp_smallk(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, static_cast<hipStream_t>(stream));
+    int v = resolve_variant(variant, R, S, I, J, K);
     // packed rows need 16-byte loads along the flat (i, j) axis; any other call runs the same tile unpacked
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
     if (variant == 0) v = tall_variant(v, R, S, I, J, K, mode);
@@ -938,6 +951,10 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
     if (J == 1 && I > 1 && variant == 0) {  // runs with the roles of i and j exchanged
         J = I;
         I = 1;
+    }
+    if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned != 0)) {
+        const int n = snprintf(buf, buf_bytes, "trt::lt2exp_smallk_kernel<%d, %d>", small_kc(K), smallk_wpr(R, S));
+        return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
     }
     int v = resolve_variant(variant, R, S, I, J, K);
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);

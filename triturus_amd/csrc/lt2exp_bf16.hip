@@ -429,6 +429,8 @@ static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, boo
     }
 }
 
+bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned);  // csrc/lt2exp.hip
+
 }  // namespace trt
 
 using namespace trt;
@@ -511,6 +513,13 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     if (J == 1 && I > 1 && variant == 0)
         return trt_lt2exp_bf16(w, b, a, c, R, S, 1, I, K, sw, sb, sa, sc, pieces, mode, variant, workspace,
                                workspace_bytes, stream);
+
+    // Outputs of at most 8 columns are a sweep over w, which the fp32 entry runs on the vector ALU
+    // (csrc/lt2exp_smallk.hpp): the matrix pipe has nothing to gain there.
+    if (variant == 0 && K <= 8 &&
+        lt2exp_takes_sweep(R, S, I, J, K, sw[2] == 1 && sw[0] % 4 == 0 && sw[1] % 4 == 0 &&
+                                              (reinterpret_cast<uintptr_t>(w) & 15) == 0))
+        return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
 
     // Rows of w of 2 or 4 values fill an eighth or a quarter of this kernel's smallest j-chunk;
     // the fp32 kernel walks such rows packed, without padding (measured 1.4-2.5x ahead on

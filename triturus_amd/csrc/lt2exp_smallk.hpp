@@ -1,0 +1,241 @@
+// lt2exp for outputs of at most 8 columns (K <= 8: one sample, or a handful, per batch -- the
+// shape of a serving call).  Such a call is a sweep over w: every weight meets K pairs of factors,
+// 2 K flops per 4 bytes, far below what the matrix pipe needs to pay for its 32-column tiles, so
+// the MFMA kernels of lt2exp.hip, which stage w through LDS one small tile per step, are bound by
+// the latency of those steps (measured: 2-4.5 TB/s of w at K = 1..32).  Here w is streamed with
+// 16-byte loads straight into registers, four in flight per lane, and contracted on the vector
+// ALU: a lane multiplies its four consecutive weights w[s, i, j..j+3] with the factors
+// exp(b[j..j+3, k] - mb[k]) and the sum with exp(a[i, k] - ma[k]), for every k, the factors
+// coming from LDS (K x J and I x K floats, computed once per workgroup).  A wavefront owns a
+// row s (or, on grids of few rows, a quarter of one) and sums over its lanes at the end.
+// No counterpart in the reference, whose kernels tile over K like the MFMA kernels here
+// (triturus/lt2exp.py:227-357); the arithmetic contract is the same (baselines/lt2exp.py:15-25).
+#pragma once
+
+#include "common.hpp"
+
+namespace trt {
+
+struct Lt2SmallArgs {
+    const float *w, *a, *b;
+    float *c;
+    int R, S, I, J, K;
+    int64_t sw0, sw1, sa0, sa1, sa2, sb0, sb1, sb2, sc0, sc1;
+    int rows_per_wg;  // rows of S that a workgroup walks
+    int s_blocks;     // workgroups per batch
+    int once;         // w is too large to be found in a cache by a later call: read-once loads
+};
+
+// Sum over the wavefront on the data-parallel-primitive path (six register moves between lanes:
+// within quads, within rows of 16, then row to row; lanes without a source read zero); the
+// result is complete in lane 63.
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_or_zero(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, ROW_MASK, 0xf, true));
+}
+__device__ __forceinline__ float wave_sum_lane63(float v) {
+    v += dpp_or_zero<0xb1, 0xf>(v);   // quad_perm [1,0,3,2]
+    v += dpp_or_zero<0x4e, 0xf>(v);   // quad_perm [2,3,0,1]
+    v += dpp_or_zero<0x114, 0xf>(v);  // row_shr 4
+    v += dpp_or_zero<0x118, 0xf>(v);  // row_shr 8
+    v += dpp_or_zero<0x142, 0xa>(v);  // row_bcast 15 into rows 1 and 3
+    v += dpp_or_zero<0x143, 0xc>(v);  // row_bcast 31 into rows 2 and 3
+    return v;
+}
+
+constexpr int kSmallThreads = 256;
+constexpr int kSmallWaves = kSmallThreads / kWave;
+constexpr int kSmallUnroll = 4;  // 16-byte loads in flight per lane
+
+// KC: columns computed (K padded to 1, 4 or 8).  WPR: wavefronts that share a row (1 or 4).
+template <int KC, int WPR>
+static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(const Lt2SmallArgs p) {
+    static_assert(KC == 1 || KC == 4 || KC == 8, "K padded to 1, 4 or 8");
+    static_assert(WPR == 1 || WPR == kSmallWaves, "a row per wavefront, or one per workgroup");
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    float *ea = lds;                          // [I][KC]: exp(a[i, k] - ma[k])
+    float *eb = ea + ((p.I * KC + 3) & ~3);   // [KC][J]: exp(b[j, k] - mb[k]), a plane per column (16-byte aligned)
+    float *red = eb + p.J * KC;     // [kSmallThreads] scratch of the reductions
+    float *mx = red + kSmallThreads;  // [2][KC]: ma, mb
+
+    const int r = (int)(blockIdx.x / (unsigned)p.s_blocks);
+    const int sblk = (int)(blockIdx.x % (unsigned)p.s_blocks);
+    const int t = (int)threadIdx.x;
+    const int lane = t & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(t / kWave);
+    const int k = t % KC;  // the column this thread serves in the prologue (kSmallThreads % KC == 0)
+    const float *ar = p.a + (int64_t)r * p.sa0;
+    const float *br = p.b + (int64_t)r * p.sb0;
+
+    // ---- column maxima of a and b (a NaN need not survive them: exp(NaN - m) is NaN for any m and
+    // poisons the sums of its column, as in the torch recipe)
+    for (int which = 0; which < 2; ++which) {
+        const float *x = which ? br : ar;
+        const int64_t s1 = which ? p.sb1 : p.sa1, s2 = which ? p.sb2 : p.sa2;
+        const int n = which ? p.J : p.I;
+        float m = -__builtin_inff();
+        if (k < p.K)
+            for (int row = t / KC; row < n; row += kSmallThreads / KC)
+                m = __builtin_fmaxf(m, x[(int64_t)row * s1 + (int64_t)k * s2]);
+        red[t] = m;
+        __syncthreads();
+        if (t < KC) {
+            float y = -__builtin_inff();
+            for (int u = t; u < kSmallThreads; u += KC) y = __builtin_fmaxf(y, red[u]);
+            mx[which * KC + t] = clamp_shift(y);
+        }
+        __syncthreads();
+    }
+    // ---- factors (columns past K: zero, they are never stored)
+    {
+        const float mak = mx[k], mbk = mx[KC + k];
+        for (int i = t / KC; i < p.I; i += kSmallThreads / KC)
+            ea[i * KC + k] = k < p.K ? exp_shifted(ar[(int64_t)i * p.sa1 + (int64_t)k * p.sa2] - mak) : 0.f;
+        for (int j = t / KC; j < p.J; j += kSmallThreads / KC)
+            eb[k * p.J + j] = k < p.K ? exp_shifted(br[(int64_t)j * p.sb1 + (int64_t)k * p.sb2] - mbk) : 0.f;
+    }
+    __syncthreads();
+
+    // ---- the sweep.  A lane's pieces lie 64 * WPR pieces apart; (i, j) of its piece advances by a
+    // fixed step per trip (J is a multiple of 4, so the four weights of a piece share their i).
+    const int n4 = p.I * p.J / 4;                        // 16-byte pieces of a row of w
+    const int lane_piece = (WPR == 1 ? 0 : wave * kWave) + lane;
+    const int stride_f = 4 * kWave * WPR;                // floats between a lane's consecutive pieces
+    const int di = stride_f / p.J, dj = stride_f % p.J;  // wave-uniform
+    const int i_first = (4 * lane_piece) / p.J, j_first = (4 * lane_piece) % p.J;
+    const uint32_t row_bytes = (uint32_t)n4 * 16u;
+    const int rows_here = WPR == 1 ? (p.rows_per_wg - wave + kSmallWaves - 1) / kSmallWaves : p.rows_per_wg;
+
+    for (int rr = 0; rr < rows_here; ++rr) {
+        const int s = sblk * p.rows_per_wg + (WPR == 1 ? wave + rr * kSmallWaves : rr);
+        if (s >= p.S) break;  // wave-uniform
+        const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(p.w + (int64_t)r * p.sw0 + (int64_t)s * p.sw1, row_bytes);
+        float acc[KC];
+#pragma unroll
+        for (int c = 0; c < KC; ++c) acc[c] = 0.f;
+        int i = i_first, j = j_first;
+        for (int base = 0; base < n4; base += kSmallUnroll * kWave * WPR) {
+            floatx4 wv[kSmallUnroll];
+#pragma unroll
+            for (int u = 0; u < kSmallUnroll; ++u) {  // pieces past the row read as zeros
+                const uint32_t off = (uint32_t)(base + u * kWave * WPR + lane_piece) * 16u;
+                wv[u] = p.once ? __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, off, 0u, kCacheNonTemporal))
+                               : buf_load_f32x4(w_rsrc, off, 0u);
+            }
+#pragma unroll
+            for (int u = 0; u < kSmallUnroll; ++u) {
+                const int ic = i < p.I ? i : p.I - 1;  // (a piece past the row: its weights are zeros)
+                const int jc = i < p.I ? j : 0;
+                if constexpr (KC == 1) {
+                    const floatx4 e = *reinterpret_cast<const floatx4 *>(&eb[jc]);
+                    const float dot = wv[u][0] * e[0] + wv[u][1] * e[1] + wv[u][2] * e[2] + wv[u][3] * e[3];
+                    acc[0] = __builtin_fmaf(ea[ic], dot, acc[0]);
+                } else {
+                    float fa[KC];
+#pragma unroll
+                    for (int q = 0; q < KC / 4; ++q) {
+                        const floatx4 v = *reinterpret_cast<const floatx4 *>(&ea[ic * KC + 4 * q]);
+                        fa[4 * q] = v[0]; fa[4 * q + 1] = v[1]; fa[4 * q + 2] = v[2]; fa[4 * q + 3] = v[3];
+                    }
+#pragma unroll
+                    for (int c = 0; c < KC; ++c) {
+                        const floatx4 e = *reinterpret_cast<const floatx4 *>(&eb[c * p.J + jc]);
+                        const float dot = wv[u][0] * e[0] + wv[u][1] * e[1] + wv[u][2] * e[2] + wv[u][3] * e[3];
+                        acc[c] = __builtin_fmaf(fa[c], dot, acc[c]);
+                    }
+                }
+                j += dj;
+                i += di;
+                if (j >= p.J) {
+                    j -= p.J;
+                    i += 1;
+                }
+            }
+        }
+        // ---- sum over the lanes (and, with WPR = 4, over the wavefronts), shift back, log, store
+#pragma unroll
+        for (int c = 0; c < KC; ++c) acc[c] = wave_sum_lane63(acc[c]);  // complete in lane 63
+        if constexpr (WPR == 1) {
+            if (lane == kWave - 1) {
+                float *crow = p.c + (int64_t)r * p.sc0 + (int64_t)s * p.sc1;
+#pragma unroll
+                for (int c = 0; c < KC; ++c)
+                    if (c < p.K) crow[c] = log_plus(acc[c], mx[c] + mx[KC + c]);
+            }
+        } else {
+            if (lane == kWave - 1)
+#pragma unroll
+                for (int c = 0; c < KC; ++c) red[wave * KC + c] = acc[c];
+            __syncthreads();
+            if (t < p.K) {
+                float sum = red[t];
+                for (int wv2 = 1; wv2 < kSmallWaves; ++wv2) sum += red[wv2 * KC + t];
+                p.c[(int64_t)r * p.sc0 + (int64_t)s * p.sc1 + t] = log_plus(sum, mx[t] + mx[KC + t]);
+            }
+            __syncthreads();  // red is written again by the next row
+        }
+    }
+}
+
+constexpr int64_t kSmallMaxK = 8;
+constexpr size_t kSmallMaxLds = 48 * 1024;
+
+static inline int small_kc(int64_t K) { return K <= 1 ? 1 : (K <= 4 ? 4 : 8); }
+static inline size_t small_lds_bytes(int64_t I, int64_t J, int64_t K) {
+    return ((size_t)(I + J) * small_kc(K) + 4 + kSmallThreads + 2 * 8) * sizeof(float);
+}
+
+// Does the call take the sweep?  At most 8 columns; rows of w that are read 16 bytes at a time
+// (J a multiple of 4, a dense flat axis, 16-byte aligned rows); factors that fit LDS; and rows
+// enough to fill the machine with wavefronts (128 and more: from 512 on a wavefront per row,
+// below that a workgroup per row).
+static inline bool smallk_applies(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned) {
+    return K <= kSmallMaxK && J % 4 == 0 && w_aligned && R * S >= 128 && I * J >= 64 &&
+           small_lds_bytes(I, J, K) <= kSmallMaxLds;
+}
+static inline int smallk_wpr(int64_t R, int64_t S) { return R * S >= 512 ? 1 : kSmallWaves; }
+
+template <int KC>
+static int launch_smallk_kc(const Lt2SmallArgs &args, int wpr, size_t lds, unsigned grid, hipStream_t stream) {
+    if (wpr == 1)
+        hipLaunchKernelGGL((lt2exp_smallk_kernel<KC, 1>), dim3(grid), dim3(kSmallThreads), lds, stream, args);
+    else
+        hipLaunchKernelGGL((lt2exp_smallk_kernel<KC, kSmallWaves>), dim3(grid), dim3(kSmallThreads), lds, stream, args);
+    return (int)hipGetLastError();
+}
+
+static int launch_lt2exp_smallk(const float *w, const float *a, const float *b, float *c, int64_t R, int64_t S,
+                                int64_t I, int64_t J, int64_t K, const int64_t sw[3], const int64_t sa[3],
+                                const int64_t sb[3], const int64_t sc[3], hipStream_t stream) {
+    Lt2SmallArgs args;
+    args.w = w; args.a = a; args.b = b; args.c = c;
+    args.R = (int)R; args.S = (int)S; args.I = (int)I; args.J = (int)J; args.K = (int)K;
+    args.sw0 = sw[0]; args.sw1 = sw[1];
+    args.sa0 = sa[0]; args.sa1 = sa[1]; args.sa2 = sa[2];
+    args.sb0 = sb[0]; args.sb1 = sb[1]; args.sb2 = sb[2];
+    args.sc0 = sc[0]; args.sc1 = sc[1];
+    const int wpr = smallk_wpr(R, S);
+    // a wavefront per row: workgroups of 4..64 rows, some 2048 of them where the rows allow
+    int64_t rows = 1;
+    if (wpr == 1) {
+        rows = ceil_div(ceil_div(R * S, 2048), kSmallWaves) * kSmallWaves;
+        if (rows < kSmallWaves) rows = kSmallWaves;
+        if (rows > 64) rows = 64;
+    }
+    // (only a w that the 256 MB memory-side cache cannot hold: the weights of a serving call are the
+    // same from call to call, and up to there ordinary loads find part of them again -- 268 MB:
+    // 46 us against 50 with read-once loads; 537 MB: 103 against 94)
+    args.once = (double)R * (double)S * (double)I * (double)J * 4.0 >= 384.0 * 1048576.0 ? 1 : 0;
+    args.rows_per_wg = (int)rows;
+    args.s_blocks = (int)ceil_div(S, rows);
+    const int64_t grid = R * args.s_blocks;
+    if (grid >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+    const size_t lds = small_lds_bytes(I, J, K);
+    switch (small_kc(K)) {
+        case 1: return launch_smallk_kc<1>(args, wpr, lds, (unsigned)grid, stream);
+        case 4: return launch_smallk_kc<4>(args, wpr, lds, (unsigned)grid, stream);
+        default: return launch_smallk_kc<8>(args, wpr, lds, (unsigned)grid, stream);
+    }
+}
+
+}  // namespace trt

@@ -98,6 +98,19 @@ def _exchange_pays(R: int, S: int, I: int, J: int, K: int) -> bool:
     return saved * kernel_s >= 1.2 * copy_s
 
 
+def _sweeps(R: int, S: int, I: int, J: int, K: int, w: torch.Tensor) -> bool:
+    """Outputs of at most 8 columns whose w the library streams once on the vector ALU
+    (csrc/lt2exp_smallk.hpp, same conditions as smallk_applies there): no front end below can
+    make such a call cheaper, a copy of w costs more than the call."""
+    if K > 8 or J % 4 != 0 or R * S < 128 or I * J < 64:
+        return False
+    kc = 1 if K <= 1 else 4 if K <= 4 else 8
+    if ((I + J) * kc + 4 + 256 + 16) * 4 > 48 * 1024:
+        return False
+    sw = w.stride()
+    return sw[2] == 1 and sw[0] % 4 == 0 and sw[1] % 4 == 0 and w.data_ptr() % 16 == 0
+
+
 def _packs(I: int, J: int) -> bool:
     """Rows of w short enough for the fp32 kernel to walk (i, j) as one flat axis (no padding of j)."""
     return J in (2, 4, 8) and (I * J) % 4 == 0 and I * J >= 32
@@ -145,6 +158,8 @@ def lt2exp(
     elif _precision not in MATRIX_PRECISIONS:
         raise ValueError(f"unknown matrix precision {_precision!r}")
     fp32 = _precision == "fp32"
+    if K <= 8 and _variant == 0 and _swap is None and _pad is None and _sweeps(R, S, I, J, K, w):
+        _swap = _pad = False
     # (the shape tests come first: most calls meet none of them and pay for no rule)
     if _variant == 0 and 2 <= J < I and not (fp32 and _packs(I, J)):
         if _swap is not None:
