@@ -563,10 +563,11 @@ def test_bf16_paths_c5_full_size(dev, precision):
 
 
 SWEEP_SHAPES = [
-    (64, 64, 64, 64, 1), (64, 64, 64, 64, 8), (16, 100, 33, 28, 3), (8, 64, 16, 4, 5),     # a wavefront per row
-    (200, 3, 5, 24, 2), (130, 1, 64, 64, 7), (3, 333, 12, 20, 4), (1, 700, 100, 8, 6),
-    (4, 64, 64, 64, 4), (2, 70, 17, 12, 1), (1, 128, 3, 300, 8), (16, 8, 40, 40, 2),      # a workgroup per row
-    (64, 64, 1, 64, 2), (64, 64, 64, 1, 2), (5, 130, 1024, 4, 3), (2, 300, 2, 1024, 8),   # J = 1 exchanged; long axes
+    (64, 64, 64, 64, 1), (64, 64, 64, 64, 8), (16, 100, 37, 28, 3), (8, 64, 64, 32, 5),     # a wavefront per row
+    (200, 3, 50, 24, 2), (130, 1, 64, 64, 7), (3, 333, 60, 20, 4), (1, 700, 300, 8, 6),
+    (4, 64, 64, 64, 4), (2, 70, 90, 12, 1), (1, 128, 7, 300, 8), (16, 8, 40, 40, 2),        # a workgroup per row
+    (64, 64, 1, 1024, 2), (64, 64, 1024, 1, 2), (5, 130, 1024, 4, 3), (2, 300, 2, 1024, 8),  # J = 1 exchanged; long axes
+    (1, 3, 64, 64, 2), (1, 1, 300, 300, 8), (8, 64, 16, 16, 5), (37, 17, 8, 16, 1), (300, 700, 4, 32, 3),  # few rows; short rows
 ]
 
 
@@ -604,7 +605,7 @@ def test_outputs_of_at_most_8_columns_take_the_sweep(dev, shape):
 
 
 def test_the_sweep_reads_strided_a_and_b_and_sliced_w_in_place(dev):
-    R, S, I, J, K = 12, 50, 24, 16, 5
+    R, S, I, J, K = 12, 50, 24, 96, 5
     g = torch.Generator().manual_seed(5)
     wide = torch.rand(R, S + 3, I, J, generator=g).to(dev)
     w = wide[:, 2:S + 2]                                           # rows stay 16-byte aligned

@@ -102,7 +102,7 @@ def _sweeps(R: int, S: int, I: int, J: int, K: int, w: torch.Tensor) -> bool:
     """Outputs of at most 8 columns whose w the library streams once on the vector ALU
     (csrc/lt2exp_smallk.hpp, same conditions as smallk_applies there): no front end below can
     make such a call cheaper, a copy of w costs more than the call."""
-    if K > 8 or J % 4 != 0 or R * S < 128 or I * J < 64:
+    if K > 8 or J % 4 != 0 or I * J < (256 if K > 4 else 128):
         return False
     kc = 1 if K <= 1 else 4 if K <= 4 else 8
     if ((I + J) * kc + 4 + 256 + 16) * 4 > 48 * 1024:
