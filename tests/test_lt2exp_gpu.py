@@ -568,6 +568,8 @@ SWEEP_SHAPES = [
     (4, 64, 64, 64, 4), (2, 70, 90, 12, 1), (1, 128, 7, 300, 8), (16, 8, 40, 40, 2),        # a workgroup per row
     (64, 64, 1, 1024, 2), (64, 64, 1024, 1, 2), (5, 130, 1024, 4, 3), (2, 300, 2, 1024, 8),  # J = 1 exchanged; long axes
     (1, 3, 64, 64, 2), (1, 1, 300, 300, 8), (8, 64, 16, 16, 5), (37, 17, 8, 16, 1), (300, 700, 4, 32, 3),  # few rows; short rows
+    (64, 64, 64, 6, 3), (8, 300, 104, 10, 8), (3, 50, 4, 73, 1), (16, 128, 20, 13, 4), (2, 7, 100, 5, 2),  # J not a multiple of 4
+    (5, 40, 160, 7, 6), (1, 600, 12, 301, 7), (33, 33, 2, 250, 1),
 ]
 
 

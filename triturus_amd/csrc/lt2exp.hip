@@ -953,7 +953,8 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
         I = 1;
     }
     if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned != 0)) {
-        const int n = snprintf(buf, buf_bytes, "trt::lt2exp_smallk_kernel<%d, %d>", small_kc(K), smallk_wpr(R, S));
+        const int n = snprintf(buf, buf_bytes, "trt::lt2exp_smallk_kernel<%d, %d, %s>", small_kc(K), smallk_wpr(R, S),
+                               J % 4 == 0 ? "false" : "true");
         return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
     }
     int v = resolve_variant(variant, R, S, I, J, K);

@@ -48,14 +48,21 @@ constexpr int kSmallWaves = kSmallThreads / kWave;
 constexpr int kSmallUnroll = 4;  // 16-byte loads in flight per lane
 
 // KC: columns computed (K padded to 1, 4 or 8).  WPR: wavefronts that share a row (1 or 4).
-template <int KC, int WPR>
+// ANYJ: J is not a multiple of 4 (but I * J is, so rows of w are still whole 16-byte pieces): the
+// four weights of a piece may lie in two rows i, i + 1 of the (i, j) plane, so every weight looks
+// its factor of b up by itself and the piece is summed in two parts, one per row of a.
+template <int KC, int WPR, bool ANYJ>
 static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(const Lt2SmallArgs p) {
     static_assert(KC == 1 || KC == 4 || KC == 8, "K padded to 1, 4 or 8");
     static_assert(WPR == 1 || WPR == kSmallWaves, "a row per wavefront, or one per workgroup");
     extern __shared__ __attribute__((aligned(16))) float lds[];
+    // ANYJ reads the factors of b one by one, consecutive lanes four values of j apart: the plane is
+    // stored "transposed by 4" -- j at (j % 4) * Q + j / 4 -- so that those reads fall into consecutive
+    // LDS banks instead of every fourth one
+    const int Q = (p.J + 3) / 4;              // pitch of a plane: 4 Q >= J floats
     float *ea = lds;                          // [I][KC]: exp(a[i, k] - ma[k])
-    float *eb = ea + ((p.I * KC + 3) & ~3);   // [KC][J]: exp(b[j, k] - mb[k]), a plane per column (16-byte aligned)
-    float *red = eb + p.J * KC;     // [kSmallThreads] scratch of the reductions
+    float *eb = ea + ((p.I * KC + 3) & ~3);   // [KC][4 Q]: exp(b[j, k] - mb[k]), a plane per column (16-byte aligned)
+    float *red = eb + 4 * Q * KC;   // [kSmallThreads] scratch of the reductions
     float *mx = red + kSmallThreads;  // [2][KC]: ma, mb
 
     const int r = (int)(blockIdx.x / (unsigned)p.s_blocks);
@@ -92,12 +99,14 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
         for (int i = t / KC; i < p.I; i += kSmallThreads / KC)
             ea[i * KC + k] = k < p.K ? exp_shifted(ar[(int64_t)i * p.sa1 + (int64_t)k * p.sa2] - mak) : 0.f;
         for (int j = t / KC; j < p.J; j += kSmallThreads / KC)
-            eb[k * p.J + j] = k < p.K ? exp_shifted(br[(int64_t)j * p.sb1 + (int64_t)k * p.sb2] - mbk) : 0.f;
+            eb[k * 4 * Q + (ANYJ ? (j & 3) * Q + (j >> 2) : j)] =
+                k < p.K ? exp_shifted(br[(int64_t)j * p.sb1 + (int64_t)k * p.sb2] - mbk) : 0.f;
     }
     __syncthreads();
 
-    // ---- the sweep.  A lane's pieces lie 64 * WPR pieces apart; (i, j) of its piece advances by a
-    // fixed step per trip (J is a multiple of 4, so the four weights of a piece share their i).
+    // ---- the sweep.  A lane's pieces lie 64 * WPR pieces apart; (i, j) of a piece's first weight
+    // advances by a fixed step per trip (with J a multiple of 4 the four weights of a piece share
+    // their i).
     const int n4 = p.I * p.J / 4;                        // 16-byte pieces of a row of w
     const int lane_piece = (WPR == 1 ? 0 : wave * kWave) + lane;
     const int stride_f = 4 * kWave * WPR;                // floats between a lane's consecutive pieces
@@ -126,7 +135,47 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
             for (int u = 0; u < kSmallUnroll; ++u) {
                 const int ic = i < p.I ? i : p.I - 1;  // (a piece past the row: its weights are zeros)
                 const int jc = i < p.I ? j : 0;
-                if constexpr (KC == 1) {
+                if constexpr (ANYJ) {
+                    // weights 0..m-1 of the piece belong to row i, the others to row i + 1 (J >= 4: at
+                    // most one row boundary inside a piece)
+                    const int m = p.J - jc;
+                    const int ih = ic + 1 < p.I ? ic + 1 : p.I - 1;
+                    int at[4];  // where the factor of b of each weight sits in a plane
+                    float wl[4], wh[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const bool low = e < m;
+                        const int jt = low ? jc + e : e - m;
+                        at[e] = (jt & 3) * Q + (jt >> 2);
+                        wl[e] = low ? wv[u][e] : 0.f;
+                        wh[e] = low ? 0.f : wv[u][e];
+                    }
+                    float fl[KC], fh[KC];
+                    if constexpr (KC == 1) {
+                        fl[0] = ea[ic];
+                        fh[0] = ea[ih];
+                    } else {
+#pragma unroll
+                        for (int q = 0; q < KC / 4; ++q) {
+                            const floatx4 v = *reinterpret_cast<const floatx4 *>(&ea[ic * KC + 4 * q]);
+                            const floatx4 h2 = *reinterpret_cast<const floatx4 *>(&ea[ih * KC + 4 * q]);
+#pragma unroll
+                            for (int x = 0; x < 4; ++x) {
+                                fl[4 * q + x] = v[x];
+                                fh[4 * q + x] = h2[x];
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int c = 0; c < KC; ++c) {
+                        const float *plane = eb + c * 4 * Q;
+                        const float e0 = plane[at[0]], e1 = plane[at[1]], e2 = plane[at[2]], e3 = plane[at[3]];
+                        const float lo = wl[0] * e0 + wl[1] * e1 + wl[2] * e2 + wl[3] * e3;
+                        const float hi = wh[0] * e0 + wh[1] * e1 + wh[2] * e2 + wh[3] * e3;
+                        acc[c] = __builtin_fmaf(fl[c], lo, acc[c]);
+                        acc[c] = __builtin_fmaf(fh[c], hi, acc[c]);
+                    }
+                } else if constexpr (KC == 1) {
                     const floatx4 e = *reinterpret_cast<const floatx4 *>(&eb[jc]);
                     const float dot = wv[u][0] * e[0] + wv[u][1] * e[1] + wv[u][2] * e[2] + wv[u][3] * e[3];
                     acc[0] = __builtin_fmaf(ea[ic], dot, acc[0]);
@@ -139,7 +188,7 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
                     }
 #pragma unroll
                     for (int c = 0; c < KC; ++c) {
-                        const floatx4 e = *reinterpret_cast<const floatx4 *>(&eb[c * p.J + jc]);
+                        const floatx4 e = *reinterpret_cast<const floatx4 *>(&eb[c * 4 * Q + jc]);
                         const float dot = wv[u][0] * e[0] + wv[u][1] * e[1] + wv[u][2] * e[2] + wv[u][3] * e[3];
                         acc[c] = __builtin_fmaf(fa[c], dot, acc[c]);
                     }
@@ -182,11 +231,12 @@ constexpr size_t kSmallMaxLds = 48 * 1024;
 
 static inline int small_kc(int64_t K) { return K <= 1 ? 1 : (K <= 4 ? 4 : 8); }
 static inline size_t small_lds_bytes(int64_t I, int64_t J, int64_t K) {
-    return ((size_t)(I + J) * small_kc(K) + 4 + kSmallThreads + 2 * 8) * sizeof(float);
+    return ((size_t)(I + (J + 3) / 4 * 4) * small_kc(K) + 4 + kSmallThreads + 2 * 8) * sizeof(float);
 }
 
 // Does the call take the sweep?  At most 8 columns; rows of w that are read 16 bytes at a time
-// (J a multiple of 4, a dense flat axis, 16-byte aligned rows); factors that fit LDS; rows of at
+// (I * J a multiple of 4 -- J itself, or any J > 4 under a fitting I --, a dense flat axis, 16-byte
+// aligned rows); factors that fit LDS; rows of at
 // least 128 weights (256 with more than 4 columns), below which the sum over the lanes at the
 // end of a row costs more than the row.  Timed against the matrix-pipe kernels on 300 random
 // shapes (K = 1..8, R = 1..256, S = 1..1024, I = 1..300, J = 4..320): the sweep is 1.5-2.8x
@@ -196,17 +246,22 @@ static inline size_t small_lds_bytes(int64_t I, int64_t J, int64_t K) {
 static inline bool smallk_applies(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned) {
     (void)R;
     (void)S;
-    return K <= kSmallMaxK && J % 4 == 0 && w_aligned && I * J >= (K > 4 ? 256 : 128) &&
-           small_lds_bytes(I, J, K) <= kSmallMaxLds;
+    if (K > kSmallMaxK || !w_aligned || small_lds_bytes(I, J, K) > kSmallMaxLds) return false;
+    if (J % 4 == 0) return I * J >= (K > 4 ? 256 : 128);
+    // (a J that is not a multiple of 4 costs every weight a look-up of its own: level with the
+    // matrix-pipe kernels on shorter rows, 0.3x at worst with 8 columns; over 120 random shapes
+    // the sweep is 1.6x ahead in the median beyond these bounds)
+    return J > 4 && (I * J) % 4 == 0 && I * J >= (K > 4 ? 1024 : 256);
 }
 static inline int smallk_wpr(int64_t R, int64_t S) { return R * S >= 512 ? 1 : kSmallWaves; }
 
-template <int KC>
+template <int KC, bool ANYJ>
 static int launch_smallk_kc(const Lt2SmallArgs &args, int wpr, size_t lds, unsigned grid, hipStream_t stream) {
     if (wpr == 1)
-        hipLaunchKernelGGL((lt2exp_smallk_kernel<KC, 1>), dim3(grid), dim3(kSmallThreads), lds, stream, args);
+        hipLaunchKernelGGL((lt2exp_smallk_kernel<KC, 1, ANYJ>), dim3(grid), dim3(kSmallThreads), lds, stream, args);
     else
-        hipLaunchKernelGGL((lt2exp_smallk_kernel<KC, kSmallWaves>), dim3(grid), dim3(kSmallThreads), lds, stream, args);
+        hipLaunchKernelGGL((lt2exp_smallk_kernel<KC, kSmallWaves, ANYJ>), dim3(grid), dim3(kSmallThreads), lds, stream,
+                           args);
     return (int)hipGetLastError();
 }
 
@@ -237,10 +292,17 @@ static int launch_lt2exp_smallk(const float *w, const float *a, const float *b, 
     const int64_t grid = R * args.s_blocks;
     if (grid >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const size_t lds = small_lds_bytes(I, J, K);
+    if (J % 4 == 0) {
+        switch (small_kc(K)) {
+            case 1: return launch_smallk_kc<1, false>(args, wpr, lds, (unsigned)grid, stream);
+            case 4: return launch_smallk_kc<4, false>(args, wpr, lds, (unsigned)grid, stream);
+            default: return launch_smallk_kc<8, false>(args, wpr, lds, (unsigned)grid, stream);
+        }
+    }
     switch (small_kc(K)) {
-        case 1: return launch_smallk_kc<1>(args, wpr, lds, (unsigned)grid, stream);
-        case 4: return launch_smallk_kc<4>(args, wpr, lds, (unsigned)grid, stream);
-        default: return launch_smallk_kc<8>(args, wpr, lds, (unsigned)grid, stream);
+        case 1: return launch_smallk_kc<1, true>(args, wpr, lds, (unsigned)grid, stream);
+        case 4: return launch_smallk_kc<4, true>(args, wpr, lds, (unsigned)grid, stream);
+        default: return launch_smallk_kc<8, true>(args, wpr, lds, (unsigned)grid, stream);
     }
 }
 
