@@ -501,6 +501,35 @@ def main() -> int:
         log(f"lm2exp smallest configuration: {eager_us:.2f} us per eager call through the Python wrapper, "
             f"{result['c1']['hip_graph_us_per_call']:.2f} us inside a HIP graph")
 
+        # ------------------------------------------------ lt2exp with few columns (HBM bound)
+        # The large configuration's weights under 1, 4 and 8 columns -- one sample per batch, or a
+        # handful: a serving call.  The contraction is then a sweep over w (67.1 MB), timed like
+        # the reductions below: 8 copies of w in turn (from HBM) and the same w again and again.
+        from benchmarks.torch_recipes import torch_lt2exp  # the eager torch recipe, on the GPU
+
+        wl = cfg["w"].to(dev)
+        wcopies = [wl] + [wl.clone() for _ in range(7)]
+        wbytes = wl.numel() * 4
+        sv = {"workload": "lt2exp R=64 S=I=J=64, K = 1, 4, 8 (a,b ~ N(-30,10))", "bytes": wbytes, "unit": "GB/s",
+              "peak": PEAK_HBM_GBPS, "protocol": "us / achieved / frac: 8 copies of w in turn (every call streams "
+                                                 "from HBM); same_operand: one w again and again"}
+        for kk in (1, 4, 8):
+            ak, bk = cfg["a"][:, :, :kk].contiguous().to(dev), cfg["b"][:, :, :kk].contiguous().to(dev)
+            fnk = lambda z: lt2exp(z, ak, bk, _precision="fp32")
+            hot = graph_time(lambda: fnk(wl), prewarm_ms=PREWARM_MS)
+            cold = graph_time(fnk, calls=24, prewarm_ms=PREWARM_MS / 2, operands=wcopies)
+            tor = graph_time(lambda: torch_lt2exp(wl, ak, bk))
+            sv[f"k{kk}"] = {"kernel": _lib.kernel_name("lt2exp", 64, 64, 64, 64, kk, _lib.MODE_AUTO, 0, 1),
+                            "us": round(cold * 1e6, 2), "achieved": round(wbytes / cold / 1e9, 1),
+                            "frac": round(wbytes / cold / 1e9 / PEAK_HBM_GBPS, 4),
+                            "same_operand": {"us": round(hot * 1e6, 2), "achieved": round(wbytes / hot / 1e9, 1)},
+                            "torch_recipe_same_operand_us": round(tor * 1e6, 2)}
+            log(f"lt2exp K={kk}: {cold * 1e6:.2f} us from HBM ({wbytes / cold / 1e9:.0f} GB/s = "
+                f"{wbytes / cold / 1e9 / PEAK_HBM_GBPS * 100:.1f}% of 8 TB/s), {hot * 1e6:.2f} us on the same w, "
+                f"torch recipe {tor * 1e6:.2f} us")
+        result["few_columns"] = sv
+        del wl, wcopies
+
         # ------------------------------------------------ max reductions (HBM bound)
         # Two figures per reduction.  `us`, `achieved`, `frac`: 8 copies of the 64 MiB operand
         # (512 MiB) taken in turn, so that every call streams from HBM -- the figure to hold

@@ -74,6 +74,39 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
     const float *ar = p.a + (int64_t)r * p.sa0;
     const float *br = p.b + (int64_t)r * p.sb0;
 
+    // ---- the sweep's geometry.  A lane's pieces lie 64 * WPR pieces apart; (i, j) of a piece's
+    // first weight advances by a fixed step per trip (with J a multiple of 4 the four weights of a
+    // piece share their i).  A trip is kSmallUnroll pieces per lane; the loads of the next trip --
+    // of the next row, at the end of a row -- are asked for before the current one is contracted,
+    // and those of the very first trip before the factors are computed, so that the prologue runs
+    // under their latency.
+    const int n4 = p.I * p.J / 4;                        // 16-byte pieces of a row of w
+    const int lane_piece = (WPR == 1 ? 0 : wave * kWave) + lane;
+    const int stride_f = 4 * kWave * WPR;                // floats between a lane's consecutive pieces
+    const int di = stride_f / p.J, dj = stride_f % p.J;  // wave-uniform
+    const int i_first = (4 * lane_piece) / p.J, j_first = (4 * lane_piece) % p.J;
+    const uint32_t row_bytes = (uint32_t)n4 * 16u;
+    constexpr int kTrip = kSmallUnroll * kWave * WPR;    // pieces of a row that a trip covers
+    const int trips_per_row = (n4 + kTrip - 1) / kTrip;
+    const int s_first = sblk * p.rows_per_wg + (WPR == 1 ? wave : 0);
+    constexpr int kRowStep = WPR == 1 ? kSmallWaves : 1;
+    const int rows_here = WPR == 1 ? (p.rows_per_wg - wave + kSmallWaves - 1) / kSmallWaves : p.rows_per_wg;
+    const int rows_left = s_first < p.S ? (p.S - s_first + kRowStep - 1) / kRowStep : 0;
+    const int rows_valid = rows_here < rows_left ? rows_here : rows_left;  // wave-uniform
+    const float *w_batch = p.w + (int64_t)r * p.sw0;
+    floatx4 nxt[kSmallUnroll];
+    auto issue = [&](int s, int trip) {  // pieces past the row read as zeros
+        const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(w_batch + (int64_t)s * p.sw1, row_bytes);
+#pragma unroll
+        for (int u = 0; u < kSmallUnroll; ++u) {
+            const uint32_t off = (uint32_t)(trip * kTrip + u * kWave * WPR + lane_piece) * 16u;
+            nxt[u] = p.once ? __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, off, 0u,
+                                                                                                kCacheNonTemporal))
+                            : buf_load_f32x4(w_rsrc, off, 0u);
+        }
+    };
+    if (rows_valid > 0) issue(s_first, 0);
+
     // ---- column maxima of a and b (a NaN need not survive them: exp(NaN - m) is NaN for any m and
     // poisons the sums of its column, as in the torch recipe)
     for (int which = 0; which < 2; ++which) {
@@ -104,32 +137,26 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
     }
     __syncthreads();
 
-    // ---- the sweep.  A lane's pieces lie 64 * WPR pieces apart; (i, j) of a piece's first weight
-    // advances by a fixed step per trip (with J a multiple of 4 the four weights of a piece share
-    // their i).
-    const int n4 = p.I * p.J / 4;                        // 16-byte pieces of a row of w
-    const int lane_piece = (WPR == 1 ? 0 : wave * kWave) + lane;
-    const int stride_f = 4 * kWave * WPR;                // floats between a lane's consecutive pieces
-    const int di = stride_f / p.J, dj = stride_f % p.J;  // wave-uniform
-    const int i_first = (4 * lane_piece) / p.J, j_first = (4 * lane_piece) % p.J;
-    const uint32_t row_bytes = (uint32_t)n4 * 16u;
-    const int rows_here = WPR == 1 ? (p.rows_per_wg - wave + kSmallWaves - 1) / kSmallWaves : p.rows_per_wg;
-
-    for (int rr = 0; rr < rows_here; ++rr) {
-        const int s = sblk * p.rows_per_wg + (WPR == 1 ? wave + rr * kSmallWaves : rr);
-        if (s >= p.S) break;  // wave-uniform
-        const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(p.w + (int64_t)r * p.sw0 + (int64_t)s * p.sw1, row_bytes);
+    // ---- the sweep
+    for (int rr = 0; rr < rows_valid; ++rr) {
+        const int s = s_first + rr * kRowStep;
         float acc[KC];
 #pragma unroll
         for (int c = 0; c < KC; ++c) acc[c] = 0.f;
         int i = i_first, j = j_first;
-        for (int base = 0; base < n4; base += kSmallUnroll * kWave * WPR) {
+        for (int trip = 0; trip < trips_per_row; ++trip) {
             floatx4 wv[kSmallUnroll];
+            if constexpr (KC < 8) {
 #pragma unroll
-            for (int u = 0; u < kSmallUnroll; ++u) {  // pieces past the row read as zeros
-                const uint32_t off = (uint32_t)(base + u * kWave * WPR + lane_piece) * 16u;
-                wv[u] = p.once ? __builtin_bit_cast(floatx4, __builtin_amdgcn_raw_buffer_load_b128(w_rsrc, off, 0u, kCacheNonTemporal))
-                               : buf_load_f32x4(w_rsrc, off, 0u);
+                for (int u = 0; u < kSmallUnroll; ++u) wv[u] = nxt[u];
+                if (trip + 1 < trips_per_row) issue(s, trip + 1);
+                else if (rr + 1 < rows_valid) issue(s + kRowStep, 0);
+            } else {
+                // (8 columns: the second set of load registers costs a wavefront per SIMD and the LDS
+                // reads of the factors, not the loads, bound the trip: measured 5-15 % slower with it)
+                if (rr + trip > 0) issue(s, trip);
+#pragma unroll
+                for (int u = 0; u < kSmallUnroll; ++u) wv[u] = nxt[u];
             }
 #pragma unroll
             for (int u = 0; u < kSmallUnroll; ++u) {
