@@ -75,7 +75,9 @@ const char *trt_error_string(int status);
  * by shape (small grids with a long contraction), 1 = never, n = n ways.  The
  * reference has no such mode for lm2exp.  When it splits, the call needs a
  * workspace of trt_lm2exp_workspace_bytes(R, I, J, K, variant, splits) bytes
- * (0 when it does not split: pass NULL, 0).
+ * (0 when it does not split: pass NULL, 0).  With variant 0, splits <= 1, at most 4 columns,
+ * J >= 1024 a multiple of 4 and 16-byte aligned rows of a, a is streamed once on the vector ALU
+ * (the few-column kernel of trt_lt2exp_f32) and no workspace is used.
  */
 int trt_lm2exp_f32(const float *a, const float *b, float *c,
                    int64_t R, int64_t I, int64_t J, int64_t K,

@@ -648,3 +648,37 @@ def test_bf16_paths_c3_full_size(dev, precision):
     assert torch.all(out <= bg.amax(1, keepdim=True) + 1e-3)
     shifted = lm2exp(ag, bg + 128.0, _precision=precision)
     assert torch.allclose(shifted, out + 128.0, rtol=1e-5, atol=1e-3)
+
+
+@pytest.mark.parametrize("shape", [(16, 512, 1024, 1), (3, 70, 2048, 4), (64, 64, 4096, 1), (1, 5, 1500, 3),
+                                   (2, 1000, 1028, 2)])
+def test_at_most_4_columns_under_a_long_contraction_take_the_sweep(dev, shape):
+    """K <= 4 and J >= 1024 with 16-byte aligned rows of a: the vector-ALU sweep of
+    csrc/lt2exp_smallk.hpp with the rows of a as the weights, against the float64 oracle (zero
+    rows, -inf and NaN columns) and against the matrix-pipe tile on the same operands."""
+    R, I, J, K = shape
+    assert "smallk_kernel" in _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1)
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(R, I, J, generator=g)
+    a[:, I // 2] = 0.0
+    b = 6 * torch.randn(R, J, K, generator=g) - 20
+    b[0, :, 0] = NINF
+    b[R - 1, J // 3, K - 1] = NINF
+    out = lm2exp(a.to(dev), b.to(dev))
+    r = oracle64.compare(out, oracle64.lm2exp64(a, b))
+    assert r["ok"], (shape, r)
+    assert torch.isneginf(out[0, :, 0]).all() and torch.isneginf(out[:, I // 2]).all()
+    assert torch.equal(out, lm2exp(a.to(dev), b.to(dev)))
+    assert torch.allclose(out, lm2exp(a.to(dev), b.to(dev), _variant=12), rtol=1e-5, atol=1e-5)
+    for prec in ("bf16x3", "bf16x6"):  # narrow outputs go to the fp32 entry, and so to the same sweep
+        assert torch.equal(out, lm2exp(a.to(dev), b.to(dev), _precision=prec))
+    bn = b.clone()
+    bn[R // 2, 7, K // 2] = float("nan")
+    outn = lm2exp(a.to(dev), bn.to(dev))
+    assert torch.isnan(outn[R // 2, :, K // 2]).all()
+    mask = torch.ones_like(outn, dtype=torch.bool)
+    mask[R // 2, :, K // 2] = False
+    assert torch.equal(outn[mask], out[mask])
+    # a transposed a is not swept (its rows are not dense): same result from the paired tiles
+    at = a.transpose(1, 2).contiguous().transpose(1, 2).to(dev)
+    assert torch.allclose(out, lm2exp(at, b.to(dev)), rtol=1e-5, atol=1e-5)

@@ -910,6 +910,12 @@ static size_t plan_workspace(const Lm2Plan &pl, int64_t R, int64_t I, int64_t K)
     return ((size_t)pl.splits * R * I * K + (size_t)pl.splits * R * K) * sizeof(float);
 }
 
+// csrc/lt2exp.hip: the sweep of csrc/lt2exp_smallk.hpp with the rows of a as the weights
+bool lm2exp_takes_sweep(int64_t R, int64_t I, int64_t J, int64_t K, bool a_aligned);
+int lm2exp_sweep(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
+                 const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], hipStream_t stream);
+int lt2exp_sweep_name(int64_t R, int64_t S, int64_t J, int64_t K, char *buf, size_t buf_bytes);
+
 }  // namespace trt
 
 using namespace trt;
@@ -938,6 +944,11 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
     if (J * sb[1] + K * sb[2] >= lim || I * sa[1] + J * sa[2] >= lim || I * sc[1] + K >= lim || I * K >= lim)
         return TRT_E_RANGE;
 
+    // at most 4 columns under a long contraction: a sweep over a on the vector ALU
+    if (variant == 0 && splits <= 1 &&
+        lm2exp_takes_sweep(R, I, J, K, sa[2] == 1 && sa[0] % 4 == 0 && sa[1] % 4 == 0 &&
+                                           (reinterpret_cast<uintptr_t>(a) & 15) == 0))
+        return lm2exp_sweep(a, b, c, R, I, J, K, sa, sb, sc, static_cast<hipStream_t>(stream));
     Lm2Plan pl = make_plan(R, I, J, K, variant, splits);
     // a trailing stride of a other than 1 (a transposed or strided view): only the
     // paired-wavefront kernel reads such a tile; a call that would take another kernel takes
@@ -1031,6 +1042,8 @@ extern "C" int trt_lm2exp_kernel_name(int64_t R, int64_t I, int64_t J, int64_t K
                                       char *buf, size_t buf_bytes) {
     if (!buf || buf_bytes == 0 || R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (variant < 0 || variant > kNumVariants || splits < 0) return TRT_E_INVALID;
+    if (variant == 0 && splits <= 1 && lm2exp_takes_sweep(R, I, J, K, a_vec != 0))
+        return lt2exp_sweep_name(R, I, J, K, buf, buf_bytes);
     const Lm2Variant &vr = kVariants[make_plan(R, I, J, K, variant, splits).variant];
     int n;
     if (vr.mode == kPair)

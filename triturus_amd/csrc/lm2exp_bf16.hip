@@ -376,6 +376,8 @@ struct LmBfVariant {
 static const LmBfVariant kLmBfVariants[] = {{4, 4}, {4, 2}, {2, 4}, {2, 2}, {1, 4}, {1, 2}, {8, 1}, {8, 2}, {3, 2}};
 constexpr int kNumLmBfVariants = sizeof(kLmBfVariants) / sizeof(kLmBfVariants[0]);
 
+bool lm2exp_takes_sweep(int64_t R, int64_t I, int64_t J, int64_t K, bool a_aligned);  // csrc/lt2exp.hip
+
 }  // namespace trt
 
 using namespace trt;
@@ -481,7 +483,10 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
                                 trt_lm2exp_workspace_bytes(R, I, J, K, 0, 0) == 0;
         // outputs of at most 32 columns: the fp32 path has a tile with its wavefronts stacked over rows
         const bool narrow = K <= 32 && I > 64;
-        if (narrow || (cut == 1 && !one_launch && (splits > 1 || small || J <= (pieces == 2 ? 16 : 32))))
+        // at most 4 columns under a long contraction: the fp32 entry sweeps a on the vector ALU
+        const bool swept = splits <= 1 && lm2exp_takes_sweep(R, I, J, K, sa[2] == 1 && sa[0] % 4 == 0 && sa[1] % 4 == 0 &&
+                                                                            (reinterpret_cast<uintptr_t>(a) & 15) == 0);
+        if (narrow || swept || (cut == 1 && !one_launch && (splits > 1 || small || J <= (pieces == 2 ? 16 : 32))))
             return trt_lm2exp_f32(a, b, c, R, I, J, K, sa, sb, sc, 0, splits, workspace, workspace_bytes, stream);
         int best_rt = 1;
         int64_t best_cost = ceil_div(I, 32) * 120;

@@ -865,6 +865,25 @@ namespace trt {
 bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned) {
     return smallk_applies(R, S, I, J, K, w_aligned);
 }
+// for trt_lm2exp_f32: c[r, i, k] = log sum_j a[r, i, j] exp(b[r, j, k]) is the same sweep with the
+// rows of a as the weights, a contracted plane of 1 x J and no factors on the other side.  Is
+// that the faster way?  Only with at most 4 columns and rows of 1024 values and more: lm2exp's
+// own tiles stream a at 3.5-4.7 TB/s, and a row ends in a sum over the lanes (timed: R=16, I=4096,
+// J=1024: K=1 60 -> 45 us, K=4 58 -> 53, K=8 57 -> 82; R=64, I=64, J=4096, K=1: 37 -> 21;
+// rows of 64..256 values: 0.2-0.8x).
+bool lm2exp_takes_sweep(int64_t R, int64_t I, int64_t J, int64_t K, bool a_aligned) {
+    return K <= 4 && J >= 1024 && smallk_applies(R, I, 1, J, K, a_aligned);
+}
+int lm2exp_sweep(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
+                 const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], hipStream_t stream) {
+    const int64_t none[3] = {0, 0, 0};
+    return launch_lt2exp_smallk(a, nullptr, b, c, R, I, 1, J, K, sa, none, sb, sc, stream);
+}
+int lt2exp_sweep_name(int64_t R, int64_t S, int64_t J, int64_t K, char *buf, size_t buf_bytes) {
+    const int n = snprintf(buf, buf_bytes, "trt::lt2exp_smallk_kernel<%d, %d, %s>", small_kc(K), smallk_wpr(R, S),
+                           J % 4 == 0 ? "false" : "true");
+    return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
+}
 }  // namespace trt
 
 extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c, int64_t R, int64_t S,
@@ -952,11 +971,7 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
         J = I;
         I = 1;
     }
-    if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned != 0)) {
-        const int n = snprintf(buf, buf_bytes, "trt::lt2exp_smallk_kernel<%d, %d, %s>", small_kc(K), smallk_wpr(R, S),
-                               J % 4 == 0 ? "false" : "true");
-        return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
-    }
+    if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned != 0)) return lt2exp_sweep_name(R, S, J, K, buf, buf_bytes);
     int v = resolve_variant(variant, R, S, I, J, K);
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
     if (variant == 0) v = tall_variant(v, R, S, I, J, K, mode);

@@ -71,7 +71,7 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
     const int lane = t & (kWave - 1);
     const int wave = __builtin_amdgcn_readfirstlane(t / kWave);
     const int k = t % KC;  // the column this thread serves in the prologue (kSmallThreads % KC == 0)
-    const float *ar = p.a + (int64_t)r * p.sa0;
+    const float *ar = p.a ? p.a + (int64_t)r * p.sa0 : nullptr;
     const float *br = p.b + (int64_t)r * p.sb0;
 
     // ---- the sweep's geometry.  A lane's pieces lie 64 * WPR pieces apart; (i, j) of a piece's
@@ -110,6 +110,10 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
     // ---- column maxima of a and b (a NaN need not survive them: exp(NaN - m) is NaN for any m and
     // poisons the sums of its column, as in the torch recipe)
     for (int which = 0; which < 2; ++which) {
+        if (which == 0 && !p.a) {  // no factors of a (the lm2exp entry: I = 1, a factor of one)
+            if (t < KC) mx[t] = 0.f;
+            continue;  // (block-uniform)
+        }
         const float *x = which ? br : ar;
         const int64_t s1 = which ? p.sb1 : p.sa1, s2 = which ? p.sb2 : p.sa2;
         const int n = which ? p.J : p.I;
@@ -130,7 +134,7 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
     {
         const float mak = mx[k], mbk = mx[KC + k];
         for (int i = t / KC; i < p.I; i += kSmallThreads / KC)
-            ea[i * KC + k] = k < p.K ? exp_shifted(ar[(int64_t)i * p.sa1 + (int64_t)k * p.sa2] - mak) : 0.f;
+            ea[i * KC + k] = k >= p.K ? 0.f : !p.a ? 1.f : exp_shifted(ar[(int64_t)i * p.sa1 + (int64_t)k * p.sa2] - mak);
         for (int j = t / KC; j < p.J; j += kSmallThreads / KC)
             eb[k * 4 * Q + (ANYJ ? (j & 3) * Q + (j >> 2) : j)] =
                 k < p.K ? exp_shifted(br[(int64_t)j * p.sb1 + (int64_t)k * p.sb2] - mbk) : 0.f;
