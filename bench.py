@@ -238,6 +238,10 @@ def profile_pass(dev) -> int:
         for _ in range(3):
             lt2exp(w, a, b, _precision=prec)
     torch.cuda.synchronize()
+    a1, b1 = a[:, :, :1].contiguous(), b[:, :, :1].contiguous()  # one column: the sweep over w
+    for _ in range(3):
+        lt2exp(w, a1, b1, _precision="fp32")
+    torch.cuda.synchronize()
     flat = b.view(-1)
     for _ in range(3):
         vmax(flat)
@@ -262,7 +266,7 @@ def profile_pass(dev) -> int:
         lm2exp(a2, b2, _precision="fp32")
         lt2exp(w4, a4, b4, _precision="fp32")
     torch.cuda.synchronize()
-    log("profile pass done: 3 x (copy 256 MiB, lt2exp large [fp32, bf16x3, bf16x6], vmax, matmax x2, "
+    log("profile pass done: 3 x (copy 256 MiB, lt2exp large [fp32, bf16x3, bf16x6, one column], vmax, matmax x2, "
         "lm2exp rectangular [fp32, bf16x3, bf16x6], lm2exp R=16 512^3, lt2exp R=16 S=64 I=J=32 K=2048)")
     return 0
 
