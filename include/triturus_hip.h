@@ -111,10 +111,10 @@ int trt_lm2exp_variant_count(void);
  * and j-chunk (tests, tuning).  With J = 1 and variant 0 the call runs with the
  * roles of (i, a) and (j, b) exchanged; with J = 2, 4 or 8, I*J a multiple of 4
  * and 16-byte aligned rows of w (base, sw[0], sw[1]) the kernel walks (i, j) as
- * one flat axis, so short rows cost no padding.  With at most 8 columns (K <= 8), I*J a
- * multiple of 4, rows of w 16-byte aligned and of at least 128 weights (more for K > 4 or a J
- * that is not a multiple of 4), variant 0 streams w once on the vector ALU instead (no cut, no
- * workspace used, whatever the mode).
+ * one flat axis, so short rows cost no padding.  With at most 8 columns (K <= 8), a dense flat
+ * axis of w (sw[2] == 1) and rows of at least 128 weights (256 for K > 4; 256 / 1024 unless J is a
+ * multiple of 4 and the rows are 16-byte aligned, and then J > 4), variant 0 streams w once on
+ * the vector ALU instead (no cut, no workspace used, whatever the mode).
  */
 int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c,
                    int64_t R, int64_t S, int64_t I, int64_t J, int64_t K,

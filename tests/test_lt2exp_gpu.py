@@ -570,6 +570,7 @@ SWEEP_SHAPES = [
     (1, 3, 64, 64, 2), (1, 1, 300, 300, 8), (8, 64, 16, 16, 5), (37, 17, 8, 16, 1), (300, 700, 4, 32, 3),  # few rows; short rows
     (64, 64, 64, 6, 3), (8, 300, 104, 10, 8), (3, 50, 4, 73, 1), (16, 128, 20, 13, 4), (2, 7, 100, 5, 2),  # J not a multiple of 4
     (5, 40, 160, 7, 6), (1, 600, 12, 301, 7), (33, 33, 2, 250, 1),
+    (228, 3, 74, 147, 3), (16, 50, 15, 73, 5), (7, 33, 9, 31, 2), (2, 5, 1, 1001, 4), (3, 9, 7, 37, 1),  # rows not 16-byte aligned
 ]
 
 
@@ -579,7 +580,7 @@ def test_outputs_of_at_most_8_columns_take_the_sweep(dev, shape):
     (csrc/lt2exp_smallk.hpp) against the float64 oracle, -inf and NaN columns included, and
     against the matrix-pipe kernel on the same operands."""
     R, S, I, J, K = shape
-    assert "smallk_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1)
+    assert "smallk_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, int((I * J) % 4 == 0))
     g = torch.Generator().manual_seed(sum(shape))
     w = torch.rand(R, S, I, J, generator=g)
     w[:, S // 2] = 0.0
@@ -604,6 +605,27 @@ def test_outputs_of_at_most_8_columns_take_the_sweep(dev, shape):
     mask = torch.ones_like(outn, dtype=torch.bool)
     mask[R // 2, :, K // 2] = False
     assert torch.equal(outn[mask], out[mask])
+
+
+@pytest.mark.parametrize("offset", [1, 2, 3])
+@pytest.mark.parametrize("shape", [(6, 40, 16, 32, 3), (2, 9, 99, 12, 8), (1, 1, 40, 40, 1)])
+def test_the_sweep_on_a_w_that_starts_off_a_16_byte_boundary(dev, shape, offset):
+    """A dense w whose first element sits 4, 8 or 12 bytes past a 16-byte boundary (a view into a
+    larger buffer): rows are read from the boundary below them, the floats before a row's start and
+    after its end weighing nothing.  The buffer around w is NaN, so a stray weight would show."""
+    R, S, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape) + offset)
+    n = R * S * I * J
+    buf = torch.full((n + 8,), float("nan"))
+    buf[offset:offset + n] = torch.rand(n, generator=g)
+    w = buf.to(dev)[offset:offset + n].view(R, S, I, J)
+    assert w.data_ptr() % 16 == 4 * offset
+    a = (3 * torch.randn(R, I, K, generator=g)).to(dev)
+    b = (3 * torch.randn(R, J, K, generator=g)).to(dev)
+    assert "smallk_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 0)
+    out = lt2exp(w, a, b)
+    r = oracle64.compare(out, oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=4))
+    assert r["ok"], (shape, offset, r)
 
 
 def test_the_sweep_reads_strided_a_and_b_and_sliced_w_in_place(dev):

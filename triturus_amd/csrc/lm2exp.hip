@@ -914,7 +914,7 @@ static size_t plan_workspace(const Lm2Plan &pl, int64_t R, int64_t I, int64_t K)
 bool lm2exp_takes_sweep(int64_t R, int64_t I, int64_t J, int64_t K, bool a_aligned);
 int lm2exp_sweep(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
                  const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], hipStream_t stream);
-int lt2exp_sweep_name(int64_t R, int64_t S, int64_t J, int64_t K, char *buf, size_t buf_bytes);
+int lt2exp_sweep_name(int64_t R, int64_t S, int64_t J, int64_t K, bool w_aligned, char *buf, size_t buf_bytes);
 
 }  // namespace trt
 
@@ -1043,7 +1043,7 @@ extern "C" int trt_lm2exp_kernel_name(int64_t R, int64_t I, int64_t J, int64_t K
     if (!buf || buf_bytes == 0 || R <= 0 || I <= 0 || J <= 0 || K <= 0) return TRT_E_INVALID;
     if (variant < 0 || variant > kNumVariants || splits < 0) return TRT_E_INVALID;
     if (variant == 0 && splits <= 1 && lm2exp_takes_sweep(R, I, J, K, a_vec != 0))
-        return lt2exp_sweep_name(R, I, J, K, buf, buf_bytes);
+        return lt2exp_sweep_name(R, I, J, K, true, buf, buf_bytes);
     const Lm2Variant &vr = kVariants[make_plan(R, I, J, K, variant, splits).variant];
     int n;
     if (vr.mode == kPair)

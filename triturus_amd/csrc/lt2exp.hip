@@ -862,8 +862,8 @@ extern "C" size_t trt_lt2exp_workspace_bytes(int64_t R, int64_t S, int64_t I, in
 namespace trt {
 // for trt_lt2exp_bf16, which hands such calls over: would trt_lt2exp_f32 take the sweep of
 // csrc/lt2exp_smallk.hpp?
-bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned) {
-    return smallk_applies(R, S, I, J, K, w_aligned);
+bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense) {
+    return smallk_applies(R, S, I, J, K, w_aligned, w_dense);
 }
 // for trt_lm2exp_f32: c[r, i, k] = log sum_j a[r, i, j] exp(b[r, j, k]) is the same sweep with the
 // rows of a as the weights, a contracted plane of 1 x J and no factors on the other side.  Is
@@ -872,16 +872,16 @@ bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, b
 // J=1024: K=1 60 -> 45 us, K=4 58 -> 53, K=8 57 -> 82; R=64, I=64, J=4096, K=1: 37 -> 21;
 // rows of 64..256 values: 0.2-0.8x).
 bool lm2exp_takes_sweep(int64_t R, int64_t I, int64_t J, int64_t K, bool a_aligned) {
-    return K <= 4 && J >= 1024 && smallk_applies(R, I, 1, J, K, a_aligned);
+    return K <= 4 && J >= 1024 && J % 4 == 0 && a_aligned && smallk_applies(R, I, 1, J, K, a_aligned);
 }
 int lm2exp_sweep(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
                  const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], hipStream_t stream) {
     const int64_t none[3] = {0, 0, 0};
-    return launch_lt2exp_smallk(a, nullptr, b, c, R, I, 1, J, K, sa, none, sb, sc, stream);
+    return launch_lt2exp_smallk(a, nullptr, b, c, R, I, 1, J, K, sa, none, sb, sc, true, stream);
 }
-int lt2exp_sweep_name(int64_t R, int64_t S, int64_t J, int64_t K, char *buf, size_t buf_bytes) {
+int lt2exp_sweep_name(int64_t R, int64_t S, int64_t J, int64_t K, bool w_aligned, char *buf, size_t buf_bytes) {
     const int n = snprintf(buf, buf_bytes, "trt::lt2exp_smallk_kernel<%d, %d, %s>", small_kc(K), smallk_wpr(R, S),
-                           J % 4 == 0 ? "false" : "true");
+                           smallk_anyj(J, w_aligned) ? "true" : "false");
     return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
 }
 }  // namespace trt
@@ -916,8 +916,8 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     const bool w_aligned = sw[2] == 1 && (sw[0] % 4 == 0) && (sw[1] % 4 == 0) && ((reinterpret_cast<uintptr_t>(w) & 15) == 0);
     // outputs of at most 8 columns: a sweep over w on the vector ALU (csrc/lt2exp_smallk.hpp); no
     // cut, no workspace, whatever the mode asks for
-    if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned))
-        return launch_lt2exp_smallk(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, static_cast<hipStream_t>(stream));
+    if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned, sw[2] == 1))
+        return launch_lt2exp_smallk(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, w_aligned, static_cast<hipStream_t>(stream));
     int v = resolve_variant(variant, R, S, I, J, K);
     // packed rows need 16-byte loads along the flat (i, j) axis; any other call runs the same tile unpacked
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
@@ -971,7 +971,8 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
         J = I;
         I = 1;
     }
-    if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned != 0)) return lt2exp_sweep_name(R, S, J, K, buf, buf_bytes);
+    // (w_aligned = 0: rows that are not 16-byte aligned, of a dense flat axis)
+    if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned != 0)) return lt2exp_sweep_name(R, S, J, K, w_aligned != 0, buf, buf_bytes);
     int v = resolve_variant(variant, R, S, I, J, K);
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
     if (variant == 0) v = tall_variant(v, R, S, I, J, K, mode);

@@ -429,7 +429,7 @@ static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, boo
     }
 }
 
-bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned);  // csrc/lt2exp.hip
+bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense);  // csrc/lt2exp.hip
 
 }  // namespace trt
 
@@ -518,7 +518,7 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     // (csrc/lt2exp_smallk.hpp): the matrix pipe has nothing to gain there.
     if (variant == 0 && K <= 8 &&
         lt2exp_takes_sweep(R, S, I, J, K, sw[2] == 1 && sw[0] % 4 == 0 && sw[1] % 4 == 0 &&
-                                              (reinterpret_cast<uintptr_t>(w) & 15) == 0))
+                                              (reinterpret_cast<uintptr_t>(w) & 15) == 0, sw[2] == 1))
         return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
 
     // Rows of w of 2 or 4 values fill an eighth or a quarter of this kernel's smallest j-chunk;

@@ -80,23 +80,32 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
     // of the next row, at the end of a row -- are asked for before the current one is contracted,
     // and those of the very first trip before the factors are computed, so that the prologue runs
     // under their latency.
-    const int n4 = p.I * p.J / 4;                        // 16-byte pieces of a row of w
+    const int n4 = (p.I * p.J + 3) / 4;                  // 16-byte pieces of a row of w
     const int lane_piece = (WPR == 1 ? 0 : wave * kWave) + lane;
     const int stride_f = 4 * kWave * WPR;                // floats between a lane's consecutive pieces
     const int di = stride_f / p.J, dj = stride_f % p.J;  // wave-uniform
     const int i_first = (4 * lane_piece) / p.J, j_first = (4 * lane_piece) % p.J;
-    const uint32_t row_bytes = (uint32_t)n4 * 16u;
+    // ANYJ also takes rows of w that do not start on a 16-byte boundary: a row is then read from the
+    // boundary below it, `mis` floats early -- those floats, the end of the row before, are given
+    // weight zero -- and (i, j) of a lane's first piece steps back by as many.
     constexpr int kTrip = kSmallUnroll * kWave * WPR;    // pieces of a row that a trip covers
-    const int trips_per_row = (n4 + kTrip - 1) / kTrip;
+    const int trips_per_row = ((ANYJ ? n4 + 1 : n4) + kTrip - 1) / kTrip;
     const int s_first = sblk * p.rows_per_wg + (WPR == 1 ? wave : 0);
     constexpr int kRowStep = WPR == 1 ? kSmallWaves : 1;
     const int rows_here = WPR == 1 ? (p.rows_per_wg - wave + kSmallWaves - 1) / kSmallWaves : p.rows_per_wg;
     const int rows_left = s_first < p.S ? (p.S - s_first + kRowStep - 1) / kRowStep : 0;
     const int rows_valid = rows_here < rows_left ? rows_here : rows_left;  // wave-uniform
     const float *w_batch = p.w + (int64_t)r * p.sw0;
+    auto row_mis = [&](int s) -> int {  // floats between the 16-byte boundary below the row and its start
+        if constexpr (!ANYJ) return 0;
+        return (int)((reinterpret_cast<uintptr_t>(w_batch + (int64_t)s * p.sw1) >> 2) & 3);
+    };
     floatx4 nxt[kSmallUnroll];
     auto issue = [&](int s, int trip) {  // pieces past the row read as zeros
-        const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(w_batch + (int64_t)s * p.sw1, row_bytes);
+        const int mis = row_mis(s);
+        // (whole pieces: what the last one holds beyond the row is given weight zero below)
+        const __amdgpu_buffer_rsrc_t w_rsrc =
+            make_rsrc(w_batch + (int64_t)s * p.sw1 - mis, (uint32_t)((p.I * p.J + mis + 3) / 4) * 16u);
 #pragma unroll
         for (int u = 0; u < kSmallUnroll; ++u) {
             const uint32_t off = (uint32_t)(trip * kTrip + u * kWave * WPR + lane_piece) * 16u;
@@ -148,6 +157,13 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
 #pragma unroll
         for (int c = 0; c < KC; ++c) acc[c] = 0.f;
         int i = i_first, j = j_first;
+        if constexpr (ANYJ) {
+            j -= row_mis(s);
+            if (j < 0) {
+                j += p.J;
+                i -= 1;
+            }
+        }
         for (int trip = 0; trip < trips_per_row; ++trip) {
             floatx4 wv[kSmallUnroll];
             if constexpr (KC < 8) {
@@ -164,13 +180,15 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
             }
 #pragma unroll
             for (int u = 0; u < kSmallUnroll; ++u) {
-                const int ic = i < p.I ? i : p.I - 1;  // (a piece past the row: its weights are zeros)
+                // (a piece past the row: its weights are zeros; i = -1: the floats before the row's start)
+                const int ic = i < p.I ? (i < 0 ? 0 : i) : p.I - 1;
                 const int jc = i < p.I ? j : 0;
                 if constexpr (ANYJ) {
                     // weights 0..m-1 of the piece belong to row i, the others to row i + 1 (J >= 4: at
                     // most one row boundary inside a piece)
                     const int m = p.J - jc;
-                    const int ih = ic + 1 < p.I ? ic + 1 : p.I - 1;
+                    const int ih = i + 1 < p.I ? i + 1 : p.I - 1;
+                    const bool before = i < 0, past_lo = i >= p.I, past_hi = i + 1 >= p.I;
                     int at[4];  // where the factor of b of each weight sits in a plane
                     float wl[4], wh[4];
 #pragma unroll
@@ -178,8 +196,8 @@ static __global__ __launch_bounds__(kSmallThreads) void lt2exp_smallk_kernel(con
                         const bool low = e < m;
                         const int jt = low ? jc + e : e - m;
                         at[e] = (jt & 3) * Q + (jt >> 2);
-                        wl[e] = low ? wv[u][e] : 0.f;
-                        wh[e] = low ? 0.f : wv[u][e];
+                        wl[e] = low && !before && !past_lo ? wv[u][e] : 0.f;
+                        wh[e] = low || past_hi ? 0.f : wv[u][e];
                     }
                     float fl[KC], fh[KC];
                     if constexpr (KC == 1) {
@@ -265,25 +283,26 @@ static inline size_t small_lds_bytes(int64_t I, int64_t J, int64_t K) {
     return ((size_t)(I + (J + 3) / 4 * 4) * small_kc(K) + 4 + kSmallThreads + 2 * 8) * sizeof(float);
 }
 
-// Does the call take the sweep?  At most 8 columns; rows of w that are read 16 bytes at a time
-// (I * J a multiple of 4 -- J itself, or any J > 4 under a fitting I --, a dense flat axis, 16-byte
-// aligned rows); factors that fit LDS; rows of at
+// Does the call take the sweep?  At most 8 columns; a dense flat axis of w (J a multiple of 4 on
+// 16-byte aligned rows: the plain build; any other J > 4 and any row alignment: ANYJ); factors that fit LDS; rows of at
 // least 128 weights (256 with more than 4 columns), below which the sum over the lanes at the
 // end of a row costs more than the row.  Timed against the matrix-pipe kernels on 300 random
 // shapes (K = 1..8, R = 1..256, S = 1..1024, I = 1..300, J = 4..320): the sweep is 1.5-2.8x
 // ahead in the median of every class of row length from 256 weights on (up to 11x), whatever
 // the number of rows, and these thresholds leave the choice 0.4 % (mean) behind the faster of
 // the two (never sweeping: 104 %).
-static inline bool smallk_applies(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned) {
+static inline bool smallk_applies(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned,
+                                  bool w_dense = true) {
     (void)R;
     (void)S;
-    if (K > kSmallMaxK || !w_aligned || small_lds_bytes(I, J, K) > kSmallMaxLds) return false;
-    if (J % 4 == 0) return I * J >= (K > 4 ? 256 : 128);
-    // (a J that is not a multiple of 4 costs every weight a look-up of its own: level with the
-    // matrix-pipe kernels on shorter rows, 0.3x at worst with 8 columns; over 120 random shapes
-    // the sweep is 1.6x ahead in the median beyond these bounds)
-    return J > 4 && (I * J) % 4 == 0 && I * J >= (K > 4 ? 1024 : 256);
+    if (K > kSmallMaxK || small_lds_bytes(I, J, K) > kSmallMaxLds) return false;
+    if (J % 4 == 0 && w_aligned) return I * J >= (K > 4 ? 256 : 128);
+    // (any other J > 4, or rows that do not start on 16-byte boundaries, cost every weight a look-up
+    // of its own: level with the matrix-pipe kernels on shorter rows, 0.3x at worst with 8
+    // columns; over 120 random shapes the sweep is 1.6x ahead in the median beyond these bounds)
+    return w_dense && J > 4 && I * J >= (K > 4 ? 1024 : 256);
 }
+static inline bool smallk_anyj(int64_t J, bool w_aligned) { return !(J % 4 == 0 && w_aligned); }
 static inline int smallk_wpr(int64_t R, int64_t S) { return R * S >= 512 ? 1 : kSmallWaves; }
 
 template <int KC, bool ANYJ>
@@ -298,7 +317,7 @@ static int launch_smallk_kc(const Lt2SmallArgs &args, int wpr, size_t lds, unsig
 
 static int launch_lt2exp_smallk(const float *w, const float *a, const float *b, float *c, int64_t R, int64_t S,
                                 int64_t I, int64_t J, int64_t K, const int64_t sw[3], const int64_t sa[3],
-                                const int64_t sb[3], const int64_t sc[3], hipStream_t stream) {
+                                const int64_t sb[3], const int64_t sc[3], bool w_aligned, hipStream_t stream) {
     Lt2SmallArgs args;
     args.w = w; args.a = a; args.b = b; args.c = c;
     args.R = (int)R; args.S = (int)S; args.I = (int)I; args.J = (int)J; args.K = (int)K;
@@ -323,7 +342,7 @@ static int launch_lt2exp_smallk(const float *w, const float *a, const float *b, 
     const int64_t grid = R * args.s_blocks;
     if (grid >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const size_t lds = small_lds_bytes(I, J, K);
-    if (J % 4 == 0) {
+    if (!smallk_anyj(J, w_aligned)) {
         switch (small_kc(K)) {
             case 1: return launch_smallk_kc<1, false>(args, wpr, lds, (unsigned)grid, stream);
             case 4: return launch_smallk_kc<4, false>(args, wpr, lds, (unsigned)grid, stream);

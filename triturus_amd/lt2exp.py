@@ -104,16 +104,13 @@ def _sweeps(R: int, S: int, I: int, J: int, K: int, w: torch.Tensor) -> bool:
     make such a call cheaper, a copy of w costs more than the call."""
     if K > 8:
         return False
-    if J % 4 == 0:
-        if I * J < (256 if K > 4 else 128):
-            return False
-    elif not (J > 4 and (I * J) % 4 == 0 and I * J >= (1024 if K > 4 else 256)):
-        return False
     kc = 1 if K <= 1 else 4 if K <= 4 else 8
     if ((I + (J + 3) // 4 * 4) * kc + 4 + 256 + 16) * 4 > 48 * 1024:
         return False
     sw = w.stride()
-    return sw[2] == 1 and sw[0] % 4 == 0 and sw[1] % 4 == 0 and w.data_ptr() % 16 == 0
+    if J % 4 == 0 and sw[2] == 1 and sw[0] % 4 == 0 and sw[1] % 4 == 0 and w.data_ptr() % 16 == 0:
+        return I * J >= (256 if K > 4 else 128)
+    return sw[2] == 1 and J > 4 and I * J >= (1024 if K > 4 else 256)
 
 
 def _packs(I: int, J: int) -> bool:
