@@ -91,6 +91,29 @@ def test_lt2exp_random(dev, seed, precision):
     assert r["ok"], (R, S, I, J, K, mode, variant, r)
 
 
+@pytest.mark.parametrize("seed", range(60))
+def test_lt2exp_random_with_few_columns(dev, seed):
+    """K = 1..9 on random shapes, a w that starts 0..12 bytes past a 16-byte boundary inside a
+    buffer of NaNs, strided a and b: the sweep over w on the vector ALU wherever the library
+    takes it (and the matrix pipe elsewhere), against the float64 oracle."""
+    rng = random.Random(3000 + seed)
+    g = torch.Generator().manual_seed(seed)
+    R, S, I, J, K = rng.randrange(1, 5), _dim(rng, 130), _dim(rng, 129), _dim(rng, 200), rng.randrange(1, 10)
+    off = rng.choice([0, 0, 1, 2, 3])
+    n = R * S * I * J
+    buf = torch.full((n + 8,), float("nan"))
+    buf[off : off + n] = torch.rand(n, generator=g) * rng.choice([1.0, 1e-4, 30.0])
+    w = buf.to(dev)[off : off + n].view(R, S, I, J)
+    if rng.random() < 0.3:
+        w[:, rng.randrange(S)] = 0.0
+    a = _sprinkle(rng, g, torch.randn(R, I, K, generator=g) * rng.choice([1.0, 10.0]) + rng.choice([0.0, -40.0]))
+    b = _sprinkle(rng, g, torch.randn(R, J, K, generator=g) * rng.choice([1.0, 10.0]) + rng.choice([0.0, 70.0]))
+    ref = oracle64.lt2exp64(w.cpu(), a, b)
+    out = lt2exp(w, _view(rng, a.to(dev)), _view(rng, b.to(dev)), mode=rng.choice(["auto", "split", "unsplit"]))
+    r = oracle64.compare(out, ref)
+    assert r["ok"], (R, S, I, J, K, off, r)
+
+
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
 def test_results_are_bit_reproducible(dev, precision):
     """Fixed summation order everywhere (no atomics, merges in split order): the same call on
