@@ -640,3 +640,82 @@ def test_the_sweep_reads_strided_a_and_b_and_sliced_w_in_place(dev):
     r = oracle64.compare(out, oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=4))
     assert r["ok"], r
     assert torch.equal(out, lt2exp(w.contiguous(), a.contiguous(), b.contiguous()))
+
+
+ROWS_FIRST_SHAPES = [
+    (2048, 1, 64, 64, 64), (130, 1, 64, 64, 12), (9, 1, 32, 8, 9), (1, 1, 31, 44, 17),       # one s per batch
+    (7, 1, 300, 300, 20), (3, 2, 245, 256, 40), (16, 4, 500, 512, 20),                          # long axes: more LDS than 64 KB
+    (5, 3, 33, 20, 70), (2, 2, 40, 12, 33), (6, 12, 29, 60, 45), (3, 9, 250, 28, 33),          # I not a multiple of 32; J = 4 (mod 8)
+    (11, 2, 7, 200, 10), (1, 5, 33, 68, 65),
+    (4, 7, 50, 36, 100), (2, 2, 64, 64, 300), (2, 5, 96, 100, 130), (2, 3, 128, 36, 257),      # several column tiles
+    (1, 16, 256, 64, 100), (3, 40, 64, 64, 12), (2, 20, 64, 128, 24),                          # s in several workgroups
+]
+
+
+@pytest.mark.parametrize("shape", ROWS_FIRST_SHAPES)
+def test_few_s_per_batch_contract_j_first(dev, shape):
+    """Few s per batch: the kernel with the rows (s, i) of w on the rows of the MFMA
+    (csrc/lt2exp_rows.hpp) against the float64 oracle, -inf and NaN columns included, and against
+    the s-row tiles on the same operands.  An infinite weight in the first row of every s but the
+    first must not leak into the s before it (rows past I of a tile are the next s's)."""
+    R, S, I, J, K = shape
+    assert "rows_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1)
+    g = torch.Generator().manual_seed(sum(shape))
+    w = torch.rand(R, S, I, J, generator=g)
+    a = 5 * torch.randn(R, I, K, generator=g) - 10
+    b = 5 * torch.randn(R, J, K, generator=g) + 3
+    a[0, :, 0] = NINF                       # a whole column of a: -inf out
+    b[R - 1, J // 2, K - 1] = NINF          # a single -inf entry: finite out
+    ref = oracle64.lt2exp64(w, a, b, batch_chunk=8)
+    out = lt2exp(w.to(dev), a.to(dev), b.to(dev))
+    r = oracle64.compare(out, ref)
+    assert r["ok"], (shape, r)
+    assert torch.isneginf(out[0, :, 0]).all()
+    assert torch.equal(out, lt2exp(w.to(dev), a.to(dev), b.to(dev)))      # the sums are added in a fixed order
+    tiles = lt2exp(w.to(dev), a.to(dev), b.to(dev), _variant=4)
+    assert torch.allclose(out, tiles, rtol=1e-4, atol=1e-5)
+    if S > 1:
+        wi = w.clone()
+        wi[:, 1:, 0, :] = float("inf")
+        outi = lt2exp(wi.to(dev), a.to(dev), b.to(dev))
+        assert torch.equal(outi[:, 0], out[:, 0])
+        ok = torch.isposinf(outi[:, 1:]) | ~torch.isfinite(out[:, 1:])
+        ok[R - 1, :, K - 1] = True             # (inf times the factor 0 of the -inf entry of b: NaN, as in the recipe)
+        assert ok.all()
+    an = a.clone()
+    an[R // 2, I // 2, K // 2] = float("nan")
+    outn = lt2exp(w.to(dev), an.to(dev), b.to(dev))
+    assert torch.isnan(outn[R // 2, :, K // 2]).all()
+    mask = torch.ones_like(outn, dtype=torch.bool)
+    mask[R // 2, :, K // 2] = False
+    assert torch.equal(outn[mask], out[mask])
+
+
+def test_j_first_reads_strided_a_and_b_and_sliced_w_in_place(dev):
+    R, S, I, J, K = 12, 3, 50, 96, 45
+    g = torch.Generator().manual_seed(6)
+    wide = torch.rand(R, S + 3, I, J, generator=g).to(dev)
+    w = wide[:, 2:S + 2]                                           # rows stay 16-byte aligned
+    a = (3 * torch.randn(R, K, I, generator=g)).to(dev).transpose(1, 2)   # K-major
+    b = (3 * torch.randn(R, J, 2 * K, generator=g)).to(dev)[:, :, ::2]    # every other column
+    assert "rows_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1)
+    out = lt2exp(w, a, b)
+    r = oracle64.compare(out, oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=4))
+    assert r["ok"], r
+    assert torch.equal(out, lt2exp(w.contiguous(), a.contiguous(), b.contiguous()))
+
+
+def test_few_s_per_batch_under_a_long_i_keep_w_as_it_lies(dev):
+    """2 <= J < I would run on a transposed copy of w under the s-row tiles; j-first takes w as it is."""
+    R, S, I, J, K = 40, 2, 300, 16, 40
+    assert "rows_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1)
+    g = torch.Generator().manual_seed(9)
+    w = torch.rand(R, S, I, J, generator=g).to(dev)
+    a = (3 * torch.randn(R, I, K, generator=g)).to(dev)
+    b = (3 * torch.randn(R, J, K, generator=g)).to(dev)
+    out = lt2exp(w, a, b)
+    assert torch.equal(out, lt2exp(w, a, b, _swap=False, _pad=False))
+    r = oracle64.compare(out, oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=4))
+    assert r["ok"], r
+    for prec in ("bf16x3", "bf16x6"):        # handed over to the same kernel
+        assert torch.equal(out, lt2exp(w, a, b, _precision=prec, _swap=False))

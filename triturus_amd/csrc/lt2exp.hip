@@ -21,6 +21,7 @@
 
 #include "common.hpp"
 #include "lt2exp_merge.hpp"
+#include "lt2exp_rows.hpp"
 #include "lt2exp_smallk.hpp"
 
 #include <cstdio>
@@ -865,6 +866,11 @@ namespace trt {
 bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense) {
     return smallk_applies(R, S, I, J, K, w_aligned, w_dense);
 }
+// likewise: would it take the kernel of csrc/lt2exp_rows.hpp (few s per batch)?
+// (margin: by how many doublings the fp32 rule's estimate must favour it)
+bool lt2exp_takes_rows(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, double margin) {
+    return rows_score(R, S, I, J, K) > margin && rows_plan(R, S, I, J, K, w_aligned).ct != 0;
+}
 // for trt_lm2exp_f32: c[r, i, k] = log sum_j a[r, i, j] exp(b[r, j, k]) is the same sweep with the
 // rows of a as the weights, a contracted plane of 1 x J and no factors on the other side.  Is
 // that the faster way?  Only with at most 4 columns and rows of 1024 values and more: lm2exp's
@@ -918,6 +924,12 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     // cut, no workspace, whatever the mode asks for
     if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned, sw[2] == 1))
         return launch_lt2exp_smallk(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, w_aligned, static_cast<hipStream_t>(stream));
+    // few s per batch: the rows (s, i) of w on the rows of the MFMA, j contracted first
+    // (csrc/lt2exp_rows.hpp); no cut and no workspace either
+    if (variant == 0 && rows_pays(R, S, I, J, K)) {
+        const RowsPlan rp = rows_plan(R, S, I, J, K, w_aligned);
+        if (rp.ct) return launch_lt2exp_rows(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, rp, static_cast<hipStream_t>(stream));
+    }
     int v = resolve_variant(variant, R, S, I, J, K);
     // packed rows need 16-byte loads along the flat (i, j) axis; any other call runs the same tile unpacked
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
@@ -973,6 +985,13 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
     }
     // (w_aligned = 0: rows that are not 16-byte aligned, of a dense flat axis)
     if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned != 0)) return lt2exp_sweep_name(R, S, J, K, w_aligned != 0, buf, buf_bytes);
+    if (variant == 0 && rows_pays(R, S, I, J, K)) {
+        const RowsPlan rp = rows_plan(R, S, I, J, K, w_aligned != 0);
+        if (rp.ct) {
+            const int n = snprintf(buf, buf_bytes, "trt::lt2exp_rows_kernel<%d>", rp.ct);
+            return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
+        }
+    }
     int v = resolve_variant(variant, R, S, I, J, K);
     if (kVariants[v].pack && !(packs(I, J) && w_aligned)) v = find_lt2_variant(kVariants[v].rt, 2, false);
     if (variant == 0) v = tall_variant(v, R, S, I, J, K, mode);

@@ -430,6 +430,7 @@ static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, boo
 }
 
 bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense);  // csrc/lt2exp.hip
+bool lt2exp_takes_rows(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, double margin);  // csrc/lt2exp.hip
 
 }  // namespace trt
 
@@ -519,6 +520,18 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     if (variant == 0 && K <= 8 &&
         lt2exp_takes_sweep(R, S, I, J, K, sw[2] == 1 && sw[0] % 4 == 0 && sw[1] % 4 == 0 &&
                                               (reinterpret_cast<uintptr_t>(w) & 15) == 0, sw[2] == 1))
+        return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
+
+    // Few s per batch: these tiles, like the fp32 ones, put s on the rows of the MFMA and pad it to
+    // 32; the fp32 kernel of csrc/lt2exp_rows.hpp puts the rows (s, i) of w there.  Where the fp32
+    // rule favours it by a factor of two (1.6 against three pieces) it beats these tiles as well
+    // (80 timed shapes with S = 1..40: 1.0-7.5x against two pieces in 36 of 41 such calls, 0.6-0.9x
+    // in five; 1.0-12x against three pieces in 38 of 44, 0.7-0.98x in six; over all 80, handing over
+    // by this rule leaves 3-4 % to the better choice per shape, never handing over 37 and 56 %)
+    // -- and it is the more exact of the two.
+    if (variant == 0 && K > 8 &&
+        lt2exp_takes_rows(R, S, I, J, K, sw[2] == 1 && sw[0] % 4 == 0 && sw[1] % 4 == 0 &&
+                                             (reinterpret_cast<uintptr_t>(w) & 15) == 0, pieces == 2 ? 1.0 : 0.7))
         return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
 
     // Rows of w of 2 or 4 values fill an eighth or a quarter of this kernel's smallest j-chunk;
