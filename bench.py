@@ -242,6 +242,15 @@ def profile_pass(dev) -> int:
     for _ in range(3):
         lt2exp(w, a1, b1, _precision="fp32")
     torch.cuda.synchronize()
+    # one s per batch: the rows (s, i) of w on the rows of the MFMA (101 MB of w, a, b and c)
+    gen = torch.Generator().manual_seed(7)
+    wf = torch.rand(2048, 1, 64, 64, generator=gen).to(dev)
+    af = (torch.randn(2048, 64, 64, generator=gen) * 10 - 30).to(dev)
+    bf = (torch.randn(2048, 64, 64, generator=gen) * 10 - 30).to(dev)
+    for _ in range(3):
+        lt2exp(wf, af, bf, _precision="fp32")
+    torch.cuda.synchronize()
+    del wf, af, bf
     flat = b.view(-1)
     for _ in range(3):
         vmax(flat)
@@ -533,6 +542,28 @@ def main() -> int:
                 f"torch recipe {tor * 1e6:.2f} us")
         result["few_columns"] = sv
         del wl, wcopies
+
+        # ------------------------------------------------ lt2exp with few s per batch
+        # Many batches of one to eight s: the library puts the rows (s, i) of w on the rows of the
+        # MFMA and contracts j first.  Bytes: w, a, b and c once (a and b outweigh w here).
+        fr = {"protocol": "the same operands again and again, inside a HIP graph", "unit": "GB/s", "peak": PEAK_HBM_GBPS}
+        gen = torch.Generator().manual_seed(7)
+        for (rr, ss, ii, jj, kk) in ((2048, 1, 64, 64, 64), (2048, 4, 64, 64, 64), (512, 2, 128, 128, 32), (128, 8, 200, 100, 64)):
+            wf = torch.rand(rr, ss, ii, jj, generator=gen).to(dev)
+            af = (torch.randn(rr, ii, kk, generator=gen) * 10 - 30).to(dev)
+            bf = (torch.randn(rr, jj, kk, generator=gen) * 10 - 30).to(dev)
+            nbytes_f = 4 * (wf.numel() + af.numel() + bf.numel() + rr * ss * kk)
+            sec = graph_time(lambda: lt2exp(wf, af, bf, _precision="fp32"), prewarm_ms=PREWARM_MS / 2)
+            tor = graph_time(lambda: torch_lt2exp(wf, af, bf), calls=5, reps=5)
+            fr[f"R{rr}_S{ss}_I{ii}_J{jj}_K{kk}"] = {
+                "kernel": _lib.kernel_name("lt2exp", rr, ss, ii, jj, kk, _lib.MODE_AUTO, 0, 1), "bytes": nbytes_f,
+                "us": round(sec * 1e6, 2), "achieved": round(nbytes_f / sec / 1e9, 1),
+                "frac": round(nbytes_f / sec / 1e9 / PEAK_HBM_GBPS, 4),
+                "tflops": round(2.0 * rr * ss * ii * jj * kk / sec / 1e12, 2), "torch_recipe_us": round(tor * 1e6, 2)}
+            log(f"lt2exp R={rr} S={ss} I={ii} J={jj} K={kk}: {sec * 1e6:.2f} us ({nbytes_f / sec / 1e9:.0f} GB/s), "
+                f"torch recipe {tor * 1e6:.2f} us")
+            del wf, af, bf
+        result["few_rows"] = fr
 
         # ------------------------------------------------ max reductions (HBM bound)
         # Two figures per reduction.  `us`, `achieved`, `frac`: 8 copies of the 64 MiB operand

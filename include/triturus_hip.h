@@ -114,7 +114,11 @@ int trt_lm2exp_variant_count(void);
  * one flat axis, so short rows cost no padding.  With at most 8 columns (K <= 8), a dense flat
  * axis of w (sw[2] == 1) and rows of at least 128 weights (256 for K > 4; 256 / 1024 unless J is a
  * multiple of 4 and the rows are 16-byte aligned, and then J > 4), variant 0 streams w once on
- * the vector ALU instead (no cut, no workspace used, whatever the mode).
+ * the vector ALU instead (no cut, no workspace used, whatever the mode).  With few s per
+ * batch (about a dozen at most), or little work altogether, J a multiple of 4 and 16-byte
+ * aligned rows of w, variant 0 contracts j first, with the rows (s, i) of w on the rows of the
+ * matrix instruction (likewise no cut and no workspace); trt_lt2exp_kernel_name tells which
+ * kernel a call takes.
  */
 int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c,
                    int64_t R, int64_t S, int64_t I, int64_t J, int64_t K,
