@@ -115,8 +115,9 @@ int trt_lm2exp_variant_count(void);
  * axis of w (sw[2] == 1) and rows of at least 128 weights (256 for K > 4; 256 / 1024 unless J is a
  * multiple of 4 and the rows are 16-byte aligned, and then J > 4), variant 0 streams w once on
  * the vector ALU instead (no cut, no workspace used, whatever the mode).  With few s per
- * batch (about a dozen at most), or little work altogether, J a multiple of 4 and 16-byte
- * aligned rows of w, variant 0 contracts j first, with the rows (s, i) of w on the rows of the
+ * batch (about a dozen at most), or little work altogether, and a dense flat axis of w
+ * (16 bytes at a time where J is a multiple of 4 and the rows are 16-byte aligned, float by
+ * float otherwise), variant 0 contracts j first, with the rows (s, i) of w on the rows of the
  * matrix instruction (likewise no cut and no workspace); trt_lt2exp_kernel_name tells which
  * kernel a call takes.
  */

@@ -68,4 +68,6 @@ def test_documented_ctypes_stubs_run(dev):
     assert scope["w"].stride(2) == 2
     exec(compile(blocks[1], "INTEGRATION.md:lt2exp", "exec"), scope)
     assert scope["status"] == 0
-    assert torch.equal(c4, lt2exp(w, a3, b3, mode="unsplit"))
+    assert torch.equal(c4, lt2exp(ws_, a3, b3, mode="unsplit"))
+    # (the dense w may run on another kernel than the strided view: the same values up to rounding)
+    assert torch.allclose(c4, lt2exp(w, a3, b3, mode="unsplit"), rtol=1e-5, atol=1e-5)

@@ -649,6 +649,8 @@ ROWS_FIRST_SHAPES = [
     (11, 2, 7, 200, 10), (1, 5, 33, 68, 65),
     (4, 7, 50, 36, 100), (2, 2, 64, 64, 300), (2, 5, 96, 100, 130), (2, 3, 128, 36, 257),      # several column tiles
     (1, 16, 256, 64, 100), (3, 40, 64, 64, 12), (2, 20, 64, 128, 24),                          # s in several workgroups
+    (3, 1, 33, 9, 10), (5, 2, 40, 13, 33), (2, 3, 64, 66, 70), (4, 1, 31, 47, 130), (2, 5, 100, 175, 40),  # J not a multiple of 4:
+    (3, 2, 245, 255, 20), (7, 4, 50, 10, 300), (40, 1, 64, 63, 64), (1, 9, 129, 30, 90),                  # rows read float by float
 ]
 
 
@@ -659,7 +661,9 @@ def test_few_s_per_batch_contract_j_first(dev, shape):
     the s-row tiles on the same operands.  An infinite weight in the first row of every s but the
     first must not leak into the s before it (rows past I of a tile are the next s's)."""
     R, S, I, J, K = shape
-    assert "rows_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1)
+    assert _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, int(J % 4 == 0)).startswith(
+        "trt::lt2exp_rows_kernel<") and _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, int(J % 4 == 0)).endswith(
+        "true>" if J % 4 == 0 else "false>")
     g = torch.Generator().manual_seed(sum(shape))
     w = torch.rand(R, S, I, J, generator=g)
     a = 5 * torch.randn(R, I, K, generator=g) - 10
@@ -705,6 +709,26 @@ def test_j_first_reads_strided_a_and_b_and_sliced_w_in_place(dev):
     assert torch.equal(out, lt2exp(w.contiguous(), a.contiguous(), b.contiguous()))
 
 
+@pytest.mark.parametrize("offset", [1, 2, 3])
+@pytest.mark.parametrize("shape", [(6, 2, 40, 32, 30), (2, 5, 33, 12, 100), (1, 1, 70, 50, 17)])
+def test_j_first_on_a_w_that_starts_off_a_16_byte_boundary(dev, shape, offset):
+    """A dense w whose first element sits 4, 8 or 12 bytes past a 16-byte boundary (a view into a
+    larger buffer of NaNs): the build that reads rows float by float, whatever J is."""
+    R, S, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape) + offset)
+    n = R * S * I * J
+    buf = torch.full((n + 8,), float("nan"))
+    buf[offset:offset + n] = torch.rand(n, generator=g)
+    w = buf.to(dev)[offset:offset + n].view(R, S, I, J)
+    assert w.data_ptr() % 16 == 4 * offset
+    a = (3 * torch.randn(R, I, K, generator=g)).to(dev)
+    b = (3 * torch.randn(R, J, K, generator=g)).to(dev)
+    assert _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 0).startswith("trt::lt2exp_rows_kernel<")
+    out = lt2exp(w, a, b)
+    r = oracle64.compare(out, oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=4))
+    assert r["ok"], (shape, offset, r)
+
+
 def test_few_s_per_batch_under_a_long_i_keep_w_as_it_lies(dev):
     """2 <= J < I would run on a transposed copy of w under the s-row tiles; j-first takes w as it is."""
     R, S, I, J, K = 40, 2, 300, 16, 40
@@ -719,3 +743,8 @@ def test_few_s_per_batch_under_a_long_i_keep_w_as_it_lies(dev):
     assert r["ok"], r
     for prec in ("bf16x3", "bf16x6"):        # handed over to the same kernel
         assert torch.equal(out, lt2exp(w, a, b, _precision=prec, _swap=False))
+    # J not a multiple of 4: no padded copies of w and b either
+    w3, b3 = w[..., :15].contiguous(), b[:, :15].contiguous()
+    assert torch.equal(lt2exp(w3, a, b3), lt2exp(w3, a, b3, _swap=False, _pad=False))
+    r = oracle64.compare(lt2exp(w3, a, b3), oracle64.lt2exp64(w3.cpu(), a.cpu(), b3.cpu(), batch_chunk=4))
+    assert r["ok"], r

@@ -116,23 +116,30 @@ def test_lt2exp_random_with_few_columns(dev, seed):
 
 @pytest.mark.parametrize("seed", range(60))
 def test_lt2exp_random_with_few_s(dev, seed):
-    """S = 1..12 on random shapes with rows of w of a multiple of 4 floats, strided a and b, every
-    precision: the kernel that contracts j first wherever the library takes it (the s-row tiles
-    elsewhere), against the float64 oracle."""
+    """S = 1..12 on random shapes, rows of w of any length, a w that starts 0..12 bytes past a
+    16-byte boundary, strided a and b, every precision: the kernel that contracts j first wherever
+    the library takes it (the s-row tiles elsewhere), against the float64 oracle."""
     rng = random.Random(4000 + seed)
     g = torch.Generator().manual_seed(seed)
-    R, S, I, J, K = rng.randrange(1, 40), rng.randrange(1, 13), _dim(rng, 300), 4 * rng.randrange(2, 80), _dim(rng, 400)
-    w = torch.rand(R, S, I, J, generator=g) * rng.choice([1.0, 1e-4, 30.0])
+    R, S, I, K = rng.randrange(1, 40), rng.randrange(1, 13), _dim(rng, 300), _dim(rng, 400)
+    J = 4 * rng.randrange(2, 80) if rng.random() < 0.5 else rng.randrange(8, 320)
+    off = rng.choice([0, 0, 0, 1, 2, 3])
+    n = R * S * I * J
+    buf = torch.full((n + 8,), float("nan"))
+    buf[off : off + n] = torch.rand(n, generator=g) * rng.choice([1.0, 1e-4, 30.0])
+    w = buf[off : off + n].view(R, S, I, J)
     if rng.random() < 0.3:
         w[:, rng.randrange(S)] = 0.0
     a = _sprinkle(rng, g, torch.randn(R, I, K, generator=g) * rng.choice([1.0, 10.0]) + rng.choice([0.0, -40.0]))
     b = _sprinkle(rng, g, torch.randn(R, J, K, generator=g) * rng.choice([1.0, 10.0]) + rng.choice([0.0, 70.0]))
     ref = oracle64.lt2exp64(w, a, b)
     precision = rng.choice(["fp32", "fp32", "bf16x3", "bf16x6"])
-    out = lt2exp(w.to(dev), _view(rng, a.to(dev)), _view(rng, b.to(dev)), mode=rng.choice(["auto", "split", "unsplit"]),
+    wg = buf.to(dev)[off : off + n].view(R, S, I, J)
+    wg.copy_(w)
+    out = lt2exp(wg, _view(rng, a.to(dev)), _view(rng, b.to(dev)), mode=rng.choice(["auto", "split", "unsplit"]),
                  _precision=precision)
     r = oracle64.compare(out, ref, **GATES[precision])
-    assert r["ok"], (R, S, I, J, K, precision, r)
+    assert r["ok"], (R, S, I, J, K, off, precision, r)
 
 
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])

@@ -868,8 +868,9 @@ bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, b
 }
 // likewise: would it take the kernel of csrc/lt2exp_rows.hpp (few s per batch)?
 // (margin: by how many doublings the fp32 rule's estimate must favour it)
-bool lt2exp_takes_rows(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, double margin) {
-    return rows_score(R, S, I, J, K) > margin && rows_plan(R, S, I, J, K, w_aligned).ct != 0;
+bool lt2exp_takes_rows(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense,
+                       double margin) {
+    return rows_score(R, S, I, J, K) > margin && rows_plan(R, S, I, J, K, w_aligned, w_dense).ct != 0;
 }
 // for trt_lm2exp_f32: c[r, i, k] = log sum_j a[r, i, j] exp(b[r, j, k]) is the same sweep with the
 // rows of a as the weights, a contracted plane of 1 x J and no factors on the other side.  Is
@@ -927,7 +928,7 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     // few s per batch: the rows (s, i) of w on the rows of the MFMA, j contracted first
     // (csrc/lt2exp_rows.hpp); no cut and no workspace either
     if (variant == 0 && rows_pays(R, S, I, J, K)) {
-        const RowsPlan rp = rows_plan(R, S, I, J, K, w_aligned);
+        const RowsPlan rp = rows_plan(R, S, I, J, K, w_aligned, sw[2] == 1);
         if (rp.ct) return launch_lt2exp_rows(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, rp, static_cast<hipStream_t>(stream));
     }
     int v = resolve_variant(variant, R, S, I, J, K);
@@ -988,7 +989,7 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
     if (variant == 0 && rows_pays(R, S, I, J, K)) {
         const RowsPlan rp = rows_plan(R, S, I, J, K, w_aligned != 0);
         if (rp.ct) {
-            const int n = snprintf(buf, buf_bytes, "trt::lt2exp_rows_kernel<%d>", rp.ct);
+            const int n = snprintf(buf, buf_bytes, "trt::lt2exp_rows_kernel<%d, %s>", rp.ct, rp.vec ? "true" : "false");
             return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
         }
     }

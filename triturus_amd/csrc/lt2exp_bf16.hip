@@ -430,7 +430,7 @@ static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, boo
 }
 
 bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense);  // csrc/lt2exp.hip
-bool lt2exp_takes_rows(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, double margin);  // csrc/lt2exp.hip
+bool lt2exp_takes_rows(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense, double margin);  // csrc/lt2exp.hip
 
 }  // namespace trt
 
@@ -535,7 +535,7 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     // batch 1 runs 1.2-1.7x faster for it from 24 to 128).
     if (variant == 0 && K > 8 &&
         lt2exp_takes_rows(R, S, I, J, K, sw[2] == 1 && sw[0] % 4 == 0 && sw[1] % 4 == 0 &&
-                                             (reinterpret_cast<uintptr_t>(w) & 15) == 0,
+                                             (reinterpret_cast<uintptr_t>(w) & 15) == 0, sw[2] == 1,
                           S <= 12 ? (pieces == 2 ? 1.0 : 0.7) : (pieces == 2 ? 0.3 : 0.0)))
         return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
 

@@ -44,7 +44,11 @@ constexpr int kRowsChunk = 64;                 // values of j per step: 8 loads 
 constexpr int kRowsGroups = kRowsChunk / 8;    // groups of 8 values of j (4 MFMAs each)
 constexpr int kRowsBlock = 16;                 // loads of a thread in flight in the prologue
 
-template <int CT>
+// VEC: rows of w of a multiple of 4 floats on 16-byte boundaries, read 16 bytes at a time; otherwise
+// (any J, any alignment of a dense w) a lane reads its row float by float -- four times the load
+// instructions, each touching 64 cache lines for 4 bytes apiece, which the narrowest column tile
+// feels (the loads of four wavefronts then take about as long as their MFMAs) and wider ones do not.
+template <int CT, bool VEC>
 static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const Lt2RowsArgs p) {
     constexpr int NT = 32 * CT;
     extern __shared__ __attribute__((aligned(16))) float lds[];
@@ -91,8 +95,16 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
         const uint32_t soff = (uint32_t)(ch * kRowsChunk) * 4u;
         const int left = n_groups - ch * kRowsGroups;  // groups of the row from this chunk on
 #pragma unroll
-        for (int g = 0; g < kRowsGroups; ++g)
-            if (g < left) nxt[g] = buf_load_f32x4(w_rsrc, voff + 32u * g, soff);
+        for (int g = 0; g < kRowsGroups; ++g) {
+            if (g < left) {
+                if constexpr (VEC) {
+                    nxt[g] = buf_load_f32x4(w_rsrc, voff + 32u * g, soff);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) nxt[g][e] = buf_load_f32(w_rsrc, voff + 32u * g + 4u * e, soff);
+                }
+            }
+        }
     };
     if (my_items > 0) issue(0, 0);
 
@@ -161,7 +173,7 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
     __syncthreads();
 
     // ---- the contraction
-    const bool odd_tail = (p.J & 7) != 0;  // J = 4 (mod 8): the upper lane half of the last group lies past the row
+    const bool ragged = (p.J & 7) != 0;  // the last group of 8 values of j ends past the row: zeros by selection
     float run[CT];                          // sums over the tiles of the current s
     int run_s = -1;
     for (int item = 0; item < my_items; ++item) {
@@ -183,7 +195,11 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
             for (int g = 0; g < kRowsGroups; ++g) {
                 if (g < left) {
                     floatx4 av = cur[g];
-                    if (odd_tail && g == left - 1 && half) av = floatx4{0.f, 0.f, 0.f, 0.f};
+                    if (ragged && g == left - 1) {
+                        const int room = p.J - 8 * (n_groups - 1) - 4 * half;  // values of j of this lane's piece inside the row
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) av[e] = e < room ? av[e] : 0.f;
+                    }
 #pragma unroll
                     for (int ct = 0; ct < CT; ++ct) {
                         const floatx4 bv =
@@ -250,14 +266,17 @@ static inline size_t rows_lds_bytes(int64_t I, int64_t J, int ct, int s_per_grou
 
 struct RowsPlan {
     int ct, s_per_group;  // ct = 0: the kernel does not apply
+    bool vec;             // 16-byte loads of w
 };
 
 // Column tile and s per workgroup.  The widest column tile that K fills and LDS holds (w is read
 // once per column tile); then as many s per workgroup as leave the grid two workgroups per
 // compute unit, where the batch and column tiles alone do not.
-static inline RowsPlan rows_plan(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned) {
-    RowsPlan none = {0, 0};
-    if (!w_aligned || J % 4 != 0 || J < 8) return none;
+static inline RowsPlan rows_plan(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned,
+                                 bool w_dense = true) {
+    RowsPlan none = {0, 0, false};
+    if (!w_dense || J < 8) return none;
+    const bool vec = w_aligned && J % 4 == 0;
     int ct = K > 64 ? 4 : (K > 32 ? 2 : 1);
     int spg = (int)(S < kRowsMaxS ? S : kRowsMaxS);
     while (ct > 1 && rows_lds_bytes(I, J, ct, spg) > kRowsMaxLds) ct /= 2;
@@ -265,7 +284,7 @@ static inline RowsPlan rows_plan(int64_t R, int64_t S, int64_t I, int64_t J, int
     const int64_t n_it = ceil_div(I, 32);
     const int64_t base = R * ceil_div(K, 32 * ct);
     while (spg > 1 && base * ceil_div(S, spg) < 512 && (int64_t)(spg / 2) * n_it >= 8) spg /= 2;
-    return RowsPlan{ct, spg};
+    return RowsPlan{ct, spg, vec};
 }
 
 // Is this kernel the faster one?  Fitted to 850 timed shapes (S = 1..256, I = 4..512, J = 8..512,
@@ -283,7 +302,10 @@ static inline RowsPlan rows_plan(int64_t R, int64_t S, int64_t I, int64_t J, int
 // Such calls need the estimate to favour this kernel by 7 %: it is the younger one.
 // Taking the kernel by this rule costs 3.2 % over the faster of the two per shape (geometric mean
 // over the fit's shapes; never taking it 53 % -- 134 % over the shapes with S <= 12 --, always
-// taking it 40 %).  Outputs of at most 8 columns have been handed to the sweep before this is asked.
+// taking it 40 %).  The rule serves the element-load build unchanged: on 250 timed shapes whose J
+// is not a multiple of 4 it stands 3.3 % behind the better choice per shape (never taking it 84 %)
+// -- the s-row tiles stage such rows element by element too.  Outputs of at most 8 columns have
+// been handed to the sweep before this is asked.
 static inline double rows_score(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
     const double ws = std::log2(32.0 * (double)ceil_div(S, 32) / (double)S);
     const double wi = std::log2(32.0 * (double)ceil_div(I, 32) / (double)I);
@@ -315,16 +337,23 @@ static int launch_lt2exp_rows(const float *w, const float *a, const float *b, fl
     const int64_t grid = R * args.n_tiles * args.s_groups;
     if (grid >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const size_t lds = rows_lds_bytes(I, J, plan.ct, plan.s_per_group);
-    if (lds > kRowsMaxLds) {  // (only the narrowest tile goes there)
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&lt2exp_rows_kernel<1>),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-        if (e != hipSuccess) return (int)e;
-    }
-    switch (plan.ct) {
-        case 1: hipLaunchKernelGGL((lt2exp_rows_kernel<1>), dim3((unsigned)grid), dim3(kRowsThreads), lds, stream, args); break;
-        case 2: hipLaunchKernelGGL((lt2exp_rows_kernel<2>), dim3((unsigned)grid), dim3(kRowsThreads), lds, stream, args); break;
-        default: hipLaunchKernelGGL((lt2exp_rows_kernel<4>), dim3((unsigned)grid), dim3(kRowsThreads), lds, stream, args); break;
-    }
+    auto launch = [&](auto kernel) -> int {
+        if (lds > kRowsMaxLds) {  // (only the narrowest tile goes there)
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return (int)e;
+        }
+        hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kRowsThreads), lds, stream, args);
+        return 0;
+    };
+    int err;
+    if (plan.vec)
+        err = plan.ct == 1 ? launch(&lt2exp_rows_kernel<1, true>)
+                           : (plan.ct == 2 ? launch(&lt2exp_rows_kernel<2, true>) : launch(&lt2exp_rows_kernel<4, true>));
+    else
+        err = plan.ct == 1 ? launch(&lt2exp_rows_kernel<1, false>)
+                           : (plan.ct == 2 ? launch(&lt2exp_rows_kernel<2, false>) : launch(&lt2exp_rows_kernel<4, false>));
+    if (err) return err;
     return (int)hipGetLastError();
 }
 

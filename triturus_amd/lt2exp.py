@@ -117,7 +117,9 @@ def _rows_first(R: int, S: int, I: int, J: int, K: int, w: torch.Tensor) -> bool
     """Would the library run this call on its kernel for few s per batch?  (Asked of the library
     itself, host side only: the rule is a fitted one and lives there.)"""
     sw = w.stride()
-    aligned = sw[2] == 1 and sw[0] % 4 == 0 and sw[1] % 4 == 0 and w.data_ptr() % 16 == 0
+    if sw[2] != 1:
+        return False
+    aligned = sw[0] % 4 == 0 and sw[1] % 4 == 0 and w.data_ptr() % 16 == 0
     return _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, int(aligned)).startswith("trt::lt2exp_rows_kernel")
 
 
@@ -171,9 +173,10 @@ def lt2exp(
     if K <= 8 and _variant == 0 and _swap is None and _pad is None and _sweeps(R, S, I, J, K, w):
         _swap = _pad = False
     # few s per batch: the library contracts j first, over the rows (s, i) of w as they lie
-    # (csrc/lt2exp_rows.hpp) -- no exchange then
-    if K > 8 and fp32 and _variant == 0 and _swap is None and 2 <= J < I and J % 4 == 0 and _rows_first(R, S, I, J, K, w):
-        _swap = False
+    # (csrc/lt2exp_rows.hpp) -- neither an exchange nor padded copies then
+    if (K > 8 and fp32 and _variant == 0 and _swap is None and _pad is None and (2 <= J < I or J % 4 != 0)
+            and _rows_first(R, S, I, J, K, w)):
+        _swap = _pad = False
     # (the shape tests come first: most calls meet none of them and pay for no rule)
     if _variant == 0 and 2 <= J < I and not (fp32 and _packs(I, J)):
         if _swap is not None:
