@@ -469,25 +469,27 @@ def test_lt2exp_cuts_64_row_tiles_where_the_contraction_is_cut_anyway():
 
 
 def test_lt2exp_few_s_per_batch_contract_j_first():
-    """Host-side rule of lt2exp for few s per batch: lt2exp_rows_kernel<column blocks of 32> puts the
+    """Host-side rule of lt2exp for few s per batch: lt2exp_rows_kernel<column blocks of 32 that a
+    wavefront contracts at once, groups of them in the workgroup's tile, 16-byte loads of w> puts the
     rows (s, i) of w on the rows of the MFMA where padding s to 32 costs more than padding i to 32,
     K is moderate and J is not too short.  Never for forced tiles or at most 8 columns (the sweep's)."""
     name = lambda *sh, variant=0, aligned=1: _lib.kernel_name("lt2exp", *sh, 0, variant, aligned)
-    assert name(2048, 1, 64, 64, 64) == "trt::lt2exp_rows_kernel<2, true>"
-    assert name(2048, 1, 64, 64, 12) == "trt::lt2exp_rows_kernel<1, true>"
-    assert name(5, 3, 33, 20, 70) == "trt::lt2exp_rows_kernel<4, true>"
-    assert name(1520, 1, 245, 256, 256) == "trt::lt2exp_rows_kernel<1, true>"      # the factors of 32 columns fill LDS
-    assert name(64, 4, 128, 128, 4096) == "trt::lt2exp_rows_kernel<1, true>"       # S = 4: 8 times the padding
+    assert name(2048, 1, 64, 64, 64) == "trt::lt2exp_rows_kernel<1, 2, true>"      # two tiles: their column blocks on four wavefronts
+    assert name(2048, 1, 64, 64, 12) == "trt::lt2exp_rows_kernel<1, 1, true>"
+    assert name(4096, 1, 32, 32, 100) == "trt::lt2exp_rows_kernel<1, 4, true>"     # one tile of four column blocks
+    assert name(5, 3, 33, 20, 70) == "trt::lt2exp_rows_kernel<4, 1, true>"
+    assert name(1520, 1, 245, 256, 256) == "trt::lt2exp_rows_kernel<1, 1, true>"      # the factors of 32 columns fill LDS
+    assert name(64, 4, 128, 128, 4096) == "trt::lt2exp_rows_kernel<1, 1, true>"       # S = 4: 8 times the padding
     assert name(64, 64, 64, 64, 4096).startswith("trt::lt2exp_kernel<")      # the large configuration: s-row tiles
     assert name(64, 16, 64, 64, 4096).startswith("trt::lt2exp_kernel<")
     # from 13 values of s on: calls of less than about a GFLOP, whatever S is
-    assert name(1, 128, 128, 128, 128) == "trt::lt2exp_rows_kernel<1, true>"
+    assert name(1, 128, 128, 128, 128) == "trt::lt2exp_rows_kernel<1, 1, true>"
     assert name(16, 128, 128, 128, 128).startswith("trt::lt2exp_kernel<")
     assert name(16, 192, 192, 192, 192).startswith("trt::lt2exp_kernel<")
     assert name(6755, 9, 5, 20, 783).startswith("trt::lt2exp_kernel<")       # I = 5 would pad to 32
     assert name(2048, 1, 64, 64, 8).startswith("trt::lt2exp_smallk_kernel<")
     assert name(2048, 1, 64, 64, 64, variant=3).startswith("trt::lt2exp_kernel<")
     # rows of w that cannot be read 16 bytes at a time: the same kernel, loading float by float
-    assert name(2048, 1, 64, 64, 64, aligned=0) == "trt::lt2exp_rows_kernel<2, false>"
-    assert name(2048, 1, 64, 66, 64) == "trt::lt2exp_rows_kernel<2, false>"  # J not a multiple of 4
+    assert name(2048, 1, 64, 64, 64, aligned=0) == "trt::lt2exp_rows_kernel<1, 2, false>"
+    assert name(2048, 1, 64, 66, 64) == "trt::lt2exp_rows_kernel<1, 2, false>"  # J not a multiple of 4
     assert name(4, 1, 5000, 5000, 64).startswith("trt::lt2exp_kernel<")      # the factors do not fit LDS

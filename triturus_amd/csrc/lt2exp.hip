@@ -989,7 +989,7 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
     if (variant == 0 && rows_pays(R, S, I, J, K)) {
         const RowsPlan rp = rows_plan(R, S, I, J, K, w_aligned != 0);
         if (rp.ct) {
-            const int n = snprintf(buf, buf_bytes, "trt::lt2exp_rows_kernel<%d, %s>", rp.ct, rp.vec ? "true" : "false");
+            const int n = snprintf(buf, buf_bytes, "trt::lt2exp_rows_kernel<%d, %d, %s>", rp.ct / rp.cts, rp.cts, rp.vec ? "true" : "false");
             return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
         }
     }

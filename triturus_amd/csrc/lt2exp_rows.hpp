@@ -48,9 +48,16 @@ constexpr int kRowsBlock = 16;                 // loads of a thread in flight in
 // (any J, any alignment of a dense w) a lane reads its row float by float -- four times the load
 // instructions, each touching 64 cache lines for 4 bytes apiece, which the narrowest column tile
 // feels (the loads of four wavefronts then take about as long as their MFMAs) and wider ones do not.
-template <int CT, bool VEC>
-static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const Lt2RowsArgs p) {
-    constexpr int NT = 32 * CT;
+// CT: column blocks of 32 that a unit of work contracts at once.  CTS: the workgroup's tile holds
+// CTS times as many, and the units of a tile split them (see below).
+// (the second launch bound keeps the register count under what 4, 3 or 2 workgroups per compute
+// unit need: a few registers more and a tile of two column blocks loses its third)
+template <int CT, int CTS, bool VEC>
+static __global__ __launch_bounds__(kRowsThreads, CT == 1 ? (VEC ? 4 : 3) : 3) void lt2exp_rows_kernel(
+    const Lt2RowsArgs p) {
+    static_assert(CT * CTS <= 4 && (CTS == 1 || CTS == 2 || CTS == 4), "a tile of at most 128 columns");
+    constexpr int NT = 32 * CT * CTS;
+    constexpr int per_shift = CTS == 4 ? 2 : (CTS == 2 ? 1 : 0);  // units per item: a power of two, at most 4
     extern __shared__ __attribute__((aligned(16))) float lds[];
     // pitches are 4 (mod 8) floats: the 16-byte reads of 8 consecutive lanes (columns) cover all banks
     float *ebT = lds;                                      // [NT][jp]: exp(b[j, n] - mb[n]), zeros past J
@@ -78,18 +85,50 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
     const uint32_t w_extent = (uint32_t)(((int64_t)(p.S - 1) * p.sw1 + (int64_t)p.I * p.J) * 4);
     const __amdgpu_buffer_rsrc_t w_rsrc = make_rsrc(wr, w_extent);
 
-    // ---- the tiles of this wavefront and their loads.  Item q of the workgroup is tile q % n_it
-    // of the group's s number q / n_it; the wavefront takes q = wave, wave + 4, ...; a step is a
-    // chunk of 64 values of j of an item.
+    // ---- the work of this wavefront and its loads.  Item q of the workgroup is tile q % n_it of the
+    // group's s number q / n_it.  A unit is an item -- or, where the workgroup holds fewer items
+    // than wavefronts, one of CTS groups of column blocks of an item, so that the MFMAs of a call of
+    // one or two tiles per workgroup run on all four SIMDs instead of one or two (each unit reads
+    // the tile's rows of w for itself, from L1).  The wavefront takes units wave, wave + 4, ...; a
+    // step is a chunk of 64 values of j of a unit.
     const int n_it = (p.I + 31) / 32;
     const int n_ch = (p.J + kRowsChunk - 1) / kRowsChunk;
     const int items = s_count * n_it;
-    const int my_items = wave < items ? (items - wave + kRowsWaves - 1) / kRowsWaves : 0;
+    const int units = items << per_shift;
+    const int my_units = wave < units ? (units - wave + kRowsWaves - 1) / kRowsWaves : 0;
     const int n_groups = (p.J + 7) / 8;  // groups of 8 values of j in a row
+    struct Unit {
+        int u, s_l, it;  // u: number of the unit in the workgroup
+    };
+    // (a wavefront's units all have the same column blocks: CTS divides the 4 wavefronts)
+    const int cb = (wave & (CTS - 1)) * CT;  // first column block of this wavefront's units
+    // (no integer division on the way from one unit to the next: it would cost as much as a
+    // quarter of a short tile's MFMAs)
+    auto first_unit = [&]() {
+        Unit x;
+        x.u = wave;
+        x.s_l = 0;
+        x.it = wave >> per_shift;
+        while (x.it >= n_it) {
+            x.it -= n_it;
+            ++x.s_l;
+        }
+        return x;
+    };
+    auto next_unit = [&](const Unit &x) {
+        Unit y;
+        y.u = x.u + kRowsWaves;
+        y.s_l = x.s_l;
+        y.it = x.it + ((y.u >> per_shift) - (x.u >> per_shift));
+        while (y.it >= n_it) {
+            y.it -= n_it;
+            ++y.s_l;
+        }
+        return y;
+    };
     floatx4 nxt[kRowsGroups];
-    auto issue = [&](int item, int ch) {
-        const int q = wave + kRowsWaves * item;
-        const int s = s_begin + q / n_it, i = (q % n_it) * 32 + n;
+    auto issue = [&](const Unit &x, int ch) {
+        const int s = s_begin + x.s_l, i = x.it * 32 + n;
         // (rows past I -- they belong to the next s -- are read past the extent: zeros)
         const uint32_t voff = i < p.I ? (uint32_t)(((int64_t)s * p.sw1 + (int64_t)i * p.J + 4 * half) * 4) : w_extent;
         const uint32_t soff = (uint32_t)(ch * kRowsChunk) * 4u;
@@ -106,7 +145,8 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
             }
         }
     };
-    if (my_items > 0) issue(0, 0);
+    Unit ahead = first_unit();  // the unit whose first chunk is in flight
+    if (my_units > 0) issue(ahead, 0);
 
     // ---- column maxima of a and b over the contracted axes, then the factors (a NaN need not
     // survive the maximum: exp(NaN - m) is NaN for any m and poisons its column's sums).  A thread
@@ -176,9 +216,11 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
     const bool ragged = (p.J & 7) != 0;  // the last group of 8 values of j ends past the row: zeros by selection
     float run[CT];                          // sums over the tiles of the current s
     int run_s = -1;
-    for (int item = 0; item < my_items; ++item) {
-        const int q = wave + kRowsWaves * item;
-        const int s_l = q / n_it, it = q % n_it;
+    const int my_cols = 32 * cb + n;
+    for (int t = 0; t < my_units; ++t) {
+        const Unit x = ahead;
+        ahead = next_unit(x);
+        const int s_l = x.s_l, it = x.it;
         floatx16 acc[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct)
@@ -188,14 +230,15 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
             floatx4 cur[kRowsGroups];
 #pragma unroll
             for (int g = 0; g < kRowsGroups; ++g) cur[g] = nxt[g];
-            if (ch + 1 < n_ch) issue(item, ch + 1);
-            else if (item + 1 < my_items) issue(item + 1, 0);
+            if (ch + 1 < n_ch) issue(x, ch + 1);
+            else if (t + 1 < my_units) issue(ahead, 0);
             const int left = n_groups - ch * kRowsGroups;
+            const int g0 = ch * kRowsGroups;  // first group of the chunk
 #pragma unroll
             for (int g = 0; g < kRowsGroups; ++g) {
                 if (g < left) {
                     floatx4 av = cur[g];
-                    if (ragged && g == left - 1) {
+                    if (ragged && g0 + g == n_groups - 1) {
                         const int room = p.J - 8 * (n_groups - 1) - 4 * half;  // values of j of this lane's piece inside the row
 #pragma unroll
                         for (int e = 0; e < 4; ++e) av[e] = e < room ? av[e] : 0.f;
@@ -203,7 +246,7 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
 #pragma unroll
                     for (int ct = 0; ct < CT; ++ct) {
                         const floatx4 bv =
-                            *reinterpret_cast<const floatx4 *>(&ebT[(32 * ct + n) * p.jp + ch * kRowsChunk + 8 * g + 4 * half]);
+                            *reinterpret_cast<const floatx4 *>(&ebT[(32 * (cb + ct) + n) * p.jp + 8 * (g0 + g) + 4 * half]);
 #pragma unroll
                         for (int e = 0; e < 4; ++e)
                             acc[ct] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[e], bv[e], acc[ct], 0, 0, 0);
@@ -216,7 +259,7 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
         if (s_l != run_s) {
             if (run_s >= 0 && half == 0) {
 #pragma unroll
-                for (int ct = 0; ct < CT; ++ct) part[(wave * p.s_per_group + run_s) * NT + 32 * ct + n] = run[ct];
+                for (int ct = 0; ct < CT; ++ct) part[(wave * p.s_per_group + run_s) * NT + 32 * ct + my_cols] = run[ct];
             }
             run_s = s_l;
 #pragma unroll
@@ -227,7 +270,7 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
             float sum = 0.f;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const floatx4 fa = *reinterpret_cast<const floatx4 *>(&eaT[(32 * ct + n) * p.ip + it * 32 + 8 * g + 4 * half]);
+                const floatx4 fa = *reinterpret_cast<const floatx4 *>(&eaT[(32 * (cb + ct) + n) * p.ip + it * 32 + 8 * g + 4 * half]);
 #pragma unroll
                 for (int e = 0; e < 4; ++e) sum = __builtin_fmaf(acc[ct][4 * g + e], fa[e], sum);
             }
@@ -237,7 +280,7 @@ static __global__ __launch_bounds__(kRowsThreads) void lt2exp_rows_kernel(const 
     }
     if (run_s >= 0 && half == 0) {
 #pragma unroll
-        for (int ct = 0; ct < CT; ++ct) part[(wave * p.s_per_group + run_s) * NT + 32 * ct + n] = run[ct];
+        for (int ct = 0; ct < CT; ++ct) part[(wave * p.s_per_group + run_s) * NT + 32 * ct + my_cols] = run[ct];
     }
     __syncthreads();
 
@@ -265,8 +308,9 @@ static inline size_t rows_lds_bytes(int64_t I, int64_t J, int ct, int s_per_grou
 }
 
 struct RowsPlan {
-    int ct, s_per_group;  // ct = 0: the kernel does not apply
+    int ct, s_per_group;  // column blocks of the workgroup's tile (0: the kernel does not apply), s per workgroup
     bool vec;             // 16-byte loads of w
+    int cts;              // a tile's work cut into cts groups of column blocks (fewer tiles than wavefronts)
 };
 
 // Column tile and s per workgroup.  The widest column tile that K fills and LDS holds (w is read
@@ -274,7 +318,7 @@ struct RowsPlan {
 // compute unit, where the batch and column tiles alone do not.
 static inline RowsPlan rows_plan(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned,
                                  bool w_dense = true) {
-    RowsPlan none = {0, 0, false};
+    RowsPlan none = {0, 0, false, 1};
     if (!w_dense || J < 8) return none;
     const bool vec = w_aligned && J % 4 == 0;
     int ct = K > 64 ? 4 : (K > 32 ? 2 : 1);
@@ -284,7 +328,12 @@ static inline RowsPlan rows_plan(int64_t R, int64_t S, int64_t I, int64_t J, int
     const int64_t n_it = ceil_div(I, 32);
     const int64_t base = R * ceil_div(K, 32 * ct);
     while (spg > 1 && base * ceil_div(S, spg) < 512 && (int64_t)(spg / 2) * n_it >= 8) spg /= 2;
-    return RowsPlan{ct, spg, vec};
+    // fewer tiles than wavefronts in a workgroup: cut a tile's work by column blocks (R=4096, S=1,
+    // I=J=32, K=100: 121 -> 48 us; R=2048, S=1, I=J=64, K=256: 144 -> 120).  Cutting the range of j
+    // as well, for tiles of a single column block, was slower (K=12: 24 -> 27 us): not done.
+    int cts = 1;
+    while ((int64_t)spg * n_it * cts < kRowsWaves && cts < ct) cts *= 2;
+    return RowsPlan{ct, spg, vec, cts};
 }
 
 // Is this kernel the faster one?  Fitted to 850 timed shapes (S = 1..256, I = 4..512, J = 8..512,
@@ -347,12 +396,13 @@ static int launch_lt2exp_rows(const float *w, const float *a, const float *b, fl
         return 0;
     };
     int err;
-    if (plan.vec)
-        err = plan.ct == 1 ? launch(&lt2exp_rows_kernel<1, true>)
-                           : (plan.ct == 2 ? launch(&lt2exp_rows_kernel<2, true>) : launch(&lt2exp_rows_kernel<4, true>));
-    else
-        err = plan.ct == 1 ? launch(&lt2exp_rows_kernel<1, false>)
-                           : (plan.ct == 2 ? launch(&lt2exp_rows_kernel<2, false>) : launch(&lt2exp_rows_kernel<4, false>));
+    const int unit_ct = plan.ct / plan.cts;  // column blocks that a unit contracts at once: the kernel's CT
+#define TRT_ROWS_LAUNCH(CT_, CTS_) \
+    (plan.vec ? launch(&lt2exp_rows_kernel<CT_, CTS_, true>) : launch(&lt2exp_rows_kernel<CT_, CTS_, false>))
+    if (plan.cts == 1) err = unit_ct == 1 ? TRT_ROWS_LAUNCH(1, 1) : (unit_ct == 2 ? TRT_ROWS_LAUNCH(2, 1) : TRT_ROWS_LAUNCH(4, 1));
+    else if (plan.cts == 2) err = unit_ct == 1 ? TRT_ROWS_LAUNCH(1, 2) : TRT_ROWS_LAUNCH(2, 2);
+    else err = TRT_ROWS_LAUNCH(1, 4);
+#undef TRT_ROWS_LAUNCH
     if (err) return err;
     return (int)hipGetLastError();
 }
