@@ -87,12 +87,12 @@ def test_c_abi_argument_errors_are_statuses():
     assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, s3(1, -1, 1), ok, ok, 0, 0, null, 0, null) == -2
     assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, s3(1, 1, -1), ok, ok, ok, 0, 0, null, 0, null) == -2
     assert lib.trt_lt2exp_f32(one, one, one, one, 1, 1, 1, 1, 1, ok, ok, ok, s3(1, 1, 2), 0, 0, null, 0, null) == -2
-    big4 = (2, 64, 16, 16, 64, s3(16384, 256, 1), s3(1024, 64, 1), s3(1024, 64, 1), s3(4096, 64, 1))
+    big4 = (64, 64, 16, 16, 4096, s3(16384, 256, 1), s3(65536, 4096, 1), s3(65536, 4096, 1), s3(262144, 4096, 1))
     assert lib.trt_lt2exp_f32(one, one, one, one, *big4, _lib.MODE_SPLIT, 0, null, 0, null) == -3  # split needs a workspace
     assert lib.trt_lt2exp_f32(one, one, one, one, *args, 0, lib.trt_lt2exp_variant_count() + 1, null, 0, null) == -1
     # short rows of w (J = 8) walked packed: a forced split still asks for its workspace
-    packed = (2, 64, 256, 8, 64, s3(64 * 2048, 2048, 1), s3(256 * 64, 64, 1), s3(8 * 64, 64, 1), s3(64 * 64, 64, 1))
-    assert lib.trt_lt2exp_workspace_bytes(2, 64, 256, 8, 64, _lib.MODE_SPLIT) > 0
+    packed = (64, 64, 256, 8, 64, s3(64 * 2048, 2048, 1), s3(256 * 64, 64, 1), s3(8 * 64, 64, 1), s3(64 * 64, 64, 1))
+    assert lib.trt_lt2exp_workspace_bytes(64, 64, 256, 8, 64, _lib.MODE_SPLIT) > 0
     assert lib.trt_lt2exp_f32(one, one, one, one, *packed, _lib.MODE_SPLIT, 0, null, 0, null) == -3
     assert lib.trt_lt2exp_bf16(one, one, one, one, *packed, 3, _lib.MODE_SPLIT, 0, null, 0, null) == -3  # handed to fp32
     # lt2exp on the bf16 matrix pipe: pieces must be 2 or 3, variant 0..4
@@ -448,10 +448,10 @@ def test_lt2exp_takes_64_column_tiles_where_128_column_tiles_would_stand_half_em
     name = lambda *sh, aligned=1: _lib.kernel_name("lt2exp", *sh, _lib.MODE_AUTO, 0, aligned)
     wm = lambda n: int(n.split(", ")[6])
     assert wm(name(1, 192, 192, 192, 192)) == 2      # one of the reference's benchmark shapes
-    assert wm(name(1, 535, 26, 64, 136)) == 2
+    assert wm(name(4, 535, 26, 64, 136)) == 2
     assert wm(name(1, 192, 192, 192, 256)) == 1      # whole 128-column tiles
     assert wm(name(1, 192, 192, 192, 448)) == 1      # 7 tiles of 64 against 4 of 128: 0.875 of the area
-    assert wm(name(1, 535, 26, 64, 136, aligned=0)) == 1 and wm(name(1, 535, 26, 24, 136)) == 1  # aligned rows, chunks of 32 only
+    assert wm(name(4, 535, 26, 64, 136, aligned=0)) == 1 and wm(name(4, 535, 26, 24, 136)) == 1  # aligned rows, chunks of 32 only
     assert name(16, 382, 10, 32, 184).endswith(", 2>")  # paired groups keep their grids
 
 
@@ -463,7 +463,7 @@ def test_lt2exp_cuts_64_row_tiles_where_the_contraction_is_cut_anyway():
     assert name(32, 64, 64, 64, 256) == "trt::lt2exp_kernel<2, 1, 4, 4, true, true, 1, 0, 1>"
     assert name(4, 170, 90, 128, 245).startswith("trt::lt2exp_kernel<2, 1, 4, 4, true, true")
     # fewer than twelve 64-row tiles, rows that 64 pads further than 32, or no cut: 32 rows
-    assert name(1, 128, 128, 128, 256).startswith("trt::lt2exp_kernel<1, 1, 4, 4, true, true")
+    assert name(1, 128, 128, 128, 512).startswith("trt::lt2exp_kernel<1, 1, 4, 4, true, true")
     assert name(32, 82, 131, 64, 184).startswith("trt::lt2exp_kernel<1, 1, 4, 4, true, true")
     assert name(32, 64, 64, 64, 256, mode=_lib.MODE_UNSPLIT).startswith("trt::lt2exp_kernel<1, 1, 4, 4, true, false")
 

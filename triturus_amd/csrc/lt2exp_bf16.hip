@@ -523,20 +523,16 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
         return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
 
     // Few s per batch: these tiles, like the fp32 ones, put s on the rows of the MFMA and pad it to
-    // 32; the fp32 kernel of csrc/lt2exp_rows.hpp puts the rows (s, i) of w there.  Up to 12 values
-    // of s, where the fp32 rule favours it by a factor of two (1.6 against three pieces) it beats
-    // these tiles as well (80 timed shapes with S = 1..40: 1.0-7.5x against two pieces in 36 of 41
-    // such calls, 0.6-0.9x in five; 1.0-12x against three pieces in 38 of 44, 0.7-0.98x in six;
-    // over all 80, handing over by this rule leaves 3-4 % to the better choice per shape, never
-    // handing over 37 and 56 %) -- and it is the more exact of the two.  Beyond 12 values of s the
-    // rule only takes calls of little work, bound by latencies in either kernel: there a score of
-    // 0.3 (two pieces) or any positive one (three) decides (90 timed shapes: 4.5 and 3.5 % behind the
-    // better choice per shape, never handing over 12 and 18 %; the reference's square sweep at
-    // batch 1 runs 1.2-1.7x faster for it from 24 to 128).
+    // 32; the fp32 kernel of csrc/lt2exp_rows.hpp puts the rows (s, i) of w there -- and is the more
+    // exact of the two.  It is taken where the fp32 rule's score (log2 of the estimated gain over the
+    // fp32 s-row tiles) exceeds a margin fitted to 260 shapes timed on all three paths: up to 12
+    // values of s 0.6 against two pieces and 0.4 against three (3.0 and 0.7 % behind the better
+    // choice per shape; never handing over 56 and 100 %), beyond that -- calls of little work, bound
+    // by latencies in either kernel -- 0.2 and 0 (3.4 and 3.7 %; never 6 and 11 %).
     if (variant == 0 && K > 8 &&
         lt2exp_takes_rows(R, S, I, J, K, sw[2] == 1 && sw[0] % 4 == 0 && sw[1] % 4 == 0 &&
                                              (reinterpret_cast<uintptr_t>(w) & 15) == 0, sw[2] == 1,
-                          S <= 12 ? (pieces == 2 ? 1.0 : 0.7) : (pieces == 2 ? 0.3 : 0.0)))
+                          S <= 12 ? (pieces == 2 ? 0.6 : 0.4) : (pieces == 2 ? 0.2 : 0.0)))
         return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
 
     // Rows of w of 2 or 4 values fill an eighth or a quarter of this kernel's smallest j-chunk;

@@ -336,33 +336,33 @@ static inline RowsPlan rows_plan(int64_t R, int64_t S, int64_t I, int64_t J, int
     return RowsPlan{ct, spg, vec, cts};
 }
 
-// Is this kernel the faster one?  Fitted to 850 timed shapes (S = 1..256, I = 4..512, J = 8..512,
-// K = 9..2048, up to 300 MB of w) as the sign of a linear score in log2 units -- the estimate of
-// log2(time of the s-row tiles / time of this kernel):
+// Is this kernel the faster one?  Fitted to 1100 timed shapes (S = 1..256, I = 4..512, J = 8..512,
+// K = 9..2048, up to 300 MB of w; a quarter of them with J not a multiple of 4) as the sign of a
+// linear score in log2 units -- the estimate of log2(time of the s-row tiles / time of this kernel):
 //   + per doubling of the padding of s to 32 rows there (0.5, not 1: small calls are bound by
 //     latencies on both sides),
-//   - 0.8-0.9 per doubling of the padding of i to 32 rows here,
-//   - per doubling of K (more column tiles fill the grid of the s-row tiles),
+//   - 0.65 per doubling of the padding of i to 32 rows here,
+//   - 0.18 per doubling of K (more column tiles fill the grid of the s-row tiles),
 //   - per halving of J below 32 (the epilogue of a tile, 16 FMAs and 4 LDS reads per column
-//     tile, against J / 2 MFMAs),
-// and, from 13 values of s on, where the padding of s no longer decides, - 0.09 per doubling of
+//     block, against J / 2 MFMAs),
+// and, from 13 values of s on, where the padding of s no longer decides, - 0.12 per doubling of
 // the work: the s-row tiles run large grids at 100-125 TFLOP/s, this kernel at 60-95, but a call
-// of less than about a GFLOP is faster here whatever S is (R=1, S=I=J=K=128: 30 -> 17 us).
-// Such calls need the estimate to favour this kernel by 7 %: it is the younger one.
-// Taking the kernel by this rule costs 3.2 % over the faster of the two per shape (geometric mean
-// over the fit's shapes; never taking it 53 % -- 134 % over the shapes with S <= 12 --, always
-// taking it 40 %).  The rule serves the element-load build unchanged: on 250 timed shapes whose J
-// is not a multiple of 4 it stands 3.3 % behind the better choice per shape (never taking it 84 %)
-// -- the s-row tiles stage such rows element by element too.  Outputs of at most 8 columns have
-// been handed to the sweep before this is asked.
+// of less than about a GFLOP is faster here whatever S is (R=1, S=I=J=K=128: 30 -> 15 us).
+// Such calls need the estimate to favour this kernel by 7 % (it costs 0.4 %, and keeps calls of
+// a few GFLOP under thousands of columns, where the two run level, on the tiles tuned for them).
+// Taking the kernel by this rule costs 2.5 % over the faster of the two per shape (geometric mean
+// over the fit's shapes; never taking it 68 % -- 154 % over the shapes with S <= 12 --, always
+// taking it 14 %).  The element-load build is served by the same rule (the s-row tiles stage
+// such rows element by element too).  Outputs of at most 8 columns have been handed to the sweep
+// before this is asked.
 static inline double rows_score(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
     const double ws = std::log2(32.0 * (double)ceil_div(S, 32) / (double)S);
     const double wi = std::log2(32.0 * (double)ceil_div(I, 32) / (double)I);
     const double lj = std::log2((double)J), lk = std::log2((double)K);
     const double short_j = lj < 5.0 ? 5.0 - lj : 0.0;
-    if (S <= 12) return 1.83 + 0.49 * ws - 0.87 * wi - 0.21 * lk - 0.62 * short_j;
+    if (S <= 12) return 1.41 + 0.52 * ws - 0.65 * wi - 0.18 * lk - 0.22 * short_j;
     const double lw = std::log2(2.0 * (double)R * (double)S * (double)I * (double)J * (double)K);
-    return 3.49 + 0.33 * ws - 0.79 * wi - 0.10 * lk - 0.40 * short_j - 0.09 * lw - 0.1;
+    return 3.77 + 0.36 * ws - 0.65 * wi - 0.27 * short_j - 0.12 * lw - 0.1;
 }
 static inline bool rows_pays(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
     return rows_score(R, S, I, J, K) > 0.0;

@@ -172,17 +172,14 @@ def lt2exp(
     fp32 = _precision == "fp32"
     if K <= 8 and _variant == 0 and _swap is None and _pad is None and _sweeps(R, S, I, J, K, w):
         _swap = _pad = False
-    # few s per batch: the library contracts j first, over the rows (s, i) of w as they lie
-    # (csrc/lt2exp_rows.hpp) -- neither an exchange nor padded copies then
-    if (K > 8 and fp32 and _variant == 0 and _swap is None and _pad is None and (2 <= J < I or J % 4 != 0)
-            and _rows_first(R, S, I, J, K, w)):
-        _swap = _pad = False
     # (the shape tests come first: most calls meet none of them and pay for no rule)
     if _variant == 0 and 2 <= J < I and not (fp32 and _packs(I, J)):
         if _swap is not None:
             swap = _swap
         elif fp32:
-            swap = _exchange_pays(R, S, I, J, K)
+            # (few s per batch: the library contracts j first, over the rows (s, i) of w as they lie
+            # -- csrc/lt2exp_rows.hpp -- and wants no exchange; asked only where one would be made)
+            swap = _exchange_pays(R, S, I, J, K) and not (K > 8 and _rows_first(R, S, I, J, K, w))
         else:
             swap = (K >= 256 and 2 * I * _padded(J) >= 3 * J * _padded(I)
                     and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS)  # worth a copy kernel: some 40 us of work
@@ -206,6 +203,8 @@ def lt2exp(
         J4 = J + (-J) % 4
         pad = (K >= _PAD_MIN_K and 2 * R * S * I * _padded(J) * K >= _RESHAPE_MIN_FLOPS
                and (not fp32 or 5 * _padded(J4) <= 4 * _padded_by_element(J))) if _pad is None else _pad
+        if pad and _pad is None and fp32 and K > 8 and _rows_first(R, S, I, J, K, w):
+            pad = False  # (the same kernel reads rows of any length in place)
         if pad:
             w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
             b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
