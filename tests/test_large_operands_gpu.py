@@ -51,6 +51,22 @@ def test_lt2exp_with_w_beyond_4_gib(big, precision):
         assert r["ok"], (r0, r)
 
 
+def test_lt2exp_with_one_s_per_batch_and_w_beyond_4_gib(big):
+    """The kernel that contracts j first (one s per batch): 64-bit batch offsets of w, a, b and c."""
+    from triturus_amd import _lib
+
+    R, S, I, J, K = 36000, 1, 128, 256, 16  # w: 4.7 GB
+    assert "rows_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1)
+    w = torch.rand(R, S, I, J, device=big)
+    a = torch.randn(R, I, K, device=big) * 3
+    b = torch.randn(R, J, K, device=big) * 3
+    c = lt2exp(w, a, b)
+    for r0 in (0, 17999, R - 8):
+        sl = slice(r0, r0 + 8)
+        r = oracle64.compare(c[sl], oracle64.lt2exp64(w[sl], a[sl], b[sl], batch_chunk=8, device=big))
+        assert r["ok"], (r0, r)
+
+
 def test_lm2exp_with_a_batch_of_b_beyond_2_gib(big):
     R, I, J, K = 2, 64, 8192, 70000  # 2.3 GB per batch of b
     a = torch.rand(R, I, J, device=big)

@@ -441,12 +441,20 @@ def test_capturable_in_a_hip_graph(dev):
     a = torch.randn(2, 16, 256, generator=g).to(dev)
     b = torch.randn(2, 32, 256, generator=g).to(dev)
     a2 = torch.rand(2, 256, 32, generator=g).to(dev)
+    w2 = w[:, :2].contiguous()                                   # two s per batch: j contracted first
+    wl = torch.rand(2, 1, 245, 256, generator=g).to(dev)         # its factors take more than 64 KB of LDS
+    al = torch.randn(2, 245, 40, generator=g).to(dev)
+    bl = torch.randn(2, 256, 40, generator=g).to(dev)
+    assert "rows_kernel" in _lib.kernel_name("lt2exp", 2, 2, 16, 32, 256, 0, 0, 1)
+    assert "rows_kernel" in _lib.kernel_name("lt2exp", 2, 1, 245, 256, 40, 0, 0, 1)
     side = torch.cuda.Stream(device=dev)
     side.wait_stream(torch.cuda.current_stream(dev))
     with torch.cuda.stream(side):
         for _ in range(2):
             lt2exp(w, a, b)
             lm2exp(a2, b)
+            lt2exp(w2, a, b)
+            lt2exp(wl, al, bl)
     torch.cuda.current_stream(dev).wait_stream(side)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
@@ -456,6 +464,8 @@ def test_capturable_in_a_hip_graph(dev):
         out_m = lm2exp(a2, b)
         out_t3 = lt2exp(w, a, b, _precision="bf16x3", _variant=1)
         out_m6 = lm2exp(a2, b, _precision="bf16x6", _variant=3)
+        out_r = lt2exp(w2, a, b)
+        out_l = lt2exp(wl, al, bl)
     for rep in range(4):
         a.copy_(torch.randn(2, 16, 256, generator=g))
         b.copy_(torch.randn(2, 32, 256, generator=g) - rep)
@@ -466,6 +476,8 @@ def test_capturable_in_a_hip_graph(dev):
         assert torch.equal(out_m, lm2exp(a2, b))
         assert torch.equal(out_t3, lt2exp(w, a, b, _precision="bf16x3", _variant=1))
         assert torch.equal(out_m6, lm2exp(a2, b, _precision="bf16x6", _variant=3))
+        assert torch.equal(out_r, lt2exp(w2, a, b))
+        assert torch.equal(out_l, lt2exp(wl, al, bl))
         torch.cuda.synchronize()
 
 

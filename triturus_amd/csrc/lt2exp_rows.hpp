@@ -20,6 +20,7 @@
 // timing.
 #pragma once
 
+#include <atomic>
 #include <cmath>
 
 #include "common.hpp"
@@ -386,11 +387,19 @@ static int launch_lt2exp_rows(const float *w, const float *a, const float *b, fl
     const int64_t grid = R * args.n_tiles * args.s_groups;
     if (grid >= ((int64_t)1 << 31)) return TRT_E_RANGE;
     const size_t lds = rows_lds_bytes(I, J, plan.ct, plan.s_per_group);
+    // (more than 64 KB of LDS must be allowed per kernel and device, once: the first such launch
+    // on a device makes that call, every later one -- one inside a stream capture, say -- does not)
     auto launch = [&](auto kernel) -> int {
         if (lds > kRowsMaxLds) {  // (only the narrowest tile goes there)
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-            if (e != hipSuccess) return (int)e;
+            static std::atomic<uint64_t> allowed{0};  // (per instance of the kernel: a bit per device)
+            int device = 0;
+            if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return TRT_E_INVALID;
+            if (!(allowed.load(std::memory_order_acquire) >> device & 1)) {
+                const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                         hipFuncAttributeMaxDynamicSharedMemorySize, (int)kRowsMaxLdsNarrow);
+                if (e != hipSuccess) return (int)e;
+                allowed.fetch_or((uint64_t)1 << device, std::memory_order_release);
+            }
         }
         hipLaunchKernelGGL(kernel, dim3((unsigned)grid), dim3(kRowsThreads), lds, stream, args);
         return 0;
