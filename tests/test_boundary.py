@@ -493,3 +493,20 @@ def test_lt2exp_few_s_per_batch_contract_j_first():
     assert name(2048, 1, 64, 64, 64, aligned=0) == "trt::lt2exp_rows_kernel<1, 2, false>"
     assert name(2048, 1, 64, 66, 64) == "trt::lt2exp_rows_kernel<1, 2, false>"  # J not a multiple of 4
     assert name(4, 1, 5000, 5000, 64).startswith("trt::lt2exp_kernel<")      # the factors do not fit LDS
+
+
+def test_lt2exp_few_units_over_many_batches_take_a_lane_per_column():
+    """Host-side rule of lt2exp for I and J of at most 16: lt2exp_cols_kernel<I and J padded to 4, 8
+    or 16, exact sizes on a dense w> where a lane's S I J FMAs stay few enough and the call is large
+    enough.  Never for forced tiles or at most 8 columns."""
+    name = lambda *sh, variant=0: _lib.kernel_name("lt2exp", *sh, 0, variant, 1)
+    assert name(8192, 8, 8, 8, 256) == "trt::lt2exp_cols_kernel<8, 8, true>"
+    assert name(8192, 4, 4, 4, 64) == "trt::lt2exp_cols_kernel<4, 4, true>"
+    assert name(4096, 4, 16, 16, 256) == "trt::lt2exp_cols_kernel<16, 16, true>"
+    assert name(1500, 3, 5, 7, 64) == "trt::lt2exp_cols_kernel<8, 8, false>"
+    assert name(2500, 7, 16, 1, 90) == "trt::lt2exp_cols_kernel<4, 16, false>"     # J = 1: i and j exchanged first
+    assert name(8192, 16, 16, 16, 256).startswith("trt::lt2exp_kernel<")            # 4096 FMAs per lane: the MFMA tiles
+    assert name(16, 8, 8, 8, 64).startswith("trt::lt2exp_kernel<")                  # a call of a few microseconds either way
+    assert name(8192, 8, 8, 17, 256).startswith("trt::lt2exp_kernel<")              # J beyond 16
+    assert name(8192, 8, 8, 8, 8).startswith("trt::lt2exp_rows_kernel<")            # 8 columns: not asked
+    assert name(8192, 8, 8, 8, 256, variant=3).startswith("trt::lt2exp_kernel<")

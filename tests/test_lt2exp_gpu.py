@@ -760,3 +760,59 @@ def test_few_s_per_batch_under_a_long_i_keep_w_as_it_lies(dev):
     assert torch.equal(lt2exp(w3, a, b3), lt2exp(w3, a, b3, _swap=False, _pad=False))
     r = oracle64.compare(lt2exp(w3, a, b3), oracle64.lt2exp64(w3.cpu(), a.cpu(), b3.cpu(), batch_chunk=4))
     assert r["ok"], r
+
+
+COLS_SHAPES = [
+    (512, 8, 8, 8, 256), (700, 4, 4, 4, 64), (400, 1, 16, 16, 512), (900, 16, 4, 8, 33), (2000, 2, 16, 4, 100),   # exact sizes
+    (1500, 3, 5, 7, 64), (3000, 5, 1, 16, 40), (2500, 7, 16, 1, 90), (5000, 1, 3, 3, 1000), (1100, 2, 13, 2, 65),    # any I and J
+]
+
+
+@pytest.mark.parametrize("shape", COLS_SHAPES)
+def test_few_units_over_many_batches_take_a_lane_per_column(dev, shape):
+    """I and J of at most 16 over many batches: the kernel with a lane per output column and the
+    batch's weights as scalar operands (csrc/lt2exp_cols.hpp) against the float64 oracle, -inf and
+    NaN columns included, and against the MFMA tiles on the same operands."""
+    R, S, I, J, K = shape
+    assert _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1).startswith("trt::lt2exp_cols_kernel<")
+    g = torch.Generator().manual_seed(sum(shape))
+    w = torch.rand(R, S, I, J, generator=g)
+    w[:, S // 2] = 0.0
+    a = 5 * torch.randn(R, I, K, generator=g) - 10
+    b = 5 * torch.randn(R, J, K, generator=g) + 3
+    a[0, :, 0] = NINF                       # a whole column of a: -inf out
+    b[R - 1, J // 2, K - 1] = NINF          # a single -inf entry
+    ref = oracle64.lt2exp64(w, a, b, batch_chunk=64)
+    out = lt2exp(w.to(dev), a.to(dev), b.to(dev))
+    r = oracle64.compare(out, ref)
+    assert r["ok"], (shape, r)
+    assert torch.isneginf(out[0, :, 0]).all() and torch.isneginf(out[:, S // 2]).all()
+    assert torch.equal(out, lt2exp(w.to(dev), a.to(dev), b.to(dev)))
+    tiles = lt2exp(w.to(dev), a.to(dev), b.to(dev), _variant=4)
+    assert torch.allclose(out, tiles, rtol=1e-5, atol=1e-5)
+    an = a.clone()
+    an[R // 2, I // 2, K // 2] = float("nan")
+    outn = lt2exp(w.to(dev), an.to(dev), b.to(dev))
+    assert torch.isnan(outn[R // 2, :, K // 2]).all()
+    mask = torch.ones_like(outn, dtype=torch.bool)
+    mask[R // 2, :, K // 2] = False
+    assert torch.equal(outn[mask], out[mask])
+
+
+def test_a_lane_per_column_reads_strided_a_and_b_and_sliced_w_in_place(dev):
+    R, S, I, J, K = 900, 6, 8, 8, 100
+    g = torch.Generator().manual_seed(8)
+    wide = torch.rand(R, S + 3, I, 2 * J, generator=g).to(dev)
+    w = wide[:, 2:S + 2, :, ::2]                                   # every other weight of a wider tensor
+    a = (3 * torch.randn(R, K, I, generator=g)).to(dev).transpose(1, 2)   # K-major
+    b = (3 * torch.randn(R, J, 2 * K, generator=g)).to(dev)[:, :, ::2]    # every other column
+    out = lt2exp(w, a, b)
+    r = oracle64.compare(out, oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=64))
+    assert r["ok"], r
+    dense = lt2exp(w.contiguous(), a.contiguous(), b.contiguous())
+    assert _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 1) == "trt::lt2exp_cols_kernel<8, 8, true>"
+    assert torch.allclose(out, dense, rtol=1e-6, atol=1e-6)        # (the general build sums in the same order)
+    for prec in ("bf16x3", "bf16x6"):
+        r = oracle64.compare(lt2exp(w, a, b, _precision=prec), oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=64),
+                             rtol=1e-4, atol=5e-5)
+        assert r["ok"], (prec, r)

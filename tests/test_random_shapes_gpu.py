@@ -142,6 +142,31 @@ def test_lt2exp_random_with_few_s(dev, seed):
     assert r["ok"], (R, S, I, J, K, off, precision, r)
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_lt2exp_random_with_few_units(dev, seed):
+    """I, J = 1..16 over hundreds to thousands of batches, any S, strided a and b, a w that is a
+    slice of a wider tensor now and then: the kernel with a lane per output column wherever the
+    library takes it, against the float64 oracle."""
+    rng = random.Random(5000 + seed)
+    g = torch.Generator().manual_seed(seed)
+    I, J, S, K = rng.randrange(1, 17), rng.randrange(1, 17), rng.choice([1, 2, 3, 5, 8, 16, 33]), _dim(rng, 300)
+    R = rng.choice([50, 400, 1500, 4000])
+    w = torch.rand(R, S, I, J, generator=g) * rng.choice([1.0, 1e-4, 30.0])
+    a = _sprinkle(rng, g, torch.randn(R, I, K, generator=g) * rng.choice([1.0, 10.0]) + rng.choice([0.0, -40.0]))
+    b = _sprinkle(rng, g, torch.randn(R, J, K, generator=g) * rng.choice([1.0, 10.0]) + rng.choice([0.0, 70.0]))
+    ref = oracle64.lt2exp64(w, a, b, batch_chunk=256)
+    wg = w.to(dev)
+    if rng.random() < 0.3:
+        wide = torch.zeros(R, S, I, 2 * J, device=dev)
+        wide[..., ::2] = wg
+        wg = wide[..., ::2]
+    precision = rng.choice(["fp32", "fp32", "bf16x3", "bf16x6"])
+    out = lt2exp(wg, _view(rng, a.to(dev)), _view(rng, b.to(dev)), mode=rng.choice(["auto", "split", "unsplit"]),
+                 _precision=precision)
+    r = oracle64.compare(out, ref, **GATES[precision])
+    assert r["ok"], (R, S, I, J, K, precision, r)
+
+
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
 def test_results_are_bit_reproducible(dev, precision):
     """Fixed summation order everywhere (no atomics, merges in split order): the same call on

@@ -21,6 +21,7 @@
 
 #include "common.hpp"
 #include "lt2exp_merge.hpp"
+#include "lt2exp_cols.hpp"
 #include "lt2exp_rows.hpp"
 #include "lt2exp_smallk.hpp"
 
@@ -866,6 +867,10 @@ namespace trt {
 bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense) {
     return smallk_applies(R, S, I, J, K, w_aligned, w_dense);
 }
+// likewise: would it take the kernel of csrc/lt2exp_cols.hpp (few units, a lane per column)?
+bool lt2exp_takes_cols(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_dense, double margin) {
+    return cols_applies(I, J, K) && cols_score(R, S, I, J, K, w_dense) > margin;
+}
 // likewise: would it take the kernel of csrc/lt2exp_rows.hpp (few s per batch)?
 // (margin: by how many doublings the fp32 rule's estimate must favour it)
 bool lt2exp_takes_rows(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense,
@@ -925,6 +930,10 @@ extern "C" int trt_lt2exp_f32(const float *w, const float *a, const float *b, fl
     // cut, no workspace, whatever the mode asks for
     if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned, sw[2] == 1))
         return launch_lt2exp_smallk(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, w_aligned, static_cast<hipStream_t>(stream));
+    // layers of few units over many batches: a lane per output column (csrc/lt2exp_cols.hpp); no cut
+    // and no workspace either
+    if (variant == 0 && cols_pays(R, S, I, J, K, sw[2] == 1))
+        return launch_lt2exp_cols(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, static_cast<hipStream_t>(stream));
     // few s per batch: the rows (s, i) of w on the rows of the MFMA, j contracted first
     // (csrc/lt2exp_rows.hpp); no cut and no workspace either
     if (variant == 0 && rows_pays(R, S, I, J, K)) {
@@ -986,6 +995,7 @@ extern "C" int trt_lt2exp_kernel_name(int64_t R, int64_t S, int64_t I, int64_t J
     }
     // (w_aligned = 0: rows that are not 16-byte aligned, of a dense flat axis)
     if (variant == 0 && smallk_applies(R, S, I, J, K, w_aligned != 0)) return lt2exp_sweep_name(R, S, J, K, w_aligned != 0, buf, buf_bytes);
+    if (variant == 0 && cols_pays(R, S, I, J, K, true)) return cols_kernel_name(I, J, true, buf, buf_bytes);
     if (variant == 0 && rows_pays(R, S, I, J, K)) {
         const RowsPlan rp = rows_plan(R, S, I, J, K, w_aligned != 0);
         if (rp.ct) {

@@ -113,14 +113,18 @@ def _sweeps(R: int, S: int, I: int, J: int, K: int, w: torch.Tensor) -> bool:
     return sw[2] == 1 and J > 4 and I * J >= (1024 if K > 4 else 256)
 
 
+_IN_PLACE_KERNELS = ("trt::lt2exp_rows_kernel", "trt::lt2exp_cols_kernel")
+
+
 def _rows_first(R: int, S: int, I: int, J: int, K: int, w: torch.Tensor) -> bool:
-    """Would the library run this call on its kernel for few s per batch?  (Asked of the library
-    itself, host side only: the rule is a fitted one and lives there.)"""
+    """Would the library run this call on one of its kernels that read any w in place -- the one for
+    few s per batch, the one for few units with a lane per column?  (Asked of the library itself,
+    host side only: the rules are fitted ones and live there.)"""
     sw = w.stride()
     if sw[2] != 1:
         return False
     aligned = sw[0] % 4 == 0 and sw[1] % 4 == 0 and w.data_ptr() % 16 == 0
-    return _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, int(aligned)).startswith("trt::lt2exp_rows_kernel")
+    return _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, int(aligned)).startswith(_IN_PLACE_KERNELS)
 
 
 def _packs(I: int, J: int) -> bool:
@@ -213,7 +217,8 @@ def lt2exp(
     # packs them (measured R=86 S=482 I=193 K=145: J = 3 574 -> 244 us, J = 5..7 576-594 -> 453-480;
     # at a tenth of that work the copies cost more than they save).
     if (_variant == 0 and fp32 and J in (3, 5, 6, 7) and I * (4 if J == 3 else 8) >= 32
-            and (2 * R * S * I * 16 * K >= _PACK_PAD_MIN_FLOPS if _pad is None else _pad)):
+            and (2 * R * S * I * 16 * K >= _PACK_PAD_MIN_FLOPS if _pad is None else _pad)
+            and not (_pad is None and I <= 16 and K > 8 and _rows_first(R, S, I, J, K, w))):
         J4 = 4 if J == 3 else 8
         w = torch.nn.functional.pad(w.view(R, S, I, J), (0, J4 - J)).view(R, S, I * J4)
         b = torch.nn.functional.pad(b, (0, 0, 0, J4 - J), value=float("-inf"))
