@@ -251,6 +251,14 @@ def profile_pass(dev) -> int:
         lt2exp(wf, af, bf, _precision="fp32")
     torch.cuda.synchronize()
     del wf, af, bf
+    # few units over many batches: a lane per output column (405 MB of w, a, b and c)
+    wf = torch.rand(8192, 4, 4, 4, generator=gen).to(dev)
+    af = (torch.randn(8192, 4, 1024, generator=gen) * 10 - 30).to(dev)
+    bf = (torch.randn(8192, 4, 1024, generator=gen) * 10 - 30).to(dev)
+    for _ in range(3):
+        lt2exp(wf, af, bf, _precision="fp32")
+    torch.cuda.synchronize()
+    del wf, af, bf
     flat = b.view(-1)
     for _ in range(3):
         vmax(flat)
@@ -564,6 +572,27 @@ def main() -> int:
                 f"torch recipe {tor * 1e6:.2f} us")
             del wf, af, bf
         result["few_rows"] = fr
+
+        # ------------------------------------------------ lt2exp on layers of few units over many batches
+        # S = I = J = 4, 8 over 8192 batches: a lane per output column, the batch's weights as scalar
+        # operands.  Bytes: w, a, b and c once.
+        fu = {"protocol": "the same operands again and again, inside a HIP graph", "unit": "GB/s", "peak": PEAK_HBM_GBPS}
+        for (rr, uu, kk) in ((8192, 4, 1024), (8192, 8, 256), (8192, 8, 1024), (2048, 16, 512)):
+            ss = 1 if uu == 16 else uu
+            wf = torch.rand(rr, ss, uu, uu, generator=gen).to(dev)
+            af = (torch.randn(rr, uu, kk, generator=gen) * 10 - 30).to(dev)
+            bf = (torch.randn(rr, uu, kk, generator=gen) * 10 - 30).to(dev)
+            nbytes_f = 4 * (wf.numel() + af.numel() + bf.numel() + rr * ss * kk)
+            sec = graph_time(lambda: lt2exp(wf, af, bf, _precision="fp32"), prewarm_ms=PREWARM_MS / 2)
+            tor = graph_time(lambda: torch_lt2exp(wf, af, bf), calls=5, reps=5)
+            fu[f"R{rr}_S{ss}_I{uu}_J{uu}_K{kk}"] = {
+                "kernel": _lib.kernel_name("lt2exp", rr, ss, uu, uu, kk, _lib.MODE_AUTO, 0, 1), "bytes": nbytes_f,
+                "us": round(sec * 1e6, 2), "achieved": round(nbytes_f / sec / 1e9, 1),
+                "frac": round(nbytes_f / sec / 1e9 / PEAK_HBM_GBPS, 4), "torch_recipe_us": round(tor * 1e6, 2)}
+            log(f"lt2exp R={rr} S={ss} I=J={uu} K={kk}: {sec * 1e6:.2f} us ({nbytes_f / sec / 1e9:.0f} GB/s = "
+                f"{nbytes_f / sec / 1e9 / PEAK_HBM_GBPS * 100:.1f}% of 8 TB/s), torch recipe {tor * 1e6:.2f} us")
+            del wf, af, bf
+        result["few_units"] = fu
 
         # ------------------------------------------------ max reductions (HBM bound)
         # Two figures per reduction.  `us`, `achieved`, `frac`: 8 copies of the 64 MiB operand

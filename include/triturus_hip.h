@@ -118,8 +118,10 @@ int trt_lm2exp_variant_count(void);
  * batch (about a dozen at most), or little work altogether, and a dense flat axis of w
  * (16 bytes at a time where J is a multiple of 4 and the rows are 16-byte aligned, float by
  * float otherwise), variant 0 contracts j first, with the rows (s, i) of w on the rows of the
- * matrix instruction (likewise no cut and no workspace); trt_lt2exp_kernel_name tells which
- * kernel a call takes.
+ * matrix instruction (likewise no cut and no workspace).  With I and J of at most 16 over many
+ * batches (and more than 8 columns), variant 0 gives every output column a lane of its own and
+ * contracts on the vector ALU where that is the faster way (likewise).  trt_lt2exp_kernel_name
+ * tells which kernel a call takes.
  */
 int trt_lt2exp_f32(const float *w, const float *a, const float *b, float *c,
                    int64_t R, int64_t S, int64_t I, int64_t J, int64_t K,

@@ -431,6 +431,7 @@ static void launch_bf_shape(const Lt2BfArgs &args, int rt, int ks, bool vec, boo
 
 bool lt2exp_takes_sweep(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense);  // csrc/lt2exp.hip
 bool lt2exp_takes_rows(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_aligned, bool w_dense, double margin);  // csrc/lt2exp.hip
+bool lt2exp_takes_cols(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_dense, double margin);  // csrc/lt2exp.hip
 
 }  // namespace trt
 
@@ -520,6 +521,14 @@ extern "C" int trt_lt2exp_bf16(const float *w, const float *a, const float *b, f
     if (variant == 0 && K <= 8 &&
         lt2exp_takes_sweep(R, S, I, J, K, sw[2] == 1 && sw[0] % 4 == 0 && sw[1] % 4 == 0 &&
                                               (reinterpret_cast<uintptr_t>(w) & 15) == 0, sw[2] == 1))
+        return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
+
+    // Layers of few units over many batches (I, J <= 16): what the fp32 entry gives to its kernel
+    // with a lane per output column (csrc/lt2exp_cols.hpp) is bound by memory there, and these tiles
+    // pad such calls as the fp32 ones do (150 timed shapes that the fp32 rule takes: 1.36x and 1.27x
+    // behind it in the geometric mean with two and three pieces; handing all of them over leaves
+    // 1.8 % to the better choice per shape).
+    if (variant == 0 && lt2exp_takes_cols(R, S, I, J, K, sw[2] == 1, 0.0))
         return trt_lt2exp_f32(w, a, b, c, R, S, I, J, K, sw, sa, sb, sc, mode, 0, workspace, workspace_bytes, stream);
 
     // Few s per batch: these tiles, like the fp32 ones, put s on the rows of the MFMA and pad it to
