@@ -504,9 +504,24 @@ def test_lt2exp_few_units_over_many_batches_take_a_lane_per_column():
     assert name(8192, 4, 4, 4, 64) == "trt::lt2exp_cols_kernel<4, 4, true>"
     assert name(4096, 4, 16, 16, 256) == "trt::lt2exp_cols_kernel<16, 16, true>"
     assert name(1500, 3, 5, 7, 64) == "trt::lt2exp_cols_kernel<8, 8, false>"
-    assert name(2500, 7, 16, 1, 90) == "trt::lt2exp_cols_kernel<4, 16, false>"     # J = 1: i and j exchanged first
+    assert name(2500, 7, 16, 1, 90) == "trt::lt2exp_cols_kernel<1, 16, true>"      # J = 1: i and j exchanged first
     assert name(8192, 16, 16, 16, 256).startswith("trt::lt2exp_kernel<")            # 4096 FMAs per lane: the MFMA tiles
     assert name(16, 8, 8, 8, 64).startswith("trt::lt2exp_kernel<")                  # a call of a few microseconds either way
     assert name(8192, 8, 8, 17, 256).startswith("trt::lt2exp_kernel<")              # J beyond 16
     assert name(8192, 8, 8, 8, 8).startswith("trt::lt2exp_rows_kernel<")            # 8 columns: not asked
     assert name(8192, 8, 8, 8, 256, variant=3).startswith("trt::lt2exp_kernel<")
+
+
+def test_lm2exp_contractions_of_at_most_16_terms_take_a_lane_per_column():
+    """Host-side rule of lm2exp for J <= 16 over many batches: the lane-per-column kernel of lt2exp
+    (lt2exp_cols_kernel<1, J padded to 4, 8 or 16, rows of exactly that many dense values>)."""
+    name = lambda *sh, variant=0, splits=0: _lib.kernel_name("lm2exp", *sh, variant, splits, 1)
+    assert name(8192, 4, 4, 1024) == "trt::lt2exp_cols_kernel<1, 4, true>"
+    assert name(8192, 8, 8, 1024) == "trt::lt2exp_cols_kernel<1, 8, true>"
+    assert name(4096, 64, 8, 256) == "trt::lt2exp_cols_kernel<1, 8, true>"
+    assert name(3000, 5, 7, 100) == "trt::lt2exp_cols_kernel<1, 8, false>"
+    assert name(64, 8, 8, 64).startswith("trt::lm2exp_kernel<")            # a call of a few microseconds either way
+    assert name(8192, 8, 17, 1024).startswith("trt::lm2exp_kernel<")       # J beyond 16
+    assert name(8192, 8, 8, 8).startswith("trt::lm2exp_kernel<")           # 8 columns: not asked
+    assert name(8192, 8, 8, 1024, variant=3).startswith("trt::lm2exp")     # forced tiles
+    assert name(8192, 8, 8, 1024, splits=2).startswith("trt::lm2exp")      # a forced cut

@@ -682,3 +682,43 @@ def test_at_most_4_columns_under_a_long_contraction_take_the_sweep(dev, shape):
     # a transposed a is not swept (its rows are not dense): same result from the paired tiles
     at = a.transpose(1, 2).contiguous().transpose(1, 2).to(dev)
     assert torch.allclose(out, lm2exp(at, b.to(dev)), rtol=1e-5, atol=1e-5)
+
+
+LM_COLS_SHAPES = [(2000, 4, 4, 300), (1500, 8, 8, 1024), (900, 16, 16, 256), (4000, 64, 8, 130), (3000, 1, 16, 64),   # rows of 4, 8, 16
+                  (3000, 5, 7, 100), (9000, 33, 3, 65), (4000, 9, 1, 200), (8000, 2, 11, 300)]                        # any J up to 16
+
+
+@pytest.mark.parametrize("shape", LM_COLS_SHAPES)
+def test_contractions_of_at_most_16_terms_over_many_batches_take_a_lane_per_column(dev, shape):
+    """J <= 16 over many batches: the lane-per-column kernel of csrc/lt2exp_cols.hpp with the rows of
+    a as the weights, against the float64 oracle (zero rows, -inf and NaN columns) and against
+    lm2exp's own tiles on the same operands; a strided a and b are read in place."""
+    R, I, J, K = shape
+    assert _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1).startswith("trt::lt2exp_cols_kernel<1, ")
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(R, I, J, generator=g)
+    a[:, I // 2] = 0.0
+    b = 6 * torch.randn(R, J, K, generator=g) - 20
+    b[0, :, 0] = NINF
+    b[R - 1, J // 3, K - 1] = NINF
+    ref = oracle64.lm2exp64(a, b)
+    out = lm2exp(a.to(dev), b.to(dev))
+    r = oracle64.compare(out, ref)
+    assert r["ok"], (shape, r)
+    assert torch.isneginf(out[0, :, 0]).all() and torch.isneginf(out[:, I // 2]).all()
+    assert torch.equal(out, lm2exp(a.to(dev), b.to(dev)))
+    assert torch.allclose(out, lm2exp(a.to(dev), b.to(dev), _variant=12), rtol=1e-5, atol=1e-5)
+    bn = b.clone()
+    bn[R // 2, J // 2, K // 2] = float("nan")
+    outn = lm2exp(a.to(dev), bn.to(dev))
+    assert torch.isnan(outn[R // 2, :, K // 2]).all()
+    mask = torch.ones_like(outn, dtype=torch.bool)
+    mask[R // 2, :, K // 2] = False
+    assert torch.equal(outn[mask], out[mask])
+    at = a.transpose(1, 2).contiguous().transpose(1, 2).to(dev)          # J-major a
+    bs = torch.nn.functional.pad(b, (0, 5)).to(dev)[:, :, :K]            # rows of b wider than K
+    r = oracle64.compare(lm2exp(at, bs), ref)
+    assert r["ok"], (shape, "strided", r)
+    for prec in ("bf16x3", "bf16x6"):
+        r = oracle64.compare(lm2exp(a.to(dev), b.to(dev), _precision=prec), ref, rtol=1e-4, atol=5e-5)
+        assert r["ok"], (shape, prec, r)

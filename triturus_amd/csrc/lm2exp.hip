@@ -915,6 +915,11 @@ bool lm2exp_takes_sweep(int64_t R, int64_t I, int64_t J, int64_t K, bool a_align
 int lm2exp_sweep(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
                  const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], hipStream_t stream);
 int lt2exp_sweep_name(int64_t R, int64_t S, int64_t J, int64_t K, bool w_aligned, char *buf, size_t buf_bytes);
+// csrc/lt2exp.hip: the lane-per-column kernel of csrc/lt2exp_cols.hpp with the rows of a as the weights
+bool lm2exp_takes_cols(int64_t R, int64_t I, int64_t J, int64_t K, bool a_dense, double margin);
+int lm2exp_cols(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
+                const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], hipStream_t stream);
+int lm2exp_cols_name(int64_t J, bool a_dense, char *buf, size_t buf_bytes);
 
 }  // namespace trt
 
@@ -949,6 +954,9 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         lm2exp_takes_sweep(R, I, J, K, sa[2] == 1 && sa[0] % 4 == 0 && sa[1] % 4 == 0 &&
                                            (reinterpret_cast<uintptr_t>(a) & 15) == 0))
         return lm2exp_sweep(a, b, c, R, I, J, K, sa, sb, sc, static_cast<hipStream_t>(stream));
+    // a contraction of at most 16 terms over many batches: a lane per output column
+    if (variant == 0 && splits <= 1 && lm2exp_takes_cols(R, I, J, K, sa[2] == 1, 0.0))
+        return lm2exp_cols(a, b, c, R, I, J, K, sa, sb, sc, static_cast<hipStream_t>(stream));
     Lm2Plan pl = make_plan(R, I, J, K, variant, splits);
     // a trailing stride of a other than 1 (a transposed or strided view): only the
     // paired-wavefront kernel reads such a tile; a call that would take another kernel takes
@@ -1044,6 +1052,7 @@ extern "C" int trt_lm2exp_kernel_name(int64_t R, int64_t I, int64_t J, int64_t K
     if (variant < 0 || variant > kNumVariants || splits < 0) return TRT_E_INVALID;
     if (variant == 0 && splits <= 1 && lm2exp_takes_sweep(R, I, J, K, a_vec != 0))
         return lt2exp_sweep_name(R, I, J, K, true, buf, buf_bytes);
+    if (variant == 0 && splits <= 1 && lm2exp_takes_cols(R, I, J, K, true, 0.0)) return lm2exp_cols_name(J, true, buf, buf_bytes);
     const Lm2Variant &vr = kVariants[make_plan(R, I, J, K, variant, splits).variant];
     int n;
     if (vr.mode == kPair)

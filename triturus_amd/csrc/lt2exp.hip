@@ -891,6 +891,27 @@ int lm2exp_sweep(const float *a, const float *b, float *c, int64_t R, int64_t I,
     const int64_t none[3] = {0, 0, 0};
     return launch_lt2exp_smallk(a, nullptr, b, c, R, I, 1, J, K, sa, none, sb, sc, true, stream);
 }
+// for trt_lm2exp_f32: lm2exp with J <= 16 is the lane-per-column kernel of csrc/lt2exp_cols.hpp with
+// the rows of a as the weights (S = I, a contracted plane of 1 x J, no factors on the other side)
+// Taken by the sign of a linear score in log2 units fitted to 350 timed shapes (J = 1..16, I = 1..256,
+// K = 9..2048, up to 100 000 batches) against lm2exp's own tiles, which pad i to 32 rows and j to a
+// chunk of 32: - 0.46 per doubling of I and - 0.48 per doubling of J (a lane's FMAs), - 0.12 per
+// doubling of K, + 0.81 for rows of exactly 4, 8 or 16 dense values (one scalar load per row),
+// + 0.2 per doubling of the call's work.  1.9 % behind the faster choice per shape (never taking it
+// 34 %, always 41 %): R=8192, I=J=4, K=1024 190 -> 60 us, I=J=8 189 -> 110.
+bool lm2exp_takes_cols(int64_t R, int64_t I, int64_t J, int64_t K, bool a_dense, double margin) {
+    if (J > 16 || K <= 8) return false;
+    const bool exact = (J == 4 || J == 8 || J == 16) && a_dense;
+    const double work = 2.0 * (double)R * (double)I * (double)J * (double)K;
+    return -1.24 - 0.46 * std::log2((double)I) - 0.475 * std::log2((double)J) - 0.12 * std::log2((double)K) +
+               (exact ? 0.81 : 0.0) + 0.196 * std::log2(work) > margin;
+}
+int lm2exp_cols(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
+                const int64_t sa[3], const int64_t sb[3], const int64_t sc[3], hipStream_t stream) {
+    const int64_t none[3] = {0, 0, 0};
+    return launch_lt2exp_cols(a, nullptr, b, c, R, I, 1, J, K, sa, none, sb, sc, stream);
+}
+int lm2exp_cols_name(int64_t J, bool a_dense, char *buf, size_t buf_bytes) { return cols_kernel_name(1, J, a_dense, buf, buf_bytes); }
 int lt2exp_sweep_name(int64_t R, int64_t S, int64_t J, int64_t K, bool w_aligned, char *buf, size_t buf_bytes) {
     const int n = snprintf(buf, buf_bytes, "trt::lt2exp_smallk_kernel<%d, %d, %s>", small_kc(K), smallk_wpr(R, S),
                            smallk_anyj(J, w_aligned) ? "true" : "false");

@@ -31,7 +31,7 @@ struct Lt2ColsArgs {
 
 constexpr int kColsThreads = 256;
 
-// IMAX, JMAX: I and J rounded up to 4, 8 or 16 (register arrays; the rows past I and J hold factors
+// IMAX, JMAX: I and J rounded up to 4, 8 or 16 -- I = 1 stays 1 -- (register arrays; the rows past I and J hold factors
 // of zero and their weights are never read).  EXACT: I = IMAX, J = JMAX and a dense flat axis of w:
 // the I * J weights of an s are one run of known length, which the compiler fetches 16 to a scalar
 // load instead of one by one.
@@ -53,11 +53,12 @@ static __global__ __launch_bounds__(kColsThreads) void lt2exp_cols_kernel(const 
     const bool live = k < p.K;
     const int kc = live ? k : p.K - 1;  // (lanes past K compute a copy of the last column and store nothing)
 
-    const float *ak = a_ + (int64_t)r * p.sa0 + (int64_t)kc * p.sa2;
+    // (no a: the lm2exp entry -- a contracted plane of 1 x J, a factor of one)
+    const float *ak = a_ ? a_ + (int64_t)r * p.sa0 + (int64_t)kc * p.sa2 : nullptr;
     const float *bk = b_ + (int64_t)r * p.sb0 + (int64_t)kc * p.sb2;
     float ea[IMAX], eb[JMAX];
 #pragma unroll
-    for (int i = 0; i < IMAX; ++i) ea[i] = i < p.I ? ak[(int64_t)i * p.sa1] : -__builtin_inff();
+    for (int i = 0; i < IMAX; ++i) ea[i] = ak && i < p.I ? ak[(int64_t)i * p.sa1] : -__builtin_inff();
 #pragma unroll
     for (int j = 0; j < JMAX; ++j) eb[j] = j < p.J ? bk[(int64_t)j * p.sb1] : -__builtin_inff();
     // (a NaN need not survive the maxima: exp(NaN - m) is NaN for any m and poisons the column)
@@ -66,10 +67,10 @@ static __global__ __launch_bounds__(kColsThreads) void lt2exp_cols_kernel(const 
     for (int i = 0; i < IMAX; ++i) ma = __builtin_fmaxf(ma, ea[i]);
 #pragma unroll
     for (int j = 0; j < JMAX; ++j) mb = __builtin_fmaxf(mb, eb[j]);
-    ma = clamp_shift(ma);
+    ma = ak ? clamp_shift(ma) : 0.f;
     mb = clamp_shift(mb);
 #pragma unroll
-    for (int i = 0; i < IMAX; ++i) ea[i] = i < p.I ? exp_shifted(ea[i] - ma) : 0.f;
+    for (int i = 0; i < IMAX; ++i) ea[i] = i < p.I ? (ak ? exp_shifted(ea[i] - ma) : 1.f) : 0.f;
 #pragma unroll
     for (int j = 0; j < JMAX; ++j) eb[j] = j < p.J ? exp_shifted(eb[j] - mb) : 0.f;
     const float shift = ma + mb;
@@ -116,6 +117,7 @@ static __global__ __launch_bounds__(kColsThreads) void lt2exp_cols_kernel(const 
 // ---- host side
 
 static inline int cols_pad(int64_t n) { return n <= 4 ? 4 : (n <= 8 ? 8 : 16); }
+static inline int cols_pad_i(int64_t n) { return n == 1 ? 1 : cols_pad(n); }
 
 static inline bool cols_applies(int64_t I, int64_t J, int64_t K) { return I <= 16 && J <= 16 && K > 8; }
 
@@ -131,7 +133,7 @@ static inline bool cols_applies(int64_t I, int64_t J, int64_t K) { return I <= 1
 // over the fit's shapes; never taking it 25 %, always taking it 98 %).  Outputs of at most 8
 // columns are not asked (a wavefront would hold 8 live lanes; the sweep takes most of them).
 static inline double cols_score(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K, bool w_dense) {
-    const int im = cols_pad(I), jm = cols_pad(J);
+    const int im = cols_pad_i(I), jm = cols_pad(J);
     const bool exact = im == I && jm == J && w_dense;
     const double fmas = (double)S * (double)(exact ? im : I) * (double)jm;
     const double work = 2.0 * (double)R * (double)S * (double)I * (double)J * (double)K;
@@ -142,7 +144,7 @@ static inline bool cols_pays(int64_t R, int64_t S, int64_t I, int64_t J, int64_t
 }
 
 static inline int cols_kernel_name(int64_t I, int64_t J, bool w_dense, char *buf, size_t buf_bytes) {
-    const int im = cols_pad(I), jm = cols_pad(J);
+    const int im = cols_pad_i(I), jm = cols_pad(J);
     const int n = snprintf(buf, buf_bytes, "trt::lt2exp_cols_kernel<%d, %d, %s>", im, jm,
                            im == I && jm == J && w_dense ? "true" : "false");
     return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
@@ -162,7 +164,7 @@ static int launch_lt2exp_cols(const float *w, const float *a, const float *b, fl
     args.total_waves = R * args.k_waves;
     const int64_t grid = ceil_div(args.total_waves, kColsThreads / kWave);
     if (grid >= ((int64_t)1 << 31)) return TRT_E_RANGE;
-    const int im = cols_pad(I), jm = cols_pad(J);
+    const int im = cols_pad_i(I), jm = cols_pad(J);
     const bool exact = im == I && jm == J && sw[2] == 1;
 #define TRT_COLS_LAUNCH(IM_, JM_)                                                                                   \
     do {                                                                                                            \
@@ -171,7 +173,11 @@ static int launch_lt2exp_cols(const float *w, const float *a, const float *b, fl
         else                                                                                                        \
             hipLaunchKernelGGL((lt2exp_cols_kernel<IM_, JM_, false>), dim3((unsigned)grid), dim3(kColsThreads), 0, stream, args, w, a, b, c); \
     } while (0)
-    if (im == 4) {
+    if (im == 1) {
+        if (jm == 4) TRT_COLS_LAUNCH(1, 4);
+        else if (jm == 8) TRT_COLS_LAUNCH(1, 8);
+        else TRT_COLS_LAUNCH(1, 16);
+    } else if (im == 4) {
         if (jm == 4) TRT_COLS_LAUNCH(4, 4);
         else if (jm == 8) TRT_COLS_LAUNCH(4, 8);
         else TRT_COLS_LAUNCH(4, 16);
