@@ -592,6 +592,21 @@ def main() -> int:
             log(f"lt2exp R={rr} S={ss} I=J={uu} K={kk}: {sec * 1e6:.2f} us ({nbytes_f / sec / 1e9:.0f} GB/s = "
                 f"{nbytes_f / sec / 1e9 / PEAK_HBM_GBPS * 100:.1f}% of 8 TB/s), torch recipe {tor * 1e6:.2f} us")
             del wf, af, bf
+        from benchmarks.torch_recipes import torch_lm2exp
+
+        for (rr, uu, kk) in ((8192, 4, 1024), (8192, 8, 1024)):   # lm2exp: the same kernel, the rows of a as the weights
+            am = torch.rand(rr, uu, uu, generator=gen).to(dev)
+            bm = (torch.randn(rr, uu, kk, generator=gen) * 10 - 30).to(dev)
+            nbytes_f = 4 * (am.numel() + bm.numel() + rr * uu * kk)
+            sec = graph_time(lambda: lm2exp(am, bm, _precision="fp32"), prewarm_ms=PREWARM_MS / 2)
+            tor = graph_time(lambda: torch_lm2exp(am, bm), calls=5, reps=5)
+            fu[f"lm2exp_R{rr}_I{uu}_J{uu}_K{kk}"] = {
+                "kernel": _lib.kernel_name("lm2exp", rr, uu, uu, kk, 0, 0, 1), "bytes": nbytes_f,
+                "us": round(sec * 1e6, 2), "achieved": round(nbytes_f / sec / 1e9, 1),
+                "frac": round(nbytes_f / sec / 1e9 / PEAK_HBM_GBPS, 4), "torch_recipe_us": round(tor * 1e6, 2)}
+            log(f"lm2exp R={rr} I=J={uu} K={kk}: {sec * 1e6:.2f} us ({nbytes_f / sec / 1e9:.0f} GB/s = "
+                f"{nbytes_f / sec / 1e9 / PEAK_HBM_GBPS * 100:.1f}% of 8 TB/s), torch recipe {tor * 1e6:.2f} us")
+            del am, bm
         result["few_units"] = fu
 
         # ------------------------------------------------ max reductions (HBM bound)

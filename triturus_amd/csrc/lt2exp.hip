@@ -898,7 +898,7 @@ int lm2exp_sweep(const float *a, const float *b, float *c, int64_t R, int64_t I,
 // chunk of 32: - 0.46 per doubling of I and - 0.48 per doubling of J (a lane's FMAs), - 0.12 per
 // doubling of K, + 0.81 for rows of exactly 4, 8 or 16 dense values (one scalar load per row),
 // + 0.2 per doubling of the call's work.  1.9 % behind the faster choice per shape (never taking it
-// 34 %, always 41 %): R=8192, I=J=4, K=1024 190 -> 60 us, I=J=8 189 -> 110.
+// 34 %, always 41 %): R=8192, I=J=4, K=1024 190 -> 42 us, I=J=8 189 -> 101.
 bool lm2exp_takes_cols(int64_t R, int64_t I, int64_t J, int64_t K, bool a_dense, double margin) {
     if (J > 16 || K <= 8) return false;
     const bool exact = (J == 4 || J == 8 || J == 16) && a_dense;
