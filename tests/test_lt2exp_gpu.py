@@ -816,3 +816,24 @@ def test_a_lane_per_column_reads_strided_a_and_b_and_sliced_w_in_place(dev):
         r = oracle64.compare(lt2exp(w, a, b, _precision=prec), oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=64),
                              rtol=1e-4, atol=5e-5)
         assert r["ok"], (prec, r)
+
+
+@pytest.mark.parametrize("offset", [1, 2, 3, 5])
+@pytest.mark.parametrize("shape", [(600, 3, 8, 8, 100), (500, 2, 16, 16, 70), (900, 5, 4, 4, 200)])
+def test_a_lane_per_column_on_a_w_that_starts_off_a_16_byte_boundary(dev, shape, offset):
+    """The exact-size build fetches 16 weights to a scalar load: from any 4-byte boundary (a view into
+    a larger buffer of NaNs)."""
+    R, S, I, J, K = shape
+    g = torch.Generator().manual_seed(sum(shape) + offset)
+    n = R * S * I * J
+    buf = torch.full((n + 8,), float("nan"))
+    buf[offset:offset + n] = torch.rand(n, generator=g)
+    w = buf.to(dev)[offset:offset + n].view(R, S, I, J)
+    assert w.data_ptr() % 64 == 4 * offset
+    a = (3 * torch.randn(R, I, K, generator=g)).to(dev)
+    b = (3 * torch.randn(R, J, K, generator=g)).to(dev)
+    assert _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 0).endswith("true>")
+    assert "cols_kernel" in _lib.kernel_name("lt2exp", R, S, I, J, K, 0, 0, 0)
+    out = lt2exp(w, a, b)
+    r = oracle64.compare(out, oracle64.lt2exp64(w.cpu(), a.cpu(), b.cpu(), batch_chunk=64))
+    assert r["ok"], (shape, offset, r)
