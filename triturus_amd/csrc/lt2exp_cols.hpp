@@ -93,7 +93,10 @@ static __global__ __launch_bounds__(kColsThreads) void lt2exp_cols_kernel(const 
     } else {
         // any I, J and flat stride: i is a real loop (unrolled over i as well, the offsets of all
         // I * J weights are loop invariants that overflow the scalar registers), so the factors of
-        // a wait in LDS, a column per thread
+        // a wait in LDS, a column per thread.  (Blocks of 2-4 rows without a branch inside -- rows and
+        // columns past I and J read again from the last ones under weights selected to zero, so that
+        // a block's scalar loads go out together -- were twice as slow: 152 -> 266 us on R=8192,
+        // S=I=J=6, K=512.)
         __shared__ float ea_lds[IMAX][kColsThreads];
 #pragma unroll
         for (int i = 0; i < IMAX; ++i) ea_lds[i][threadIdx.x] = ea[i];  // (read back by the same thread only)
@@ -104,9 +107,23 @@ static __global__ __launch_bounds__(kColsThreads) void lt2exp_cols_kernel(const 
 #pragma unroll 1
             for (int i = 0; i < p.I; ++i, wi += row) {
                 float t = 0.f;
+                if (p.sw2 == 1) {  // (wave-uniform) dense rows: four weights to a scalar load, the tail one by one
 #pragma unroll
-                for (int j = 0; j < JMAX; ++j)
-                    if (j < p.J) t = __builtin_fmaf(wi[(int64_t)j * p.sw2], eb[j], t);
+                    for (int jq = 0; jq < JMAX / 4; ++jq) {
+                        if (4 * jq + 4 <= p.J) {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) t = __builtin_fmaf(wi[4 * jq + e], eb[4 * jq + e], t);
+                        } else {
+#pragma unroll
+                            for (int e = 0; e < 4; ++e)
+                                if (4 * jq + e < p.J) t = __builtin_fmaf(wi[4 * jq + e], eb[4 * jq + e], t);
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int j = 0; j < JMAX; ++j)
+                        if (j < p.J) t = __builtin_fmaf(wi[(int64_t)j * p.sw2], eb[j], t);
+                }
                 sum = __builtin_fmaf(ea_lds[i][threadIdx.x], t, sum);
             }
             if (live) ck[(int64_t)s * p.sc1] = log_plus(sum, shift);
