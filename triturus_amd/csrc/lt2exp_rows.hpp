@@ -347,15 +347,18 @@ static inline RowsPlan rows_plan(int64_t R, int64_t S, int64_t I, int64_t J, int
 //   - per halving of J below 32 (the epilogue of a tile, 16 FMAs and 4 LDS reads per column
 //     block, against J / 2 MFMAs),
 // and, from 13 values of s on, where the padding of s no longer decides, - 0.12 per doubling of
-// the work: the s-row tiles run large grids at 100-125 TFLOP/s, this kernel at 60-95, but a call
-// of less than about a GFLOP is faster here whatever S is (R=1, S=I=J=K=128: 30 -> 15 us).
-// Such calls need the estimate to favour this kernel by 7 % (it costs 0.4 %, and keeps calls of
-// a few GFLOP under thousands of columns, where the two run level, on the tiles tuned for them).
-// Taking the kernel by this rule costs 2.5 % over the faster of the two per shape (geometric mean
-// over the fit's shapes; never taking it 68 % -- 154 % over the shapes with S <= 12 --, always
-// taking it 14 %).  The element-load build is served by the same rule (the s-row tiles stage
-// such rows element by element too).  Outputs of at most 8 columns have been handed to the sweep
-// before this is asked.
+// the work and + 0.25 per halving of K below 64: the s-row tiles run large grids at 100-125
+// TFLOP/s, this kernel at 60-95, but a call of less than about a GFLOP is faster here whatever S
+// is (R=1, S=I=J=K=128: 30 -> 15 us), and under 64 columns most of the four wavefronts that the
+// s-row tiles set side by side over 128 columns stand idle (R=2048, S=16, I=J=64, K=32: 509 ->
+// 127 us; S=32, I=J=32, K=32: 137 -> 78).  Such calls need the estimate to favour this kernel by
+// 10 % (which keeps calls of a few GFLOP under thousands of columns, where the two run level, on
+// the tiles tuned for them).
+// Taking the kernel by this rule costs 2.5-3 % over the faster of the two per shape (geometric
+// mean over the fit's shapes; never taking it 68 % -- 154 % over the shapes with S <= 12, 23 % over
+// 400 shapes with S = 13..128 and K up to 512 --, always taking it 14 %).  The element-load build
+// is served by the same rule (the s-row tiles stage such rows element by element too).  Outputs
+// of at most 8 columns have been handed to the sweep before this is asked.
 static inline double rows_score(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
     const double ws = std::log2(32.0 * (double)ceil_div(S, 32) / (double)S);
     const double wi = std::log2(32.0 * (double)ceil_div(I, 32) / (double)I);
@@ -363,7 +366,7 @@ static inline double rows_score(int64_t R, int64_t S, int64_t I, int64_t J, int6
     const double short_j = lj < 5.0 ? 5.0 - lj : 0.0;
     if (S <= 12) return 1.41 + 0.52 * ws - 0.65 * wi - 0.18 * lk - 0.22 * short_j;
     const double lw = std::log2(2.0 * (double)R * (double)S * (double)I * (double)J * (double)K);
-    return 3.77 + 0.36 * ws - 0.65 * wi - 0.27 * short_j - 0.12 * lw - 0.1;
+    return 3.62 + 0.36 * ws - 0.65 * wi - 0.27 * short_j - 0.12 * lw + 0.25 * (lk < 6.0 ? 6.0 - lk : 0.0);
 }
 static inline bool rows_pays(int64_t R, int64_t S, int64_t I, int64_t J, int64_t K) {
     return rows_score(R, S, I, J, K) > 0.0;
