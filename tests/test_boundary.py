@@ -420,7 +420,8 @@ def test_lm2exp_outputs_of_at_most_64_columns_take_the_narrow_tiles():
     assert name(101, 1510, 48, 48) == "trt::lm2exp_pair_kernel<2, 2, 2, 0>"           # 2424 tiles of 64 rows
     assert name(14, 2464, 2688, 48) == "trt::lm2exp_pair_kernel<2, 2, 2, 0>"          # 546, a long contraction
     assert name(203, 267, 2788, 63) == "trt::lm2exp_kernel<1, 1, 2, 2, 4, true, 1>"   # 128 rows would pad 267 to 384
-    assert name(40, 30, 500, 20) == "trt::lm2exp_kernel<1, 1, 1, 4, 4, true, 1>"      # I <= 32: the 32 x 128 tile
+    # I <= 32: the 32 x 128 tile (here with rows of a that are not 16-byte aligned; aligned ones: the next test)
+    assert _lib.kernel_name("lm2exp", 40, 30, 500, 20, 0, 0, 0) == "trt::lm2exp_kernel<1, 1, 1, 4, 4, false, 1>"
 
 
 def test_paired_wavefront_groups_take_grids_of_at_most_two_tiles_per_cu():
@@ -525,3 +526,21 @@ def test_lm2exp_contractions_of_at_most_16_terms_take_a_lane_per_column():
     assert name(8192, 8, 8, 8).startswith("trt::lm2exp_kernel<")           # 8 columns: not asked
     assert name(8192, 8, 8, 1024, variant=3).startswith("trt::lm2exp")     # forced tiles
     assert name(8192, 8, 8, 1024, splits=2).startswith("trt::lm2exp")      # a forced cut
+
+
+def test_lm2exp_narrow_outputs_of_few_rows_cut_the_contraction_over_the_wavefronts():
+    """Host-side rule of lm2exp for at most 64 columns under few rows per batch: lm2exp_jsplit_kernel<column
+    blocks of 32> gives a workgroup one tile and each wavefront a quarter of J."""
+    name = lambda *sh, variant=0, splits=0, aligned=1: _lib.kernel_name("lm2exp", *sh, variant, splits, aligned)
+    assert name(8192, 1, 256, 16) == "trt::lm2exp_jsplit_kernel<1>"
+    assert name(4438, 16, 256, 16) == "trt::lm2exp_jsplit_kernel<1>"
+    assert name(2000, 40, 128, 48) == "trt::lm2exp_jsplit_kernel<2>"
+    assert name(40, 30, 500, 20) == "trt::lm2exp_jsplit_kernel<1>"
+    assert name(508, 16, 256, 256).startswith("trt::lm2exp_kernel<")        # more than 64 columns
+    assert name(4000, 8, 66, 20).startswith("trt::lm2exp_kernel<")          # J not a multiple of 4
+    assert name(8192, 1, 256, 16, aligned=0).startswith("trt::lm2exp_kernel<")
+    assert name(30, 283, 2788, 10).startswith("trt::lm2exp_kernel<")        # nine row tiles per batch on a small grid
+    assert name(8192, 1, 256, 16, variant=3).startswith("trt::lm2exp")      # forced tiles
+    assert name(8192, 1, 256, 16, splits=2).startswith("trt::lm2exp_")      # a forced cut over workgroups
+    assert "jsplit" not in name(8192, 1, 256, 16, splits=2)
+    assert name(8192, 8, 8, 16).startswith("trt::lt2exp_cols_kernel<")      # short contractions: a lane per column

@@ -722,3 +722,45 @@ def test_contractions_of_at_most_16_terms_over_many_batches_take_a_lane_per_colu
     for prec in ("bf16x3", "bf16x6"):
         r = oracle64.compare(lm2exp(a.to(dev), b.to(dev), _precision=prec), ref, rtol=1e-4, atol=5e-5)
         assert r["ok"], (shape, prec, r)
+
+
+JSPLIT_SHAPES = [(3000, 1, 256, 16), (900, 16, 256, 16), (700, 8, 64, 32), (500, 40, 128, 48), (3000, 33, 100, 64),   # one or two column blocks
+                 (60, 4, 4096, 32), (40, 30, 500, 20), (1200, 5, 36, 9), (800, 32, 44, 33), (300, 7, 1000, 40)]        # long and ragged contractions, small grids
+
+
+@pytest.mark.parametrize("shape", JSPLIT_SHAPES)
+def test_narrow_outputs_of_few_rows_cut_the_contraction_over_the_wavefronts(dev, shape):
+    """At most 64 columns under few rows per batch: lm2exp_jsplit_kernel (csrc/lm2exp_jsplit.hpp) against
+    the float64 oracle (zero rows, -inf and NaN columns, a strided b) and against lm2exp's own tiles."""
+    R, I, J, K = shape
+    assert _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1).startswith("trt::lm2exp_jsplit_kernel<")
+    g = torch.Generator().manual_seed(sum(shape))
+    a = torch.rand(R, I, J, generator=g)
+    a[:, I // 2] = 0.0
+    b = 6 * torch.randn(R, J, K, generator=g) - 20
+    b[0, :, 0] = NINF
+    b[R - 1, J // 3, K - 1] = NINF
+    ref = oracle64.lm2exp64(a, b)
+    out = lm2exp(a.to(dev), b.to(dev))
+    r = oracle64.compare(out, ref)
+    assert r["ok"], (shape, r)
+    assert torch.isneginf(out[0, :, 0]).all() and torch.isneginf(out[:, I // 2]).all()
+    assert torch.equal(out, lm2exp(a.to(dev), b.to(dev)))                      # fixed order of the partial tiles
+    assert torch.allclose(out, lm2exp(a.to(dev), b.to(dev), _variant=12), rtol=1e-5, atol=1e-5)
+    bn = b.clone()
+    bn[R // 2, J // 2, K // 2] = float("nan")
+    outn = lm2exp(a.to(dev), bn.to(dev))
+    assert torch.isnan(outn[R // 2, :, K // 2]).all()
+    mask = torch.ones_like(outn, dtype=torch.bool)
+    mask[R // 2, :, K // 2] = False
+    assert torch.equal(outn[mask], out[mask])
+    bs = torch.nn.functional.pad(b, (0, 5)).to(dev)[:, :, :K]                  # rows of b wider than K
+    bt = b.transpose(1, 2).contiguous().transpose(1, 2).to(dev)                # K-major b
+    for bv in (bs, bt):
+        r = oracle64.compare(lm2exp(a.to(dev), bv), ref)
+        assert r["ok"], (shape, "strided b", r)
+    ai = a.clone()                                                             # an infinite weight in the row after
+    if I > 1:
+        ai[:, 1, 0] = float("inf")
+        outi = lm2exp(ai.to(dev), b.to(dev))
+        assert torch.equal(outi[:, 0], out[:, 0])

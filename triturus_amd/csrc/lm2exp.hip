@@ -56,6 +56,7 @@ constexpr int kPair = 4;      // lm2exp_pair_kernel: exact column maximum first,
 
 }  // namespace trt
 
+#include "lm2exp_jsplit.hpp"
 #include "lm2exp_pair.hpp"
 
 namespace trt {
@@ -954,6 +955,11 @@ extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t 
         lm2exp_takes_sweep(R, I, J, K, sa[2] == 1 && sa[0] % 4 == 0 && sa[1] % 4 == 0 &&
                                            (reinterpret_cast<uintptr_t>(a) & 15) == 0))
         return lm2exp_sweep(a, b, c, R, I, J, K, sa, sb, sc, static_cast<hipStream_t>(stream));
+    // at most 64 columns under few rows per batch: one tile per batch, its contraction cut over the
+    // wavefronts (csrc/lm2exp_jsplit.hpp)
+    if (variant == 0 && splits <= 1 &&
+        jsplit_pays(R, I, J, K, sa[2] == 1 && sa[0] % 4 == 0 && sa[1] % 4 == 0 && (reinterpret_cast<uintptr_t>(a) & 15) == 0))
+        return launch_lm2exp_jsplit(a, b, c, R, I, J, K, sa, sb, sc, static_cast<hipStream_t>(stream));
     // a contraction of at most 16 terms over many batches: a lane per output column
     if (variant == 0 && splits <= 1 && lm2exp_takes_cols(R, I, J, K, sa[2] == 1, 0.0))
         return lm2exp_cols(a, b, c, R, I, J, K, sa, sb, sc, static_cast<hipStream_t>(stream));
@@ -1052,6 +1058,10 @@ extern "C" int trt_lm2exp_kernel_name(int64_t R, int64_t I, int64_t J, int64_t K
     if (variant < 0 || variant > kNumVariants || splits < 0) return TRT_E_INVALID;
     if (variant == 0 && splits <= 1 && lm2exp_takes_sweep(R, I, J, K, a_vec != 0))
         return lt2exp_sweep_name(R, I, J, K, true, buf, buf_bytes);
+    if (variant == 0 && splits <= 1 && jsplit_pays(R, I, J, K, a_vec != 0)) {
+        const int n = snprintf(buf, buf_bytes, "trt::lm2exp_jsplit_kernel<%d>", K > 32 ? 2 : 1);
+        return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
+    }
     if (variant == 0 && splits <= 1 && lm2exp_takes_cols(R, I, J, K, true, 0.0)) return lm2exp_cols_name(J, true, buf, buf_bytes);
     const Lm2Variant &vr = kVariants[make_plan(R, I, J, K, variant, splits).variant];
     int n;
