@@ -609,6 +609,25 @@ def main() -> int:
             del am, bm
         result["few_units"] = fu
 
+        # ------------------------------------------------ lm2exp on narrow outputs of few rows per batch
+        # At most 64 columns and 32 rows: one tile per batch, its contraction cut over the four
+        # wavefronts.  Bytes: a, b and c once (b outweighs the rest).
+        nw = {"protocol": "the same operands again and again, inside a HIP graph", "unit": "GB/s", "peak": PEAK_HBM_GBPS}
+        for (rr, ii, jj, kk) in ((8192, 1, 256, 16), (4096, 16, 256, 16), (8192, 32, 64, 16), (4096, 1, 256, 32)):
+            am = torch.rand(rr, ii, jj, generator=gen).to(dev)
+            bm = (torch.randn(rr, jj, kk, generator=gen) * 10 - 30).to(dev)
+            nbytes_f = 4 * (am.numel() + bm.numel() + rr * ii * kk)
+            sec = graph_time(lambda: lm2exp(am, bm, _precision="fp32"), prewarm_ms=PREWARM_MS / 2)
+            tor = graph_time(lambda: torch_lm2exp(am, bm), calls=5, reps=5)
+            nw[f"lm2exp_R{rr}_I{ii}_J{jj}_K{kk}"] = {
+                "kernel": _lib.kernel_name("lm2exp", rr, ii, jj, kk, 0, 0, 1), "bytes": nbytes_f,
+                "us": round(sec * 1e6, 2), "achieved": round(nbytes_f / sec / 1e9, 1),
+                "frac": round(nbytes_f / sec / 1e9 / PEAK_HBM_GBPS, 4), "torch_recipe_us": round(tor * 1e6, 2)}
+            log(f"lm2exp R={rr} I={ii} J={jj} K={kk}: {sec * 1e6:.2f} us ({nbytes_f / sec / 1e9:.0f} GB/s = "
+                f"{nbytes_f / sec / 1e9 / PEAK_HBM_GBPS * 100:.1f}% of 8 TB/s), torch recipe {tor * 1e6:.2f} us")
+            del am, bm
+        result["narrow"] = nw
+
         # ------------------------------------------------ max reductions (HBM bound)
         # Two figures per reduction.  `us`, `achieved`, `frac`: 8 copies of the 64 MiB operand
         # (512 MiB) taken in turn, so that every call streams from HBM -- the figure to hold
