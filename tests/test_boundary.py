@@ -532,13 +532,18 @@ def test_lm2exp_narrow_outputs_of_few_rows_cut_the_contraction_over_the_wavefron
     """Host-side rule of lm2exp for at most 64 columns under few rows per batch: lm2exp_jsplit_kernel<column
     blocks of 32> gives a workgroup one tile and each wavefront a quarter of J."""
     name = lambda *sh, variant=0, splits=0, aligned=1: _lib.kernel_name("lm2exp", *sh, variant, splits, aligned)
-    assert name(8192, 1, 256, 16) == "trt::lm2exp_jsplit_kernel<1>"
-    assert name(4438, 16, 256, 16) == "trt::lm2exp_jsplit_kernel<1>"
+    assert name(8192, 20, 256, 16) == "trt::lm2exp_jsplit_kernel<1>"
     assert name(2000, 40, 128, 48) == "trt::lm2exp_jsplit_kernel<2>"
     assert name(40, 30, 500, 20) == "trt::lm2exp_jsplit_kernel<1>"
     assert name(508, 16, 256, 256).startswith("trt::lm2exp_kernel<")        # more than 64 columns
-    assert name(4000, 8, 66, 20).startswith("trt::lm2exp_kernel<")          # J not a multiple of 4
-    assert name(8192, 1, 256, 16, aligned=0).startswith("trt::lm2exp_kernel<")
+    assert name(4000, 24, 66, 20).startswith("trt::lm2exp_kernel<")         # J not a multiple of 4
+    assert name(8192, 20, 256, 16, aligned=0).startswith("trt::lm2exp_kernel<")
+    # at most 16 rows and 32 columns: the 16 x 16 x 4 MFMA's tile, <column blocks of 16>, any J and layout of a
+    assert name(8192, 1, 256, 16) == "trt::lm2exp_jsplit16_kernel<1>"
+    assert name(4438, 16, 256, 16) == "trt::lm2exp_jsplit16_kernel<1>"
+    assert name(4000, 8, 66, 20) == "trt::lm2exp_jsplit16_kernel<2>"
+    assert name(8192, 1, 255, 16, aligned=0) == "trt::lm2exp_jsplit16_kernel<1>"
+    assert name(8, 2, 3848, 24).startswith("trt::lm2exp_kernel<")           # a few batches under a long contraction: tiles cut over J
     assert name(30, 283, 2788, 10).startswith("trt::lm2exp_kernel<")        # nine row tiles per batch on a small grid
     assert name(8192, 1, 256, 16, variant=3).startswith("trt::lm2exp")      # forced tiles
     assert name(8192, 1, 256, 16, splits=2).startswith("trt::lm2exp_")      # a forced cut over workgroups

@@ -725,15 +725,18 @@ def test_contractions_of_at_most_16_terms_over_many_batches_take_a_lane_per_colu
 
 
 JSPLIT_SHAPES = [(3000, 1, 256, 16), (900, 16, 256, 16), (700, 8, 64, 32), (500, 40, 128, 48), (3000, 33, 100, 64),   # one or two column blocks
-                 (60, 4, 4096, 32), (40, 30, 500, 20), (1200, 5, 36, 9), (800, 32, 44, 33), (300, 7, 1000, 40)]        # long and ragged contractions, small grids
+                 (60, 4, 4096, 32), (40, 30, 500, 20), (1200, 5, 36, 9), (800, 32, 44, 33), (300, 7, 1000, 40),        # long and ragged contractions, small grids
+                 (2000, 5, 73, 20), (1000, 7, 1001, 11), (1500, 16, 33, 9), (900, 12, 130, 25), (200, 3, 4099, 32),    # at most 16 rows and 32 columns: any J
+                 (20000, 2, 32, 16), (700, 9, 515, 17)]
 
 
 @pytest.mark.parametrize("shape", JSPLIT_SHAPES)
 def test_narrow_outputs_of_few_rows_cut_the_contraction_over_the_wavefronts(dev, shape):
-    """At most 64 columns under few rows per batch: lm2exp_jsplit_kernel (csrc/lm2exp_jsplit.hpp) against
-    the float64 oracle (zero rows, -inf and NaN columns, a strided b) and against lm2exp's own tiles."""
+    """At most 64 columns under few rows per batch: lm2exp_jsplit_kernel and, for at most 16 rows and 32
+    columns, lm2exp_jsplit16_kernel (csrc/lm2exp_jsplit.hpp) against the float64 oracle (zero rows, -inf and NaN columns, a strided b) and against lm2exp's own tiles."""
     R, I, J, K = shape
-    assert _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1).startswith("trt::lm2exp_jsplit_kernel<")
+    kernel = _lib.kernel_name("lm2exp", R, I, J, K, 0, 0, 1)
+    assert kernel.startswith("trt::lm2exp_jsplit16_kernel<" if I <= 16 and K <= 32 else "trt::lm2exp_jsplit_kernel<")
     g = torch.Generator().manual_seed(sum(shape))
     a = torch.rand(R, I, J, generator=g)
     a[:, I // 2] = 0.0
@@ -759,6 +762,11 @@ def test_narrow_outputs_of_few_rows_cut_the_contraction_over_the_wavefronts(dev,
     for bv in (bs, bt):
         r = oracle64.compare(lm2exp(a.to(dev), bv), ref)
         assert r["ok"], (shape, "strided b", r)
+    at = a.transpose(1, 2).contiguous().transpose(1, 2).to(dev)                # J-major a, and a off the 16-byte grid
+    ao = torch.nn.functional.pad(a, (1, 2)).to(dev)[:, :, 1:J + 1]
+    for av in (at, ao):
+        r = oracle64.compare(lm2exp(av, bs), ref)
+        assert r["ok"], (shape, "strided a", r)
     ai = a.clone()                                                             # an infinite weight in the row after
     if I > 1:
         ai[:, 1, 0] = float("inf")

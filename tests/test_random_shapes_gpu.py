@@ -167,6 +167,25 @@ def test_lt2exp_random_with_few_units(dev, seed):
     assert r["ok"], (R, S, I, J, K, precision, r)
 
 
+@pytest.mark.parametrize("seed", range(40))
+def test_lm2exp_random_with_narrow_outputs(dev, seed):
+    """At most 40 rows and 9..64 columns per batch over hundreds to thousands of batches, any J from
+    32 on, strided a and b: the kernels that cut a batch's one tile over the wavefronts wherever the
+    library takes them, against the float64 oracle."""
+    rng = random.Random(7000 + seed)
+    g = torch.Generator().manual_seed(seed)
+    I, J, K = rng.randrange(1, 41), rng.choice([32, 33, 47, 64, 100, 129, 256, 515, 1000, 2050]), rng.randrange(9, 65)
+    R = rng.choice([30, 300, 1200, 3000])
+    a = torch.rand(R, I, J, generator=g) * rng.choice([1.0, 1e-4, 30.0])
+    a[torch.rand(R, I, J, generator=g) < 0.1] = 0.0
+    b = _sprinkle(rng, g, torch.randn(R, J, K, generator=g) * rng.choice([1.0, 10.0]) + rng.choice([0.0, 70.0, -90.0]))
+    ref = oracle64.lm2exp64(a, b)
+    precision = rng.choice(["fp32", "fp32", "fp32", "bf16x3"])
+    out = lm2exp(_view(rng, a.to(dev)), _view(rng, b.to(dev)), _precision=precision)
+    r = oracle64.compare(out, ref, **GATES[precision])
+    assert r["ok"], (R, I, J, K, precision, r)
+
+
 @pytest.mark.parametrize("precision", ["fp32", "bf16x3", "bf16x6"])
 def test_results_are_bit_reproducible(dev, precision):
     """Fixed summation order everywhere (no atomics, merges in split order): the same call on

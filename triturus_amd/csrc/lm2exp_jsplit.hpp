@@ -14,6 +14,7 @@
 #pragma once
 
 #include <cmath>
+#include <cstdio>
 
 #include "common.hpp"
 
@@ -23,7 +24,7 @@ struct Lm2JsplitArgs {
     const float *a, *b;
     float *c;
     int R, I, J, K;
-    int64_t sa0, sa1, sb0, sb1, sb2, sc0, sc1;  // (rows of a: dense, 16-byte aligned, J a multiple of 4)
+    int64_t sa0, sa1, sa2, sb0, sb1, sb2, sc0, sc1;  // (32-row kernel: rows of a dense, 16-byte aligned, J a multiple of 4)
     int n_tiles, i_tiles;
 };
 
@@ -160,6 +161,137 @@ static __global__ __launch_bounds__(kJsplitThreads) void lm2exp_jsplit_kernel(co
     }
 }
 
+// At most 16 rows and at most 32 columns: the same plan on the 16 x 16 x 4 MFMA, whose tile such a
+// batch fills (half of a 32 x 32 x 2 tile's rows or columns would be padding, and its MFMAs are a
+// quarter of the time here).  Lane (n, q), n = lane % 16, q = lane / 16, holds a[n, j] and
+// exp(b[j, n] - m) for j = 4 u + q of MFMA u: 64 lanes read 4 consecutive rows of b, 256
+// consecutive bytes where K = 16.  The wavefronts split J in units of 4 (one MFMA), so any J of
+// at least 32 is spread evenly; rows of a are read 4 bytes at a time and need no alignment.
+// CT: column blocks of 16 per workgroup (K <= 16 CT)
+template <int CT>
+static __global__ __launch_bounds__(kJsplitThreads) void lm2exp_jsplit16_kernel(const Lm2JsplitArgs p) {
+    constexpr int NT = 16 * CT;
+    __shared__ float part[kJsplitWaves][CT][4][kWave];  // the wavefronts' partial tiles
+    __shared__ float red[kJsplitWaves][NT];
+    __shared__ float shift[NT];
+
+    const int tid = (int)threadIdx.x;
+    const int lane = tid & (kWave - 1);
+    const int wave = __builtin_amdgcn_readfirstlane(tid / kWave);
+    const int n = lane & 15, q = lane >> 4;
+    const int r = (int)blockIdx.x;
+
+    // this wavefront's part of j: a quarter, in whole units of 4
+    const int n_units = (p.J + 3) / 4;
+    const int u_lo = n_units * wave / kJsplitWaves, u_hi = n_units * (wave + 1) / kJsplitWaves;
+
+    const float *br = p.b + (int64_t)r * p.sb0;
+    const __amdgpu_buffer_rsrc_t b_rsrc =
+        make_rsrc(br, (uint32_t)(((int64_t)(p.J - 1) * p.sb1 + (int64_t)(p.K - 1) * p.sb2 + 1) * 4));
+    const uint32_t b_row = (uint32_t)p.sb1 * 4u;  // bytes between two values of j
+    uint32_t bcol[CT];  // this lane's column of b and its row q in bytes (columns past K: the last one again, never stored)
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) {
+        const int k = 16 * ct + n;
+        bcol[ct] = (uint32_t)((int64_t)(k < p.K ? k : p.K - 1) * p.sb2) * 4u + (uint32_t)q * b_row;
+    }
+
+    // ---- column maxima: lane (n, q) takes j = 4 u + q (rows past J are read past the extent as
+    // zeros and set aside)
+    {
+        float m[CT];
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) m[ct] = -__builtin_inff();
+#pragma unroll 4
+        for (int u = u_lo; u < u_hi; ++u) {
+            const bool inside = 4 * u + q < p.J;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const float v = buf_load_f32(b_rsrc, bcol[ct], (uint32_t)(4 * u) * b_row);
+                m[ct] = __builtin_fmaxf(m[ct], inside ? v : -__builtin_inff());
+            }
+        }
+#pragma unroll
+        for (int ct = 0; ct < CT; ++ct) {
+            m[ct] = __builtin_fmaxf(m[ct], __shfl_xor(m[ct], 16, kWave));
+            m[ct] = __builtin_fmaxf(m[ct], __shfl_xor(m[ct], 32, kWave));
+            if (q == 0) red[wave][16 * ct + n] = m[ct];
+        }
+        __syncthreads();
+        if (tid < NT) {
+            float y = red[0][tid];
+#pragma unroll
+            for (int w = 1; w < kJsplitWaves; ++w) y = __builtin_fmaxf(y, red[w][tid]);
+            shift[tid] = clamp_shift(y);
+        }
+        __syncthreads();
+    }
+    float mk[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct) mk[ct] = shift[16 * ct + n];
+
+    // ---- the contraction over this wavefront's units, four at a time
+    const float *ar = p.a + (int64_t)r * p.sa0;
+    const uint32_t a_extent = (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + (int64_t)(p.J - 1) * p.sa2 + 1) * 4);
+    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ar, a_extent);
+    const uint32_t a_col = (uint32_t)p.sa2 * 4u;  // bytes between two values of j
+    // (rows past I are read past the extent: zeros)
+    const uint32_t a_voff = n < p.I ? (uint32_t)((int64_t)n * p.sa1 * 4) + (uint32_t)q * a_col : a_extent;
+    floatx4 acc[CT];
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) acc[ct][v] = 0.f;
+
+    float a_next[4], b_next[CT][4];
+    auto issue = [&](int u) {  // (units past u_hi: a neighbour's values or zeros, never used)
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            a_next[e] = buf_load_f32(a_rsrc, a_voff, (uint32_t)(4 * (u + e)) * a_col);
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) b_next[ct][e] = buf_load_f32(b_rsrc, bcol[ct], (uint32_t)(4 * (u + e)) * b_row);
+        }
+    };
+    if (u_lo < u_hi) issue(u_lo);
+    for (int u = u_lo; u < u_hi; u += 4) {
+        float av[4], bv[CT][4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            av[e] = a_next[e];
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) bv[ct][e] = b_next[ct][e];
+        }
+        if (u + 4 < u_hi) issue(u + 4);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const bool inside = u + e < u_hi && 4 * (u + e) + q < p.J;
+            const float aw = inside ? av[e] : 0.f;
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct) {
+                const float f = inside ? exp_shifted(bv[ct][e] - mk[ct]) : 0.f;
+                acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(aw, f, acc[ct], 0, 0, 0);
+            }
+        }
+    }
+
+    // ---- the four partial tiles, added in a fixed order; accumulator v of a lane is row 4 q + v
+    // of the tile, column n
+#pragma unroll
+    for (int ct = 0; ct < CT; ++ct)
+#pragma unroll
+        for (int v = 0; v < 4; ++v) part[wave][ct][v][lane] = acc[ct][v];
+    __syncthreads();
+    for (int t = tid; t < CT * 4 * kWave; t += kJsplitThreads) {
+        const int l = t & (kWave - 1), v = (t >> 6) & 3, ct = t >> 8;
+        const int orow = 4 * (l >> 4) + v, col = 16 * ct + (l & 15);
+        if (orow >= p.I || col >= p.K) continue;
+        float sum = part[0][ct][v][l];
+#pragma unroll
+        for (int w = 1; w < kJsplitWaves; ++w) sum += part[w][ct][v][l];
+        p.c[(int64_t)r * p.sc0 + (int64_t)orow * p.sc1 + col] = log_plus(sum, shift[col]);
+    }
+}
+
 // ---- host side
 
 // (rows of a read 16 bytes at a time; J of at least 32 so that every wavefront has a group)
@@ -180,8 +312,27 @@ static inline double jsplit_score(int64_t R, int64_t I, int64_t J, int64_t K) {
     return 1.51 - 0.08 * std::log2((double)K) - 0.031 * std::log2((double)J) - 0.156 * (lgrid < 10.0 ? 10.0 - lgrid : 0.0) -
            0.311 * std::log2(tiles) - (K > 32 ? 0.44 : 0.0);
 }
+// The 16-row kernel (any layout of a): against lm2exp's own tiles on 300 timed shapes (I = 1..16,
+// J = 32..4096, half of them no multiple of 4, K = 9..32, up to 60 000 batches) it is 2.0 times
+// faster in the geometric mean and behind only on grids of a few dozen batches under contractions of
+// thousands of terms, which the tiles cut over J: 1.1 doublings ahead to begin with, + 0.17 per
+// doubling of J, - 0.26 per doubling of K, - 0.30 per halving of the grid below 1024 batches
+// (0.8 % behind the faster choice per shape; always taking it 0.4 %).  Where both kernels apply it
+// is 1.23 times faster than the 32-row one (which is ahead by up to 10 % at I = 16, K = 16: its
+// 16-byte loads of a).
+static inline bool jsplit16_applies(int64_t I, int64_t J, int64_t K) { return I <= 16 && J >= 32 && K <= 32 && K > 8; }
+static inline double jsplit16_score(int64_t R, int64_t J, int64_t K) {
+    const double lr = std::log2((double)R);
+    return 1.13 - 0.26 * std::log2((double)K) + 0.17 * std::log2((double)J) - 0.30 * (lr < 10.0 ? 10.0 - lr : 0.0);
+}
 static inline bool jsplit_pays(int64_t R, int64_t I, int64_t J, int64_t K, bool a_aligned) {
+    if (jsplit16_applies(I, J, K)) return jsplit16_score(R, J, K) > 0.0;
     return jsplit_applies(I, J, K, a_aligned) && jsplit_score(R, I, J, K) > 0.0;
+}
+// (the kernel a call that takes this path runs)
+static inline int jsplit_kernel_name(char *buf, size_t bytes, int64_t I, int64_t J, int64_t K) {
+    if (jsplit16_applies(I, J, K)) return snprintf(buf, bytes, "trt::lm2exp_jsplit16_kernel<%d>", K > 16 ? 2 : 1);
+    return snprintf(buf, bytes, "trt::lm2exp_jsplit_kernel<%d>", K > 32 ? 2 : 1);
 }
 
 static int launch_lm2exp_jsplit(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J, int64_t K,
@@ -189,9 +340,17 @@ static int launch_lm2exp_jsplit(const float *a, const float *b, float *c, int64_
     Lm2JsplitArgs args;
     args.a = a; args.b = b; args.c = c;
     args.R = (int)R; args.I = (int)I; args.J = (int)J; args.K = (int)K;
-    args.sa0 = sa[0]; args.sa1 = sa[1];
+    args.sa0 = sa[0]; args.sa1 = sa[1]; args.sa2 = sa[2];
     args.sb0 = sb[0]; args.sb1 = sb[1]; args.sb2 = sb[2];
     args.sc0 = sc[0]; args.sc1 = sc[1];
+    if (jsplit16_applies(I, J, K)) {
+        if (R >= ((int64_t)1 << 31)) return TRT_E_RANGE;
+        if (K <= 16)
+            hipLaunchKernelGGL((lm2exp_jsplit16_kernel<1>), dim3((unsigned)R), dim3(kJsplitThreads), 0, stream, args);
+        else
+            hipLaunchKernelGGL((lm2exp_jsplit16_kernel<2>), dim3((unsigned)R), dim3(kJsplitThreads), 0, stream, args);
+        return (int)hipGetLastError();
+    }
     const int ct = K > 32 ? 2 : 1;
     args.n_tiles = (int)ceil_div(K, 32 * ct);
     args.i_tiles = (int)ceil_div(I, 32);
