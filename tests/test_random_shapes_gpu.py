@@ -174,7 +174,7 @@ def test_lm2exp_random_with_narrow_outputs(dev, seed):
     library takes them, against the float64 oracle."""
     rng = random.Random(7000 + seed)
     g = torch.Generator().manual_seed(seed)
-    I, J, K = rng.randrange(1, 41), rng.choice([32, 33, 47, 64, 100, 129, 256, 515, 1000, 2050]), rng.randrange(9, 65)
+    I, J, K = rng.randrange(1, 41), rng.choice([32, 33, 47, 64, 100, 129, 256, 380, 500, 515, 1000, 2050]), rng.randrange(9, 65)
     R = rng.choice([30, 300, 1200, 3000])
     a = torch.rand(R, I, J, generator=g) * rng.choice([1.0, 1e-4, 30.0])
     a[torch.rand(R, I, J, generator=g) < 0.1] = 0.0

@@ -167,8 +167,16 @@ static __global__ __launch_bounds__(kJsplitThreads) void lm2exp_jsplit_kernel(co
 // exp(b[j, n] - m) for j = 4 u + q of MFMA u: 64 lanes read 4 consecutive rows of b, 256
 // consecutive bytes where K = 16.  The wavefronts split J in units of 4 (one MFMA), so any J of
 // at least 32 is spread evenly; rows of a are read 4 bytes at a time and need no alignment.
-// CT: column blocks of 16 per workgroup (K <= 16 CT)
-template <int CT>
+// CT: column blocks of 16 per workgroup (K <= 16 CT).  KEEP > 0: J of at most 512 (384 above 16 columns), a wavefront's
+// quarter of at most KEEP units: its values of b stay in registers between the maxima and the
+// exponentials (b is read once, and the loads of a are in flight across the barrier).
+static inline int jsplit16_keep(int64_t J, int64_t K) {  // (0: the wavefronts walk their quarters twice)
+    const int64_t share = ceil_div(ceil_div(J, 4), kJsplitWaves);
+    for (int keep : {2, 4, 6, 8, 12, 16, 24, 32})
+        if (share <= keep) return keep;
+    return 0;
+}
+template <int CT, int KEEP>
 static __global__ __launch_bounds__(kJsplitThreads) void lm2exp_jsplit16_kernel(const Lm2JsplitArgs p) {
     constexpr int NT = 16 * CT;
     __shared__ float part[kJsplitWaves][CT][4][kWave];  // the wavefronts' partial tiles
@@ -198,17 +206,44 @@ static __global__ __launch_bounds__(kJsplitThreads) void lm2exp_jsplit16_kernel(
 
     // ---- column maxima: lane (n, q) takes j = 4 u + q (rows past J are read past the extent as
     // zeros and set aside)
+    const float *ar = p.a + (int64_t)r * p.sa0;
+    const uint32_t a_extent = (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + (int64_t)(p.J - 1) * p.sa2 + 1) * 4);
+    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ar, a_extent);
+    const uint32_t a_col = (uint32_t)p.sa2 * 4u;  // bytes between two values of j
+    // (rows past I are read past the extent: zeros)
+    const uint32_t a_voff = n < p.I ? (uint32_t)((int64_t)n * p.sa1 * 4) + (uint32_t)q * a_col : a_extent;
+    float b_keep[KEEP ? CT : 1][KEEP ? KEEP : 1], a_keep[KEEP ? KEEP : 1];  // (KEEP: -inf and 0 outside the wavefront's units)
     {
         float m[CT];
 #pragma unroll
         for (int ct = 0; ct < CT; ++ct) m[ct] = -__builtin_inff();
-#pragma unroll 4
-        for (int u = u_lo; u < u_hi; ++u) {
-            const bool inside = 4 * u + q < p.J;
+        if constexpr (KEEP > 0) {
 #pragma unroll
-            for (int ct = 0; ct < CT; ++ct) {
-                const float v = buf_load_f32(b_rsrc, bcol[ct], (uint32_t)(4 * u) * b_row);
-                m[ct] = __builtin_fmaxf(m[ct], inside ? v : -__builtin_inff());
+            for (int t = 0; t < KEEP; ++t) {
+                const int u = u_lo + t;
+                const bool inside = u < u_hi && 4 * u + q < p.J;
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    const float v = buf_load_f32(b_rsrc, bcol[ct], (uint32_t)(4 * u) * b_row);
+                    b_keep[ct][t] = inside ? v : -__builtin_inff();
+                    m[ct] = __builtin_fmaxf(m[ct], b_keep[ct][t]);
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < KEEP; ++t) {
+                const int u = u_lo + t;
+                const float v = buf_load_f32(a_rsrc, a_voff, (uint32_t)(4 * u) * a_col);
+                a_keep[t] = (u < u_hi && 4 * u + q < p.J) ? v : 0.f;
+            }
+        } else {
+#pragma unroll 4
+            for (int u = u_lo; u < u_hi; ++u) {
+                const bool inside = 4 * u + q < p.J;
+#pragma unroll
+                for (int ct = 0; ct < CT; ++ct) {
+                    const float v = buf_load_f32(b_rsrc, bcol[ct], (uint32_t)(4 * u) * b_row);
+                    m[ct] = __builtin_fmaxf(m[ct], inside ? v : -__builtin_inff());
+                }
             }
         }
 #pragma unroll
@@ -231,18 +266,19 @@ static __global__ __launch_bounds__(kJsplitThreads) void lm2exp_jsplit16_kernel(
     for (int ct = 0; ct < CT; ++ct) mk[ct] = shift[16 * ct + n];
 
     // ---- the contraction over this wavefront's units, four at a time
-    const float *ar = p.a + (int64_t)r * p.sa0;
-    const uint32_t a_extent = (uint32_t)(((int64_t)(p.I - 1) * p.sa1 + (int64_t)(p.J - 1) * p.sa2 + 1) * 4);
-    const __amdgpu_buffer_rsrc_t a_rsrc = make_rsrc(ar, a_extent);
-    const uint32_t a_col = (uint32_t)p.sa2 * 4u;  // bytes between two values of j
-    // (rows past I are read past the extent: zeros)
-    const uint32_t a_voff = n < p.I ? (uint32_t)((int64_t)n * p.sa1 * 4) + (uint32_t)q * a_col : a_extent;
     floatx4 acc[CT];
 #pragma unroll
     for (int ct = 0; ct < CT; ++ct)
 #pragma unroll
         for (int v = 0; v < 4; ++v) acc[ct][v] = 0.f;
 
+    if constexpr (KEEP > 0) {
+#pragma unroll
+        for (int t = 0; t < KEEP; ++t)
+#pragma unroll
+            for (int ct = 0; ct < CT; ++ct)  // (outside: exp(-inf) = 0 times 0)
+                acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(a_keep[t], exp_shifted(b_keep[ct][t] - mk[ct]), acc[ct], 0, 0, 0);
+    } else {
     float a_next[4], b_next[CT][4];
     auto issue = [&](int u) {  // (units past u_hi: a neighbour's values or zeros, never used)
 #pragma unroll
@@ -272,6 +308,7 @@ static __global__ __launch_bounds__(kJsplitThreads) void lm2exp_jsplit16_kernel(
                 acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(aw, f, acc[ct], 0, 0, 0);
             }
         }
+    }
     }
 
     // ---- the four partial tiles, added in a fixed order; accumulator v of a lane is row 4 q + v
@@ -331,7 +368,8 @@ static inline bool jsplit_pays(int64_t R, int64_t I, int64_t J, int64_t K, bool 
 }
 // (the kernel a call that takes this path runs)
 static inline int jsplit_kernel_name(char *buf, size_t bytes, int64_t I, int64_t J, int64_t K) {
-    if (jsplit16_applies(I, J, K)) return snprintf(buf, bytes, "trt::lm2exp_jsplit16_kernel<%d>", K > 16 ? 2 : 1);
+    if (jsplit16_applies(I, J, K))
+        return snprintf(buf, bytes, "trt::lm2exp_jsplit16_kernel<%d, %d>", K > 16 ? 2 : 1, jsplit16_keep(J, K));
     return snprintf(buf, bytes, "trt::lm2exp_jsplit_kernel<%d>", K > 32 ? 2 : 1);
 }
 
@@ -345,10 +383,27 @@ static int launch_lm2exp_jsplit(const float *a, const float *b, float *c, int64_
     args.sc0 = sc[0]; args.sc1 = sc[1];
     if (jsplit16_applies(I, J, K)) {
         if (R >= ((int64_t)1 << 31)) return TRT_E_RANGE;
-        if (K <= 16)
-            hipLaunchKernelGGL((lm2exp_jsplit16_kernel<1>), dim3((unsigned)R), dim3(kJsplitThreads), 0, stream, args);
-        else
-            hipLaunchKernelGGL((lm2exp_jsplit16_kernel<2>), dim3((unsigned)R), dim3(kJsplitThreads), 0, stream, args);
+#define TRT_JSPLIT16_LAUNCH(CT_, KEEP_) \
+    hipLaunchKernelGGL((lm2exp_jsplit16_kernel<CT_, KEEP_>), dim3((unsigned)R), dim3(kJsplitThreads), 0, stream, args)
+#define TRT_JSPLIT16_KEEP(CT_) \
+    switch (jsplit16_keep(J, K)) { \
+        case 2: TRT_JSPLIT16_LAUNCH(CT_, 2); break; \
+        case 4: TRT_JSPLIT16_LAUNCH(CT_, 4); break; \
+        case 6: TRT_JSPLIT16_LAUNCH(CT_, 6); break; \
+        case 8: TRT_JSPLIT16_LAUNCH(CT_, 8); break; \
+        case 12: TRT_JSPLIT16_LAUNCH(CT_, 12); break; \
+        case 16: TRT_JSPLIT16_LAUNCH(CT_, 16); break; \
+        case 24: TRT_JSPLIT16_LAUNCH(CT_, 24); break; \
+        case 32: TRT_JSPLIT16_LAUNCH(CT_, 32); break; \
+        default: TRT_JSPLIT16_LAUNCH(CT_, 0); break; \
+    }
+        if (K <= 16) {
+            TRT_JSPLIT16_KEEP(1)
+        } else {
+            TRT_JSPLIT16_KEEP(2)
+        }
+#undef TRT_JSPLIT16_KEEP
+#undef TRT_JSPLIT16_LAUNCH
         return (int)hipGetLastError();
     }
     const int ct = K > 32 ? 2 : 1;
