@@ -80,9 +80,9 @@ const char *trt_error_string(int status);
  * (the few-column kernel of trt_lt2exp_f32) and no workspace is used.  With variant 0,
  * splits <= 1, more than 8 columns and J <= 16 over many batches, every output column gets a lane
  * of its own (the few-unit kernel of trt_lt2exp_f32) where that is the faster way; likewise no
- * workspace.  With at most 64 columns under few rows per batch, J >= 32 a multiple of 4 and
- * 16-byte aligned rows of a, a workgroup takes a batch's one tile and cuts its contraction over
- * its wavefronts (likewise).  trt_lm2exp_kernel_name tells which kernel a call takes.
+ * workspace.  With at most 64 columns under few rows per batch and J >= 32 (above 16 rows or 32
+ * columns: J a multiple of 4 and 16-byte aligned rows of a), a workgroup takes a batch's one
+ * tile and cuts its contraction over its wavefronts (likewise).  trt_lm2exp_kernel_name tells which kernel a call takes.
  */
 int trt_lm2exp_f32(const float *a, const float *b, float *c,
                    int64_t R, int64_t I, int64_t J, int64_t K,

@@ -11,6 +11,8 @@
 // (lane = column, consecutive lanes on consecutive k: whole cache lines), and multiplies by its
 // rows of a, which it reads straight into the A layout (lane = row, 16 bytes per load).  Nothing
 // passes through LDS but the four partial tiles at the end, which are added in a fixed order.
+// lm2exp_jsplit16_kernel, below, is the same plan on the 16 x 16 x 4 MFMA for at most 16 rows and 32
+// columns.
 #pragma once
 
 #include <cmath>
