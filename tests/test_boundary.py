@@ -541,13 +541,19 @@ def test_lm2exp_narrow_outputs_of_few_rows_cut_the_contraction_over_the_wavefron
     # at most 16 rows and 32 columns: the 16 x 16 x 4 MFMA's tile, <column blocks of 16>, any J and layout of a
     # (second argument: the units of 4 values of j that a wavefront keeps in registers between the maxima
     # and the exponentials, 0 where its quarter of J is longer than 32 units)
-    assert name(8192, 1, 256, 16) == "trt::lm2exp_jsplit16_kernel<1, 16>"
-    assert name(4438, 16, 256, 16) == "trt::lm2exp_jsplit16_kernel<1, 16>"
-    assert name(4000, 8, 66, 20) == "trt::lm2exp_jsplit16_kernel<2, 6>"
-    assert name(8192, 1, 255, 16, aligned=0) == "trt::lm2exp_jsplit16_kernel<1, 16>"
-    assert name(8192, 1, 32, 16) == "trt::lm2exp_jsplit16_kernel<1, 2>"
-    assert name(4000, 8, 512, 32) == "trt::lm2exp_jsplit16_kernel<2, 32>"
-    assert name(4000, 8, 513, 32) == "trt::lm2exp_jsplit16_kernel<2, 0>"
+    assert name(8192, 1, 256, 16) == "trt::lm2exp_jsplit16_kernel<1, 16, false>"
+    assert name(4000, 8, 66, 20) == "trt::lm2exp_jsplit16_kernel<2, 6, false>"
+    assert name(8192, 1, 255, 16, aligned=0) == "trt::lm2exp_jsplit16_kernel<1, 16, false>"
+    assert name(8192, 1, 32, 16) == "trt::lm2exp_jsplit16_kernel<1, 2, false>"
+    assert name(4000, 8, 512, 32) == "trt::lm2exp_jsplit16_kernel<2, 32, false>"
+    assert name(4000, 8, 513, 32) == "trt::lm2exp_jsplit16_kernel<2, 0, false>"
+    # (third argument: from 12 rows on, dense aligned rows of a and whole groups of four units are read
+    # 16 bytes at a time and transposed among the four lanes of a row)
+    assert name(4438, 16, 256, 16) == "trt::lm2exp_jsplit16_kernel<1, 16, true>"
+    assert name(4438, 16, 256, 16, aligned=0) == "trt::lm2exp_jsplit16_kernel<1, 16, false>"
+    assert name(4000, 12, 512, 32) == "trt::lm2exp_jsplit16_kernel<2, 32, true>"
+    assert name(4000, 12, 96, 32) == "trt::lm2exp_jsplit16_kernel<2, 6, false>"
+    assert name(4000, 11, 512, 32) == "trt::lm2exp_jsplit16_kernel<2, 32, false>"
     assert name(8, 2, 3848, 24).startswith("trt::lm2exp_kernel<")           # a few batches under a long contraction: tiles cut over J
     assert name(30, 283, 2788, 10).startswith("trt::lm2exp_kernel<")        # nine row tiles per batch on a small grid
     assert name(8192, 1, 256, 16, variant=3).startswith("trt::lm2exp")      # forced tiles

@@ -727,7 +727,8 @@ def test_contractions_of_at_most_16_terms_over_many_batches_take_a_lane_per_colu
 JSPLIT_SHAPES = [(3000, 1, 256, 16), (900, 16, 256, 16), (700, 8, 64, 32), (500, 40, 128, 48), (3000, 33, 100, 64),   # one or two column blocks
                  (60, 4, 4096, 32), (40, 30, 500, 20), (1200, 5, 36, 9), (800, 32, 44, 33), (300, 7, 1000, 40),        # long and ragged contractions, small grids
                  (2000, 5, 73, 20), (1000, 7, 1001, 11), (1500, 16, 33, 9), (900, 12, 130, 25), (200, 3, 4099, 32),    # at most 16 rows and 32 columns: any J
-                 (20000, 2, 32, 16), (700, 9, 515, 17), (600, 6, 120, 12), (500, 10, 380, 30), (500, 3, 509, 14)]
+                 (20000, 2, 32, 16), (700, 9, 515, 17), (600, 6, 120, 12), (500, 10, 380, 30), (500, 3, 509, 14),
+                 (800, 14, 64, 20), (600, 13, 128, 30), (400, 15, 192, 16), (300, 16, 384, 32), (300, 12, 512, 10)]    # 12 to 16 rows: a read 16 bytes at a time
 
 
 @pytest.mark.parametrize("shape", JSPLIT_SHAPES)

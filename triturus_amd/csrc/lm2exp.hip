@@ -1059,7 +1059,7 @@ extern "C" int trt_lm2exp_kernel_name(int64_t R, int64_t I, int64_t J, int64_t K
     if (variant == 0 && splits <= 1 && lm2exp_takes_sweep(R, I, J, K, a_vec != 0))
         return lt2exp_sweep_name(R, I, J, K, true, buf, buf_bytes);
     if (variant == 0 && splits <= 1 && jsplit_pays(R, I, J, K, a_vec != 0)) {
-        const int n = jsplit_kernel_name(buf, buf_bytes, I, J, K);
+        const int n = jsplit_kernel_name(buf, buf_bytes, I, J, K, a_vec != 0);
         return n > 0 && (size_t)n < buf_bytes ? 0 : TRT_E_RANGE;
     }
     if (variant == 0 && splits <= 1 && lm2exp_takes_cols(R, I, J, K, true, 0.0)) return lm2exp_cols_name(J, true, buf, buf_bytes);
