@@ -934,6 +934,16 @@ extern "C" size_t trt_lm2exp_workspace_bytes(int64_t R, int64_t I, int64_t J, in
     return plan_workspace(make_plan(R, I, J, K, variant, splits), R, I, K);
 }
 
+namespace trt {
+// (for the split-bf16 entry, csrc/lm2exp_bf16.hip: outputs of at most 16 rows and 32 columns per batch
+// are bound by the reads of b, not by the matrix pipe, and go to the fp32 entry's kernel for them --
+// R=8192, I=1, J=256, K=16: 97 -> 26 us; R=3000, I=7, J=1001, K=11: 145 -> 54; the 32-row kernel against
+// the bf16 tiles is 0.6 to 1.2 times their speed and is not handed to)
+bool lm2exp_takes_jsplit16(int64_t R, int64_t I, int64_t J, int64_t K) {
+    return jsplit16_applies(I, J, K) && jsplit16_score(R, J, K) > 0.0;
+}
+}  // namespace trt
+
 extern "C" int trt_lm2exp_f32(const float *a, const float *b, float *c, int64_t R, int64_t I, int64_t J,
                               int64_t K, const int64_t sa[3], const int64_t sb[3], const int64_t sc[3],
                               int variant, int splits, void *workspace, size_t workspace_bytes, void *stream) {

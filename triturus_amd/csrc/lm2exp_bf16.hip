@@ -377,6 +377,7 @@ static const LmBfVariant kLmBfVariants[] = {{4, 4}, {4, 2}, {2, 4}, {2, 2}, {1, 
 constexpr int kNumLmBfVariants = sizeof(kLmBfVariants) / sizeof(kLmBfVariants[0]);
 
 bool lm2exp_takes_sweep(int64_t R, int64_t I, int64_t J, int64_t K, bool a_aligned);  // csrc/lt2exp.hip
+bool lm2exp_takes_jsplit16(int64_t R, int64_t I, int64_t J, int64_t K);  // csrc/lm2exp.hip
 
 }  // namespace trt
 
@@ -486,7 +487,9 @@ extern "C" int trt_lm2exp_bf16(const float *a, const float *b, float *c, int64_t
         // at most 4 columns under a long contraction: the fp32 entry sweeps a on the vector ALU
         const bool swept = splits <= 1 && lm2exp_takes_sweep(R, I, J, K, sa[2] == 1 && sa[0] % 4 == 0 && sa[1] % 4 == 0 &&
                                                                             (reinterpret_cast<uintptr_t>(a) & 15) == 0);
-        if (narrow || swept || (cut == 1 && !one_launch && (splits > 1 || small || J <= (pieces == 2 ? 16 : 32))))
+        // at most 16 rows and 32 columns per batch: one tile per batch, bound by the reads of b
+        const bool one_tile = splits <= 1 && lm2exp_takes_jsplit16(R, I, J, K);
+        if (narrow || swept || one_tile || (cut == 1 && !one_launch && (splits > 1 || small || J <= (pieces == 2 ? 16 : 32))))
             return trt_lm2exp_f32(a, b, c, R, I, J, K, sa, sb, sc, 0, splits, workspace, workspace_bytes, stream);
         int best_rt = 1;
         int64_t best_cost = ceil_div(I, 32) * 120;
